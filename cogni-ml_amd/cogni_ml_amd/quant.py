@@ -1,0 +1,121 @@
+"""QuantMatmul / Dequant on the GPU: Python (ctypes) binding of the operator layer in libcogni_hip.so.
+
+Signatures follow the reference's CPU operators so a caller switches by renaming the module:
+  dequantize(data, type, n_elements)                              src/ml/gguf/dequant.cr:19
+  matmul_add(x, rows, in_dim, w_raw, w_type, out_dim, bias)       src/ml/gguf/quant_matmul.cr:20
+  QuantWeight(raw, type, out_dim, in_dim, route_tag)              src/ml/gguf/compute.cr:20-30
+"""
+import ctypes
+
+import numpy as np
+
+from . import hip
+from .types import TensorType
+
+MAX_GEMV_TOKENS = 8
+
+
+class QuantError(RuntimeError):
+    def __init__(self, code):
+        self.code = code
+        super().__init__(hip.lib().cogni_last_error().decode())
+
+
+def _check(code):
+    if code != 0:
+        raise QuantError(code)
+
+
+def init(ordinal=0):
+    """Load the gfx950 code object on device `ordinal`. Raises if there is no such GPU."""
+    _check(hip.lib().cogni_quant_init(ordinal))
+
+
+def shutdown():
+    _check(hip.lib().cogni_quant_shutdown())
+
+
+def gemv_kernel_name(w_type, tokens=1, add=False):
+    n = hip.lib().cogni_gemv_kernel_name(int(w_type), tokens, int(add))
+    return n.decode() if n else None
+
+
+def dequantize_kernel_name(w_type):
+    n = hip.lib().cogni_dequantize_kernel_name(int(w_type))
+    return n.decode() if n else None
+
+
+def gemv_launch_dims(out_dim):
+    g, b = ctypes.c_uint32(), ctypes.c_uint32()
+    _check(hip.lib().cogni_gemv_launch_dims(out_dim, ctypes.byref(g), ctypes.byref(b)))
+    return g.value, b.value
+
+
+def dequantize_dev(w_ptr, w_type, n_elements, out_ptr, stream=None):
+    _check(hip.lib().cogni_dequantize_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)),
+                                          ctypes.c_uint64(n_elements), ctypes.c_uint64(out_ptr), stream))
+
+
+def gemv_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens=1, residual_ptr=0, stream=None):
+    _check(hip.lib().cogni_gemv_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(x_ptr),
+                                    ctypes.c_uint64(residual_ptr), ctypes.c_uint64(out_ptr), ctypes.c_uint32(in_dim),
+                                    ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
+def dequantize(data, w_type, n_elements):
+    """Dequant.dequantize: raw bytes -> float32[n_elements], computed on the GPU."""
+    d = np.ascontiguousarray(np.frombuffer(data, dtype=np.uint8) if not isinstance(data, np.ndarray) else data,
+                             dtype=np.uint8)
+    out = np.empty(int(n_elements), dtype=np.float32)
+    _check(hip.lib().cogni_dequantize(ctypes.c_void_p(d.ctypes.data), ctypes.c_size_t(d.size),
+                                      ctypes.c_uint32(int(w_type)), ctypes.c_int64(int(n_elements)),
+                                      ctypes.c_void_p(out.ctypes.data)))
+    return out
+
+
+def matmul_add(x, rows, in_dim, w_raw, w_type, out_dim, bias):
+    """QuantMatmul.matmul_add: float32[rows*out_dim] = bias + x @ deq(W)^T, computed on the GPU."""
+    xa = np.ascontiguousarray(x, dtype=np.float32)
+    wa = np.ascontiguousarray(w_raw, dtype=np.uint8)
+    ba = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    if xa.size < rows * in_dim:
+        raise ValueError("x has %d elements, rows*in_dim is %d" % (xa.size, rows * in_dim))
+    if ba is not None and ba.size < out_dim:
+        raise ValueError("bias has %d elements, out_dim is %d" % (ba.size, out_dim))
+    res = np.empty(rows * out_dim, dtype=np.float32)
+    _check(hip.lib().cogni_matmul_add(ctypes.c_void_p(xa.ctypes.data), ctypes.c_int32(rows), ctypes.c_int32(in_dim),
+                                      ctypes.c_void_p(wa.ctypes.data), ctypes.c_size_t(wa.size),
+                                      ctypes.c_uint32(int(w_type)), ctypes.c_int32(out_dim),
+                                      ctypes.c_void_p(ba.ctypes.data if ba is not None else None),
+                                      ctypes.c_void_p(res.ctypes.data)))
+    return res
+
+
+class QuantWeight:
+    """compute.cr:20-45: {raw, type, out_dim, in_dim, route_tag} plus the resident device copy."""
+
+    def __init__(self, raw, w_type, out_dim, in_dim, route_tag=None):
+        self.raw = np.ascontiguousarray(raw, dtype=np.uint8)
+        self.type, self.out_dim, self.in_dim, self.route_tag = TensorType(int(w_type)), out_dim, in_dim, route_tag
+        self._handle = ctypes.c_void_p()
+        _check(hip.lib().cogni_weight_create(ctypes.byref(self._handle), ctypes.c_void_p(self.raw.ctypes.data),
+                                             ctypes.c_size_t(self.raw.size), ctypes.c_uint32(int(w_type)),
+                                             ctypes.c_int32(out_dim), ctypes.c_int32(in_dim)))
+
+    @property
+    def device_ptr(self):
+        return hip.lib().cogni_weight_device_ptr(self._handle)
+
+    def matmul(self, x, rows=1, bias=None):
+        xa = np.ascontiguousarray(x, dtype=np.float32)
+        ba = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        res = np.empty(rows * self.out_dim, dtype=np.float32)
+        _check(hip.lib().cogni_weight_matmul(self._handle, ctypes.c_void_p(xa.ctypes.data), ctypes.c_int32(rows),
+                                             ctypes.c_void_p(ba.ctypes.data if ba is not None else None),
+                                             ctypes.c_void_p(res.ctypes.data)))
+        return res
+
+    def close(self):
+        if self._handle:
+            hip.lib().cogni_weight_destroy(self._handle)
+            self._handle = None

@@ -1,0 +1,370 @@
+// Quantized-matmul operators over the gfx950 code object. See include/cogni_quant.h.
+//
+// The kernels live in a separately compiled code object that is embedded in this library
+// (hsaco_blob.S) and loaded with hipModuleLoadData; every launch goes through
+// hipModuleLaunchKernel with the kernel ABI the header documents. There is no host fallback.
+#include "cogni_quant.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+extern "C" const unsigned char cogni_hsaco_begin[];
+extern "C" const unsigned char cogni_hsaco_end[];
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string& what) {
+  g_err = what;
+  return code;
+}
+
+int hip_fail(hipError_t e, const std::string& what) {
+  char buf[64];
+  std::snprintf(buf, sizeof buf, " failed with HIP error %d (", (int)e);
+  g_err = what + buf + hipGetErrorName(e) + ")";
+  return (int)e;
+}
+
+#define HIP_TRY(call, what)                          \
+  do {                                               \
+    hipError_t e__ = (call);                         \
+    if (e__ != hipSuccess) return hip_fail(e__, what); \
+  } while (0)
+
+struct Runtime {
+  bool ready = false;
+  int ordinal = -1;
+  int compute_units = 0;
+  hipModule_t mod = nullptr;
+  std::unordered_map<std::string, hipFunction_t> fns;
+};
+Runtime g_rt;
+std::mutex g_mu;
+
+int get_fn(const char* name, hipFunction_t* out) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (!g_rt.ready) return fail(COGNI_ERR_NOT_INITIALIZED, "cogni_quant_init has not been called");
+  auto it = g_rt.fns.find(name);
+  if (it != g_rt.fns.end()) {
+    *out = it->second;
+    return 0;
+  }
+  hipFunction_t fn = nullptr;
+  HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
+  g_rt.fns.emplace(name, fn);
+  *out = fn;
+  return 0;
+}
+
+int launch(const char* name, uint32_t grid, uint32_t block, void** params, void* stream) {
+  hipFunction_t fn = nullptr;
+  int rc = get_fn(name, &fn);
+  if (rc != 0) return rc;
+  HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, 0, (hipStream_t)stream, params, nullptr),
+          std::string("hipModuleLaunchKernel(") + name + ")");
+  return 0;
+}
+
+const char* type_prefix(uint32_t type) {
+  switch (type) {
+    case COGNI_TYPE_Q8_0: return "q8_0";
+    case COGNI_TYPE_Q4_K: return "q4_k";
+    case COGNI_TYPE_Q5_K: return "q5_k";
+    case COGNI_TYPE_Q6_K: return "q6_k";
+    case COGNI_TYPE_IQ4_NL: return "iq4_nl";
+    case COGNI_TYPE_F16: return "f16";
+    case COGNI_TYPE_F32: return "f32";
+    default: return nullptr;
+  }
+}
+
+const char* type_name(uint32_t type) {
+  switch (type) {
+    case COGNI_TYPE_Q8_0: return "Q8_0";
+    case COGNI_TYPE_Q4_K: return "Q4_K";
+    case COGNI_TYPE_Q5_K: return "Q5_K";
+    case COGNI_TYPE_Q6_K: return "Q6_K";
+    case COGNI_TYPE_IQ4_NL: return "IQ4_NL";
+    case COGNI_TYPE_F16: return "F16";
+    case COGNI_TYPE_F32: return "F32";
+    default: return "unknown";
+  }
+}
+
+bool gemv_type(uint32_t t) {
+  return t == COGNI_TYPE_Q8_0 || t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q5_K || t == COGNI_TYPE_Q6_K;
+}
+bool k_quant(uint32_t t) { return t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q5_K || t == COGNI_TYPE_Q6_K; }
+
+// Bytes of one weight row, the reference's row_bytes (quant_matmul.cr:46-47, 241-242).
+size_t row_bytes_of(uint32_t type, uint32_t in_dim) {
+  const size_t be = (size_t)cogni_block_elements(type), bb = (size_t)cogni_block_bytes(type);
+  return ((in_dim + be - 1) / be) * bb;
+}
+
+struct DeviceMem {  // frees on scope exit; host-buffer operators are synchronous
+  void* p = nullptr;
+  ~DeviceMem() {
+    if (p) (void)hipFree(p);
+  }
+  uint64_t addr() const { return (uint64_t)(uintptr_t)p; }
+};
+
+}  // namespace
+
+struct cogni_quant_weight {
+  void* dev = nullptr;
+  size_t bytes = 0;
+  uint32_t type = 0;
+  int32_t out_dim = 0, in_dim = 0;
+};
+
+extern "C" {
+
+const char* cogni_last_error(void) { return g_err.c_str(); }
+
+// ---- geometry (reader.cr:51-78, 119-127) -----------------------------------------------------
+int32_t cogni_block_bytes(uint32_t type) {
+  switch (type) {
+    case 0: return 4;    case 1: return 2;    case 2: return 18;   case 3: return 20;
+    case 6: return 22;   case 7: return 24;   case 8: return 34;   case 10: return 84;
+    case 11: return 110; case 12: return 144; case 13: return 176; case 14: return 210;
+    case 15: return 292; case 20: return 18;
+    default: return -1;
+  }
+}
+
+int32_t cogni_block_elements(uint32_t type) {
+  switch (type) {
+    case 0: case 1: return 1;
+    case 2: case 3: case 6: case 7: case 8: case 20: return 32;
+    case 10: case 11: case 12: case 13: case 14: case 15: return 256;
+    default: return -1;
+  }
+}
+
+int64_t cogni_data_bytes(uint32_t type, int64_t n_elements) {
+  const int64_t bb = cogni_block_bytes(type), be = cogni_block_elements(type);
+  if (bb < 0) return -1;
+  if (type == COGNI_TYPE_F32 || type == COGNI_TYPE_F16) return n_elements * bb;
+  return ((n_elements + be - 1) / be) * bb;
+}
+
+// ---- code object ----------------------------------------------------------------------------------
+int cogni_quant_code_object(const void** image, size_t* size) {
+  if (!image || !size) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_quant_code_object: null argument");
+  *image = cogni_hsaco_begin;
+  *size = (size_t)(cogni_hsaco_end - cogni_hsaco_begin);
+  return 0;
+}
+
+const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add) {
+  static thread_local char buf[64];
+  if (!gemv_type(type) || tokens < 1 || tokens > COGNI_MAX_GEMV_TOKENS) return nullptr;
+  if (tokens == 1)
+    std::snprintf(buf, sizeof buf, "%s_gemv_%sf32", type_prefix(type), add ? "add_" : "");
+  else
+    std::snprintf(buf, sizeof buf, "%s_gemv_%sf32_tbatch%u", type_prefix(type), add ? "add_" : "", tokens);
+  return buf;
+}
+
+int cogni_gemv_launch_dims(uint32_t out_dim, uint32_t* grid_x, uint32_t* block_x) {
+  if (!grid_x || !block_x || out_dim == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_launch_dims: bad argument");
+  *grid_x = (out_dim + 15) / 16;
+  *block_x = 256;
+  return 0;
+}
+
+const char* cogni_dequantize_kernel_name(uint32_t type) {
+  static thread_local char buf[64];
+  const char* p = type_prefix(type);
+  if (!p) return nullptr;
+  std::snprintf(buf, sizeof buf, "dequantize_%s_f32", p);
+  return buf;
+}
+
+// ---- initialisation -------------------------------------------------------------------------------
+int cogni_quant_init(int32_t ordinal) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_rt.ready) {
+    if (g_rt.ordinal == ordinal) return 0;
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_quant_init: already initialised on another device");
+  }
+  hipError_t e = hipInit(0);
+  if (e != hipSuccess) return fail(COGNI_ERR_NO_DEVICE, std::string("hipInit failed (") + hipGetErrorName(e) + "): no GPU, and there is no CPU fallback");
+  int count = 0;
+  e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= ordinal || ordinal < 0)
+    return fail(COGNI_ERR_NO_DEVICE, "no HIP device with the requested ordinal; there is no CPU fallback");
+  HIP_TRY(hipSetDevice(ordinal), "hipSetDevice");
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, ordinal), "hipGetDeviceProperties");
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(COGNI_ERR_NO_DEVICE, std::string("device is ") + prop.gcnArchName + ", the code object is gfx950 only");
+  HIP_TRY(hipModuleLoadData(&g_rt.mod, cogni_hsaco_begin), "hipModuleLoadData(cogni_quant gfx950 code object)");
+  g_rt.compute_units = prop.multiProcessorCount;
+  g_rt.ordinal = ordinal;
+  g_rt.ready = true;
+  return 0;
+}
+
+int cogni_quant_shutdown(void) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (!g_rt.ready) return 0;
+  (void)hipModuleUnload(g_rt.mod);
+  g_rt = Runtime();
+  return 0;
+}
+
+// ---- device-pointer operators -----------------------------------------------------------------------
+int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, uint64_t out, void* stream) {
+  const char* name = cogni_dequantize_kernel_name(w_type);
+  if (!name) return fail(COGNI_ERR_UNSUPPORTED_TYPE, "Unsupported dequantization type: " + std::to_string(w_type));
+  if (n_elements == 0) return 0;
+  if (!w_raw || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_dequantize_dev: null device pointer");
+  // one wavefront step produces 256 floats; 4 wavefronts per workgroup; grid-stride beyond the cap
+  uint64_t groups = (n_elements + 1023) / 1024;
+  const uint64_t cap = 65536;
+  uint32_t grid = (uint32_t)(groups < cap ? groups : cap);
+  if (grid == 0) grid = 1;
+  unsigned long long n = n_elements;
+  void* params[] = {&w_raw, &out, &n};
+  return launch(name, grid, 256, params, stream);
+}
+
+int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out, uint32_t in_dim,
+                   uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (!gemv_type(w_type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for fused matmul: ") + type_name(w_type));
+  if (!w_raw || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: null device pointer");
+  if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: zero dimension");
+  if (k_quant(w_type) && (in_dim % 256) != 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  uint32_t grid = 0, block = 0;
+  cogni_gemv_launch_dims(out_dim, &grid, &block);
+  for (uint32_t t0 = 0; t0 < tokens; t0 += COGNI_MAX_GEMV_TOKENS) {
+    const uint32_t m = tokens - t0 < COGNI_MAX_GEMV_TOKENS ? tokens - t0 : COGNI_MAX_GEMV_TOKENS;
+    uint64_t xm = x + (uint64_t)t0 * in_dim * 4, om = out + (uint64_t)t0 * out_dim * 4;
+    uint64_t rm = residual ? residual + (uint64_t)t0 * out_dim * 4 : 0;
+    const std::string name = cogni_gemv_kernel_name(w_type, m, residual != 0);
+    int rc;
+    if (residual) {
+      void* params[] = {&w_raw, &xm, &rm, &om, &in_dim, &out_dim};
+      rc = launch(name.c_str(), grid, block, params, stream);
+    } else {
+      void* params[] = {&w_raw, &xm, &om, &in_dim, &out_dim};
+      rc = launch(name.c_str(), grid, block, params, stream);
+    }
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+
+// ---- host-buffer operators --------------------------------------------------------------------------
+int cogni_dequantize(const void* data, size_t data_bytes, uint32_t type, int64_t n_elements, float* out) {
+  if (!cogni_dequantize_kernel_name(type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, "Unsupported dequantization type: " + std::to_string(type));
+  if (n_elements < 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_dequantize: negative n_elements");
+  if (n_elements == 0) return 0;
+  if (!data || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_dequantize: null buffer");
+  // K-quants read floor(n/256) blocks (dequant.cr:107,147,198); the 32-element formats ceil(n/32).
+  const size_t need = k_quant(type) ? (size_t)(n_elements / 256) * (size_t)cogni_block_bytes(type)
+                                    : (size_t)cogni_data_bytes(type, n_elements);
+  if (data_bytes < need)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_dequantize: data has " + std::to_string(data_bytes) + " bytes, needs " + std::to_string(need));
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_rt.ready) return fail(COGNI_ERR_NOT_INITIALIZED, "cogni_quant_init has not been called");
+  }
+  DeviceMem dw, dout;
+  HIP_TRY(hipMalloc(&dw.p, need ? need : 16), "hipMalloc(dequantize input)");
+  HIP_TRY(hipMalloc(&dout.p, (size_t)n_elements * 4), "hipMalloc(dequantize output)");
+  if (need) HIP_TRY(hipMemcpyHtoD(dw.p, const_cast<void*>(data), need), "hipMemcpyHtoD(dequantize input)");
+  int rc = cogni_dequantize_dev(dw.addr(), type, (uint64_t)n_elements, dout.addr(), nullptr);
+  if (rc != 0) return rc;
+  HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize(dequantize)");
+  HIP_TRY(hipMemcpyDtoH(out, dout.p, (size_t)n_elements * 4), "hipMemcpyDtoH(dequantize output)");
+  return 0;
+}
+
+int cogni_weight_create(cogni_quant_weight** qw, const void* raw, size_t raw_bytes, uint32_t type, int32_t out_dim,
+                        int32_t in_dim) {
+  if (!qw || !raw) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_create: null argument");
+  if (!gemv_type(type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for fused matmul: ") + type_name(type));
+  if (out_dim <= 0 || in_dim <= 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_create: dimensions must be positive");
+  if (k_quant(type) && in_dim % 256 != 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(type)) + " requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  const size_t need = (size_t)out_dim * row_bytes_of(type, (uint32_t)in_dim);
+  if (raw_bytes < need)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "weight has " + std::to_string(raw_bytes) + " bytes, shape needs " + std::to_string(need));
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_rt.ready) return fail(COGNI_ERR_NOT_INITIALIZED, "cogni_quant_init has not been called");
+  }
+  cogni_quant_weight* w = new cogni_quant_weight();
+  hipError_t e = hipMalloc(&w->dev, need);
+  if (e == hipSuccess) e = hipMemcpyHtoD(w->dev, const_cast<void*>(raw), need);
+  if (e != hipSuccess) {
+    if (w->dev) (void)hipFree(w->dev);
+    delete w;
+    return hip_fail(e, "upload of quantized weight");
+  }
+  w->bytes = need;
+  w->type = type;
+  w->out_dim = out_dim;
+  w->in_dim = in_dim;
+  *qw = w;
+  return 0;
+}
+
+uint64_t cogni_weight_device_ptr(const cogni_quant_weight* qw) { return qw ? (uint64_t)(uintptr_t)qw->dev : 0; }
+
+int cogni_weight_destroy(cogni_quant_weight* qw) {
+  if (!qw) return 0;
+  if (qw->dev) (void)hipFree(qw->dev);
+  delete qw;
+  return 0;
+}
+
+int cogni_weight_matmul(const cogni_quant_weight* qw, const float* x, int32_t rows, const float* bias, float* result) {
+  if (!qw || !x || !result) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_matmul: null argument");
+  if (rows <= 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_matmul: rows must be positive");
+  const size_t xin = (size_t)rows * qw->in_dim * 4, xout = (size_t)rows * qw->out_dim * 4;
+  DeviceMem dx, dres, dout;
+  HIP_TRY(hipMalloc(&dx.p, xin), "hipMalloc(x)");
+  HIP_TRY(hipMalloc(&dout.p, xout), "hipMalloc(result)");
+  HIP_TRY(hipMemcpyHtoD(dx.p, const_cast<float*>(x), xin), "hipMemcpyHtoD(x)");
+  if (bias) {  // bias[o] is added to every row: stage it as a [rows][out_dim] residual
+    std::vector<float> tiled((size_t)rows * qw->out_dim);
+    for (int32_t r = 0; r < rows; r++) std::memcpy(&tiled[(size_t)r * qw->out_dim], bias, (size_t)qw->out_dim * 4);
+    HIP_TRY(hipMalloc(&dres.p, xout), "hipMalloc(bias)");
+    HIP_TRY(hipMemcpyHtoD(dres.p, tiled.data(), xout), "hipMemcpyHtoD(bias)");
+  }
+  int rc = cogni_gemv_dev((uint64_t)(uintptr_t)qw->dev, qw->type, dx.addr(), dres.addr(), dout.addr(),
+                          (uint32_t)qw->in_dim, (uint32_t)qw->out_dim, (uint32_t)rows, nullptr);
+  if (rc != 0) return rc;
+  HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize(matmul)");
+  HIP_TRY(hipMemcpyDtoH(result, dout.p, xout), "hipMemcpyDtoH(result)");
+  return 0;
+}
+
+int cogni_matmul_add(const float* x, int32_t rows, int32_t in_dim, const void* w_raw, size_t w_bytes, uint32_t w_type,
+                     int32_t out_dim, const float* bias, float* result) {
+  cogni_quant_weight* qw = nullptr;
+  int rc = cogni_weight_create(&qw, w_raw, w_bytes, w_type, out_dim, in_dim);
+  if (rc != 0) return rc;
+  rc = cogni_weight_matmul(qw, x, rows, bias, result);
+  cogni_weight_destroy(qw);
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,132 @@
+/*
+ * cogni_quant.h - C ABI of the quantized-matmul operators (libcogni_hip.so).
+ *
+ * Replaces, for one MI355X (gfx950), the reference's CPU operators
+ *   ML::GGUF::QuantMatmul.matmul_add   src/ml/gguf/quant_matmul.cr:20-36
+ *   ML::GGUF::Dequant.dequantize       src/ml/gguf/dequant.cr:19-31
+ * and the GPU kernels its CUDA probes launch (src/ml/cuda/kernels/q{4,5,6}k_gemv_probe.ptx,
+ * bin/cuda_q8_gemv_probe.cr:39-227). Weights are the raw GGUF bytes, row-major
+ * [out_dim][in_dim / block_elements][block_bytes]; nothing is repacked on the host.
+ *
+ * Three levels, lowest first:
+ *   1. the code object: kernels are unmangled symbols, launched by name through
+ *      ml_hip_driver.h exactly as the reference launches PTX entries
+ *      (cogni_quant_code_object, cogni_kernel_name, cogni_gemv_grid);
+ *   2. device-pointer operators, asynchronous on a stream (cogni_*_dev);
+ *   3. host-buffer operators with the reference's CPU signatures (cogni_dequantize,
+ *      cogni_matmul_add) and the QuantWeight handle that keeps weights resident.
+ *
+ * Every function returns 0 on success, a positive hipError_t value when a HIP call failed, or one
+ * of the negative COGNI_ERR_* codes. cogni_last_error() gives the text for the calling thread.
+ * There is no CPU fallback: without a gfx950 device every operator fails with an error.
+ */
+#ifndef COGNI_QUANT_H
+#define COGNI_QUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml tensor type ids, src/ml/gguf/reader.cr:34-49 */
+enum {
+  COGNI_TYPE_F32 = 0,
+  COGNI_TYPE_F16 = 1,
+  COGNI_TYPE_Q8_0 = 8,
+  COGNI_TYPE_Q4_K = 12,
+  COGNI_TYPE_Q5_K = 13,
+  COGNI_TYPE_Q6_K = 14,
+  COGNI_TYPE_IQ4_NL = 20
+};
+
+enum {
+  COGNI_ERR_INVALID_ARGUMENT = -1, /* the reference raises ArgumentError / a size check fails */
+  COGNI_ERR_UNSUPPORTED_TYPE = -2, /* "Unsupported ... type", quant_matmul.cr:33-34, dequant.cr:29-30 */
+  COGNI_ERR_NOT_INITIALIZED = -3,  /* cogni_quant_init has not succeeded in this process */
+  COGNI_ERR_NO_DEVICE = -4         /* no gfx950 device: there is no fallback path */
+};
+
+enum { COGNI_MAX_GEMV_TOKENS = 8 }; /* tokens one weight-stationary GEMV launch handles */
+
+/* ---- geometry: TensorType#block_bytes / #block_elements / TensorInfo#data_bytes,
+ *      src/ml/gguf/reader.cr:51-78,119-127. Return -1 for an unknown type id. No GPU needed. */
+int32_t cogni_block_bytes(uint32_t type);
+int32_t cogni_block_elements(uint32_t type);
+int64_t cogni_data_bytes(uint32_t type, int64_t n_elements);
+
+/* ---- level 1: the code object ---------------------------------------------------------------- */
+
+/* The embedded gfx950 code object, suitable for hipModuleLoadData / mlhip_module_load_data. Takes the
+ * place of the PTX text the reference embeds (bin/cuda_q4k_gemv_probe.cr:39, driver.cr:115-119).
+ * No GPU needed. */
+int cogni_quant_code_object(const void** image, size_t* size);
+
+/* Kernel symbol for (type, tokens, add): "q4_k_gemv_f32", "q6_k_gemv_add_f32_tbatch4", ...
+ * tokens in 1..COGNI_MAX_GEMV_TOKENS. Parameters of the kernel, in order:
+ *   (w_raw:u64, x:u64, out:u64, in_dim:u32, out_dim:u32)              q4k_gemv_probe.ptx:5-11
+ *   (w_raw, x, residual, out, in_dim, out_dim) for the *_add_* kernels  q4k_gemv_probe.ptx:1572-1578
+ * x rows at stride in_dim floats, out/residual rows at stride out_dim floats (q4k_gemv_probe.ptx:747-768).
+ * Returns NULL for an unsupported combination. No GPU needed. */
+const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add);
+/* Launch geometry of every GEMV kernel: block = 256 threads, grid_x = ceil(out_dim / 16), no dynamic
+ * shared memory. (The reference's kernels use grid ceil(out_dim/4) x block 128,
+ * bin/cuda_q4k_gemv_probe.cr:225-230.) */
+int cogni_gemv_launch_dims(uint32_t out_dim, uint32_t* grid_x, uint32_t* block_x);
+/* Kernel symbol "dequantize_<type>_f32"; parameters (w_raw:u64, out:u64, n_elements:u64); block = 256
+ * threads, any grid (grid-stride). NULL for an unsupported type. No GPU needed. */
+const char* cogni_dequantize_kernel_name(uint32_t type);
+
+/* ---- initialisation --------------------------------------------------------------------------- */
+
+/* Select device `ordinal`, check that it is gfx950, load the code object and resolve the kernels.
+ * Idempotent per process for the same ordinal. */
+int cogni_quant_init(int32_t ordinal);
+/* Unload the module and free cached scratch buffers. */
+int cogni_quant_shutdown(void);
+
+/* ---- level 2: device-pointer operators (asynchronous on `stream`; NULL = the null stream) ----- */
+
+/* Dequant.dequantize on device memory: out[0..n_elements) float32. dequant.cr:19-31. */
+int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, uint64_t out, void* stream);
+
+/* Decode GEMV, weights read once for all tokens:
+ *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
+ * fp32 accumulation. tokens >= 1; more than COGNI_MAX_GEMV_TOKENS are issued as consecutive launches
+ * of up to 8 tokens. in_dim must be a multiple of 256 (Q4_K/Q5_K/Q6_K; the reference requires the
+ * same, bin/cuda_q4k_gemv_probe.cr:125) or of 32... Q8_0 accepts any in_dim >= 1 (its last block is clipped,
+ * quant_matmul.cr:241,259). Types: Q8_0, Q4_K, Q5_K, Q6_K. */
+int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
+                   uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
+
+/* ---- level 3: host-buffer operators with the reference's CPU signatures (synchronous) -------- */
+
+/* Dequant.dequantize(data, type, n_elements) : Array(Float32)   dequant.cr:19
+ * `out` receives n_elements floats. data_bytes is checked against the type's geometry. */
+int cogni_dequantize(const void* data, size_t data_bytes, uint32_t type, int64_t n_elements, float* out);
+
+/* QuantMatmul.matmul_add(x, rows, in_dim, w_raw, w_type, out_dim, bias) : Array(Float32)   quant_matmul.cr:20
+ * result[r*out_dim + o] = bias[o] + sum_j x[r*in_dim + j] * deq(W[o][j]); `result` receives rows*out_dim floats. */
+int cogni_matmul_add(const float* x, int32_t rows, int32_t in_dim, const void* w_raw, size_t w_bytes,
+                     uint32_t w_type, int32_t out_dim, const float* bias, float* result);
+
+/* QuantWeight {raw, type, out_dim, in_dim} (src/ml/gguf/compute.cr:20-30) with its bytes uploaded once
+ * and kept resident, the role of fallback_metal_buffer (compute.cr:36-43). */
+typedef struct cogni_quant_weight cogni_quant_weight;
+int cogni_weight_create(cogni_quant_weight** qw, const void* raw, size_t raw_bytes, uint32_t type,
+                        int32_t out_dim, int32_t in_dim);
+uint64_t cogni_weight_device_ptr(const cogni_quant_weight* qw);
+/* matmul(x, rows, qw, bias): ComputeBackend#matmul, compute.cr:50; bias may be NULL (qmatvec_nobias,
+ * src/ml/gguf/qwen35_cpu.cr:1462-1468). */
+int cogni_weight_matmul(const cogni_quant_weight* qw, const float* x, int32_t rows, const float* bias,
+                        float* result);
+int cogni_weight_destroy(cogni_quant_weight* qw);
+
+/* Text of the last failure on the calling thread ("hipModuleLoadData failed with HIP error 209 (...)"). */
+const char* cogni_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COGNI_QUANT_H */

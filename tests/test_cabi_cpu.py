@@ -1,0 +1,134 @@
+"""CPU-side checks of the C-ABI boundary: the library loads, exports every declared symbol, embeds a
+gfx950 code object with the documented kernel symbols, and fails loudly when there is no GPU."""
+import ctypes
+import os
+import re
+import struct
+
+import pytest
+
+from cogni_ml_amd import hip, quant
+from cogni_ml_amd.types import TensorType
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:mlhip|cogni)_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.mark.parametrize("header", ["ml_hip_driver.h", "cogni_quant.h"])
+def test_every_declared_symbol_is_exported(header):
+    L = hip.lib()
+    names = declared_functions(header)
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(L, n), "%s declared in %s but not exported" % (n, header)
+
+
+def test_geometry_matches_reference_table():
+    L = hip.lib()
+    for t in TensorType:
+        assert L.cogni_block_bytes(int(t)) == t.block_bytes
+        assert L.cogni_block_elements(int(t)) == t.block_elements
+    assert L.cogni_data_bytes(12, 12288 * 4096) == 28311552
+    assert L.cogni_data_bytes(14, 151936 * 4096) == 510504960
+    assert L.cogni_data_bytes(8, 3584 * 1024) == 3899392
+    assert L.cogni_block_bytes(99) == -1 and L.cogni_data_bytes(99, 10) == -1
+
+
+def code_object():
+    img, size = ctypes.c_void_p(), ctypes.c_size_t()
+    assert hip.lib().cogni_quant_code_object(ctypes.byref(img), ctypes.byref(size)) == 0
+    return ctypes.string_at(img, size.value)
+
+
+def test_code_object_is_amdgpu_elf_with_kernel_symbols():
+    blob = code_object()
+    assert blob[:4] == b"\x7fELF" and blob[4] == 2                      # ELF64
+    assert struct.unpack_from("<H", blob, 18)[0] == 224                  # EM_AMDGPU
+    assert struct.unpack_from("<I", blob, 48)[0] & 0xFF == 0x4F          # EF_AMDGPU_MACH_AMDGCN_GFX950
+    for t in (8, 12, 13, 14):
+        for m in range(1, 9):
+            for add in (0, 1):
+                name = quant.gemv_kernel_name(t, m, add)
+                assert name and (name.encode() + b"\x00") in blob, name
+    for t in (0, 1, 8, 12, 13, 14, 20):
+        assert (quant.dequantize_kernel_name(t).encode() + b"\x00") in blob
+    assert quant.gemv_kernel_name(12, 1) == "q4_k_gemv_f32"               # the reference's naming scheme
+    assert quant.gemv_kernel_name(14, 4, True) == "q6_k_gemv_add_f32_tbatch4"
+    assert quant.gemv_kernel_name(20, 1) is None and quant.gemv_kernel_name(12, 9) is None
+    assert quant.dequantize_kernel_name(10) is None
+
+
+def test_gemv_launch_dims():
+    assert quant.gemv_launch_dims(12288) == (768, 256)
+    assert quant.gemv_launch_dims(17) == (2, 256)
+
+
+def test_argument_errors_do_not_need_a_gpu():
+    import numpy as np
+    x = np.zeros(256, dtype=np.float32)
+    w = np.zeros(144, dtype=np.uint8)
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for fused matmul: IQ4_NL") as e:
+        quant.matmul_add(x, 1, 256, w, 20, 1, None)
+    assert e.value.code == -2
+    with pytest.raises(quant.QuantError, match="requires in_dim multiple of 256") as e:
+        quant.matmul_add(x, 1, 100, w, 12, 1, None)
+    assert e.value.code == -1
+    with pytest.raises(quant.QuantError, match="shape needs 288") as e:
+        quant.matmul_add(x, 1, 256, w, 12, 2, None)
+    assert e.value.code == -1
+    with pytest.raises(quant.QuantError, match="Unsupported dequantization type") as e:
+        quant.dequantize(w, 10, 256)
+    assert e.value.code == -2
+
+
+def gpu_present():
+    return os.path.exists("/dev/kfd")
+
+
+@pytest.mark.skipif(gpu_present(), reason="checks the no-GPU failure mode")
+def test_no_gpu_means_error_not_fallback():
+    import numpy as np
+    with pytest.raises(quant.QuantError, match="no CPU fallback") as e:
+        quant.init(0)
+    assert e.value.code == -4
+    with pytest.raises(quant.QuantError, match="cogni_quant_init has not been called") as e:
+        quant.dequantize(np.zeros(144, dtype=np.uint8), 12, 256)
+    assert e.value.code == -3
+
+
+# ---- ResidentSequenceRunner: the reference's three examples (spec/cuda_resident_sequence_runner_spec.cr:5-50)
+
+def test_runner_runs_only_the_active_token_prefix():
+    seen = []
+    r = hip.ResidentSequenceRunner(4, lambda: None, lambda: None, seen.append)
+    r.active_tokens = 2
+    r.run_sequence()
+    assert seen == [0, 1]
+    assert r.run_repeated(3) == 6
+
+
+def test_runner_passes_active_count_to_override():
+    seen = []
+    r = hip.ResidentSequenceRunner(8, lambda: None, lambda: None, lambda tok: None, None, seen.append)
+    r.active_tokens = 4
+    r.run_sequence()
+    assert seen == [4]
+
+
+def test_runner_rejects_invalid_active_counts():
+    r = hip.ResidentSequenceRunner(4, lambda: None, lambda: None, lambda tok: None)
+    with pytest.raises(ValueError, match="active_tokens must be positive"):
+        r.active_tokens = 0
+    with pytest.raises(ValueError, match="active_tokens must be <= tokens"):
+        r.active_tokens = 5
+    with pytest.raises(ValueError, match="tokens must be positive"):
+        hip.ResidentSequenceRunner(0, lambda: None, lambda: None, lambda tok: None)
+    with pytest.raises(ValueError, match="reps must be positive"):
+        r.run_repeated(0)
+    r.reset_active_tokens()
+    assert r.active_tokens == 4

@@ -1,0 +1,158 @@
+"""GPU decode GEMV (M = 1..8, optional residual) vs the CPU oracle.
+
+Tolerance (fp32 path): max|err| <= 1e-4 * ||x||_2 * max|w_row| per token and output row. The
+reference's own probe gate (cos >= 0.99999 and max_diff <= 1e-3, bin/cuda_q4k_gemv_probe.cr:289)
+is asserted as well where the output scale makes it meaningful.
+"""
+import numpy as np
+import pytest
+
+from cogni_ml_amd import quant, synth
+from gpu_common import DevArray, gpu  # noqa: F401
+from helpers import BLOCK, Q4_K, Q5_K, Q6_K, Q8_0, cosine, gemv_tolerance
+
+pytestmark = pytest.mark.gpu
+TYPES = [Q8_0, Q4_K, Q5_K, Q6_K]
+
+
+def run_gemv(raw, type_id, x, in_dim, out_dim, tokens, residual=None):
+    w, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim)
+    rd = DevArray(residual) if residual is not None else None
+    quant.gemv_dev(w.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, tokens, rd.ptr if rd else 0)
+    out = od.read(np.float32, tokens * out_dim)
+    for a in (w, xd, od, rd):
+        if a:
+            a.close()
+    return out
+
+
+def check(oracle, raw, type_id, x, in_dim, out_dim, tokens, residual=None, what=""):
+    got = run_gemv(raw, type_id, x, in_dim, out_dim, tokens, residual)
+    zero = np.zeros(out_dim, dtype=np.float32)
+    want = oracle.matmul_add(x, tokens, in_dim, raw, type_id, out_dim, zero, threads=8).astype(np.float64)
+    if residual is not None:
+        want = (want.astype(np.float32) + residual).astype(np.float64)
+    dense = np.abs(oracle.dequantize(raw, type_id, out_dim * (raw.size // out_dim // BLOCK[type_id][0]) * BLOCK[type_id][1])
+                   ).reshape(out_dim, -1)
+    tol = gemv_tolerance(x, dense, tokens, in_dim).reshape(-1)
+    err = np.abs(got.astype(np.float64) - want)
+    worst = int(np.argmax(err / np.maximum(tol, 1e-30)))
+    assert np.all(err <= tol), "%s: err %.3e > tol %.3e at %d" % (what, err[worst], tol[worst], worst)
+    return got, want, float(np.max(err / np.maximum(tol, 1e-30)))
+
+
+@pytest.mark.parametrize("type_id", TYPES)
+@pytest.mark.parametrize("tokens", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("add", [False, True])
+def test_small_shapes_all_token_counts(gpu, oracle, type_id, tokens, add):
+    rng = np.random.default_rng(1000 * type_id + 10 * tokens + add)
+    be = BLOCK[type_id][1]
+    out_dim = 37                                  # not a multiple of the 16 rows a workgroup covers
+    in_dim = be * 9 if be == 256 else 1024 + 96   # K-quants: 9 blocks = one full + one partial column set
+    raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = rng.standard_normal(tokens * out_dim).astype(np.float32) if add else None
+    check(oracle, raw, type_id, x, in_dim, out_dim, tokens, res, "type %d M=%d add=%s" % (type_id, tokens, add))
+
+
+@pytest.mark.parametrize("in_dim", [32, 80, 1000, 1024, 2048 + 32])
+def test_q8_0_row_lengths_including_clipped_tail(gpu, oracle, in_dim):
+    rng = np.random.default_rng(in_dim)
+    raw = synth.make_weights(rng, Q8_0, 21, in_dim)
+    x = synth.make_activations(rng, 2, in_dim)
+    check(oracle, raw, Q8_0, x, in_dim, 21, 2, None, "Q8_0 in=%d" % in_dim)
+
+
+@pytest.mark.parametrize("type_id", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("nb", [1, 7, 8, 16, 17, 33])
+def test_k_quant_block_counts(gpu, oracle, type_id, nb):
+    rng = np.random.default_rng(77 * type_id + nb)
+    raw = synth.make_weights(rng, type_id, 16, 256 * nb)
+    x = synth.make_activations(rng, 1, 256 * nb)
+    check(oracle, raw, type_id, x, 256 * nb, 16, 1, None, "type %d nb=%d" % (type_id, nb))
+
+
+def test_single_output_row_and_many_tokens(gpu, oracle):
+    rng = np.random.default_rng(5)
+    raw = synth.make_weights(rng, Q4_K, 1, 512)
+    check(oracle, raw, Q4_K, synth.make_activations(rng, 1, 512), 512, 1, 1)
+    raw = synth.make_weights(rng, Q6_K, 40, 512)
+    res = rng.standard_normal(19 * 40).astype(np.float32)
+    check(oracle, raw, Q6_K, synth.make_activations(rng, 19, 512), 512, 40, 19, res, "19 tokens = 8 + 8 + 3")
+
+
+CONFIGS = [
+    ("cfg1 Q8_0 ffn_up 0.8B", Q8_0, 3584, 1024, [1]),
+    ("cfg2 Q4_K gate/up", Q4_K, 12288, 4096, [1, 4, 8]),
+    ("cfg2 Q4_K down", Q4_K, 4096, 12288, [1, 8]),
+    ("cfg3 Q6_K down", Q6_K, 4096, 12288, [1, 4, 8]),
+    ("cfg3 Q5_K", Q5_K, 4096, 4096, [1, 8]),
+    ("cfg5 Q4_K k/v", Q4_K, 1024, 4096, [1, 8]),
+]
+
+
+@pytest.mark.parametrize("name,type_id,out_dim,in_dim,token_list", CONFIGS)
+def test_configured_shapes(gpu, oracle, name, type_id, out_dim, in_dim, token_list):
+    rng = np.random.default_rng(abs(hash(name)) % (1 << 31))
+    raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+    for tokens in token_list:
+        x = synth.make_activations(rng, tokens, in_dim)
+        got, want, frac = check(oracle, raw, type_id, x, in_dim, out_dim, tokens, None, "%s M=%d" % (name, tokens))
+        assert cosine(got, want) >= 0.99999
+        assert np.max(np.abs(got - want)) <= 1e-3
+        print("%s M=%d: max err / tolerance = %.4f" % (name, tokens, frac))
+
+
+def test_q6_k_output_head_shape(gpu, oracle):
+    """The 4096 -> 151936 Q6_K head (510 MB of weights): sampled rows against the oracle."""
+    rng = np.random.default_rng(151936)
+    out_dim, in_dim = 151936, 4096
+    raw = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    x = synth.make_activations(rng, 1, in_dim)
+    got = run_gemv(raw, Q6_K, x, in_dim, out_dim, 1)
+    rb = 16 * 210
+    for lo in (0, 70000, out_dim - 4096):
+        sub = raw[lo * rb:(lo + 4096) * rb]
+        want = oracle.matmul_add(x, 1, in_dim, sub, Q6_K, 4096, np.zeros(4096, dtype=np.float32), threads=8)
+        dense = np.abs(oracle.dequantize(sub, Q6_K, 4096 * in_dim)).reshape(4096, in_dim)
+        tol = gemv_tolerance(x, dense, 1, in_dim).reshape(-1)
+        assert np.all(np.abs(got[lo:lo + 4096].astype(np.float64) - want) <= tol)
+
+
+def test_matmul_add_host_signature_with_bias(gpu, oracle):
+    """QuantMatmul.matmul_add through the host-buffer entry point, with the reference spec's
+    deterministic x and bias (spec/q4k_matmul_spec.cr:66-73)."""
+    rng = np.random.default_rng(12)
+    out_dim, in_dim, rows = 256, 1024, 2
+    i = np.arange(rows * in_dim, dtype=np.uint64)
+    x = (((i * 2654435761) % (1 << 32) % 2000).astype(np.int64) - 1000).astype(np.float32) / np.float32(1000.0)
+    bias = ((np.arange(out_dim) % 10) / np.float32(100.0)).astype(np.float32)
+    for t in TYPES:
+        raw = synth.make_weights(rng, t, out_dim, in_dim)
+        mine = quant.matmul_add(x, rows, in_dim, raw, t, out_dim, bias)
+        ref = oracle.matmul_add(x, rows, in_dim, raw, t, out_dim, bias)
+        assert cosine(mine, ref) >= 0.9999999
+        assert np.max(np.abs(mine - ref)) / np.max(np.abs(ref)) <= 1e-5     # the reference's own gate
+        qw = quant.QuantWeight(raw, t, out_dim, in_dim, "test")
+        assert qw.device_ptr != 0
+        assert np.array_equal(qw.matmul(x, rows, bias), mine)
+        nobias = qw.matmul(x[:in_dim], 1)
+        assert np.allclose(nobias, ref[:out_dim] - bias, rtol=0, atol=1e-4)
+        qw.close()
+
+
+def test_linearity_and_determinism_at_full_size(gpu):
+    """Size-independent properties at the headline shape: same input -> same bits; f(2a) == 2 f(a) exactly;
+    f(a) + f(b) ~= f(a + b)."""
+    rng = np.random.default_rng(99)
+    out_dim, in_dim = 12288, 4096
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    a, b = synth.make_activations(rng, 1, in_dim), synth.make_activations(rng, 1, in_dim)
+    fa = run_gemv(raw, Q4_K, a, in_dim, out_dim, 1)
+    assert np.array_equal(fa, run_gemv(raw, Q4_K, a, in_dim, out_dim, 1))
+    assert np.array_equal(run_gemv(raw, Q4_K, 2 * a, in_dim, out_dim, 1), 2 * fa)
+    fb, fab = run_gemv(raw, Q4_K, b, in_dim, out_dim, 1), run_gemv(raw, Q4_K, a + b, in_dim, out_dim, 1)
+    assert np.max(np.abs((fa + fb) - fab)) <= 1e-4 * np.max(np.abs(fab))
+    # tokens batched in one launch give the same bits as one launch per token
+    both = run_gemv(raw, Q4_K, np.concatenate([a, b]), in_dim, out_dim, 2)
+    assert np.array_equal(both[:out_dim], fa) and np.array_equal(both[out_dim:], fb)
