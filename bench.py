@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+Headline (the JSON line on stdout): Q4_K decode GEMV, W = 12288 x 4096 (in_dim 4096 -> out_dim 12288,
+the ffn_gate/ffn_up shape), M = 1, fp32 activations and accumulation. One "step" is one GEMV launch.
+Weights are seeded synthetic super-blocks, already resident in HBM; consecutive steps read different
+copies of the matrix (more bytes in total than the 256 MB last-level cache) so every step streams
+its 28 MB from HBM. The K timed steps are captured into one HIP graph and bracketed by HIP events
+on the launch stream.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+  python bench.py --mode cases      per-shape table (key=value blocks, stderr) + the JSON line
+  python bench.py --mode pmc        plain launches of the dominant kernel and of a copy kernel of
+                                    known size, for rocprofv3 --pmc / --kernel-trace runs
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "cogni-ml_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import numpy as np  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
+LLC_BYTES = 256 << 20           # last-level (Infinity) cache
+Q4_K, Q5_K, Q6_K, Q8_0 = 12, 13, 14, 8
+TYPE_NAME = {Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", Q8_0: "Q8_0"}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gemv_bytes(w_bytes, in_dim, out_dim, tokens):
+    """Algorithmic bytes of one GEMV: weights once + activations in + results out."""
+    return w_bytes + 4 * tokens * in_dim + 4 * tokens * out_dim
+
+
+class GemvCase:
+    """Rotating weight copies + activations + output for one (type, shape, tokens)."""
+
+    def __init__(self, hip, quant, synth, rng, w_type, out_dim, in_dim, tokens, min_total_bytes=2 * LLC_BYTES,
+                 max_copies=24):
+        from cogni_ml_amd.types import TensorType
+        self.hip, self.quant = hip, quant
+        self.w_type, self.out_dim, self.in_dim, self.tokens = w_type, out_dim, in_dim, tokens
+        self.w_bytes = TensorType(w_type).data_bytes(in_dim) * out_dim
+        self.copies = int(max(1, min(max_copies, -(-min_total_bytes // self.w_bytes))))
+        self.host_w = synth.make_weights(rng, w_type, out_dim, in_dim)
+        self.host_x = synth.make_activations(rng, tokens, in_dim)
+        self.w = []
+        for c in range(self.copies):
+            buf = hip.DeviceBuffer(self.w_bytes)
+            # copy 0 is the matrix checked against the oracle; the others are the same bytes rotated, so that
+            # every copy holds different data at every address
+            src = self.host_w if c == 0 else np.roll(self.host_w, 4096 * c + 17)
+            hip.copy_htod(buf.ptr, src, self.w_bytes, "weights")
+            self.w.append(buf)
+        self.x = hip.DeviceBuffer(self.host_x.nbytes)
+        hip.copy_htod(self.x.ptr, self.host_x, self.host_x.nbytes, "x")
+        self.out = hip.DeviceBuffer(4 * tokens * out_dim)
+        self.bytes_per_step = gemv_bytes(self.w_bytes, in_dim, out_dim, tokens)
+
+    def launch(self, step, stream):
+        self.quant.gemv_dev(self.w[step % self.copies].ptr, self.w_type, self.x.ptr, self.out.ptr, self.in_dim,
+                            self.out_dim, self.tokens, 0, stream.handle)
+
+    def read_out(self):
+        out = np.empty(self.tokens * self.out_dim, dtype=np.float32)
+        self.hip.synchronize()
+        self.hip.copy_dtoh(out, self.out.ptr, out.nbytes, "out")
+        return out
+
+    def close(self):
+        for b in self.w + [self.x, self.out]:
+            b.close()
+
+
+def time_steps(hip, stream, launch, steps, warmup):
+    """Run `warmup` untimed and exactly `steps` timed launches on `stream`; returns ms for the timed region.
+    The timed launches are captured into one HIP graph so host launch latency does not gate the GPU."""
+    for i in range(warmup):
+        launch(i, stream)
+    stream.synchronize()
+    graph = exe = None
+    try:
+        stream.begin_capture(1)
+        for i in range(steps):
+            launch(warmup + i, stream)
+        graph = stream.end_capture()
+        exe = graph.instantiate()
+        exe.upload(stream)
+        stream.synchronize()
+    except Exception as e:  # stream capture unavailable: fall back to direct launches
+        log("graph capture failed (%s); timing direct launches" % e)
+        exe = None
+    e0, e1 = hip.Event(), hip.Event()
+    hip.synchronize()
+    e0.record(stream)
+    if exe is not None:
+        exe.launch(stream)
+    else:
+        for i in range(steps):
+            launch(warmup + i, stream)
+    e1.record(stream)
+    e1.synchronize()
+    hip.synchronize()
+    ms = e0.elapsed_ms(e1)
+    for o in (exe, graph):
+        if o is not None:
+            o.close()
+    e0.close()
+    e1.close()
+    return ms, exe is not None
+
+
+def cpu_baseline(oracle, case, budget_s=10.0):
+    """The CPU oracle (C restatement of QuantMatmul.matmul_add, 1 thread, f64 accumulation) on the same matrix."""
+    zero = np.zeros(case.out_dim, dtype=np.float32)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        ref = oracle.matmul_add(case.host_x, case.tokens, case.in_dim, case.host_w, case.w_type, case.out_dim, zero)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el >= budget_s and reps >= 3 or reps >= 200:
+            break
+    return ref, reps, el
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--mode", choices=["headline", "cases", "pmc"], default="headline")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--seed", type=int, default=1234)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the path has no multi-GPU part (run with --gpus 1)")
+    if args.steps <= 0 or args.warmup < 0:
+        sys.exit("--steps must be positive and --warmup non-negative")
+
+    from cogni_ml_amd import hip, quant, synth
+    from oracle import oracle
+
+    ctx = hip.Context.create(0)
+    quant.init(0)
+    log("device=%s arch=%s compute_units=%d clock_mhz=%d host_cores=%d" % (
+        ctx.device_name, ctx.arch, ctx.compute_units, ctx.clock_khz // 1000, os.cpu_count()))
+    rng = np.random.default_rng(args.seed)
+    stream = hip.HIPStream()
+
+    head = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1)
+
+    if args.mode == "pmc":
+        # plain (uncaptured) launches so a profiler attributes counters per dispatch; the copy kernel moves a
+        # known number of bytes and calibrates the counters' units
+        mod = hip.HIPModule.load_builtin()
+        copy_fn = mod.function("copy_bytes_16")
+        import ctypes
+        nbytes = 512 << 20
+        src, dst = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(nbytes)
+        params = hip.KernelParams(ctypes.c_uint64(src.ptr), ctypes.c_uint64(dst.ptr), ctypes.c_uint64(nbytes))
+        with hip.with_stream(stream):
+            for i in range(args.warmup + args.steps):
+                head.launch(i, stream)
+            for i in range(8):
+                hip.launch(copy_fn, 8192, 1, 1, 256, 1, 1, params, "copy_bytes_16")
+        stream.synchronize()
+        log("pmc mode: %d x %s over %d weight copies, 8 x copy_bytes_16 of %d bytes" % (
+            args.warmup + args.steps, quant.gemv_kernel_name(Q4_K, 1), head.copies, nbytes))
+        return
+
+    # ---- parity spot check of the measured kernel against the oracle, and the CPU baseline ------------
+    head.launch(0, stream)
+    stream.synchronize()
+    got = head.read_out()
+    ref, cpu_reps, cpu_s = cpu_baseline(oracle, head, args.cpu_seconds)
+    dense_max = float(np.max(np.abs(oracle.dequantize(head.host_w[:16 * 144 * 256], Q4_K, 256 * 4096))))
+    max_diff = float(np.max(np.abs(got - ref)))
+    cos = float(got.astype(np.float64) @ ref.astype(np.float64) /
+                np.sqrt((got.astype(np.float64) @ got.astype(np.float64)) * (ref.astype(np.float64) @ ref.astype(np.float64))))
+    ok = cos >= 0.99999 and max_diff <= 1e-3
+    cpu_gbps = head.bytes_per_step * cpu_reps / cpu_s / 1e9
+
+    # ---- timed region ------------------------------------------------------------------------------------
+    ms, graphed = time_steps(hip, stream, head.launch, args.steps, args.warmup)
+    ms_per_step = ms / args.steps
+    gbps = head.bytes_per_step / (ms_per_step * 1e-3) / 1e9
+
+    # cache-resident figure (one copy only), reported beside the HBM one
+    hot_ms, _ = time_steps(hip, stream, lambda i, s: head.launch(0, s), args.steps, args.warmup)
+    hot_gbps = head.bytes_per_step / (hot_ms / args.steps * 1e-3) / 1e9
+
+    log("case=q4_k_gemv ffn_up\ntype=Q4_K\nshape=%dx%d\ntokens=1\nraw_bytes=%d\ncopies=%d\nreps=%d\nwarmup=%d\n"
+        "hip_ms=%.5f\ncpu_ms=%.3f\ncos=%.8f\nmax_diff=%g\nok=%s\ngbps_hbm=%.1f\ngbps_cache_hot=%.1f\ngraph=%s" % (
+            head.in_dim, head.out_dim, head.w_bytes, head.copies, args.steps, args.warmup, ms_per_step,
+            cpu_s / cpu_reps * 1e3, cos, max_diff, str(ok).lower(), gbps, hot_gbps, graphed))
+
+    extra = {}
+    if args.mode == "cases":
+        table = [
+            ("q8_0 ffn_up 0.8B", Q8_0, 3584, 1024, 1), ("q4_k ffn_down", Q4_K, 4096, 12288, 1),
+            ("q6_k ffn_down", Q6_K, 4096, 12288, 1), ("q5_k attn_qkv-like", Q5_K, 4096, 4096, 1),
+            ("q6_k output head", Q6_K, 151936, 4096, 1),
+            ("q4_k ffn_up M=4", Q4_K, 12288, 4096, 4), ("q4_k ffn_up M=8", Q4_K, 12288, 4096, 8),
+        ]
+        for name, t, out_dim, in_dim, tokens in table:
+            c = GemvCase(hip, quant, synth, rng, t, out_dim, in_dim, tokens)
+            steps = max(20, min(args.steps, int(2e9 // c.bytes_per_step)))
+            cms, _ = time_steps(hip, stream, c.launch, steps, min(args.warmup, steps))
+            cg = c.bytes_per_step / (cms / steps * 1e-3) / 1e9
+            extra[name] = {"gbps": round(cg, 1), "ms": round(cms / steps, 5), "frac_hbm": round(cg / HBM_PEAK_GBPS, 4)}
+            log("case=%s\ntype=%s\nshape=%dx%d\ntokens=%d\nraw_bytes=%d\ncopies=%d\nreps=%d\nhip_ms=%.5f\ngbps_hbm=%.1f\n" % (
+                name, TYPE_NAME[t], in_dim, out_dim, tokens, c.w_bytes, c.copies, steps, cms / steps, cg))
+            c.close()
+
+    result = {
+        "metric": "Q4_K GEMV GB/s 4096x12288 M=1",
+        "value": round(gbps, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "Q4_K decode GEMV, W 12288x4096 (in 4096 -> out 12288), M=1, fp32 x, fp32 accumulate",
+            "weight_bytes": head.w_bytes, "bytes_per_step": head.bytes_per_step,
+            "weight_copies_rotated": head.copies, "timed_region": "hip graph of K launches" if graphed else "K direct launches",
+        },
+        "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "cache_hot_gbps": round(hot_gbps, 1),
+        "parity": {"cos": round(cos, 8), "max_diff": max_diff, "ok": ok, "tol_1e-4_x_wmax": 1e-4 * float(np.linalg.norm(head.host_x)) * dense_max},
+        "roofline": {
+            "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+        },
+        "cpu_baseline": {
+            "value": round(cpu_gbps, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d x the same 12288x4096 Q4_K GEMV (M=1) through the C restatement of QuantMatmul.matmul_add, "
+                      "1 thread, %.1f s" % (cpu_reps, cpu_s),
+        },
+    }
+    if extra:
+        result["cases"] = extra
+    head.close()
+    stream.close()
+    ctx.close()
+    print(json.dumps(result), flush=True)
+    if not ok:
+        sys.exit(1)
+
+
+if __name__ == "__main__":
+    main()
