@@ -137,7 +137,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--mode", choices=["headline", "cases", "pmc"], default="headline")
+    ap.add_argument("--mode", choices=["headline", "cases", "pmc", "ceiling"], default="headline")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--seed", type=int, default=1234)
     args = ap.parse_args()
@@ -175,6 +175,32 @@ def main():
         stream.synchronize()
         log("pmc mode: %d x %s over %d weight copies, 8 x copy_bytes_16 of %d bytes" % (
             args.warmup + args.steps, quant.gemv_kernel_name(Q4_K, 1), head.copies, nbytes))
+        return
+
+    if args.mode == "ceiling":
+        # what the machine gives a trivial kernel under the same timing method: an empty launch, and a
+        # read-only stream over the same rotating weight buffers
+        import ctypes
+        mod = hip.HIPModule.load_builtin()
+        copy_fn, read_fn = mod.function("copy_bytes_16"), mod.function("read_bytes_16")
+        sink = hip.DeviceBuffer(4 * 65536)
+        nul = hip.KernelParams(ctypes.c_uint64(head.w[0].ptr), ctypes.c_uint64(sink.ptr), ctypes.c_uint64(0))
+
+        def empty(i, st):
+            with hip.with_stream(st):
+                hip.launch(copy_fn, 768, 1, 1, 256, 1, 1, nul, "empty")
+        ms, _ = time_steps(hip, stream, empty, args.steps, args.warmup)
+        log("empty_kernel_us=%.3f" % (ms / args.steps * 1e3))
+        for grid in (256, 512, 1024, 2048, 4096, 8192):
+            boxes = [hip.KernelParams(ctypes.c_uint64(b.ptr), ctypes.c_uint64(sink.ptr), ctypes.c_uint64(head.w_bytes))
+                     for b in head.w]
+
+            def rd(i, st, grid=grid, boxes=boxes):
+                with hip.with_stream(st):
+                    hip.launch(read_fn, grid, 1, 1, 256, 1, 1, boxes[i % len(boxes)], "read")
+            ms, _ = time_steps(hip, stream, rd, args.steps, args.warmup)
+            us = ms / args.steps * 1e3
+            log("read_only grid=%d us=%.3f gbps=%.1f" % (grid, us, head.w_bytes / us / 1e3))
         return
 
     # ---- parity spot check of the measured kernel against the oracle, and the CPU baseline ------------

@@ -45,10 +45,12 @@ def dequantize_kernel_name(w_type):
     return n.decode() if n else None
 
 
-def gemv_launch_dims(out_dim):
-    g, b = ctypes.c_uint32(), ctypes.c_uint32()
-    _check(hip.lib().cogni_gemv_launch_dims(out_dim, ctypes.byref(g), ctypes.byref(b)))
-    return g.value, b.value
+def gemv_launch_dims(w_type, tokens, in_dim, out_dim):
+    """(grid_x, block_x, shared_mem_bytes) of the GEMV kernel for this type, token count and shape."""
+    g, b, s = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+    _check(hip.lib().cogni_gemv_launch_dims(int(w_type), tokens, in_dim, out_dim, ctypes.byref(g), ctypes.byref(b),
+                                            ctypes.byref(s)))
+    return g.value, b.value, s.value
 
 
 def dequantize_dev(w_ptr, w_type, n_elements, out_ptr, stream=None):

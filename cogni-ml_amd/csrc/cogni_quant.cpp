@@ -4,6 +4,7 @@
 // (hsaco_blob.S) and loaded with hipModuleLoadData; every launch goes through
 // hipModuleLaunchKernel with the kernel ABI the header documents. There is no host fallback.
 #include "cogni_quant.h"
+#include "kernels/gemv_config.h"
 
 #include <hip/hip_runtime_api.h>
 
@@ -64,11 +65,11 @@ int get_fn(const char* name, hipFunction_t* out) {
   return 0;
 }
 
-int launch(const char* name, uint32_t grid, uint32_t block, void** params, void* stream) {
+int launch(const char* name, uint32_t grid, uint32_t block, uint32_t shmem, void** params, void* stream) {
   hipFunction_t fn = nullptr;
   int rc = get_fn(name, &fn);
   if (rc != 0) return rc;
-  HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, 0, (hipStream_t)stream, params, nullptr),
+  HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, shmem, (hipStream_t)stream, params, nullptr),
           std::string("hipModuleLaunchKernel(") + name + ")");
   return 0;
 }
@@ -176,10 +177,14 @@ const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add) {
   return buf;
 }
 
-int cogni_gemv_launch_dims(uint32_t out_dim, uint32_t* grid_x, uint32_t* block_x) {
-  if (!grid_x || !block_x || out_dim == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_launch_dims: bad argument");
-  *grid_x = (out_dim + 15) / 16;
-  *block_x = 256;
+int cogni_gemv_launch_dims(uint32_t type, uint32_t tokens, uint32_t in_dim, uint32_t out_dim, uint32_t* grid_x,
+                           uint32_t* block_x, uint32_t* shared_mem_bytes) {
+  const int rows = (tokens >= 1 && tokens <= COGNI_MAX_GEMV_TOKENS) ? gemv_rows_per_block(type, (int)tokens) : 0;
+  if (!grid_x || !block_x || !shared_mem_bytes || out_dim == 0 || in_dim == 0 || rows == 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_launch_dims: bad argument");
+  *grid_x = (out_dim + (uint32_t)rows - 1) / (uint32_t)rows;
+  *block_x = GEMV_BLOCK;
+  *shared_mem_bytes = gemv_lds_bytes(type, (int)tokens, in_dim);
   return 0;
 }
 
@@ -237,7 +242,7 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
   if (grid == 0) grid = 1;
   unsigned long long n = n_elements;
   void* params[] = {&w_raw, &out, &n};
-  return launch(name, grid, 256, params, stream);
+  return launch(name, grid, 256, 0, params, stream);
 }
 
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out, uint32_t in_dim,
@@ -248,20 +253,21 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: zero dimension");
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
-  uint32_t grid = 0, block = 0;
-  cogni_gemv_launch_dims(out_dim, &grid, &block);
   for (uint32_t t0 = 0; t0 < tokens; t0 += COGNI_MAX_GEMV_TOKENS) {
-    const uint32_t m = tokens - t0 < COGNI_MAX_GEMV_TOKENS ? tokens - t0 : COGNI_MAX_GEMV_TOKENS;
+    const uint32_t left = tokens - t0, cap = COGNI_MAX_GEMV_TOKENS;
+    const uint32_t m = left < cap ? left : cap;
+    uint32_t grid = 0, block = 0, shmem = 0;
+    cogni_gemv_launch_dims(w_type, m, in_dim, out_dim, &grid, &block, &shmem);
     uint64_t xm = x + (uint64_t)t0 * in_dim * 4, om = out + (uint64_t)t0 * out_dim * 4;
     uint64_t rm = residual ? residual + (uint64_t)t0 * out_dim * 4 : 0;
     const std::string name = cogni_gemv_kernel_name(w_type, m, residual != 0);
     int rc;
     if (residual) {
       void* params[] = {&w_raw, &xm, &rm, &om, &in_dim, &out_dim};
-      rc = launch(name.c_str(), grid, block, params, stream);
+      rc = launch(name.c_str(), grid, block, shmem, params, stream);
     } else {
       void* params[] = {&w_raw, &xm, &om, &in_dim, &out_dim};
-      rc = launch(name.c_str(), grid, block, params, stream);
+      rc = launch(name.c_str(), grid, block, shmem, params, stream);
     }
     if (rc != 0) return rc;
   }

@@ -6,29 +6,30 @@
 //   *_gemv_add_f32        (w_raw, x, residual, out, in_dim, out_dim)           (q4k_gemv_probe.ptx:1572-1578)
 //   *_gemv_f32_tbatchM    same, M tokens: x rows at stride in_dim, out/residual rows at stride out_dim
 //   *_gemv_add_f32_tbatchM
-// Launch: block = 256 threads (4 wavefronts), grid = ceil(out_dim / 16), no dynamic shared memory.
-// w_raw is row-major [out_dim][in_dim/QK][block_bytes]; in_dim must be a multiple of the block size
-// (256 for the K-quants, 32 for Q8_0). Accumulation is fp32.
+// Launch: block = 256 threads (4 wavefronts), grid = ceil(out_dim / rows_per_block), dynamic shared
+// memory = gemv_lds_bytes(type, tokens, in_dim), both from gemv_config.h. w_raw is row-major [out_dim][in_dim/QK][block_bytes];
+// in_dim must be a multiple of 256 for the K-quants (Q8_0 takes any in_dim). Accumulation is fp32.
 //
-// Work split. A wavefront owns GEMV_ROWS consecutive output rows and walks the row in "column sets":
-// the span of blocks one 16-byte-per-lane load instruction covers (Q4_K/Q5_K: 8 lanes per 256-value
-// super-block -> 8 blocks; Q6_K: 4 lanes per block -> 16 blocks; Q8_0: 2 lanes per 32-value block ->
-// 32 blocks). A lane always sits at the same position inside a block, so the activations it needs
-// for a column set are fixed: they are staged once per workgroup into LDS in lane order
-// ([float4 index][lane], conflict-free 16-byte reads), pulled into registers, and reused for all rows
-// of the wavefront. Each weight byte is loaded exactly once, 16 bytes per lane, and the 6-bit
-// scale/min fields are unpacked in registers.
+// Work split. A wavefront owns R consecutive output rows and walks them in "column sets": the span
+// of blocks the 64 lanes cover side by side (Q4_K/Q5_K/Q6_K: 4 lanes per 256-value super-block ->
+// 16 blocks; Q8_0: 2 lanes per 32-value block -> 32 blocks), all loads 16 bytes per lane. A lane always sits at the same position inside a block, so the activations it needs
+// for a column set are fixed: the workgroup stages x into LDS already in lane order
+// ([float4 index][lane]: conflict-free 16-byte reads), each lane pulls its share into registers and
+// reuses it for all R rows. Every weight byte is loaded exactly once, 16 bytes per lane; the loads of
+// column set s+2 are issued while set s is being consumed (two register stages), so a row of up to
+// two column sets is requested in full before the first byte is used.
 //
-// Arithmetic per 32-value sub-block uses sum_j x_j*(d*sc*q_j - dmin*m) = d*sc*sum(q_j x_j) - dmin*m*sum(x_j):
-// the integer codes are converted with v_cvt_f32_ubyte and multiplied into fp32 accumulators; the
-// per-lane sum(x_j) is computed once per column set.
+// Arithmetic. Per 32-value sub-block sum_j x_j*(d*sc*q_j - dmin*m) = d*sc*sum(q_j x_j) - dmin*m*sum(x_j);
+// sum(x_j) is per lane and computed once per column set. The integer codes are not converted to
+// float one by one: a masked pair of codes (two 16-bit halves of a dword, values < 1024) read as two
+// binary16 numbers is exactly code * 2^-24 (a subnormal) or, for codes sitting 4 bits up, code * 2^-20.
+// v_fma_mix_f32 multiplies such a half by an fp32 activation into an fp32 accumulator, subnormals
+// honoured, so a code costs one mask per pair plus one fused multiply-add; the power of two is folded
+// into the block scale.
 #pragma once
 #include "common.cuh"
+#include "gemv_config.h"
 
-#define GEMV_BLOCK 256
-#define GEMV_WAVES (GEMV_BLOCK / WAVE)
-#define GEMV_ROWS 4                           // rows per wavefront
-#define GEMV_ROWS_PER_BLOCK (GEMV_WAVES * GEMV_ROWS)
 
 __device__ __forceinline__ float4 ldx4(const float* p) {
   float4 v;
@@ -37,27 +38,438 @@ __device__ __forceinline__ float4 ldx4(const float* p) {
 }
 __device__ __forceinline__ float hsum4(float4 v) { return (v.x + v.y) + (v.z + v.w); }
 
-template <int B>
-__device__ __forceinline__ float f4c(const float4& v) {
-  return B == 0 ? v.x : (B == 1 ? v.y : (B == 2 ? v.z : v.w));
+// acc + lo16(t) * a + hi16(t) * b with the halves of t read as binary16 (two v_fma_mix_f32)
+__device__ __forceinline__ float mix2(u32 t, float a, float b, float acc) {
+  const __half2 h = *reinterpret_cast<const __half2*>(&t);
+  acc = fmaf(__low2float(h), a, acc);
+  acc = fmaf(__high2float(h), b, acc);
+  return acc;
 }
 
-// acc[mm] += sum_b byte_b(q) * xv[mm].b
-template <int MG, int NF4, int IDX>
-__device__ __forceinline__ void dot4_bytes(u32 q, const float4 (&xr)[MG][NF4], float (&acc)[MG]) {
-  const float f0 = ubyte_f<0>(q), f1 = ubyte_f<1>(q), f2 = ubyte_f<2>(q), f3 = ubyte_f<3>(q);
-#pragma unroll
-  for (int mm = 0; mm < MG; mm++) {
-    acc[mm] = fmaf(f0, xr[mm][IDX].x, acc[mm]);
-    acc[mm] = fmaf(f1, xr[mm][IDX].y, acc[mm]);
-    acc[mm] = fmaf(f2, xr[mm][IDX].z, acc[mm]);
-    acc[mm] = fmaf(f3, xr[mm][IDX].w, acc[mm]);
+#define TWO_P24 16777216.0f
+#define TWO_P20 1048576.0f
+
+// ---------------------------------------------------------------------------------------------
+// Q4_K (144 B: d, dmin, scales[12], qs[128]) and Q5_K (176 B: d, dmin, scales[12], qh[32], ql[128]).
+// Lane = (jb, g): block jb of the column set (16 blocks), 64-value group g of the block: the 32 bytes
+// qs[32g, 32g+32) as two 16-byte loads. Byte l holds element 64g+l (low nibble, sub-block 2g) and
+// element 64g+32+l (high nibble, sub-block 2g+1); Q5_K adds bit 2g / 2g+1 of qh[l]. One (scale, min)
+// pair decode per lane and row serves 64 weights.
+// x registers: float4 i<8 -> low elements 4i..4i+3, i>=8 -> high elements 4(i-8)..
+// ---------------------------------------------------------------------------------------------
+template <bool Q5>
+struct FmtK45 {
+  static constexpr int BB = Q5 ? 176 : 144;
+  static constexpr int QOFF = Q5 ? 48 : 16;
+  static constexpr int BPS = 16;   // blocks per column set
+  static constexpr int NF4 = 16;   // float4 of x per lane per column set and token
+  static constexpr int NSUM = 2;
+  static constexpr int MG_MAX = 2;
+  static constexpr int SPI = 1;   // sets per iteration: a column set is 4096 values
+  static constexpr int rows(int m) { return Q5 ? GEMV_ROWS_Q5K(m) : GEMV_ROWS_Q4K(m); }
+
+  struct Lane {
+    int jb, g;
+    u32 sh, sh2, shm, m1, m2;   // constants of the branch-free 6-bit field decode below
+    bool upper;
+    __device__ __forceinline__ explicit Lane(int lane) : jb(lane >> 2), g(lane & 3) {
+      upper = g >= 2;
+      sh = 16u * (g & 1);
+      sh2 = sh + 2;
+      shm = upper ? sh + 4 : sh;
+      m1 = upper ? 0x0F0Fu : 0x3F3Fu;
+      m2 = upper ? 0x3030u : 0u;
+    }
+  };
+  template <int R>
+  struct Stage {
+    uint4 hdr[R], q0[R], q1[R], h0[R], h1[R];
+  };
+
+  static __device__ __forceinline__ u32 nblocks(u32 in_dim) { return in_dim >> 8; }
+  static __device__ __forceinline__ size_t row_bytes(u32 nb) { return (size_t)nb * BB; }
+  // first element (in the row) of float4 i of lane l in column set `set`
+  static __device__ __forceinline__ u32 x_elem(u32 set, u32 l, u32 i) {
+    return (set * 16 + (l >> 2)) * 256 + (l & 3) * 64 + (i >> 3) * 32 + (i & 7) * 4;
   }
-}
+  static __device__ __forceinline__ float4 load_x(const float* xrow, u32 e, u32 in_dim) {
+    return e < in_dim ? ldx4(xrow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
 
-template <int R, int M, bool ADD>
-__device__ __forceinline__ void gemv_epilogue(float (&acc)[R][M], const float* residual, float* out, u32 row0,
-                                              u32 out_dim, int lane) {
+  template <int R>
+  static __device__ __forceinline__ void load(Stage<R>& st, const uint8_t* const (&rowp)[R], const Lane& ln,
+                                              u32 set, u32 nb) {
+    const u32 off = min(set * 16 + ln.jb, nb - 1) * BB;   // a row is far below 4 GiB
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      st.hdr[r] = ld16(rowp[r] + off);
+      st.q0[r] = ld16(rowp[r] + (off + QOFF + 32 * ln.g));
+      st.q1[r] = ld16(rowp[r] + (off + QOFF + 32 * ln.g + 16));
+      st.h0[r] = Q5 ? ld16(rowp[r] + (off + 16)) : make_uint4(0u, 0u, 0u, 0u);
+      st.h1[r] = Q5 ? ld16(rowp[r] + (off + 32)) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+
+  // contribution of this lane's 64 weights of row r to MG tokens
+  template <int R, int MG>
+  static __device__ __forceinline__ void compute(const Stage<R>& st, int r, const Lane& ln,
+                                                 const float4 (&xr)[MG][NF4], const float (&sx)[MG][NSUM],
+                                                 float (&c)[MG]) {
+    const float d = h2f(st.hdr[r].x), dmin = h2f(st.hdr[r].x >> 16);
+    const float d24 = d * TWO_P24, d20 = d * TWO_P20;
+    // (scale, min) of sub-blocks 2g and 2g+1 as byte pairs (dequant.cr:240-249 for j = 2g, 2g+1 at once):
+    //   g < 2 : sc = s[2g..] & 63,                         m = s[2g+4..] & 63
+    //   g >= 2: sc = (s[2g+4..] & 15) | (s[2g-4..] >> 6 << 4), m = (s[2g+4..] >> 4) | (s[2g..] >> 6 << 4)
+    // with s0/s1/s2 the three dwords of the field, both cases are
+    //   sc = ((P >> sh) & m1) | ((s0 >> (sh+2)) & m2),  m = ((Q >> shm) & m1) | ((s1 >> (sh+2)) & m2)
+    const u32 s0 = st.hdr[r].y, s1 = st.hdr[r].z, s2 = st.hdr[r].w;
+    const u32 P = ln.upper ? s2 : s0, Q = ln.upper ? s2 : s1;
+    const u32 scp = ((P >> ln.sh) & ln.m1) | ((s0 >> ln.sh2) & ln.m2);
+    const u32 mp = ((Q >> ln.shm) & ln.m1) | ((s1 >> ln.sh2) & ln.m2);
+    const float dsl = d24 * ubyte_f<0>(scp), dsh = d20 * ubyte_f<1>(scp);
+    const float dml = dmin * ubyte_f<0>(mp), dmh = dmin * ubyte_f<1>(mp);
+    const u32 qd[8] = {st.q0[r].x, st.q0[r].y, st.q0[r].z, st.q0[r].w, st.q1[r].x, st.q1[r].y, st.q1[r].z, st.q1[r].w};
+    const u32 hd[8] = {st.h0[r].x, st.h0[r].y, st.h0[r].z, st.h0[r].w, st.h1[r].x, st.h1[r].y, st.h1[r].z, st.h1[r].w};
+    u32 t0[8], t1[8], t2[8], t3[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const u32 q = qd[i], q8 = q >> 8;
+      t0[i] = q & 0x000F000Fu;    // low nibbles of bytes 0,2   (x 2^-24)
+      t1[i] = q & 0x00F000F0u;    // high nibbles of bytes 0,2  (x 2^-20)
+      t2[i] = q8 & 0x000F000Fu;   // low nibbles of bytes 1,3
+      t3[i] = q8 & 0x00F000F0u;   // high nibbles of bytes 1,3
+      if (Q5) {
+        const u32 tq = hd[i] >> (2 * ln.g);  // per byte: bit 0 -> 5th bit of the low element, bit 1 -> high element
+        t0[i] |= (tq << 4) & 0x00100010u;
+        t2[i] |= (tq >> 4) & 0x00100010u;
+        t1[i] |= (tq << 7) & 0x01000100u;
+        t3[i] |= (tq >> 1) & 0x01000100u;
+      }
+    }
+#pragma unroll
+    for (int mm = 0; mm < MG; mm++) {
+      float dl0 = 0.0f, dl1 = 0.0f, dh0 = 0.0f, dh1 = 0.0f;   // two chains each to shorten the dependency
+#pragma unroll
+      for (int i = 0; i < 8; i += 2) {
+        dl0 = mix2(t0[i], xr[mm][i].x, xr[mm][i].z, dl0);
+        dl0 = mix2(t2[i], xr[mm][i].y, xr[mm][i].w, dl0);
+        dl1 = mix2(t0[i + 1], xr[mm][i + 1].x, xr[mm][i + 1].z, dl1);
+        dl1 = mix2(t2[i + 1], xr[mm][i + 1].y, xr[mm][i + 1].w, dl1);
+        dh0 = mix2(t1[i], xr[mm][8 + i].x, xr[mm][8 + i].z, dh0);
+        dh0 = mix2(t3[i], xr[mm][8 + i].y, xr[mm][8 + i].w, dh0);
+        dh1 = mix2(t1[i + 1], xr[mm][9 + i].x, xr[mm][9 + i].z, dh1);
+        dh1 = mix2(t3[i + 1], xr[mm][9 + i].y, xr[mm][9 + i].w, dh1);
+      }
+      float v = fmaf(dsl, dl0 + dl1, -(dml * sx[mm][0]));
+      v = fmaf(dsh, dh0 + dh1, v);
+      c[mm] = fmaf(-dmh, sx[mm][1], v);
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Q6_K (210 B: ql[128], qh[64], scales:i8[16], d). Lane = (jb, n, v): block jb of the column set,
+// 128-value half n, 16-byte slice v of the half's 32 "l" positions. With l = 16v+i:
+//   A = ql[64n+l], B = ql[64n+32+l], H = qh[32n+l]
+//   quarter k element 128n + 32k + l  <-  (A&15|H<<4&48, B&15|H<<2&48, A>>4|H&48, B>>4|H>>2&48)[k] - 32
+//   scales sc[8n + v + 2k]
+// x registers: float4 4k+c -> quarter k, l = 16v+4c..+3. Blocks are 2-byte aligned only; the
+// 16-byte loads are issued at their natural addresses.
+// ---------------------------------------------------------------------------------------------
+struct FmtQ6K {
+  static constexpr int BB = 210;
+  static constexpr int BPS = 16;
+  static constexpr int NF4 = 16;
+  static constexpr int NSUM = 4;
+  static constexpr int MG_MAX = 2;
+  static constexpr int SPI = 1;
+  static constexpr int rows(int m) { return GEMV_ROWS_Q6K(m); }
+
+  struct Lane {
+    int jb, n, v;
+    __device__ __forceinline__ explicit Lane(int lane) : jb(lane >> 2), n((lane & 3) >> 1), v(lane & 1) {}
+  };
+  template <int R>
+  struct Stage {
+    uint4 qa[R], qb[R], qh[R];
+    uint2 sc[R];
+    u32 d[R];
+  };
+
+  static __device__ __forceinline__ u32 nblocks(u32 in_dim) { return in_dim >> 8; }
+  static __device__ __forceinline__ size_t row_bytes(u32 nb) { return (size_t)nb * BB; }
+  static __device__ __forceinline__ u32 x_elem(u32 set, u32 l, u32 i) {
+    return (set * 16 + (l >> 2)) * 256 + ((l & 3) >> 1) * 128 + (i >> 2) * 32 + (l & 1) * 16 + (i & 3) * 4;
+  }
+  static __device__ __forceinline__ float4 load_x(const float* xrow, u32 e, u32 in_dim) {
+    return e < in_dim ? ldx4(xrow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void load(Stage<R>& st, const uint8_t* const (&rowp)[R], const Lane& ln,
+                                              u32 set, u32 nb) {
+    const u32 off = min(set * 16 + ln.jb, nb - 1) * BB;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      st.qa[r] = ld16(rowp[r] + (off + 64 * ln.n + 16 * ln.v));
+      st.qb[r] = ld16(rowp[r] + (off + 64 * ln.n + 32 + 16 * ln.v));
+      st.qh[r] = ld16(rowp[r] + (off + 128 + 32 * ln.n + 16 * ln.v));
+      st.sc[r] = ld8(rowp[r] + (off + 192 + 8 * ln.n));
+      st.d[r] = ld2(rowp[r] + (off + 208));
+    }
+  }
+
+  template <int R, int MG>
+  static __device__ __forceinline__ void compute(const Stage<R>& st, int r, const Lane& ln,
+                                                 const float4 (&xr)[MG][NF4], const float (&sx)[MG][NSUM],
+                                                 float (&c)[MG]) {
+    const float d = h2f(st.d[r]);
+    // scale bytes v, v+2, v+4, v+6 of the half's eight
+    const u32 s01 = st.sc[r].x >> (8 * ln.v), s23 = st.sc[r].y >> (8 * ln.v);
+    const float sc0 = d * (float)(int)(signed char)(s01 & 0xFFu);
+    const float sc1 = d * (float)(int)(signed char)((s01 >> 16) & 0xFFu);
+    const float sc2 = d * (float)(int)(signed char)(s23 & 0xFFu);
+    const float sc3 = d * (float)(int)(signed char)((s23 >> 16) & 0xFFu);
+    const u32 a4[4] = {st.qa[r].x, st.qa[r].y, st.qa[r].z, st.qa[r].w};
+    const u32 b4[4] = {st.qb[r].x, st.qb[r].y, st.qb[r].z, st.qb[r].w};
+    const u32 h4[4] = {st.qh[r].x, st.qh[r].y, st.qh[r].z, st.qh[r].w};
+    // 6-bit codes as pairs of binary16 subnormals: [k][c][0] = bytes 0,2, [k][c][1] = bytes 1,3 of dword c
+    u32 q[4][4][2];
+#pragma unroll
+    for (int cc = 0; cc < 4; cc++) {
+      const u32 A = a4[cc], B = b4[cc], H = h4[cc];
+      const u32 A8 = A >> 8, B8 = B >> 8, Hl4 = H << 4, Hr4 = H >> 4, Hl2 = H << 2, Hr6 = H >> 6;
+      q[0][cc][0] = (A & 0x000F000Fu) | (Hl4 & 0x00300030u);
+      q[0][cc][1] = (A8 & 0x000F000Fu) | (Hr4 & 0x00300030u);
+      q[1][cc][0] = (B & 0x000F000Fu) | (Hl2 & 0x00300030u);
+      q[1][cc][1] = (B8 & 0x000F000Fu) | (Hr6 & 0x00300030u);
+      q[2][cc][0] = (A & 0x00F000F0u) | (Hl4 & 0x03000300u);
+      q[2][cc][1] = (A8 & 0x00F000F0u) | (Hr4 & 0x03000300u);
+      q[3][cc][0] = (B & 0x00F000F0u) | (Hl2 & 0x03000300u);
+      q[3][cc][1] = (B8 & 0x00F000F0u) | (Hr6 & 0x03000300u);
+    }
+#pragma unroll
+    for (int mm = 0; mm < MG; mm++) {
+      float dk[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) {
+        float a = 0.0f;
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) {
+          a = mix2(q[k][cc][0], xr[mm][4 * k + cc].x, xr[mm][4 * k + cc].z, a);
+          a = mix2(q[k][cc][1], xr[mm][4 * k + cc].y, xr[mm][4 * k + cc].w, a);
+        }
+        dk[k] = a;
+      }
+      // sum (q-32) x = sum q x - 32 sum x; quarters 0,1 carry 2^-24, quarters 2,3 carry 2^-20
+      float v = sc0 * fmaf(TWO_P24, dk[0], -32.0f * sx[mm][0]);
+      v = fmaf(sc1, fmaf(TWO_P24, dk[1], -32.0f * sx[mm][1]), v);
+      v = fmaf(sc2, fmaf(TWO_P20, dk[2], -32.0f * sx[mm][2]), v);
+      c[mm] = fmaf(sc3, fmaf(TWO_P20, dk[3], -32.0f * sx[mm][3]), v);
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Q8_0 (34 B: d, qs:i8[32]). Lane = (jb, hf): block jb of the column set (32 blocks = 1024 values),
+// 16-byte half hf of its codes. Signed codes are read as unsigned with the top bit flipped:
+// sum q x = sum (q^0x80) x - 128 sum x. in_dim may end inside a block (the tail is clipped).
+// ---------------------------------------------------------------------------------------------
+struct FmtQ80 {
+  static constexpr int BB = 34;
+  static constexpr int BPS = 32;
+  static constexpr int NF4 = 4;
+  static constexpr int NSUM = 1;
+  static constexpr int MG_MAX = 4;
+  static constexpr int SPI = 2;   // sets per iteration: a column set is 1024 values
+  static constexpr int rows(int m) { return GEMV_ROWS_Q80(m); }
+
+  struct Lane {
+    int jb, hf;
+    __device__ __forceinline__ explicit Lane(int lane) : jb(lane >> 1), hf(lane & 1) {}
+  };
+  template <int R>
+  struct Stage {
+    uint4 qs[R];
+    u32 d[R];
+  };
+
+  static __device__ __forceinline__ u32 nblocks(u32 in_dim) { return (in_dim + 31) >> 5; }
+  static __device__ __forceinline__ size_t row_bytes(u32 nb) { return (size_t)nb * BB; }
+  static __device__ __forceinline__ u32 x_elem(u32 set, u32 l, u32 i) {
+    return (set * 32 + (l >> 1)) * 32 + (l & 1) * 16 + i * 4;
+  }
+  static __device__ __forceinline__ float4 load_x(const float* xrow, u32 e, u32 in_dim) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (e + 4 <= in_dim) {
+      v = ldx4(xrow + e);
+    } else {  // clipped tail of the last block
+      if (e + 0 < in_dim) v.x = xrow[e + 0];
+      if (e + 1 < in_dim) v.y = xrow[e + 1];
+      if (e + 2 < in_dim) v.z = xrow[e + 2];
+    }
+    return v;
+  }
+
+  template <int R>
+  static __device__ __forceinline__ void load(Stage<R>& st, const uint8_t* const (&rowp)[R], const Lane& ln,
+                                              u32 set, u32 nb) {
+    const u32 off = min(set * 32 + ln.jb, nb - 1) * BB;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      st.qs[r] = ld16(rowp[r] + (off + 2 + 16 * ln.hf));
+      st.d[r] = ld2(rowp[r] + off);
+    }
+  }
+
+  template <int R, int MG>
+  static __device__ __forceinline__ void compute(const Stage<R>& st, int r, const Lane&,
+                                                 const float4 (&xr)[MG][NF4], const float (&sx)[MG][NSUM],
+                                                 float (&c)[MG]) {
+    const float d24 = h2f(st.d[r]) * TWO_P24, d = h2f(st.d[r]);
+    const u32 qd[4] = {st.qs[r].x ^ 0x80808080u, st.qs[r].y ^ 0x80808080u, st.qs[r].z ^ 0x80808080u,
+                       st.qs[r].w ^ 0x80808080u};
+#pragma unroll
+    for (int mm = 0; mm < MG; mm++) {
+      float a = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        a = mix2(qd[i] & 0x00FF00FFu, xr[mm][i].x, xr[mm][i].z, a);         // bytes 0,2 as code * 2^-24
+        a = mix2((qd[i] >> 8) & 0x00FF00FFu, xr[mm][i].y, xr[mm][i].w, a);  // bytes 1,3
+      }
+      c[mm] = fmaf(d24, a, -128.0f * (d * sx[mm][0]));
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+template <class F, int M, bool ADD>
+__device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                          const float* __restrict__ residual, float* __restrict__ out,
+                                          u32 in_dim, u32 out_dim) {
+  constexpr int R = F::rows(M);
+  constexpr int MG = M < F::MG_MAX ? M : F::MG_MAX;   // tokens held in registers at a time
+  constexpr int NG = (M + MG - 1) / MG;
+  constexpr int NF4 = F::NF4, NSUM = F::NSUM;
+  constexpr int SET_F4 = NF4 * 64;                     // float4 per token and column set
+  extern __shared__ float4 xs[];                       // [token][set in chunk][float4 index][lane]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const typename F::Lane ln(lane);
+  const u32 nb = F::nblocks(in_dim);
+  const u32 ncs = (nb + F::BPS - 1) / F::BPS;
+  // column sets staged in LDS at a time (the host sizes the dynamic LDS with the same formula);
+  // with several token groups each set is staged per group
+  const u32 CH = NG > 1 ? 1u : (u32)gemv_chunk_sets(MG * SET_F4, ncs);
+  const size_t row_bytes = F::row_bytes(nb);
+  const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
+
+  const uint8_t* rowp[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) rowp[r] = w + (size_t)min(row0 + r, out_dim - 1) * row_bytes;
+
+  float acc[R][M];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
+
+  float* xsum = reinterpret_cast<float*>(xs + (size_t)(MG * SET_F4) * CH);   // [token][set in chunk][k][lane]
+  constexpr int FU = 4;                                 // float4 a thread keeps in flight while staging
+  const u32 stage_n = (u32)(MG * SET_F4) * CH;          // float4 staged per chunk and token group
+
+  // Staging of the activations of column sets [s0, s0+CH), token group mg, is split in two so that
+  // the global loads of x can be issued ahead of the weight loads (loads return in order, and x is
+  // needed first): stage_begin issues the first FU loads per thread, stage_end stores them, handles the
+  // rest, and builds the per-lane sums.
+  auto stage_addr = [&](u32 idx, u32 s0, int mg, const float*& xrow, u32& e) -> bool {
+    const u32 l = idx & 63, i = (idx >> 6) % NF4, cm = idx / SET_F4;
+    const u32 cset = s0 + cm % CH, m = mg * MG + cm / CH;
+    xrow = x + (size_t)m * in_dim;
+    e = F::x_elem(cset, l, i);
+    return cset < ncs && m < (u32)M;
+  };
+  auto stage_begin = [&](u32 s0, int mg, float4 (&buf)[FU]) {
+#pragma unroll
+    for (int k = 0; k < FU; k++) {
+      const u32 idx = tid + k * GEMV_BLOCK;
+      const float* xrow;
+      u32 e;
+      buf[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (idx < stage_n && stage_addr(idx, s0, mg, xrow, e)) buf[k] = F::load_x(xrow, e, in_dim);
+    }
+  };
+  auto stage_end = [&](u32 s0, int mg, const float4 (&buf)[FU]) {
+    __syncthreads();   // every wavefront is done with the previous contents
+#pragma unroll
+    for (int k = 0; k < FU; k++) {
+      const u32 idx = tid + k * GEMV_BLOCK;
+      if (idx < stage_n) xs[idx] = buf[k];
+    }
+    for (u32 idx = tid + FU * GEMV_BLOCK; idx < stage_n; idx += GEMV_BLOCK) {
+      const float* xrow;
+      u32 e;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (stage_addr(idx, s0, mg, xrow, e)) v = F::load_x(xrow, e, in_dim);
+      xs[idx] = v;
+    }
+    __syncthreads();
+    // per-lane sums of the staged activations, one per scale group of the lane
+    for (u32 idx = tid; idx < (u32)(MG * NSUM * 64) * CH; idx += GEMV_BLOCK) {
+      const u32 l = idx & 63, k = (idx >> 6) % NSUM, cm = idx / (NSUM * 64);
+      float a = 0.0f;
+#pragma unroll
+      for (int i = 0; i < NF4 / NSUM; i++) a += hsum4(xs[(cm * NF4 + k * (NF4 / NSUM) + i) * 64 + l]);
+      xsum[idx] = a;
+    }
+    __syncthreads();
+  };
+
+  auto step = [&](const typename F::template Stage<R>& st, u32 s) {
+    const bool valid = s * F::BPS + ln.jb < nb;
+#pragma unroll
+    for (int mg = 0; mg < NG; mg++) {
+      if (NG > 1) {   // several token groups share the weight registers: stage each group in turn
+        float4 buf[FU];
+        stage_begin(s, mg, buf);
+        stage_end(s, mg, buf);
+      }
+      float4 xr[MG][NF4];
+      float sx[MG][NSUM];
+#pragma unroll
+      for (int mm = 0; mm < MG; mm++) {
+        const u32 cm = mm * CH + (s % CH);
+#pragma unroll
+        for (int i = 0; i < NF4; i++) xr[mm][i] = xs[(cm * NF4 + i) * 64 + lane];
+#pragma unroll
+        for (int k = 0; k < NSUM; k++) sx[mm][k] = xsum[(cm * NSUM + k) * 64 + lane];
+      }
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        float c[MG];
+        F::template compute<R, MG>(st, r, ln, xr, sx, c);
+#pragma unroll
+        for (int mm = 0; mm < MG; mm++)
+          if (mg * MG + mm < M) acc[r][mg * MG + mm] += valid ? c[mm] : 0.0f;
+      }
+    }
+  };
+
+  // Column sets are taken F::SPI at a time: all their weight loads are issued before the first is consumed.
+  for (u32 s = 0; s < ncs; s += F::SPI) {
+    const bool restage = NG == 1 && (s % CH) == 0;   // CH is a multiple of SPI or covers the whole row
+    float4 buf[FU];
+    if (restage) stage_begin(s, 0, buf);
+    typename F::template Stage<R> stA, stB;
+    F::template load<R>(stA, rowp, ln, s, nb);
+    const bool two = F::SPI == 2 && s + 1 < ncs;
+    if (two) F::template load<R>(stB, rowp, ln, s + 1, nb);
+    if (restage) stage_end(s, 0, buf);
+    step(stA, s);
+    if (two) step(stB, s + 1);
+  }
+
 #pragma unroll
   for (int r = 0; r < R; r++) {
 #pragma unroll
@@ -73,385 +485,40 @@ __device__ __forceinline__ void gemv_epilogue(float (&acc)[R][M], const float* r
   }
 }
 
-// ---------------------------------------------------------------------------------------------
-// Q4_K (144 B: d, dmin, scales[12], qs[128]) and Q5_K (176 B: d, dmin, scales[12], qh[32], ql[128]).
-// Lane = (jb, t): block jb of the column set, 16-byte chunk t of its nibble array. Chunk t = 2g+h
-// holds bytes [16h,16h+16) of group g: low nibbles are elements 64g+16h+i (sub-block 2g), high
-// nibbles are elements 64g+32+16h+i (sub-block 2g+1). Q5_K adds bit 2g / 2g+1 of qh[16h+i].
-// ---------------------------------------------------------------------------------------------
-template <int M, bool Q5, bool ADD>
-__device__ __forceinline__ void k45_gemv(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                         const float* __restrict__ residual, float* __restrict__ out, u32 in_dim,
-                                         u32 out_dim) {
-  constexpr int R = GEMV_ROWS;
-  constexpr int BB = Q5 ? 176 : 144;
-  constexpr int QOFF = Q5 ? 48 : 16;
-  constexpr int MG = M < 4 ? M : 4;          // tokens held in registers at a time
-  constexpr int NG = (M + MG - 1) / MG;
-  __shared__ float4 xs[MG * 8 * 64];          // [token][float4 index][lane]
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int t = lane & 7, jb = lane >> 3, g = t >> 1, h = t & 1;
-  const u32 nb = in_dim >> 8;
-  const u32 ncs = (nb + 7) >> 3;
-  const size_t row_bytes = (size_t)nb * BB;
-  const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
-  const u32 sh = 16u * (g & 1);
-  const bool upper = g >= 2;
-
-  float acc[R][M];
-#pragma unroll
-  for (int r = 0; r < R; r++)
-#pragma unroll
-    for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
-
-  for (u32 cs = 0; cs < ncs; cs++) {
-    const u32 blk = cs * 8 + jb;
-    const bool valid = blk < nb;
-    const u32 blkc = valid ? blk : nb - 1;
-    uint4 hdr[R], qs[R], qh[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      const u32 row = min(row0 + r, out_dim - 1);
-      const uint8_t* bp = w + (size_t)row * row_bytes + (size_t)blkc * BB;
-      hdr[r] = ld16(bp);
-      qs[r] = ld16(bp + QOFF + 16 * t);
-      qh[r] = Q5 ? ld16(bp + 16 + 16 * h) : make_uint4(0u, 0u, 0u, 0u);
-    }
-
-#pragma unroll
-    for (int mg = 0; mg < NG; mg++) {
-      __syncthreads();
-      // stage x of tokens [mg*MG, mg*MG+MG) for this column set, already in lane order
-      for (u32 idx = tid; idx < (u32)(MG * 8 * 64); idx += GEMV_BLOCK) {
-        const u32 l = idx & 63, i = (idx >> 6) & 7, mm = idx >> 9;
-        const u32 m = mg * MG + mm;
-        const u32 b = cs * 8 + (l >> 3);
-        const u32 e = b * 256 + ((l & 7) >> 1) * 64 + (i >> 2) * 32 + (l & 1) * 16 + (i & 3) * 4;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (b < nb && m < (u32)M) v = ldx4(x + (size_t)m * in_dim + e);
-        xs[idx] = v;
-      }
-      __syncthreads();
-
-      float4 xr[MG][8];
-      float sxl[MG], sxh[MG];
-#pragma unroll
-      for (int mm = 0; mm < MG; mm++) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) xr[mm][i] = xs[(mm * 8 + i) * 64 + lane];
-        sxl[mm] = (hsum4(xr[mm][0]) + hsum4(xr[mm][1])) + (hsum4(xr[mm][2]) + hsum4(xr[mm][3]));
-        sxh[mm] = (hsum4(xr[mm][4]) + hsum4(xr[mm][5])) + (hsum4(xr[mm][6]) + hsum4(xr[mm][7]));
-      }
-
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        const float d = h2f(hdr[r].x), dmin = h2f(hdr[r].x >> 16);
-        u32 scp, mp;
-        k4_pair(hdr[r].y, hdr[r].z, hdr[r].w, sh, upper, scp, mp);
-        const float dsl = d * (float)(scp & 0xFFu), dsh = d * (float)(scp >> 8);
-        const float dml = dmin * (float)(mp & 0xFFu), dmh = dmin * (float)(mp >> 8);
-        float dl[MG], dh[MG];
-#pragma unroll
-        for (int mm = 0; mm < MG; mm++) dl[mm] = dh[mm] = 0.0f;
-        const u32 qd[4] = {qs[r].x, qs[r].y, qs[r].z, qs[r].w};
-        const u32 hd[4] = {qh[r].x, qh[r].y, qh[r].z, qh[r].w};
-        u32 lo[4], hi[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          lo[i] = qd[i] & 0x0F0F0F0Fu;
-          hi[i] = (qd[i] >> 4) & 0x0F0F0F0Fu;
-          if (Q5) {
-            const u32 tq = hd[i] >> (2 * g);
-            lo[i] |= (tq << 4) & 0x10101010u;
-            hi[i] |= (tq << 3) & 0x10101010u;
-          }
-        }
-        dot4_bytes<MG, 8, 0>(lo[0], xr, dl);
-        dot4_bytes<MG, 8, 1>(lo[1], xr, dl);
-        dot4_bytes<MG, 8, 2>(lo[2], xr, dl);
-        dot4_bytes<MG, 8, 3>(lo[3], xr, dl);
-        dot4_bytes<MG, 8, 4>(hi[0], xr, dh);
-        dot4_bytes<MG, 8, 5>(hi[1], xr, dh);
-        dot4_bytes<MG, 8, 6>(hi[2], xr, dh);
-        dot4_bytes<MG, 8, 7>(hi[3], xr, dh);
-#pragma unroll
-        for (int mm = 0; mm < MG; mm++) {
-          if (mg * MG + mm < M) {
-            float c = fmaf(dsl, dl[mm], -(dml * sxl[mm]));
-            c = fmaf(dsh, dh[mm], c);
-            c = fmaf(-dmh, sxh[mm], c);
-            acc[r][mg * MG + mm] += valid ? c : 0.0f;
-          }
-        }
-      }
-    }
-  }
-  gemv_epilogue<R, M, ADD>(acc, residual, out, row0, out_dim, lane);
-}
-
-// ---------------------------------------------------------------------------------------------
-// Q6_K (210 B: ql[128], qh[64], scales:i8[16], d). Lane = (jb, n, v): block jb of the column set,
-// 128-value half n, 16-byte slice v of the half's 32 "l" positions. With l = 16v+i:
-//   A = ql[64n+l], B = ql[64n+32+l], H = qh[32n+l]
-//   elements 128n + {0,32,64,96} + l  <-  (A&15|H<<4&48, B&15|H<<2&48, A>>4|H&48, B>>4|H>>2&48) - 32
-//   scales sc[8n + v + {0,2,4,6}]
-// Blocks are 2-byte aligned only; the 16-byte loads are issued at their natural addresses.
-// ---------------------------------------------------------------------------------------------
-template <int M, bool ADD>
-__device__ __forceinline__ void q6k_gemv(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                         const float* __restrict__ residual, float* __restrict__ out, u32 in_dim,
-                                         u32 out_dim) {
-  constexpr int R = GEMV_ROWS;
-  constexpr int MG = M < 2 ? M : 2;
-  constexpr int NG = (M + MG - 1) / MG;
-  __shared__ float4 xs[MG * 16 * 64];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int s = lane & 3, jb = lane >> 2, n = s >> 1, v = s & 1;
-  const u32 nb = in_dim >> 8;
-  const u32 ncs = (nb + 15) >> 4;
-  const size_t row_bytes = (size_t)nb * 210;
-  const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
-
-  float acc[R][M];
-#pragma unroll
-  for (int r = 0; r < R; r++)
-#pragma unroll
-    for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
-
-  for (u32 cs = 0; cs < ncs; cs++) {
-    const u32 blk = cs * 16 + jb;
-    const bool valid = blk < nb;
-    const u32 blkc = valid ? blk : nb - 1;
-    uint4 qa[R], qb[R], qh[R];
-    uint2 scb[R];
-    u32 db[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      const u32 row = min(row0 + r, out_dim - 1);
-      const uint8_t* bp = w + (size_t)row * row_bytes + (size_t)blkc * 210;
-      qa[r] = ld16(bp + 64 * n + 16 * v);
-      qb[r] = ld16(bp + 64 * n + 32 + 16 * v);
-      qh[r] = ld16(bp + 128 + 32 * n + 16 * v);
-      scb[r] = ld8(bp + 192 + 8 * n);
-      db[r] = ld2(bp + 208);
-    }
-
-#pragma unroll
-    for (int mg = 0; mg < NG; mg++) {
-      __syncthreads();
-      // float4 index i = 4*quarter + c: elements 128n + 32*quarter + 16v + 4c .. +3
-      for (u32 idx = tid; idx < (u32)(MG * 16 * 64); idx += GEMV_BLOCK) {
-        const u32 l = idx & 63, i = (idx >> 6) & 15, mm = idx >> 10;
-        const u32 m = mg * MG + mm;
-        const u32 b = cs * 16 + (l >> 2);
-        const u32 e = b * 256 + ((l & 3) >> 1) * 128 + (i >> 2) * 32 + (l & 1) * 16 + (i & 3) * 4;
-        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (b < nb && m < (u32)M) val = ldx4(x + (size_t)m * in_dim + e);
-        xs[idx] = val;
-      }
-      __syncthreads();
-
-      float4 xr[MG][16];
-      float sx[MG][4];
-#pragma unroll
-      for (int mm = 0; mm < MG; mm++) {
-#pragma unroll
-        for (int i = 0; i < 16; i++) xr[mm][i] = xs[(mm * 16 + i) * 64 + lane];
-#pragma unroll
-        for (int k = 0; k < 4; k++)
-          sx[mm][k] = (hsum4(xr[mm][4 * k]) + hsum4(xr[mm][4 * k + 1])) +
-                      (hsum4(xr[mm][4 * k + 2]) + hsum4(xr[mm][4 * k + 3]));
-      }
-
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        const float d = h2f(db[r]);
-        // scale bytes v, v+2, v+4, v+6 of the half's 8
-        const u32 s01 = scb[r].x >> (8 * v), s23 = scb[r].y >> (8 * v);
-        const float sc0 = d * (float)(int)(signed char)(s01 & 0xFFu);
-        const float sc1 = d * (float)(int)(signed char)((s01 >> 16) & 0xFFu);
-        const float sc2 = d * (float)(int)(signed char)(s23 & 0xFFu);
-        const float sc3 = d * (float)(int)(signed char)((s23 >> 16) & 0xFFu);
-        const u32 a4[4] = {qa[r].x, qa[r].y, qa[r].z, qa[r].w};
-        const u32 b4[4] = {qb[r].x, qb[r].y, qb[r].z, qb[r].w};
-        const u32 h4[4] = {qh[r].x, qh[r].y, qh[r].z, qh[r].w};
-        float d0[MG], d1[MG], d2[MG], d3[MG];
-#pragma unroll
-        for (int mm = 0; mm < MG; mm++) d0[mm] = d1[mm] = d2[mm] = d3[mm] = 0.0f;
-        u32 q0[4], q1[4], q2[4], q3[4];
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-          q0[c] = (a4[c] & 0x0F0F0F0Fu) | ((h4[c] << 4) & 0x30303030u);
-          q1[c] = (b4[c] & 0x0F0F0F0Fu) | ((h4[c] << 2) & 0x30303030u);
-          q2[c] = ((a4[c] >> 4) & 0x0F0F0F0Fu) | (h4[c] & 0x30303030u);
-          q3[c] = ((b4[c] >> 4) & 0x0F0F0F0Fu) | ((h4[c] >> 2) & 0x30303030u);
-        }
-        dot4_bytes<MG, 16, 0>(q0[0], xr, d0);
-        dot4_bytes<MG, 16, 1>(q0[1], xr, d0);
-        dot4_bytes<MG, 16, 2>(q0[2], xr, d0);
-        dot4_bytes<MG, 16, 3>(q0[3], xr, d0);
-        dot4_bytes<MG, 16, 4>(q1[0], xr, d1);
-        dot4_bytes<MG, 16, 5>(q1[1], xr, d1);
-        dot4_bytes<MG, 16, 6>(q1[2], xr, d1);
-        dot4_bytes<MG, 16, 7>(q1[3], xr, d1);
-        dot4_bytes<MG, 16, 8>(q2[0], xr, d2);
-        dot4_bytes<MG, 16, 9>(q2[1], xr, d2);
-        dot4_bytes<MG, 16, 10>(q2[2], xr, d2);
-        dot4_bytes<MG, 16, 11>(q2[3], xr, d2);
-        dot4_bytes<MG, 16, 12>(q3[0], xr, d3);
-        dot4_bytes<MG, 16, 13>(q3[1], xr, d3);
-        dot4_bytes<MG, 16, 14>(q3[2], xr, d3);
-        dot4_bytes<MG, 16, 15>(q3[3], xr, d3);
-#pragma unroll
-        for (int mm = 0; mm < MG; mm++) {
-          if (mg * MG + mm < M) {
-            // sum (q-32) x = sum q x - 32 sum x
-            float c = sc0 * fmaf(-32.0f, sx[mm][0], d0[mm]);
-            c = fmaf(sc1, fmaf(-32.0f, sx[mm][1], d1[mm]), c);
-            c = fmaf(sc2, fmaf(-32.0f, sx[mm][2], d2[mm]), c);
-            c = fmaf(sc3, fmaf(-32.0f, sx[mm][3], d3[mm]), c);
-            acc[r][mg * MG + mm] += valid ? c : 0.0f;
-          }
-        }
-      }
-    }
-  }
-  gemv_epilogue<R, M, ADD>(acc, residual, out, row0, out_dim, lane);
-}
-
-// ---------------------------------------------------------------------------------------------
-// Q8_0 (34 B: d, qs:i8[32]). Lane = (jb, hf): block jb of the column set (32 blocks = 1024 values),
-// 16-byte half hf of its codes. Signed codes are read as unsigned with the top bit flipped:
-// sum q x = sum (q^0x80) x - 128 sum x. in_dim may end inside a block (the tail is clipped).
-// ---------------------------------------------------------------------------------------------
-template <int M, bool ADD>
-__device__ __forceinline__ void q80_gemv(const uint8_t* __restrict__ w, const float* __restrict__ x,
-                                         const float* __restrict__ residual, float* __restrict__ out, u32 in_dim,
-                                         u32 out_dim) {
-  constexpr int R = GEMV_ROWS;
-  constexpr int MG = M < 4 ? M : 4;
-  constexpr int NG = (M + MG - 1) / MG;
-  __shared__ float4 xs[MG * 4 * 64];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int hf = lane & 1, jb = lane >> 1;
-  const u32 nb = (in_dim + 31) >> 5;
-  const u32 ncs = (nb + 31) >> 5;
-  const size_t row_bytes = (size_t)nb * 34;
-  const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
-
-  float acc[R][M];
-#pragma unroll
-  for (int r = 0; r < R; r++)
-#pragma unroll
-    for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
-
-  for (u32 cs = 0; cs < ncs; cs++) {
-    const u32 blk = cs * 32 + jb;
-    const bool valid = blk < nb;
-    const u32 blkc = valid ? blk : nb - 1;
-    uint4 qs[R];
-    u32 db[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      const u32 row = min(row0 + r, out_dim - 1);
-      const uint8_t* bp = w + (size_t)row * row_bytes + (size_t)blkc * 34;
-      qs[r] = ld16(bp + 2 + 16 * hf);
-      db[r] = ld2(bp);
-    }
-
-#pragma unroll
-    for (int mg = 0; mg < NG; mg++) {
-      __syncthreads();
-      for (u32 idx = tid; idx < (u32)(MG * 4 * 64); idx += GEMV_BLOCK) {
-        const u32 l = idx & 63, i = (idx >> 6) & 3, mm = idx >> 8;
-        const u32 m = mg * MG + mm;
-        const u32 e = (cs * 32 + (l >> 1)) * 32 + (l & 1) * 16 + i * 4;
-        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (m < (u32)M) {
-          const float* xp = x + (size_t)m * in_dim;
-          if (e + 4 <= in_dim) {
-            val = ldx4(xp + e);
-          } else {                      // clipped tail of the last block
-            if (e + 0 < in_dim) val.x = xp[e + 0];
-            if (e + 1 < in_dim) val.y = xp[e + 1];
-            if (e + 2 < in_dim) val.z = xp[e + 2];
-          }
-        }
-        xs[idx] = val;
-      }
-      __syncthreads();
-
-      float4 xr[MG][4];
-      float sx[MG];
-#pragma unroll
-      for (int mm = 0; mm < MG; mm++) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) xr[mm][i] = xs[(mm * 4 + i) * 64 + lane];
-        sx[mm] = (hsum4(xr[mm][0]) + hsum4(xr[mm][1])) + (hsum4(xr[mm][2]) + hsum4(xr[mm][3]));
-      }
-
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        const float d = h2f(db[r]);
-        float dt[MG];
-#pragma unroll
-        for (int mm = 0; mm < MG; mm++) dt[mm] = 0.0f;
-        dot4_bytes<MG, 4, 0>(qs[r].x ^ 0x80808080u, xr, dt);
-        dot4_bytes<MG, 4, 1>(qs[r].y ^ 0x80808080u, xr, dt);
-        dot4_bytes<MG, 4, 2>(qs[r].z ^ 0x80808080u, xr, dt);
-        dot4_bytes<MG, 4, 3>(qs[r].w ^ 0x80808080u, xr, dt);
-#pragma unroll
-        for (int mm = 0; mm < MG; mm++) {
-          if (mg * MG + mm < M) {
-            const float c = d * fmaf(-128.0f, sx[mm], dt[mm]);
-            acc[r][mg * MG + mm] += valid ? c : 0.0f;
-          }
-        }
-      }
-    }
-  }
-  gemv_epilogue<R, M, ADD>(acc, residual, out, row0, out_dim, lane);
-}
-
 // ---- entry points ---------------------------------------------------------------------------
-#define GEMV_ENTRY(NAME, BODY, M)                                                                                  \
-  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) void NAME(const uint8_t* w, const float* x, float* out,      \
-                                                                 u32 in_dim, u32 out_dim) {                        \
-    BODY(M, false)(w, x, nullptr, out, in_dim, out_dim);                                                          \
+#define GEMV_ENTRY(NAME, FMT, M)                                                                                \
+  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) void NAME(const uint8_t* w, const float* x, float* out,   \
+                                                                 u32 in_dim, u32 out_dim) {                     \
+    gemv_core<FMT, M, false>(w, x, nullptr, out, in_dim, out_dim);                                              \
   }
-#define GEMV_ADD_ENTRY(NAME, BODY, M)                                                                              \
-  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) void NAME(const uint8_t* w, const float* x,                  \
-                                                                 const float* residual, float* out, u32 in_dim,    \
-                                                                 u32 out_dim) {                                    \
-    BODY(M, true)(w, x, residual, out, in_dim, out_dim);                                                          \
+#define GEMV_ADD_ENTRY(NAME, FMT, M)                                                                            \
+  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) void NAME(const uint8_t* w, const float* x,               \
+                                                                 const float* residual, float* out, u32 in_dim, \
+                                                                 u32 out_dim) {                                 \
+    gemv_core<FMT, M, true>(w, x, residual, out, in_dim, out_dim);                                              \
   }
-#define BODY_Q4K(M, ADD) k45_gemv<M, false, ADD>
-#define BODY_Q5K(M, ADD) k45_gemv<M, true, ADD>
-#define BODY_Q6K(M, ADD) q6k_gemv<M, ADD>
-#define BODY_Q80(M, ADD) q80_gemv<M, ADD>
 
-#define GEMV_FAMILY(PFX, BODY)                        \
-  GEMV_ENTRY(PFX##_gemv_f32, BODY, 1)                 \
-  GEMV_ENTRY(PFX##_gemv_f32_tbatch2, BODY, 2)         \
-  GEMV_ENTRY(PFX##_gemv_f32_tbatch3, BODY, 3)         \
-  GEMV_ENTRY(PFX##_gemv_f32_tbatch4, BODY, 4)         \
-  GEMV_ENTRY(PFX##_gemv_f32_tbatch5, BODY, 5)         \
-  GEMV_ENTRY(PFX##_gemv_f32_tbatch6, BODY, 6)         \
-  GEMV_ENTRY(PFX##_gemv_f32_tbatch7, BODY, 7)         \
-  GEMV_ENTRY(PFX##_gemv_f32_tbatch8, BODY, 8)         \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32, BODY, 1)         \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch2, BODY, 2) \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch3, BODY, 3) \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch4, BODY, 4) \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch5, BODY, 5) \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch6, BODY, 6) \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch7, BODY, 7) \
-  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch8, BODY, 8)
+#define GEMV_FAMILY(PFX, FMT)                        \
+  GEMV_ENTRY(PFX##_gemv_f32, FMT, 1)                 \
+  GEMV_ENTRY(PFX##_gemv_f32_tbatch2, FMT, 2)         \
+  GEMV_ENTRY(PFX##_gemv_f32_tbatch3, FMT, 3)         \
+  GEMV_ENTRY(PFX##_gemv_f32_tbatch4, FMT, 4)         \
+  GEMV_ENTRY(PFX##_gemv_f32_tbatch5, FMT, 5)         \
+  GEMV_ENTRY(PFX##_gemv_f32_tbatch6, FMT, 6)         \
+  GEMV_ENTRY(PFX##_gemv_f32_tbatch7, FMT, 7)         \
+  GEMV_ENTRY(PFX##_gemv_f32_tbatch8, FMT, 8)         \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32, FMT, 1)         \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch2, FMT, 2) \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch3, FMT, 3) \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch4, FMT, 4) \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch5, FMT, 5) \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch6, FMT, 6) \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch7, FMT, 7) \
+  GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch8, FMT, 8)
 
-GEMV_FAMILY(q4_k, BODY_Q4K)
-GEMV_FAMILY(q5_k, BODY_Q5K)
-GEMV_FAMILY(q6_k, BODY_Q6K)
-GEMV_FAMILY(q8_0, BODY_Q80)
+typedef FmtK45<false> FmtQ4K;
+typedef FmtK45<true> FmtQ5K;
+GEMV_FAMILY(q4_k, FmtQ4K)
+GEMV_FAMILY(q5_k, FmtQ5K)
+GEMV_FAMILY(q6_k, FmtQ6K)
+GEMV_FAMILY(q8_0, FmtQ80)

@@ -11,7 +11,7 @@
  * Three levels, lowest first:
  *   1. the code object: kernels are unmangled symbols, launched by name through
  *      ml_hip_driver.h exactly as the reference launches PTX entries
- *      (cogni_quant_code_object, cogni_kernel_name, cogni_gemv_grid);
+ *      (cogni_quant_code_object, cogni_gemv_kernel_name, cogni_gemv_launch_dims);
  *   2. device-pointer operators, asynchronous on a stream (cogni_*_dev);
  *   3. host-buffer operators with the reference's CPU signatures (cogni_dequantize,
  *      cogni_matmul_add) and the QuantWeight handle that keeps weights resident.
@@ -70,10 +70,14 @@ int cogni_quant_code_object(const void** image, size_t* size);
  * x rows at stride in_dim floats, out/residual rows at stride out_dim floats (q4k_gemv_probe.ptx:747-768).
  * Returns NULL for an unsupported combination. No GPU needed. */
 const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add);
-/* Launch geometry of every GEMV kernel: block = 256 threads, grid_x = ceil(out_dim / 16), no dynamic
- * shared memory. (The reference's kernels use grid ceil(out_dim/4) x block 128,
- * bin/cuda_q4k_gemv_probe.cr:225-230.) */
-int cogni_gemv_launch_dims(uint32_t out_dim, uint32_t* grid_x, uint32_t* block_x);
+/* Launch geometry of the GEMV kernel for (type, tokens) at this shape: block_x = 256 threads, grid_x =
+ * ceil(out_dim / rows_per_block) where rows_per_block depends on the type and token count, all other
+ * grid/block extents 1, and shared_mem_bytes of dynamic shared memory (the staged activations), which
+ * goes into the shared_mem_bytes argument of the launch (driver.cr:278-286). (The reference's kernels
+ * use grid ceil(out_dim/4) x block 128 and no dynamic shared memory, bin/cuda_q4k_gemv_probe.cr:225-230.)
+ * No GPU needed. */
+int cogni_gemv_launch_dims(uint32_t type, uint32_t tokens, uint32_t in_dim, uint32_t out_dim, uint32_t* grid_x,
+                           uint32_t* block_x, uint32_t* shared_mem_bytes);
 /* Kernel symbol "dequantize_<type>_f32"; parameters (w_raw:u64, out:u64, n_elements:u64); block = 256
  * threads, any grid (grid-stride). NULL for an unsupported type. No GPU needed. */
 const char* cogni_dequantize_kernel_name(uint32_t type);
@@ -94,8 +98,8 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 /* Decode GEMV, weights read once for all tokens:
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
  * fp32 accumulation. tokens >= 1; more than COGNI_MAX_GEMV_TOKENS are issued as consecutive launches
- * of up to 8 tokens. in_dim must be a multiple of 256 (Q4_K/Q5_K/Q6_K; the reference requires the
- * same, bin/cuda_q4k_gemv_probe.cr:125) or of 32... Q8_0 accepts any in_dim >= 1 (its last block is clipped,
+ * of up to 8 tokens. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
+ * same, bin/cuda_q4k_gemv_probe.cr:125); Q8_0 accepts any in_dim >= 1 (its last block is clipped,
  * quant_matmul.cr:241,259). Types: Q8_0, Q4_K, Q5_K, Q6_K. */
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
                    uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);

@@ -64,8 +64,21 @@ def test_code_object_is_amdgpu_elf_with_kernel_symbols():
 
 
 def test_gemv_launch_dims():
-    assert quant.gemv_launch_dims(12288) == (768, 256)
-    assert quant.gemv_launch_dims(17) == (2, 256)
+    for t in (8, 12, 13, 14):
+        for m in range(1, 9):
+            grid, block, lds = quant.gemv_launch_dims(t, m, 4096, 12288)
+            assert block == 256 and 12288 % grid == 0 and 4 <= 12288 // grid <= 32
+            assert 0 < lds <= 49152 and lds % 256 == 0
+    # M = 1: the whole activation vector (plus 1/16 of it for the per-lane sums) is staged once when it fits
+    assert quant.gemv_launch_dims(12, 1, 4096, 12288)[2] == 4096 * 4 * 17 // 16
+    assert quant.gemv_launch_dims(12, 1, 8192, 4096)[2] == 8192 * 4 * 17 // 16
+    assert quant.gemv_launch_dims(12, 1, 65536, 4096)[2] <= 49152
+    g1 = quant.gemv_launch_dims(12, 1, 256, 17)[0]
+    assert g1 == -(-17 // (12288 // quant.gemv_launch_dims(12, 1, 4096, 12288)[0]))
+    with pytest.raises(quant.QuantError):
+        quant.gemv_launch_dims(20, 1, 256, 16)
+    with pytest.raises(quant.QuantError):
+        quant.gemv_launch_dims(12, 9, 256, 16)
 
 
 def test_argument_errors_do_not_need_a_gpu():
