@@ -130,36 +130,34 @@ struct FmtK45 {
     const float dml = dmin * ubyte_f<0>(mp), dmh = dmin * ubyte_f<1>(mp);
     const u32 qd[8] = {st.q0[r].x, st.q0[r].y, st.q0[r].z, st.q0[r].w, st.q1[r].x, st.q1[r].y, st.q1[r].z, st.q1[r].w};
     const u32 hd[8] = {st.h0[r].x, st.h0[r].y, st.h0[r].z, st.h0[r].w, st.h1[r].x, st.h1[r].y, st.h1[r].z, st.h1[r].w};
-    u32 t0[8], t1[8], t2[8], t3[8];
+    float dl[MG][2], dh[MG][2];   // two chains each to shorten the dependency
+#pragma unroll
+    for (int mm = 0; mm < MG; mm++) dl[mm][0] = dl[mm][1] = dh[mm][0] = dh[mm][1] = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
       const u32 q = qd[i], q8 = q >> 8;
-      t0[i] = q & 0x000F000Fu;    // low nibbles of bytes 0,2   (x 2^-24)
-      t1[i] = q & 0x00F000F0u;    // high nibbles of bytes 0,2  (x 2^-20)
-      t2[i] = q8 & 0x000F000Fu;   // low nibbles of bytes 1,3
-      t3[i] = q8 & 0x00F000F0u;   // high nibbles of bytes 1,3
+      u32 t0 = q & 0x000F000Fu;    // low nibbles of bytes 0,2   (x 2^-24)
+      u32 t1 = q & 0x00F000F0u;    // high nibbles of bytes 0,2  (x 2^-20)
+      u32 t2 = q8 & 0x000F000Fu;   // low nibbles of bytes 1,3
+      u32 t3 = q8 & 0x00F000F0u;   // high nibbles of bytes 1,3
       if (Q5) {
         const u32 tq = hd[i] >> (2 * ln.g);  // per byte: bit 0 -> 5th bit of the low element, bit 1 -> high element
-        t0[i] |= (tq << 4) & 0x00100010u;
-        t2[i] |= (tq >> 4) & 0x00100010u;
-        t1[i] |= (tq << 7) & 0x01000100u;
-        t3[i] |= (tq >> 1) & 0x01000100u;
+        t0 |= (tq << 4) & 0x00100010u;
+        t2 |= (tq >> 4) & 0x00100010u;
+        t1 |= (tq << 7) & 0x01000100u;
+        t3 |= (tq >> 1) & 0x01000100u;
+      }
+#pragma unroll
+      for (int mm = 0; mm < MG; mm++) {
+        dl[mm][i & 1] = mix2(t0, xr[mm][i].x, xr[mm][i].z, dl[mm][i & 1]);
+        dl[mm][i & 1] = mix2(t2, xr[mm][i].y, xr[mm][i].w, dl[mm][i & 1]);
+        dh[mm][i & 1] = mix2(t1, xr[mm][8 + i].x, xr[mm][8 + i].z, dh[mm][i & 1]);
+        dh[mm][i & 1] = mix2(t3, xr[mm][8 + i].y, xr[mm][8 + i].w, dh[mm][i & 1]);
       }
     }
 #pragma unroll
     for (int mm = 0; mm < MG; mm++) {
-      float dl0 = 0.0f, dl1 = 0.0f, dh0 = 0.0f, dh1 = 0.0f;   // two chains each to shorten the dependency
-#pragma unroll
-      for (int i = 0; i < 8; i += 2) {
-        dl0 = mix2(t0[i], xr[mm][i].x, xr[mm][i].z, dl0);
-        dl0 = mix2(t2[i], xr[mm][i].y, xr[mm][i].w, dl0);
-        dl1 = mix2(t0[i + 1], xr[mm][i + 1].x, xr[mm][i + 1].z, dl1);
-        dl1 = mix2(t2[i + 1], xr[mm][i + 1].y, xr[mm][i + 1].w, dl1);
-        dh0 = mix2(t1[i], xr[mm][8 + i].x, xr[mm][8 + i].z, dh0);
-        dh0 = mix2(t3[i], xr[mm][8 + i].y, xr[mm][8 + i].w, dh0);
-        dh1 = mix2(t1[i + 1], xr[mm][9 + i].x, xr[mm][9 + i].z, dh1);
-        dh1 = mix2(t3[i + 1], xr[mm][9 + i].y, xr[mm][9 + i].w, dh1);
-      }
+      const float dl0 = dl[mm][0], dl1 = dl[mm][1], dh0 = dh[mm][0], dh1 = dh[mm][1];
       float v = fmaf(dsl, dl0 + dl1, -(dml * sx[mm][0]));
       v = fmaf(dsh, dh0 + dh1, v);
       c[mm] = fmaf(-dmh, sx[mm][1], v);
@@ -486,13 +484,15 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
 }
 
 // ---- entry points ---------------------------------------------------------------------------
+// M = 1, 2: ask for at least 3 wavefronts per SIMD so a 12288-row matrix is resident in one round
+#define GEMV_OCC(M) __attribute__((amdgpu_waves_per_eu((M) <= 1 ? 3 : 1)))
 #define GEMV_ENTRY(NAME, FMT, M)                                                                                \
-  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) void NAME(const uint8_t* w, const float* x, float* out,   \
+  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(M) void NAME(const uint8_t* w, const float* x, float* out,   \
                                                                  u32 in_dim, u32 out_dim) {                     \
     gemv_core<FMT, M, false>(w, x, nullptr, out, in_dim, out_dim);                                              \
   }
 #define GEMV_ADD_ENTRY(NAME, FMT, M)                                                                            \
-  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) void NAME(const uint8_t* w, const float* x,               \
+  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(M) void NAME(const uint8_t* w, const float* x,               \
                                                                  const float* residual, float* out, u32 in_dim, \
                                                                  u32 out_dim) {                                 \
     gemv_core<FMT, M, true>(w, x, residual, out, in_dim, out_dim);                                              \

@@ -6,7 +6,7 @@
 #define GEMV_WAVES 4
 
 #define GEMV_ROWS_Q4K(M) ((M) <= 2 ? 4 : 2)
-#define GEMV_ROWS_Q5K(M) ((M) <= 2 ? 4 : 2)
+#define GEMV_ROWS_Q5K(M) 2
 #define GEMV_ROWS_Q6K(M) 2
 #define GEMV_ROWS_Q80(M) 4
 
