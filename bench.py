@@ -27,6 +27,7 @@ for p in (ROOT, os.path.join(ROOT, "cogni-ml_amd")):
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 matrix peak, published
 LLC_BYTES = 256 << 20           # last-level (Infinity) cache
 Q4_K, Q5_K, Q6_K, Q8_0 = 12, 13, 14, 8
 TYPE_NAME = {Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", Q8_0: "Q8_0"}
@@ -117,6 +118,25 @@ def time_steps(hip, stream, launch, steps, warmup):
     e0.close()
     e1.close()
     return ms, exe is not None
+
+
+def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, warmup):
+    """Q4_K prefill GEMM (x repack + MFMA kernel) at `tokens`; returns (ms per call, TFLOP/s)."""
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens)
+    bufs = [hip.DeviceBuffer(n) for n in (raw.nbytes, x.nbytes, 4 * tokens * out_dim, wsb)]
+    hip.copy_htod(bufs[0].ptr, raw, raw.nbytes, "w")
+    hip.copy_htod(bufs[1].ptr, x, x.nbytes, "x")
+
+    def launch(i, st):
+        quant.gemm_dev(bufs[0].ptr, Q4_K, bufs[1].ptr, bufs[2].ptr, in_dim, out_dim, tokens, bufs[3].ptr, wsb, 0,
+                       st.handle)
+    ms, _ = time_steps(hip, stream, launch, steps, warmup)
+    for b in bufs:
+        b.close()
+    per = ms / steps
+    return per, 2.0 * tokens * out_dim * in_dim / (per * 1e-3) / 1e12
 
 
 def cpu_baseline(oracle, case, budget_s=10.0):
@@ -229,6 +249,14 @@ def main():
             head.in_dim, head.out_dim, head.w_bytes, head.copies, args.steps, args.warmup, ms_per_step,
             cpu_s / cpu_reps * 1e3, cos, max_diff, str(ok).lower(), gbps, hot_gbps, graphed))
 
+    gemm = {}
+    for tokens in ((64, 512, 2048) if args.mode == "cases" else (512,)):
+        gsteps = max(10, min(200, args.steps // 10))
+        per, tf = bench_gemm(hip, quant, synth, rng, stream, tokens, 12288, 4096, gsteps, 5)
+        gemm["M=%d" % tokens] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
+            tokens, gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
+
     extra = {}
     if args.mode == "cases":
         table = [
@@ -267,6 +295,7 @@ def main():
         },
         "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "cache_hot_gbps": round(hot_gbps, 1),
+        "prefill_gemm_q4k_12288x4096": gemm,
         "parity": {"cos": round(cos, 8), "max_diff": max_diff, "ok": ok, "tol_1e-4_x_wmax": 1e-4 * float(np.linalg.norm(head.host_x)) * dense_max},
         "roofline": {
             "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

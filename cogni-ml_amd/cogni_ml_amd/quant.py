@@ -64,6 +64,37 @@ def gemv_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens=1, residual_
                                     ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+def gemm_workspace_bytes(w_type, in_dim, tokens):
+    f = hip.lib().cogni_gemm_workspace_bytes
+    f.restype = ctypes.c_size_t
+    return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens))
+
+
+def gemm_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_ptr, workspace_bytes, bias_ptr=0,
+             stream=None):
+    _check(hip.lib().cogni_gemm_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(x_ptr),
+                                    ctypes.c_uint64(bias_ptr), ctypes.c_uint64(out_ptr), ctypes.c_uint32(in_dim),
+                                    ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), ctypes.c_uint64(workspace_ptr),
+                                    ctypes.c_size_t(workspace_bytes), stream))
+
+
+def matmul_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_ptr=0, workspace_bytes=0, bias_ptr=0,
+               stream=None):
+    """The GEMV/GEMM router (tokens > threshold and Q4_K -> GEMM)."""
+    _check(hip.lib().cogni_matmul_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(x_ptr),
+                                      ctypes.c_uint64(bias_ptr), ctypes.c_uint64(out_ptr), ctypes.c_uint32(in_dim),
+                                      ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens),
+                                      ctypes.c_uint64(workspace_ptr), ctypes.c_size_t(workspace_bytes), stream))
+
+
+def set_gemm_threshold(tokens):
+    _check(hip.lib().cogni_set_gemm_threshold(ctypes.c_int32(tokens)))
+
+
+def get_gemm_threshold():
+    return hip.lib().cogni_get_gemm_threshold()
+
+
 def dequantize(data, w_type, n_elements):
     """Dequant.dequantize: raw bytes -> float32[n_elements], computed on the GPU."""
     d = np.ascontiguousarray(np.frombuffer(data, dtype=np.uint8) if not isinstance(data, np.ndarray) else data,

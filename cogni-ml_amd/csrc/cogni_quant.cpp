@@ -9,6 +9,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -274,6 +275,65 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   return 0;
 }
 
+int g_gemm_threshold = -1;   // -1: not resolved yet
+
+size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {
+  if (w_type != COGNI_TYPE_Q4_K || in_dim == 0 || tokens == 0) return 0;
+  const size_t mtiles = ((size_t)tokens + 127) / 128;
+  return mtiles * 128 * (size_t)in_dim * 2;
+}
+
+int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
+                   uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream) {
+  if (w_type != COGNI_TYPE_Q4_K)
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the prefill GEMM: ") + type_name(w_type));
+  if (!w_raw || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: null device pointer");
+  if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: zero dimension");
+  if ((in_dim % 256) != 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "Q4_K GEMM requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  const size_t need = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
+  if (!workspace || workspace_bytes < need)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: workspace has " + std::to_string(workspace_bytes) + " bytes, needs " + std::to_string(need));
+  const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 191) / 192;
+  {
+    const uint64_t pieces = (uint64_t)need / 16;
+    uint64_t g = (pieces + 255) / 256;
+    uint32_t grid = (uint32_t)(g < 16384 ? g : 16384);
+    void* params[] = {&x, &workspace, &tokens, &in_dim};
+    int rc = launch("pack_x_f16_q4k", grid, 256, 0, params, stream);
+    if (rc != 0) return rc;
+  }
+  void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};
+  return launch("q4_k_gemm_f16", mtiles * ntiles, 256, 131072, params, stream);
+}
+
+int cogni_set_gemm_threshold(int32_t tokens) {
+  if (tokens < 1) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_set_gemm_threshold: threshold must be >= 1");
+  g_gemm_threshold = tokens;
+  return 0;
+}
+
+int32_t cogni_get_gemm_threshold(void) {
+  if (g_gemm_threshold < 0) {
+    g_gemm_threshold = 8;
+    if (const char* e = std::getenv("QWEN35_GEMM_BATCH_THRESHOLD")) {
+      const int v = std::atoi(e);
+      if (v >= 1) g_gemm_threshold = v;
+    }
+  }
+  return g_gemm_threshold;
+}
+
+int cogni_matmul_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
+                     uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream) {
+  if (w_type == COGNI_TYPE_Q4_K && tokens > (uint32_t)cogni_get_gemm_threshold())
+    return cogni_gemm_dev(w_raw, w_type, x, bias, out, in_dim, out_dim, tokens, workspace, workspace_bytes, stream);
+  if (bias && tokens != 1)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_matmul_dev: a [out_dim] bias is only accepted with one token or on the GEMM path; "
+                                            "pass a [tokens][out_dim] residual to cogni_gemv_dev");
+  return cogni_gemv_dev(w_raw, w_type, x, bias, out, in_dim, out_dim, tokens, stream);
+}
+
 // ---- host-buffer operators --------------------------------------------------------------------------
 int cogni_dequantize(const void* data, size_t data_bytes, uint32_t type, int64_t n_elements, float* out) {
   if (!cogni_dequantize_kernel_name(type))
@@ -349,14 +409,31 @@ int cogni_weight_matmul(const cogni_quant_weight* qw, const float* x, int32_t ro
   HIP_TRY(hipMalloc(&dx.p, xin), "hipMalloc(x)");
   HIP_TRY(hipMalloc(&dout.p, xout), "hipMalloc(result)");
   HIP_TRY(hipMemcpyHtoD(dx.p, const_cast<float*>(x), xin), "hipMemcpyHtoD(x)");
-  if (bias) {  // bias[o] is added to every row: stage it as a [rows][out_dim] residual
+  const bool gemm_path = qw->type == COGNI_TYPE_Q4_K && rows > cogni_get_gemm_threshold();
+  if (bias && !gemm_path) {  // bias[o] is added to every row: stage it as a [rows][out_dim] residual
     std::vector<float> tiled((size_t)rows * qw->out_dim);
     for (int32_t r = 0; r < rows; r++) std::memcpy(&tiled[(size_t)r * qw->out_dim], bias, (size_t)qw->out_dim * 4);
     HIP_TRY(hipMalloc(&dres.p, xout), "hipMalloc(bias)");
     HIP_TRY(hipMemcpyHtoD(dres.p, tiled.data(), xout), "hipMemcpyHtoD(bias)");
   }
-  int rc = cogni_gemv_dev((uint64_t)(uintptr_t)qw->dev, qw->type, dx.addr(), dres.addr(), dout.addr(),
-                          (uint32_t)qw->in_dim, (uint32_t)qw->out_dim, (uint32_t)rows, nullptr);
+  int rc;
+  if (gemm_path) {
+    DeviceMem dws, dbias;
+    const size_t wsb = cogni_gemm_workspace_bytes(qw->type, (uint32_t)qw->in_dim, (uint32_t)rows);
+    HIP_TRY(hipMalloc(&dws.p, wsb), "hipMalloc(gemm workspace)");
+    if (bias) {
+      HIP_TRY(hipMalloc(&dbias.p, (size_t)qw->out_dim * 4), "hipMalloc(bias)");
+      HIP_TRY(hipMemcpyHtoD(dbias.p, const_cast<float*>(bias), (size_t)qw->out_dim * 4), "hipMemcpyHtoD(bias)");
+    }
+    rc = cogni_gemm_dev((uint64_t)(uintptr_t)qw->dev, qw->type, dx.addr(), dbias.addr(), dout.addr(),
+                        (uint32_t)qw->in_dim, (uint32_t)qw->out_dim, (uint32_t)rows, dws.addr(), wsb, nullptr);
+    if (rc != 0) return rc;
+    HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize(matmul)");
+    HIP_TRY(hipMemcpyDtoH(result, dout.p, xout), "hipMemcpyDtoH(result)");
+    return 0;
+  }
+  rc = cogni_gemv_dev((uint64_t)(uintptr_t)qw->dev, qw->type, dx.addr(), dres.addr(), dout.addr(),
+                      (uint32_t)qw->in_dim, (uint32_t)qw->out_dim, (uint32_t)rows, nullptr);
   if (rc != 0) return rc;
   HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize(matmul)");
   HIP_TRY(hipMemcpyDtoH(result, dout.p, xout), "hipMemcpyDtoH(result)");

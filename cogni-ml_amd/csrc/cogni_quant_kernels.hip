@@ -3,4 +3,5 @@
 // its PTX modules (src/ml/cuda/driver.cr:115-127).
 #include "kernels/dequant.cuh"
 #include "kernels/gemv.cuh"
+#include "kernels/gemm_q4k.cuh"
 #include "kernels/util.cuh"

@@ -104,6 +104,29 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
                    uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 
+/* Prefill GEMM for `tokens` > 8 (Q4_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
+ * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
+ * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:
+ * 97-105,678-686); expect about 5e-4 of max|out| where the GEMV path gives 1e-6. `workspace` is caller-owned
+ * device memory of at least cogni_gemm_workspace_bytes(...) bytes (x repacked as fp16); nothing is allocated.
+ * Kernels: pack_x_f16_q4k (x, workspace, tokens, in_dim) then
+ *          q4_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,
+ *          grid ceil(tokens/128)*ceil(out_dim/192), 131072 bytes of dynamic shared memory. */
+size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
+int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
+                   uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream);
+
+/* The router of the reference's GPU arm (Qwen35Metal.matmul, src/ml/gguf/qwen35_metal.cr:11404-11449):
+ * tokens > threshold and a type with a GEMM kernel -> cogni_gemm_dev, else cogni_gemv_dev. The threshold
+ * defaults to 8 (GEMM_BATCH_THRESHOLD, qwen35_metal.cr:70-75) and can be changed with
+ * cogni_set_gemm_threshold or the QWEN35_GEMM_BATCH_THRESHOLD environment variable the reference reads.
+ * `bias` ([out_dim], may be 0) is only accepted with tokens == 1 or on the GEMM path. `workspace` may be 0
+ * when the call stays on the GEMV path. */
+int cogni_matmul_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
+                     uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream);
+int cogni_set_gemm_threshold(int32_t tokens);
+int32_t cogni_get_gemm_threshold(void);
+
 /* ---- level 3: host-buffer operators with the reference's CPU signatures (synchronous) -------- */
 
 /* Dequant.dequantize(data, type, n_elements) : Array(Float32)   dequant.cr:19

@@ -69,9 +69,9 @@ def test_gemv_launch_dims():
             grid, block, lds = quant.gemv_launch_dims(t, m, 4096, 12288)
             assert block == 256 and 12288 % grid == 0 and 4 <= 12288 // grid <= 32
             assert 0 < lds <= 49152 and lds % 256 == 0
-    # M = 1: the whole activation vector (plus 1/16 of it for the per-lane sums) is staged once when it fits
-    assert quant.gemv_launch_dims(12, 1, 4096, 12288)[2] == 4096 * 4 * 17 // 16
-    assert quant.gemv_launch_dims(12, 1, 8192, 4096)[2] == 8192 * 4 * 17 // 16
+    # M = 1: the whole activation vector is staged once when it fits, plus two per-lane sums per 4096-value column set
+    assert quant.gemv_launch_dims(12, 1, 4096, 12288)[2] == 4096 * 4 + 512
+    assert quant.gemv_launch_dims(12, 1, 8192, 4096)[2] == 8192 * 4 + 1024
     assert quant.gemv_launch_dims(12, 1, 65536, 4096)[2] <= 49152
     g1 = quant.gemv_launch_dims(12, 1, 256, 17)[0]
     assert g1 == -(-17 // (12288 // quant.gemv_launch_dims(12, 1, 4096, 12288)[0]))

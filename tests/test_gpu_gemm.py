@@ -1,0 +1,116 @@
+"""GPU prefill GEMM (Q4_K, fp16 MFMA path) vs the CPU oracle.
+
+Tolerance (fp16-MFMA path): max|err| <= 2e-3 * max|ref| over the output, plus cos >= 0.9999 -- the
+reference's own convention for its Metal GEMM (spec/qwen35_metal_spec.cr:78,104 uses 0.05 * max|cpu|).
+The figure normalised the fp32 way, max|err| / (||x||_2 * max|w_row|), is printed beside it.
+"""
+import numpy as np
+import pytest
+
+from cogni_ml_amd import quant, synth
+from gpu_common import DevArray, gpu  # noqa: F401
+from helpers import Q4_K, Q6_K, cosine
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gemm(raw, x, in_dim, out_dim, tokens, bias=None, router=False):
+    w, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim)
+    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens)
+    ws = DevArray(nbytes=wsb)
+    bd = DevArray(bias) if bias is not None else None
+    fn = quant.matmul_dev if router else quant.gemm_dev
+    fn(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens, ws.ptr, wsb, bd.ptr if bd else 0)
+    out = od.read(np.float32, tokens * out_dim)
+    for a in (w, xd, od, ws, bd):
+        if a:
+            a.close()
+    return out
+
+
+def check(oracle, raw, x, in_dim, out_dim, tokens, bias=None, what="", router=False, sample_tokens=None):
+    got = run_gemm(raw, x, in_dim, out_dim, tokens, bias, router).reshape(tokens, out_dim)
+    b = bias if bias is not None else np.zeros(out_dim, dtype=np.float32)
+    rows = np.arange(tokens) if sample_tokens is None else np.asarray(sample_tokens)
+    xs = x.reshape(tokens, in_dim)[rows]
+    want = oracle.matmul_add(xs.reshape(-1), len(rows), in_dim, raw, Q4_K, out_dim, b, threads=16).reshape(len(rows), out_dim)
+    err = np.max(np.abs(got[rows].astype(np.float64) - want))
+    ref_max = np.max(np.abs(want))
+    dense_max = np.max(np.abs(oracle.dequantize(raw, Q4_K, out_dim * in_dim)))
+    fp32_style = err / (np.max(np.linalg.norm(xs, axis=1)) * dense_max)
+    print("%s: max|err|/max|ref| = %.3e, max|err|/(||x|| max|w|) = %.3e" % (what, err / ref_max, fp32_style))
+    assert cosine(got[rows].reshape(-1), want.reshape(-1)) >= 0.9999, what
+    assert err <= 2e-3 * ref_max, "%s: err %.3e > 2e-3 * %.3e" % (what, err, ref_max)
+    return got
+
+
+@pytest.mark.parametrize("tokens,out_dim,in_dim", [(9, 192, 256), (16, 48, 512), (64, 200, 1024), (128, 192, 256),
+                                                     (130, 400, 768), (257, 31, 256)])
+def test_small_shapes_and_tails(gpu, oracle, tokens, out_dim, in_dim):
+    rng = np.random.default_rng(tokens * 1000 + out_dim)
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    check(oracle, raw, x, in_dim, out_dim, tokens, None, "M=%d N=%d K=%d" % (tokens, out_dim, in_dim))
+
+
+def test_bias_and_router(gpu, oracle):
+    rng = np.random.default_rng(4)
+    out_dim, in_dim = 384, 512
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    bias = rng.standard_normal(out_dim).astype(np.float32)
+    x = synth.make_activations(rng, 40, in_dim)
+    check(oracle, raw, x, in_dim, out_dim, 40, bias, "bias M=40", router=True)
+    # at or below the threshold the router takes the fp32 GEMV path: agreement with the oracle is ~1e-6
+    assert quant.get_gemm_threshold() == 8
+    got = run_gemm(raw, x[:8 * in_dim], in_dim, out_dim, 8, None, router=True)
+    want = oracle.matmul_add(x[:8 * in_dim], 8, in_dim, raw, Q4_K, out_dim, np.zeros(out_dim, dtype=np.float32))
+    assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+    # host-level matmul_add with rows > 8 goes through the GEMM as well
+    mine = quant.matmul_add(x, 40, in_dim, raw, Q4_K, out_dim, bias)
+    ref = oracle.matmul_add(x, 40, in_dim, raw, Q4_K, out_dim, bias)
+    assert np.max(np.abs(mine - ref)) <= 2e-3 * np.max(np.abs(ref))
+    quant.set_gemm_threshold(64)
+    try:
+        mine32 = quant.matmul_add(x, 40, in_dim, raw, Q4_K, out_dim, bias)
+        assert np.max(np.abs(mine32 - ref)) <= 1e-5 * np.max(np.abs(ref))
+    finally:
+        quant.set_gemm_threshold(8)
+
+
+def test_argument_checks(gpu):
+    w, x, o = DevArray(nbytes=4096), DevArray(nbytes=4096), DevArray(nbytes=4096)
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for the prefill GEMM") as e:
+        quant.gemm_dev(w.ptr, Q6_K, x.ptr, o.ptr, 256, 1, 16, w.ptr, 4096)
+    assert e.value.code == -2
+    with pytest.raises(quant.QuantError, match="workspace has 16 bytes, needs 65536"):
+        quant.gemm_dev(w.ptr, Q4_K, x.ptr, o.ptr, 256, 1, 16, w.ptr, 16)
+    with pytest.raises(quant.QuantError, match="in_dim multiple of 256"):
+        quant.gemm_dev(w.ptr, Q4_K, x.ptr, o.ptr, 100, 1, 16, w.ptr, 1 << 20)
+    with pytest.raises(quant.QuantError, match="bias is only accepted"):
+        quant.matmul_dev(w.ptr, Q4_K, x.ptr, o.ptr, 256, 1, 4, 0, 0, bias_ptr=o.ptr)
+    for a in (w, x, o):
+        a.close()
+
+
+@pytest.mark.parametrize("tokens", [64, 512])
+def test_configured_prefill_shapes(gpu, oracle, tokens):
+    """Config 4: X tokens x 4096, W Q4_K 12288 x 4096."""
+    rng = np.random.default_rng(4096 + tokens)
+    out_dim, in_dim = 12288, 4096
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    sample = None if tokens <= 64 else np.concatenate([np.arange(0, 24), np.arange(250, 262), np.arange(tokens - 12, tokens)])
+    check(oracle, raw, x, in_dim, out_dim, tokens, None, "cfg4 M=%d" % tokens, sample_tokens=sample)
+
+
+def test_m2048_row_identity(gpu, oracle):
+    """M = 2048: a sample of tokens against the oracle, and every token against the same token run through a
+    smaller GEMM (the result for a token does not depend on which tile it sits in)."""
+    rng = np.random.default_rng(2048)
+    out_dim, in_dim, tokens = 12288, 4096, 2048
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    got = check(oracle, raw, x, in_dim, out_dim, tokens, None, "cfg4 M=2048",
+                sample_tokens=[0, 1, 127, 128, 1000, 1023, 1024, 2046, 2047])
+    part = run_gemm(raw, x[1900 * in_dim:], in_dim, out_dim, tokens - 1900).reshape(-1, out_dim)
+    assert np.array_equal(part, got[1900:])
