@@ -105,9 +105,12 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const size_t row_bytes = (size_t)nkb * 144;
   const u32 sh = 16u * (kg >> 1);
 
-  const uint8_t* rowp[3];
+  // uniform base of the wavefront's rows + a 32-bit per-lane offset (48 rows are far below 4 GiB)
+  const u32 base_row = min(n0, out_dim - 1);
+  const uint8_t* wbase = w + (size_t)base_row * row_bytes;
+  u32 rowoff[3];
 #pragma unroll
-  for (int c = 0; c < 3; c++) rowp[c] = w + (size_t)min(n0 + 16 * c + j, out_dim - 1) * row_bytes;
+  for (int c = 0; c < 3; c++) rowoff[c] = (min(n0 + 16 * c + j, out_dim - 1) - base_row) * (u32)row_bytes + 16 * kg;
   const uint4* xtile = xp + (size_t)mt * nkb * 4096;
 
   float4_t acc[8][3];
@@ -117,12 +120,12 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     for (int c = 0; c < 3; c++) acc[r][c] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
   auto load_raw = [&](GemmRaw (&raw)[3], u32 kb) {
+    const uint8_t* kbase = wbase + (size_t)kb * 144;   // uniform
 #pragma unroll
     for (int c = 0; c < 3; c++) {
-      const uint8_t* bp = rowp[c] + (size_t)kb * 144;
-      raw[c].hdr = ld16(bp);
-      raw[c].q0 = ld16(bp + 16 + 16 * kg);
-      raw[c].q1 = ld16(bp + 80 + 16 * kg);
+      raw[c].hdr = ld16(kbase + (rowoff[c] - 16 * kg));
+      raw[c].q0 = ld16(kbase + (rowoff[c] + 16));
+      raw[c].q1 = ld16(kbase + (rowoff[c] + 80));
     }
   };
 
@@ -130,15 +133,18 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   GemmRaw cur[3];
   load_raw(cur, 0);
 #pragma unroll
-  for (int i = 0; i < 16; i++) lds[tid + 256 * i] = xtile[tid + 256 * i];
+  for (int i = 0; i < 16; i++) lds[tid + 256 * i] = (xtile + 256 * i)[tid];
   __syncthreads();
 
   for (u32 kb = 0; kb < nkb; kb++) {
     const u32 cb = (kb & 1) * 4096, nb_ = 4096 - cb;
-    const bool more = kb + 1 < nkb;
+    const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
     GemmRaw nxt[3];
-    if (more) load_raw(nxt, kb + 1);
-    const uint4* xnext = xtile + (size_t)(kb + 1) * 4096;
+    load_raw(nxt, kn);
+    const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
+    uint4 xbuf[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) xbuf[i] = (xnext + 256 * i)[tid];
 
     // per-row scales of this super-block as duplicated half2: [c][u][lo scale, lo -min, hi scale, hi -min]
     u32 S[3][2][4];
@@ -159,15 +165,10 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       S[c][1][3] = h2_dup(-(dm * ubyte_f<1>(mU)));
     }
 
+    const uint4* arow = lds + cb + j * 4 + kg;
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) {
       const int u = ks >> 2, op = ks & 3, hi = op >> 1;
-      // copy a quarter of the next x tile during k-steps 0, 2, 4, 6
-      uint4 xbuf[4];
-      if ((ks & 1) == 0 && more) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) xbuf[i] = xnext[tid + 256 * (4 * (ks >> 1) + i)];
-      }
       half8_t B[3];
 #pragma unroll
       for (int c = 0; c < 3; c++) {
@@ -186,21 +187,18 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       }
 #pragma unroll
       for (int r = 0; r < 8; r++) {
-        const uint4 av = lds[cb + (ks * 128 + r * 16 + j) * 4 + kg];
+        const uint4 av = arow[(ks * 128 + r * 16) * 4];
         const half8_t A = *reinterpret_cast<const half8_t*>(&av);
 #pragma unroll
         for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B[c], acc[r][c], 0, 0, 0);
       }
-      if ((ks & 1) == 0 && more) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) lds[nb_ + tid + 256 * (4 * (ks >> 1) + i)] = xbuf[i];
-      }
     }
+    // the other buffer was last read in the previous iteration, which ended with a barrier
+#pragma unroll
+    for (int i = 0; i < 16; i++) lds[nb_ + tid + 256 * i] = xbuf[i];
     __syncthreads();
-    if (more) {
 #pragma unroll
-      for (int c = 0; c < 3; c++) cur[c] = nxt[c];
-    }
+    for (int c = 0; c < 3; c++) cur[c] = nxt[c];
   }
 
   // D layout: lane holds column j (weight row) and rows 4*kg + v (tokens) of each 16x16 tile
