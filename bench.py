@@ -82,14 +82,20 @@ class GemvCase:
             b.close()
 
 
-def time_steps(hip, stream, launch, steps, warmup):
+def graph_ok(wanted):
+    return bool(wanted)
+
+
+def time_steps(hip, stream, launch, steps, warmup, graph=True):
     """Run `warmup` untimed and exactly `steps` timed launches on `stream`; returns ms for the timed region.
     The timed launches are captured into one HIP graph so host launch latency does not gate the GPU."""
     for i in range(warmup):
         launch(i, stream)
     stream.synchronize()
-    graph = exe = None
+    graph, exe = None, None
     try:
+        if not graph_ok(graph_wanted := graph):
+            raise RuntimeError("direct launches requested")
         stream.begin_capture(1)
         for i in range(steps):
             launch(warmup + i, stream)
@@ -97,9 +103,10 @@ def time_steps(hip, stream, launch, steps, warmup):
         exe = graph.instantiate()
         exe.upload(stream)
         stream.synchronize()
-    except Exception as e:  # stream capture unavailable: fall back to direct launches
-        log("graph capture failed (%s); timing direct launches" % e)
-        exe = None
+    except Exception as e:  # stream capture unavailable or not wanted: direct launches
+        if graph_wanted:
+            log("graph capture failed (%s); timing direct launches" % e)
+        graph, exe = None, None
     e0, e1 = hip.Event(), hip.Event()
     hip.synchronize()
     e0.record(stream)
@@ -120,7 +127,7 @@ def time_steps(hip, stream, launch, steps, warmup):
     return ms, exe is not None
 
 
-def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, warmup):
+def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, warmup, graph=True):
     """Q4_K prefill GEMM (x repack + MFMA kernel) at `tokens`; returns (ms per call, TFLOP/s)."""
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
@@ -132,7 +139,7 @@ def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, w
     def launch(i, st):
         quant.gemm_dev(bufs[0].ptr, Q4_K, bufs[1].ptr, bufs[2].ptr, in_dim, out_dim, tokens, bufs[3].ptr, wsb, 0,
                        st.handle)
-    ms, _ = time_steps(hip, stream, launch, steps, warmup)
+    ms, _ = time_steps(hip, stream, launch, steps, warmup, graph)
     for b in bufs:
         b.close()
     per = ms / steps
@@ -157,7 +164,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--mode", choices=["headline", "cases", "pmc", "ceiling"], default="headline")
+    ap.add_argument("--mode", choices=["headline", "cases", "pmc", "pmc-gemm", "ceiling"], default="headline")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--seed", type=int, default=1234)
     args = ap.parse_args()
@@ -175,6 +182,12 @@ def main():
         ctx.device_name, ctx.arch, ctx.compute_units, ctx.clock_khz // 1000, os.cpu_count()))
     rng = np.random.default_rng(args.seed)
     stream = hip.HIPStream()
+
+    if args.mode == "pmc-gemm":
+        # plain launches of the prefill GEMM (M = 512) for profiler runs
+        per, tf = bench_gemm(hip, quant, synth, rng, stream, 512, 12288, 4096, args.steps, args.warmup, graph=False)
+        log("pmc-gemm mode: M=512 ms=%.5f tflops=%.1f" % (per, tf))
+        return
 
     head = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1)
 

@@ -304,7 +304,7 @@ int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, u
     if (rc != 0) return rc;
   }
   void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};
-  return launch("q4_k_gemm_f16", mtiles * ntiles, 256, 131072, params, stream);
+  return launch("q4_k_gemm_f16", mtiles * ntiles, 256, 0, params, stream);
 }
 
 int cogni_set_gemm_threshold(int32_t tokens) {

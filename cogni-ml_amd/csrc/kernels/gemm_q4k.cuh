@@ -1,48 +1,52 @@
 // Prefill GEMM over raw Q4_K weights: out[m][n] = (bias[n] +) sum_k x[m][k] * deq(W[n][k]), M >= 9.
-// fp16 operands, v_mfma_f32_16x16x32_f16, fp32 accumulation (the precision of the reference's Metal
+// fp16 operands, v_mfma_f32_32x32x16_f16, fp32 accumulation (the precision of the reference's Metal
 // prefill kernels, which round both x and the dequantized weights to half:
-// src/ml/gguf/kernels/gemm_q4k.metal:97-105,678-686).
+// src/ml/gguf/kernels/gemm_q4k.metal:97-105,678-686). On gfx950 the 32x32x16 instruction sustains twice
+// the rate of 16x16x32 (about 32 vs 2 x 32 clocks for the same 32768 flops per SIMD), hence the tile shape.
 //
 // Two kernels:
 //   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, any grid
 //   q4_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
-//                   block 256, grid ceil(m/128) * ceil(out_dim/192), dynamic LDS 131072 bytes
+//                   block 256, grid ceil(m/128) * ceil(out_dim/192), no dynamic LDS (128 KiB static)
 //
-// Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows; a wavefront owns all 128 tokens
-// x 48 rows, so every weight is dequantized by exactly one wavefront of the workgroup and reused for
-// 128 tokens, and 512 x 12288 gives 256 workgroups, one per CU. K is walked one 256-value super-block
-// at a time, eight MFMA k-steps of 32.
+// Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows, so 512 x 12288 gives 256
+// workgroups, one per CU. K is walked one 256-value super-block at a time = 16 MFMA k-steps of 16.
+// The four wavefronts split the tile as (row half nh) x (k-step half kh): a wavefront accumulates
+// 128 tokens x 96 rows (4 x 3 tiles of 32 x 32, 192 accumulator registers) over 8 of the 16 k-steps of
+// every super-block; the two k halves are added through LDS once, at the end. Every weight is
+// dequantized by exactly one wavefront and reused for 128 tokens.
 //
-// Weights never touch LDS: a lane holds 16-byte chunks of "its" weight row (row = lane % 16, k-group
-// = lane / 16) and turns their nibbles into the MFMA B operand in registers. A masked dword
-// (q & 0x000F000F) | 0x64006400 is the half2 (1024 + n0, 1024 + n4); subtracting 1024 and one packed
-// fma give fp16(d*sc*n - dmin*m) for two weights. The eight k values a lane contributes to one k-step
-// therefore come in nibble order (bytes 0,2,1,3,4,6,5,7 of eight consecutive bytes); pack_x_f16_q4k
-// writes x in exactly that order, already laid out as the LDS image [k-step][token][k-group][8 halves]
-// of each (128-token tile, super-block), so staging x is a straight 64 KiB copy and the A operand
-// is one conflict-free ds_read_b128 per lane.
+// Weights never touch LDS. In MFMA terms a lane is (weight row j = lane % 32, k-group kg = lane / 32)
+// and supplies 8 k values per k-step. Lane (j, kg) of a kh wavefront owns the 64-value group
+// g = 2*kg + kh of its row's super-block: the 32 bytes qs[32g, 32g+32) as two 16-byte loads, one
+// (scale, min) pair decode. Eight consecutive bytes give two k-steps: their low nibbles (sub-block 2g)
+// and their high nibbles (sub-block 2g+1). A masked dword (q & 0x000F000F) | 0x64006400 is the half2
+// (1024 + n0, 1024 + n4); subtracting 1024 and one packed fma give fp16(d*sc*n - dmin*m) for two
+// weights. The 8 k values of a lane therefore come in nibble order (bytes 0,2,1,3,4,6,5,7);
+// pack_x_f16_q4k writes x in exactly that order, already laid out as the LDS image
+// [k-step][k-group][token][8 halves] of each (128-token tile, super-block), so staging x is a straight
+// 64 KiB copy (global_load_lds_dwordx4, no registers) and an A operand is one conflict-free ds_read_b128.
 //
-// The only LDS traffic is the activations: 8 KiB read per wavefront and k-step for 24 MFMAs.
-// The x tile of the next super-block is copied global -> LDS while the current one is consumed
-// (two 64 KiB buffers), and the raw weight chunks of the next super-block are prefetched into
-// registers.
+// The only LDS traffic in the loop is the activations: 4 KiB read per wavefront and k-step for 12
+// MFMAs. The x tile of the next super-block is copied while the current one is consumed (two 64 KiB
+// buffers) and the raw weight bytes of the next super-block are prefetched into registers.
 #pragma once
 #include "common.cuh"
 
 #define GEMM_BM 128
 #define GEMM_BN 192
-#define GEMM_WN 48          // weight rows per wavefront (3 column tiles of 16)
-#define GEMM_LDS_BYTES 131072
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
-typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void gbl_void;
 
-// Element (0..255) of a super-block that k-slot (kstep, kg, e) of the MFMA stands for.
-// kstep = 4u + op: u = 64-byte half of the nibble array, op&1 = upper 8 bytes of the lane's chunk,
-// op>>1 = high nibbles.
-__device__ __forceinline__ u32 gemm_k_element(u32 kstep, u32 kg, u32 e) {
-  const u32 u = kstep >> 2, op = kstep & 3;
-  const u32 chunk = 4 * u + kg, g = chunk >> 1, h = chunk & 1;
+// Element (0..255) of a super-block that k-slot (ks, kg, e) of the MFMA stands for. ks = 8*kh + 4*h + op:
+// kh = k half (which wavefront), h = 16-byte half of the lane's group, op & 1 = upper 8 bytes of that
+// half, op >> 1 = high nibbles. The group is g = 2*kg + kh.
+__device__ __forceinline__ u32 gemm_k_element(u32 ks, u32 kg, u32 e) {
+  const u32 kh = ks >> 3, h = (ks >> 2) & 1, op = ks & 3;
+  const u32 g = 2 * kg + kh;
   const u32 perm = ((e & 1) << 1) | ((e >> 1) & 1) | (e & 4);   // 0,2,1,3,4,6,5,7
   return 64 * g + 32 * (op >> 1) + 16 * h + 8 * (op & 1) + perm;
 }
@@ -54,13 +58,13 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q4k(const float* __
   const u64 total = (u64)mtiles * nkb * 4096;   // 16-byte pieces
   const u64 step = (u64)gridDim.x * blockDim.x;
   for (u64 idx = (u64)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += step) {
-    const u32 kg = idx & 3, tok = (idx >> 2) & 127, kstep = (idx >> 9) & 7;
+    const u32 tok = idx & 127, kg = (idx >> 7) & 1, ks = (idx >> 8) & 15;
     const u64 tile = idx >> 12;
     const u32 kb = (u32)(tile % nkb), mt = (u32)(tile / nkb);
     const u32 row = mt * GEMM_BM + tok;
     uint4 o = make_uint4(0u, 0u, 0u, 0u);
     if (row < m) {
-      const float* src = x + (size_t)row * in_dim + kb * 256 + gemm_k_element(kstep, kg, 0);   // e = 0 is the base
+      const float* src = x + (size_t)row * in_dim + kb * 256 + gemm_k_element(ks, kg, 0);   // e = 0 is the base
       float4 a, b;
       __builtin_memcpy(&a, src, 16);
       __builtin_memcpy(&b, src + 4, 16);
@@ -85,99 +89,118 @@ __device__ __forceinline__ u32 h2_fma_off(u32 t, u32 off, u32 scale, u32 negmin)
   return *reinterpret_cast<const u32*>(&w);
 }
 
-struct GemmRaw {   // raw bytes of one super-block of one weight row, as a lane sees them
-  uint4 hdr, q0, q1;
+// The two x-tile buffers are separate objects so the compiler can tell the LDS-direct loads into one from
+// the operand reads out of the other (otherwise every read would first wait for all loads in flight).
+__shared__ uint4 gemm_xbuf0[4096];   // [16 k-steps][2 k-groups][128 tokens] uint4
+__shared__ uint4 gemm_xbuf1[4096];
+
+struct GemmRaw {   // raw bytes of one group of one super-block of one weight row, as a lane sees them
+  uint4 hdr, qa, qb;
 };
 
-extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_f16(const uint8_t* __restrict__ w,
-                                                                 const uint4* __restrict__ xp,
-                                                                 const float* __restrict__ bias,
-                                                                 float* __restrict__ out, u32 in_dim, u32 out_dim,
-                                                                 u32 m) {
-  extern __shared__ uint4 lds[];   // 2 x [8 k-steps][128 tokens][4 k-groups] uint4
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
+  // (no __restrict__ on w / xp: loads the compiler knows to be invariant are rematerialised next to
+  // their use, which would undo the prefetch distance set up below)
   const u32 tid = threadIdx.x, lane = tid & 63;
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const u32 j = lane & 15, kg = lane >> 4;
+  const u32 nh = wave & 1, kh = wave >> 1;
+  const u32 j = lane & 31, kg = lane >> 5;
+  const u32 g = 2 * kg + kh;
   const u32 nkb = in_dim >> 8;
   const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM;
   const u32 mt = blockIdx.x % mtiles, nt = blockIdx.x / mtiles;
-  const u32 n0 = nt * GEMM_BN + wave * GEMM_WN;      // first weight row of this wavefront
+  const u32 n0 = nt * GEMM_BN + nh * 96;             // first weight row of this wavefront
   const size_t row_bytes = (size_t)nkb * 144;
-  const u32 sh = 16u * (kg >> 1);
+  const u32 sh = 16u * (g & 1);
+  const bool upper = g >= 2;
 
-  // uniform base of the wavefront's rows + a 32-bit per-lane offset (48 rows are far below 4 GiB)
+  // uniform base of the wavefront's rows + a 32-bit per-lane offset (96 rows are far below 4 GiB)
   const u32 base_row = min(n0, out_dim - 1);
   const uint8_t* wbase = w + (size_t)base_row * row_bytes;
   u32 rowoff[3];
 #pragma unroll
-  for (int c = 0; c < 3; c++) rowoff[c] = (min(n0 + 16 * c + j, out_dim - 1) - base_row) * (u32)row_bytes + 16 * kg;
+  for (int c = 0; c < 3; c++) rowoff[c] = (min(n0 + 32 * c + j, out_dim - 1) - base_row) * (u32)row_bytes;
   const uint4* xtile = xp + (size_t)mt * nkb * 4096;
 
-  float4_t acc[8][3];
+  float16_t acc[4][3];
 #pragma unroll
-  for (int r = 0; r < 8; r++)
+  for (int r = 0; r < 4; r++)
 #pragma unroll
-    for (int c = 0; c < 3; c++) acc[r][c] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
   auto load_raw = [&](GemmRaw (&raw)[3], u32 kb) {
     const uint8_t* kbase = wbase + (size_t)kb * 144;   // uniform
 #pragma unroll
     for (int c = 0; c < 3; c++) {
-      raw[c].hdr = ld16(kbase + (rowoff[c] - 16 * kg));
-      raw[c].q0 = ld16(kbase + (rowoff[c] + 16));
-      raw[c].q1 = ld16(kbase + (rowoff[c] + 80));
+      raw[c].hdr = ld16(kbase + rowoff[c]);
+      raw[c].qa = ld16(kbase + (rowoff[c] + 16 + 32 * g));
+      raw[c].qb = ld16(kbase + (rowoff[c] + 32 + 32 * g));
     }
   };
 
-  // stage super-block 0 of x and the first weights
+  // Stage super-block 0 of x and the first weights. The main loop below takes super-blocks in pairs with
+  // fixed buffer roles (buffer 0 then buffer 1) and no branch in its body; with an odd number of
+  // super-blocks the first one is taken alone out of buffer 1.
+  const bool odd = nkb & 1;
   GemmRaw cur[3];
   load_raw(cur, 0);
+  if (odd) {
 #pragma unroll
-  for (int i = 0; i < 16; i++) lds[tid + 256 * i] = (xtile + 256 * i)[tid];
+    for (int i = 0; i < 16; i++)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf1 + 256 * i + wave * 64),
+                                       16, 0, 0);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
+                                       16, 0, 0);
+  }
   __syncthreads();
 
-  for (u32 kb = 0; kb < nkb; kb++) {
-    const u32 cb = (kb & 1) * 4096, nb_ = 4096 - cb;
+  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt) {
     const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
+    // The next x tile goes global -> LDS without passing through registers (global_load_lds_dwordx4:
+    // lane l of a wavefront lands at LDS base + 16*l), into the buffer that was last read in the previous
+    // iteration, which ended with a barrier. Loads complete in issue order, so these (L2 hits) go ahead of
+    // the raw weights of the next super-block (HBM).
+    const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64),
+                                       16, 0, 0);
     GemmRaw nxt[3];
     load_raw(nxt, kn);
-    const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
-    uint4 xbuf[16];
-#pragma unroll
-    for (int i = 0; i < 16; i++) xbuf[i] = (xnext + 256 * i)[tid];
+    __builtin_amdgcn_sched_barrier(0);   // keep the prefetches up here
 
-    // per-row scales of this super-block as duplicated half2: [c][u][lo scale, lo -min, hi scale, hi -min]
-    u32 S[3][2][4];
+    // (scale, -min) of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles) as duplicated half2
+    u32 S[3][4];
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const float d = h2f(cur[c].hdr.x), dm = h2f(cur[c].hdr.x >> 16);
-      const u32 a0 = cur[c].hdr.y >> sh, a1 = cur[c].hdr.z >> sh, a2 = cur[c].hdr.w >> sh;
-      const u32 scL = a0 & 0x3F3Fu, mL = a1 & 0x3F3Fu;                       // sub-blocks 2g, 2g+1, g = kg>>1
-      const u32 scU = (a2 & 0x0F0Fu) | ((a0 >> 2) & 0x3030u);                // sub-blocks 2g+4, 2g+5
-      const u32 mU = ((a2 >> 4) & 0x0F0Fu) | ((a1 >> 2) & 0x3030u);
-      S[c][0][0] = h2_dup(d * ubyte_f<0>(scL));
-      S[c][0][1] = h2_dup(-(dm * ubyte_f<0>(mL)));
-      S[c][0][2] = h2_dup(d * ubyte_f<1>(scL));
-      S[c][0][3] = h2_dup(-(dm * ubyte_f<1>(mL)));
-      S[c][1][0] = h2_dup(d * ubyte_f<0>(scU));
-      S[c][1][1] = h2_dup(-(dm * ubyte_f<0>(mU)));
-      S[c][1][2] = h2_dup(d * ubyte_f<1>(scU));
-      S[c][1][3] = h2_dup(-(dm * ubyte_f<1>(mU)));
+      const u32 s0 = cur[c].hdr.y, s1 = cur[c].hdr.z, s2 = cur[c].hdr.w;
+      const u32 a0 = s0 >> sh, a1 = s1 >> sh, a2 = s2 >> sh;
+      const u32 scp = upper ? ((a2 & 0x0F0Fu) | ((a0 >> 2) & 0x3030u)) : (a0 & 0x3F3Fu);
+      const u32 mp = upper ? (((a2 >> 4) & 0x0F0Fu) | ((a1 >> 2) & 0x3030u)) : (a1 & 0x3F3Fu);
+      S[c][0] = h2_dup(d * ubyte_f<0>(scp));
+      S[c][1] = h2_dup(-(dm * ubyte_f<0>(mp)));
+      S[c][2] = h2_dup(d * ubyte_f<1>(scp));
+      S[c][3] = h2_dup(-(dm * ubyte_f<1>(mp)));
     }
 
-    const uint4* arow = lds + cb + j * 4 + kg;
-#pragma unroll
-    for (int ks = 0; ks < 8; ks++) {
-      const int u = ks >> 2, op = ks & 3, hi = op >> 1;
-      half8_t B[3];
+    const uint4* arow = xcur + (16 * kh + kg) * 128 + j;   // k-steps 8*kh .. 8*kh+7; 32 lanes read 512 contiguous bytes
+    auto build_b = [&](half8_t (&B)[3], int t) {
+      const int h = t >> 2, op = t & 3, hi = op >> 1;
 #pragma unroll
       for (int c = 0; c < 3; c++) {
-        const uint4 Q = u ? cur[c].q1 : cur[c].q0;
+        const uint4 Q = h ? cur[c].qb : cur[c].qa;
         const u32 qa = (op & 1) ? Q.z : Q.x, qb = (op & 1) ? Q.w : Q.y;
         const u32 mask = hi ? 0x00F000F0u : 0x000F000Fu;
         const u32 magic = hi ? 0x54005400u : 0x64006400u;     // 64 + n (n sits 4 bits up) : 1024 + n
         const u32 off = hi ? 0xD400D400u : 0xE400E400u;       // half2(-64) : half2(-1024)
-        const u32 sc = S[c][u][2 * hi], nm = S[c][u][2 * hi + 1];
+        const u32 sc = S[c][2 * hi], nm = S[c][2 * hi + 1];
         uint4 bw;
         bw.x = h2_fma_off((qa & mask) | magic, off, sc, nm);
         bw.y = h2_fma_off(((qa >> 8) & mask) | magic, off, sc, nm);
@@ -185,35 +208,71 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
         bw.w = h2_fma_off(((qb >> 8) & mask) | magic, off, sc, nm);
         B[c] = *reinterpret_cast<const half8_t*>(&bw);
       }
+    };
+
+    // software pipeline over the wavefront's eight k-steps: while the MFMAs of step t run, the A operands
+    // of step t+1 are read from LDS and its B operands are built
+    uint4 A[2][4];
+    half8_t B[2][3];
 #pragma unroll
-      for (int r = 0; r < 8; r++) {
-        const uint4 av = arow[(ks * 128 + r * 16) * 4];
-        const half8_t A = *reinterpret_cast<const half8_t*>(&av);
+    for (int r = 0; r < 4; r++) A[0][r] = arow[r * 32];
+    build_b(B[0], 0);
 #pragma unroll
-        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B[c], acc[r][c], 0, 0, 0);
+    for (int t = 0; t < 8; t++) {
+      const int p = t & 1;
+      if (t < 7) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) A[p ^ 1][r] = arow[(t + 1) * 256 + r * 32];
+        build_b(B[p ^ 1], t + 1);
       }
-    }
-    // the other buffer was last read in the previous iteration, which ended with a barrier
 #pragma unroll
-    for (int i = 0; i < 16; i++) lds[nb_ + tid + 256 * i] = xbuf[i];
-    __syncthreads();
+      for (int r = 0; r < 4; r++) {
+        const half8_t Ar = *reinterpret_cast<const half8_t*>(&A[p][r]);
+#pragma unroll
+        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Ar, B[p][c], acc[r][c], 0, 0, 0);
+      }
+      // scheduling window = one k-step: its MFMAs interleave with the operand preparation of the next
+      // step, but the preparation of later steps is not pulled forward (it would only occupy registers)
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();   // waits for the LDS-direct loads of this wavefront, then for everybody's
 #pragma unroll
     for (int c = 0; c < 3; c++) cur[c] = nxt[c];
+  };
+  if (odd) iteration(0, gemm_xbuf1, gemm_xbuf0);
+  for (u32 kb = odd; kb < nkb; kb += 2) {
+    iteration(kb, gemm_xbuf0, gemm_xbuf1);
+    iteration(kb + 1, gemm_xbuf1, gemm_xbuf0);
   }
 
-  // D layout: lane holds column j (weight row) and rows 4*kg + v (tokens) of each 16x16 tile
+  // add the two k halves: kh = 1 wavefronts hand their accumulators to their kh = 0 partners through LDS
+  // (48 KiB each, [r][c][v][lane]; the x buffers are free after the final barrier above)
+  float* xch = reinterpret_cast<float*>(nh ? gemm_xbuf1 : gemm_xbuf0);
+  if (kh == 1) {
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+      for (int c = 0; c < 3; c++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) xch[((r * 3 + c) * 16 + v) * 64 + lane] = acc[r][c][v];
+  }
+  __syncthreads();
+  if (kh == 1) return;
+
+  // D layout of a 32x32 tile: register v of lane (j, kg) is row 8*(v/4) + 4*kg + v%4 (token), column j (weight row)
 #pragma unroll
   for (int c = 0; c < 3; c++) {
-    const u32 n = n0 + 16 * c + j;
+    const u32 n = n0 + 32 * c + j;
     if (n < out_dim) {
       const float b = bias ? bias[n] : 0.0f;
 #pragma unroll
-      for (int r = 0; r < 8; r++) {
+      for (int r = 0; r < 4; r++) {
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-          const u32 row = mt * GEMM_BM + 16 * r + 4 * kg + v;
-          if (row < m) out[(size_t)row * out_dim + n] = acc[r][c][v] + b;
+        for (int v = 0; v < 16; v++) {
+          const u32 row = mt * GEMM_BM + 32 * r + 8 * (v >> 2) + 4 * kg + (v & 3);
+          if (row < m) out[(size_t)row * out_dim + n] = acc[r][c][v] + xch[((r * 3 + c) * 16 + v) * 64 + lane] + b;
         }
+        __builtin_amdgcn_sched_barrier(0);   // one tile at a time: keeps the LDS reads from piling up in registers
       }
     }
   }
