@@ -291,6 +291,28 @@ def main():
                 name, TYPE_NAME[t], in_dim, out_dim, tokens, c.w_bytes, c.copies, steps, cms / steps, cg))
             c.close()
 
+    if args.mode == "cases":
+        # config 5: the mixed-quant projection stack, resident, back to back in one stream
+        from cogni_ml_amd.projection_stack import QwenProjectionStackRunner, Weights
+        wts = Weights.synthetic(rng)
+        for tokens in (1, 4, 8):
+            runner = QwenProjectionStackRunner.from_weights(wts, tokens, synth.make_activations(rng, tokens, wts.hidden))
+            runner.upload_weights()
+            runner.reset_sequence()
+
+            def seq(i, st, runner=runner):
+                with hip.with_stream(st):
+                    runner.run_sequence()
+            reps = max(20, min(args.steps // 4, 300))
+            sms, _ = time_steps(hip, stream, seq, reps, 10)
+            sg = runner.bytes_per_sequence() / (sms / reps * 1e-3) / 1e9
+            extra["projection stack M=%d" % tokens] = {"gbps": round(sg, 1), "ms": round(sms / reps, 5),
+                                                        "frac_hbm": round(sg / HBM_PEAK_GBPS, 4)}
+            log("case=projection stack (q,k,v,o,gate,up Q4_K + down Q6_K)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\n"
+                "gbps=%.1f\nnote=weights %.0f MB stay in the 256 MB last-level cache between repetitions\n" % (
+                    tokens, wts.raw_bytes, reps, sms / reps, sg, wts.raw_bytes / 1e6))
+            runner.close()
+
     result = {
         "metric": "Q4_K GEMV GB/s 4096x12288 M=1",
         "value": round(gbps, 1),

@@ -1,0 +1,152 @@
+"""Resident decoder-layer projection stack on one HIP stream.
+
+The HIP counterpart of the reference's resident projection runners
+(src/ml/cuda/qwen_full_attn_projection_runner.cr: q/k/v bundle; bin/cuda_ffn_sequence_probe.cr:
+gate/up/down): weights and activations stay on the device, every projection of every token group is
+launched back to back into the current stream, and the lifecycle goes through ResidentSequenceRunner
+(upload_weights -> reset_sequence -> run_sequence x reps -> synchronize -> read_outputs).
+
+Where the reference runs either one launch per token or weight-stationary groups of 4 tokens
+(`tbatch4`, qwen_full_attn_projection_runner.cr:274-301), this runner hands groups of up to 8 tokens
+to one weight-stationary launch.
+"""
+import numpy as np
+
+from . import hip, quant
+from .types import TensorType
+
+# (name, input, weight type, out_dim, in_dim) at the shapes of the benchmark's mixed-quant layer:
+# hidden 4096, 32 query / 8 KV heads of 128, FFN 12288; q/k/v/o/gate/up Q4_K, down Q6_K
+QWEN_LAYER_4096 = [
+    ("q", "x", TensorType.Q4_K, 4096, 4096),
+    ("k", "x", TensorType.Q4_K, 1024, 4096),
+    ("v", "x", TensorType.Q4_K, 1024, 4096),
+    ("o", "q", TensorType.Q4_K, 4096, 4096),
+    ("gate", "x", TensorType.Q4_K, 12288, 4096),
+    ("up", "x", TensorType.Q4_K, 12288, 4096),
+    ("down", "gate", TensorType.Q6_K, 4096, 12288),
+]
+
+
+class Weights:
+    """Raw GGUF bytes per projection: {name: (raw, type, out_dim, in_dim, input name)}."""
+
+    def __init__(self, hidden, entries):
+        self.hidden = hidden
+        self.entries = entries        # ordered list of (name, input, type, out_dim, in_dim, raw)
+
+    @classmethod
+    def synthetic(cls, rng, layout=QWEN_LAYER_4096):
+        from . import synth
+        hidden = layout[0][4]
+        return cls(hidden, [(n, src, t, o, i, synth.make_weights(rng, t, o, i)) for n, src, t, o, i in layout])
+
+    @property
+    def raw_bytes(self):
+        return sum(e[5].size for e in self.entries)
+
+
+class QwenProjectionStackRunner:
+    def __init__(self, weights, tokens, xs):
+        if not tokens > 0:
+            raise ValueError("tokens must be positive")
+        if len(xs) != tokens * weights.hidden:
+            raise ValueError("xs size mismatch")
+        self.weights, self.tokens, self.hidden = weights, tokens, weights.hidden
+        self._xs = np.ascontiguousarray(xs, dtype=np.float32)
+        self._buffers = []
+        self._w = {}
+        self._act = {"x": self._alloc(4 * tokens * self.hidden)}
+        for name, src, t, out_dim, in_dim, raw in weights.entries:
+            self._w[name] = self._alloc(raw.size)
+            self._act[name] = self._alloc(4 * tokens * out_dim)
+        self.outputs = {}
+        self._runner = hip.ResidentSequenceRunner(
+            tokens, self._upload_weights, self._reset_sequence, self._run_token, self._read_outputs,
+            self._run_sequence)
+
+    @classmethod
+    def from_weights(cls, weights, tokens, xs):
+        return cls(weights, tokens, xs)
+
+    def _alloc(self, nbytes):
+        b = hip.DeviceBuffer(nbytes)
+        self._buffers.append(b)
+        return b
+
+    # ---- closures handed to ResidentSequenceRunner -------------------------------------------------
+    def _upload_weights(self):
+        for name, src, t, out_dim, in_dim, raw in self.weights.entries:
+            hip.copy_htod(self._w[name].ptr, raw, raw.size, "%s weights" % name)
+
+    def _reset_sequence(self):
+        hip.copy_htod(self._act["x"].ptr, self._xs, self._xs.nbytes, "sequence input")
+
+    def _launch(self, tok0, count):
+        stream = hip.current_stream_handle()
+        for name, src, t, out_dim, in_dim, raw in self.weights.entries:
+            quant.gemv_dev(self._w[name].ptr, t, self._act[src].ptr + 4 * tok0 * in_dim,
+                           self._act[name].ptr + 4 * tok0 * out_dim, in_dim, out_dim, count, 0, stream)
+
+    def _run_token(self, tok):
+        self._launch(tok, 1)
+
+    def _run_sequence(self, active_tokens):
+        for tok0 in range(0, active_tokens, quant.MAX_GEMV_TOKENS):
+            self._launch(tok0, min(quant.MAX_GEMV_TOKENS, active_tokens - tok0))
+
+    def _read_outputs(self):
+        hip.synchronize("hipDeviceSynchronize(read_outputs)")
+        for name, src, t, out_dim, in_dim, raw in self.weights.entries:
+            out = np.empty(self.tokens * out_dim, dtype=np.float32)
+            hip.copy_dtoh(out, self._act[name].ptr, out.nbytes, "%s output" % name)
+            self.outputs[name] = out
+
+    # ---- public lifecycle, as the reference runner's (qwen_full_attn_projection_runner.cr:111-165) ----
+    def upload_weights(self):
+        self._runner.upload_weights()
+
+    def replace_sequence_input(self, xs):
+        if len(xs) != self.tokens * self.hidden:
+            raise ValueError("xs size mismatch")
+        self._xs = np.ascontiguousarray(xs, dtype=np.float32)
+
+    def reset_sequence(self):
+        self._runner.reset_sequence()
+
+    def run_sequence(self):
+        self._runner.run_sequence()
+
+    def run_repeated(self, reps):
+        return self._runner.run_repeated(reps)
+
+    @property
+    def active_tokens(self):
+        return self._runner.active_tokens
+
+    @active_tokens.setter
+    def active_tokens(self, count):
+        self._runner.active_tokens = count
+
+    def reset_active_tokens(self):
+        self._runner.reset_active_tokens()
+
+    def read_outputs(self):
+        self._runner.read_outputs()
+
+    def device_ptr(self, name):
+        return self._act[name].ptr
+
+    def bytes_per_sequence(self, active_tokens=None):
+        """Algorithmic bytes of one run_sequence: every weight once per group of up to 8 tokens, x in, out out."""
+        m = self.tokens if active_tokens is None else active_tokens
+        groups = -(-m // quant.MAX_GEMV_TOKENS)
+        total = 0
+        for name, src, t, out_dim, in_dim, raw in self.weights.entries:
+            total += groups * raw.size + 4 * m * (in_dim + out_dim)
+        return total
+
+    def close(self):
+        for b in self._buffers:
+            b.close()
+        self._buffers = []
