@@ -3,6 +3,7 @@
 #include "ml_hip_driver.h"
 
 #include <hip/hip_runtime_api.h>
+#include <cstdio>
 #include <cstring>
 
 extern "C" {
@@ -17,7 +18,12 @@ int mlhip_device_get(int32_t* device, int32_t ordinal) {
 }
 
 int mlhip_device_get_name(char* name, int32_t len, int32_t device) {
-  return (int)hipDeviceGetName(name, len, (hipDevice_t)device);
+  hipError_t e = hipDeviceGetName(name, len, (hipDevice_t)device);
+  if (e == hipSuccess && name && len > 0 && name[0] == '\0') {   // some containers expose no marketing name
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) std::snprintf(name, (size_t)len, "AMD %s", prop.gcnArchName);
+  }
+  return (int)e;
 }
 
 int mlhip_device_compute_capability(int32_t* major, int32_t* minor, int32_t device) {
