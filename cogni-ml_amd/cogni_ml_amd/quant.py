@@ -53,6 +53,15 @@ def gemv_launch_dims(w_type, tokens, in_dim, out_dim):
     return g.value, b.value, s.value
 
 
+def gemv_plan(w_type, tokens, in_dim, out_dim, add=False):
+    """(kernel_name, grid_x, block_x, shared_mem_bytes) the library launches for this shape."""
+    k = ctypes.c_char_p()
+    g, b, s = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+    _check(hip.lib().cogni_gemv_plan(int(w_type), tokens, int(add), in_dim, out_dim, ctypes.byref(k), ctypes.byref(g),
+                                     ctypes.byref(b), ctypes.byref(s)))
+    return k.value.decode(), g.value, b.value, s.value
+
+
 def dequantize_dev(w_ptr, w_type, n_elements, out_ptr, stream=None):
     _check(hip.lib().cogni_dequantize_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)),
                                           ctypes.c_uint64(n_elements), ctypes.c_uint64(out_ptr), stream))

@@ -246,6 +246,25 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
   return launch(name, grid, 256, 0, params, stream);
 }
 
+int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, uint32_t out_dim, const char** kernel,
+                    uint32_t* grid_x, uint32_t* block_x, uint32_t* shared_mem_bytes) {
+  static thread_local char buf[64];
+  if (!kernel || !grid_x || !block_x || !shared_mem_bytes || !gemv_type(type) || tokens < 1 ||
+      tokens > COGNI_MAX_GEMV_TOKENS || in_dim == 0 || out_dim == 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_plan: bad argument");
+  // two to four tokens of a Q4_K matrix go to the matrix-core kernel; one token is faster on the vector ALU
+  if (tokens >= 2 && gemv_mfma_supported(type, (int)tokens, in_dim)) {
+    std::snprintf(buf, sizeof buf, "q4_k_gemv_mfma_%sf32_tbatch%u", add ? "add_" : "", tokens);
+    *kernel = buf;
+    *grid_x = gemv_mfma_grid((int)tokens, in_dim, out_dim);
+    *block_x = GEMV_MFMA_WAVES * 64;
+    *shared_mem_bytes = gemv_mfma_lds_bytes((int)tokens, in_dim);
+    return 0;
+  }
+  *kernel = cogni_gemv_kernel_name(type, tokens, add);
+  return cogni_gemv_launch_dims(type, tokens, in_dim, out_dim, grid_x, block_x, shared_mem_bytes);
+}
+
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out, uint32_t in_dim,
                    uint32_t out_dim, uint32_t tokens, void* stream) {
   if (!gemv_type(w_type))
@@ -254,15 +273,20 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: zero dimension");
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
-  for (uint32_t t0 = 0; t0 < tokens; t0 += COGNI_MAX_GEMV_TOKENS) {
-    const uint32_t left = tokens - t0, cap = COGNI_MAX_GEMV_TOKENS;
+  // tokens per launch: groups of up to 4 where the matrix-core kernel takes the shape (two passes over the
+  // weights for 5..8 tokens are still far cheaper than one pass on the vector ALU), else up to 8
+  const uint32_t cap = gemv_mfma_supported(w_type, GEMV_MFMA_MAX_TOKENS, in_dim) ? (uint32_t)GEMV_MFMA_MAX_TOKENS
+                                                                                : (uint32_t)COGNI_MAX_GEMV_TOKENS;
+  for (uint32_t t0 = 0; t0 < tokens; t0 += cap) {
+    const uint32_t left = tokens - t0;
     const uint32_t m = left < cap ? left : cap;
     uint32_t grid = 0, block = 0, shmem = 0;
-    cogni_gemv_launch_dims(w_type, m, in_dim, out_dim, &grid, &block, &shmem);
+    const char* kernel = nullptr;
+    int rc = cogni_gemv_plan(w_type, m, residual != 0, in_dim, out_dim, &kernel, &grid, &block, &shmem);
+    if (rc != 0) return rc;
+    const std::string name = kernel;
     uint64_t xm = x + (uint64_t)t0 * in_dim * 4, om = out + (uint64_t)t0 * out_dim * 4;
     uint64_t rm = residual ? residual + (uint64_t)t0 * out_dim * 4 : 0;
-    const std::string name = cogni_gemv_kernel_name(w_type, m, residual != 0);
-    int rc;
     if (residual) {
       void* params[] = {&w_raw, &xm, &rm, &om, &in_dim, &out_dim};
       rc = launch(name.c_str(), grid, block, shmem, params, stream);

@@ -3,5 +3,13 @@
 // its PTX modules (src/ml/cuda/driver.cr:115-127).
 #include "kernels/dequant.cuh"
 #include "kernels/gemv.cuh"
+#include "kernels/gemv_mfma.cuh"
 #include "kernels/gemm_q4k.cuh"
 #include "kernels/util.cuh"
+
+GEMV_MFMA_ENTRY(q4_k_gemv_mfma_f32_tbatch2, 2)
+GEMV_MFMA_ENTRY(q4_k_gemv_mfma_f32_tbatch3, 3)
+GEMV_MFMA_ENTRY(q4_k_gemv_mfma_f32_tbatch4, 4)
+GEMV_MFMA_ADD_ENTRY(q4_k_gemv_mfma_add_f32_tbatch2, 2)
+GEMV_MFMA_ADD_ENTRY(q4_k_gemv_mfma_add_f32_tbatch3, 3)
+GEMV_MFMA_ADD_ENTRY(q4_k_gemv_mfma_add_f32_tbatch4, 4)

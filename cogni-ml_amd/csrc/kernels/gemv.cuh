@@ -46,6 +46,12 @@ __device__ __forceinline__ float mix2(u32 t, float a, float b, float acc) {
   return acc;
 }
 
+struct gemv_true { static constexpr bool value = true; };
+struct gemv_false { static constexpr bool value = false; };
+#ifndef GEMV_PIPELINED
+#define GEMV_PIPELINED 1
+#endif
+#define GEMV_PIPELINE_MAX_GRID 4096u
 #define TWO_P24 16777216.0f
 #define TWO_P20 1048576.0f
 
@@ -99,15 +105,18 @@ struct FmtK45 {
   template <int R>
   static __device__ __forceinline__ void load(Stage<R>& st, const uint8_t* const (&rowp)[R], const Lane& ln,
                                               u32 set, u32 nb) {
-    const u32 off = min(set * 16 + ln.jb, nb - 1) * BB;   // a row is far below 4 GiB
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      st.hdr[r] = ld16(rowp[r] + off);
-      st.q0[r] = ld16(rowp[r] + (off + QOFF + 32 * ln.g));
-      st.q1[r] = ld16(rowp[r] + (off + QOFF + 32 * ln.g + 16));
-      st.h0[r] = Q5 ? ld16(rowp[r] + (off + 16)) : make_uint4(0u, 0u, 0u, 0u);
-      st.h1[r] = Q5 ? ld16(rowp[r] + (off + 32)) : make_uint4(0u, 0u, 0u, 0u);
-    }
+    for (int r = 0; r < R; r++) load_row<R>(st, r, rowp[r], ln, set, nb);
+  }
+  template <int R>
+  static __device__ __forceinline__ void load_row(Stage<R>& st, int r, const uint8_t* rp, const Lane& ln, u32 set,
+                                                  u32 nb) {
+    const u32 off = min(set * 16 + ln.jb, nb - 1) * BB;   // a row is far below 4 GiB
+    st.hdr[r] = ld16(rp + off);
+    st.q0[r] = ld16(rp + (off + QOFF + 32 * ln.g));
+    st.q1[r] = ld16(rp + (off + QOFF + 32 * ln.g + 16));
+    st.h0[r] = Q5 ? ld16(rp + (off + 16)) : make_uint4(0u, 0u, 0u, 0u);
+    st.h1[r] = Q5 ? ld16(rp + (off + 32)) : make_uint4(0u, 0u, 0u, 0u);
   }
 
   // contribution of this lane's 64 weights of row r to MG tokens
@@ -206,15 +215,18 @@ struct FmtQ6K {
   template <int R>
   static __device__ __forceinline__ void load(Stage<R>& st, const uint8_t* const (&rowp)[R], const Lane& ln,
                                               u32 set, u32 nb) {
-    const u32 off = min(set * 16 + ln.jb, nb - 1) * BB;
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      st.qa[r] = ld16(rowp[r] + (off + 64 * ln.n + 16 * ln.v));
-      st.qb[r] = ld16(rowp[r] + (off + 64 * ln.n + 32 + 16 * ln.v));
-      st.qh[r] = ld16(rowp[r] + (off + 128 + 32 * ln.n + 16 * ln.v));
-      st.sc[r] = ld8(rowp[r] + (off + 192 + 8 * ln.n));
-      st.d[r] = ld2(rowp[r] + (off + 208));
-    }
+    for (int r = 0; r < R; r++) load_row<R>(st, r, rowp[r], ln, set, nb);
+  }
+  template <int R>
+  static __device__ __forceinline__ void load_row(Stage<R>& st, int r, const uint8_t* rp, const Lane& ln, u32 set,
+                                                  u32 nb) {
+    const u32 off = min(set * 16 + ln.jb, nb - 1) * BB;
+    st.qa[r] = ld16(rp + (off + 64 * ln.n + 16 * ln.v));
+    st.qb[r] = ld16(rp + (off + 64 * ln.n + 32 + 16 * ln.v));
+    st.qh[r] = ld16(rp + (off + 128 + 32 * ln.n + 16 * ln.v));
+    st.sc[r] = ld8(rp + (off + 192 + 8 * ln.n));
+    st.d[r] = ld2(rp + (off + 208));
   }
 
   template <int R, int MG>
@@ -312,12 +324,15 @@ struct FmtQ80 {
   template <int R>
   static __device__ __forceinline__ void load(Stage<R>& st, const uint8_t* const (&rowp)[R], const Lane& ln,
                                               u32 set, u32 nb) {
-    const u32 off = min(set * 32 + ln.jb, nb - 1) * BB;
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-      st.qs[r] = ld16(rowp[r] + (off + 2 + 16 * ln.hf));
-      st.d[r] = ld2(rowp[r] + off);
-    }
+    for (int r = 0; r < R; r++) load_row<R>(st, r, rowp[r], ln, set, nb);
+  }
+  template <int R>
+  static __device__ __forceinline__ void load_row(Stage<R>& st, int r, const uint8_t* rp, const Lane& ln, u32 set,
+                                                  u32 nb) {
+    const u32 off = min(set * 32 + ln.jb, nb - 1) * BB;
+    st.qs[r] = ld16(rp + (off + 2 + 16 * ln.hf));
+    st.d[r] = ld2(rp + off);
   }
 
   template <int R, int MG>
@@ -454,6 +469,56 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     }
   };
 
+  // (one token only: with two the registers no longer allow it; and only while the grid is a few
+  // workgroups per compute unit - a long grid keeps the memory pipeline full by itself and is better off
+  // with every load queued at once)
+  if (M == 1 && NG == 1 && F::SPI == 1 && GEMV_PIPELINED && gridDim.x <= GEMV_PIPELINE_MAX_GRID) {
+    // Rolling pipeline over (column set, row): PF rows are in flight while one is consumed. A compute unit
+    // accepts only so many loads at a time and serves its oldest wavefronts first, so a wavefront that
+    // queues all its loads up front sits in the issue of them, and the ones served last still have all
+    // their arithmetic to do when the last byte arrives. Here the arithmetic of a row starts as soon as
+    // that row is there, and what is left after the last byte is one row's worth.
+    constexpr int PF = R >= 4 ? 2 : 1;
+    typename F::template Stage<R> st;
+    float4 buf[FU];
+    stage_begin(0, 0, buf);
+#pragma unroll
+    for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nb);
+    stage_end(0, 0, buf);
+    // one column set; `last` (a compile-time tag) says that no column set follows, so the prefetches that
+    // would wrap into the next set are left out and the number of loads in flight stays a constant
+    auto column_set = [&](u32 s, auto last) {
+      if (s > 0 && (s % CH) == 0) {
+        stage_begin(s, 0, buf);
+        stage_end(s, 0, buf);
+      }
+      const bool valid = s * F::BPS + ln.jb < nb;
+      float4 xr[MG][NF4];
+      float sx[MG][NSUM];
+#pragma unroll
+      for (int mm = 0; mm < MG; mm++) {
+        const u32 cm = mm * CH + (s % CH);
+#pragma unroll
+        for (int i = 0; i < NF4; i++) xr[mm][i] = xs[(cm * NF4 + i) * 64 + lane];
+#pragma unroll
+        for (int k = 0; k < NSUM; k++) sx[mm][k] = xsum[(cm * NSUM + k) * 64 + lane];
+      }
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const int rr = (r + PF) % R;
+        if (r + PF < R) F::template load_row<R>(st, rr, rowp[rr], ln, s, nb);
+        else if constexpr (!decltype(last)::value) F::template load_row<R>(st, rr, rowp[rr], ln, s + 1, nb);
+        __builtin_amdgcn_sched_barrier(0);
+        float c[MG];
+        F::template compute<R, MG>(st, r, ln, xr, sx, c);
+#pragma unroll
+        for (int mm = 0; mm < MG; mm++) acc[r][mm] += valid ? c[mm] : 0.0f;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    for (u32 s = 0; s + 1 < ncs; s++) column_set(s, gemv_false{});
+    column_set(ncs - 1, gemv_true{});
+  } else
   // Column sets are taken F::SPI at a time: all their weight loads are issued before the first is consumed.
   for (u32 s = 0; s < ncs; s += F::SPI) {
     const bool restage = NG == 1 && (s % CH) == 0;   // CH is a multiple of SPI or covers the whole row

@@ -63,3 +63,42 @@ static inline unsigned gemv_lds_bytes(unsigned type, int tokens, unsigned in_dim
   const int ch = ng > 1 ? 1 : gemv_chunk_sets(per_set_f4, ncs);
   return (unsigned)(per_set_f4 * ch) * 16u + (unsigned)(mg * nsum * 64 * ch) * 4u;
 }
+
+// ---- matrix-core GEMV (gemv_mfma.cuh): 8 wavefronts per workgroup ------------------------------------
+#define GEMV_MFMA_WAVES 8
+#define GEMV_MFMA_TMAX 3            // 16-row tiles a wavefront carries at most
+#define GEMV_MFMA_MAX_TOKENS 4
+// (token, super-block) pairs of activations a workgroup stages (tokens * in_dim / 256) at most
+#define GEMV_MFMA_MAX_UNITS(M) ((M) >= 3 ? 64 : 96)
+
+// log2 of the k-slices a workgroup's wavefronts form: the largest power of two <= min(8, super-blocks)
+static inline GEMV_HD unsigned gemv_mfma_log2_kslices(unsigned nsb) {
+  unsigned lg = 0;
+  while (lg < 3 && (2u << lg) <= nsb) lg++;
+  return lg;
+}
+// Shapes the matrix-core kernel takes: Q4_K, 1..4 tokens, in_dim a multiple of 256, all activations staged at once.
+static inline int gemv_mfma_supported(unsigned type, int tokens, unsigned in_dim) {
+  if (type != 12 || tokens < 1 || tokens > GEMV_MFMA_MAX_TOKENS || in_dim == 0 || (in_dim & 255u)) return 0;
+  return (unsigned)tokens * (in_dim >> 8) <= (unsigned)GEMV_MFMA_MAX_UNITS(tokens);
+}
+// 16-row tiles per row group and the grid: aim at one workgroup per compute unit (256 of them)
+static inline unsigned gemv_mfma_tiles(int tokens, unsigned in_dim, unsigned out_dim) {
+  (void)tokens;
+  const unsigned nwr = GEMV_MFMA_WAVES >> gemv_mfma_log2_kslices(in_dim >> 8);
+  const unsigned ntiles = (out_dim + 15) / 16, tmax = (unsigned)GEMV_MFMA_TMAX;
+  unsigned t = ntiles / (nwr * 256u);
+  if (t < 1) t = 1;
+  if (t > tmax) t = tmax;
+  return t;
+}
+static inline unsigned gemv_mfma_grid(int tokens, unsigned in_dim, unsigned out_dim) {
+  const unsigned nwr = GEMV_MFMA_WAVES >> gemv_mfma_log2_kslices(in_dim >> 8);
+  const unsigned ntiles = (out_dim + 15) / 16, per_wg = nwr * gemv_mfma_tiles(tokens, in_dim, out_dim);
+  return (ntiles + per_wg - 1) / per_wg;
+}
+static inline unsigned gemv_mfma_lds_bytes(int tokens, unsigned in_dim) {
+  const int mp = tokens <= 1 ? 1 : (tokens <= 2 ? 2 : 4);
+  return 64u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * 1024u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * (unsigned)mp * 64u +
+         (unsigned)tokens * (in_dim >> 8) * (4u + 32u + 1024u);
+}

@@ -78,6 +78,13 @@ const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add);
  * No GPU needed. */
 int cogni_gemv_launch_dims(uint32_t type, uint32_t tokens, uint32_t in_dim, uint32_t out_dim, uint32_t* grid_x,
                            uint32_t* block_x, uint32_t* shared_mem_bytes);
+/* The kernel the library itself launches for this shape, with its geometry: for 2..4 tokens of a Q4_K matrix
+ * whose activations fit the staging buffer (tokens * in_dim / 256 <= 96, or 64 from 3 tokens) that is the
+ * matrix-core variant "q4_k_gemv_mfma_[add_]f32_tbatchM" (same parameter list, block 512), otherwise the kernel
+ * cogni_gemv_kernel_name / cogni_gemv_launch_dims describe. *kernel points at thread-local storage that the
+ * next call on the thread overwrites. tokens in 1..COGNI_MAX_GEMV_TOKENS. No GPU needed. */
+int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, uint32_t out_dim, const char** kernel,
+                    uint32_t* grid_x, uint32_t* block_x, uint32_t* shared_mem_bytes);
 /* Kernel symbol "dequantize_<type>_f32"; parameters (w_raw:u64, out:u64, n_elements:u64); block = 256
  * threads, any grid (grid-stride). NULL for an unsupported type. No GPU needed. */
 const char* cogni_dequantize_kernel_name(uint32_t type);
@@ -97,8 +104,8 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 
 /* Decode GEMV, weights read once for all tokens:
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
- * fp32 accumulation. tokens >= 1; more than COGNI_MAX_GEMV_TOKENS are issued as consecutive launches
- * of up to 8 tokens. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
+ * fp32 accumulation. tokens >= 1; they are issued as consecutive launches of up to 8 tokens (up to 4 where
+ * cogni_gemv_plan picks the matrix-core kernel). in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
  * same, bin/cuda_q4k_gemv_probe.cr:125); Q8_0 accepts any in_dim >= 1 (its last block is clipped,
  * quant_matmul.cr:241,259). Types: Q8_0, Q4_K, Q5_K, Q6_K. */
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,

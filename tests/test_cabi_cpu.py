@@ -81,6 +81,26 @@ def test_gemv_launch_dims():
         quant.gemv_launch_dims(12, 9, 256, 16)
 
 
+def test_gemv_plan_picks_the_kernel_for_the_shape():
+    # one token: the vector-ALU kernel and its geometry
+    assert quant.gemv_plan(12, 1, 4096, 12288) == ("q4_k_gemv_f32",) + quant.gemv_launch_dims(12, 1, 4096, 12288)
+    # 2..4 tokens of a Q4_K matrix: the matrix-core kernel, 8 wavefronts, one workgroup per 48 rows at 12288 rows
+    name, grid, block, lds = quant.gemv_plan(12, 4, 4096, 12288)
+    assert (name, grid, block) == ("q4_k_gemv_mfma_f32_tbatch4", 256, 512)
+    assert lds == 64 + 8 * 3 * 1024 + 8 * 3 * 4 * 64 + 4 * 16 * (4 + 32 + 1024)
+    assert quant.gemv_plan(12, 2, 4096, 12288, add=True)[0] == "q4_k_gemv_mfma_add_f32_tbatch2"
+    assert quant.gemv_plan(12, 2, 4096, 4096)[1] == 256 and quant.gemv_plan(12, 2, 1024, 3584)[1] == 112
+    # activations that do not fit the staging buffer, other types, more tokens: the vector-ALU kernels
+    assert quant.gemv_plan(12, 4, 12288, 4096)[0] == "q4_k_gemv_f32_tbatch4"
+    assert quant.gemv_plan(12, 2, 12288, 4096)[0] == "q4_k_gemv_mfma_f32_tbatch2"
+    assert quant.gemv_plan(14, 4, 4096, 4096)[0] == "q6_k_gemv_f32_tbatch4"
+    assert quant.gemv_plan(12, 8, 4096, 4096)[0] == "q4_k_gemv_f32_tbatch8"
+    with pytest.raises(quant.QuantError):
+        quant.gemv_plan(12, 9, 4096, 4096)
+    with pytest.raises(quant.QuantError):
+        quant.gemv_plan(20, 1, 4096, 4096)
+
+
 def test_argument_errors_do_not_need_a_gpu():
     import numpy as np
     x = np.zeros(256, dtype=np.float32)

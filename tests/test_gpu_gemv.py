@@ -154,6 +154,53 @@ def test_linearity_and_determinism_at_full_size(gpu):
     assert np.array_equal(run_gemv(raw, Q4_K, 2 * a, in_dim, out_dim, 1), 2 * fa)
     fb, fab = run_gemv(raw, Q4_K, b, in_dim, out_dim, 1), run_gemv(raw, Q4_K, a + b, in_dim, out_dim, 1)
     assert np.max(np.abs((fa + fb) - fab)) <= 1e-4 * np.max(np.abs(fab))
-    # tokens batched in one launch give the same bits as one launch per token
+    # two tokens in one launch (the matrix-core kernel for this shape): reproducible, and the same values as
+    # one launch per token up to the order of the fp32 additions
     both = run_gemv(raw, Q4_K, np.concatenate([a, b]), in_dim, out_dim, 2)
-    assert np.array_equal(both[:out_dim], fa) and np.array_equal(both[out_dim:], fb)
+    assert np.array_equal(both, run_gemv(raw, Q4_K, np.concatenate([a, b]), in_dim, out_dim, 2))
+    scale = np.max(np.abs(fab))
+    assert np.max(np.abs(both[:out_dim] - fa)) <= 2e-5 * scale and np.max(np.abs(both[out_dim:] - fb)) <= 2e-5 * scale
+    # a token's result does not depend on its neighbours in the launch
+    swapped = run_gemv(raw, Q4_K, np.concatenate([b, a]), in_dim, out_dim, 2)
+    assert np.array_equal(swapped[out_dim:], both[:out_dim]) and np.array_equal(swapped[:out_dim], both[out_dim:])
+
+
+MFMA_SHAPES = [(256, 17), (512, 100), (768, 33), (1024, 3584), (2048, 48), (2304, 250), (4096, 1024), (8192, 300)]
+
+
+@pytest.mark.parametrize("in_dim,out_dim", MFMA_SHAPES)
+@pytest.mark.parametrize("tokens", [2, 3, 4, 7])
+def test_q4_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
+    """2..4 tokens of a Q4_K matrix run on the matrix cores where the activations fit the staging buffer:
+    odd row counts, every k-slice split (1, 2, 3, 4, 8, 9, 16, 32 super-blocks), with and without residual."""
+    rng = np.random.default_rng(in_dim * 131 + out_dim * 7 + tokens)
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = rng.standard_normal(tokens * out_dim).astype(np.float32)
+    m = min(tokens, 4)
+    name = quant.gemv_plan(Q4_K, m, in_dim, out_dim)[0]
+    expect_mfma = m * (in_dim // 256) <= (64 if m >= 3 else 96)
+    assert ("mfma" in name) == expect_mfma, name
+    check(oracle, raw, Q4_K, x, in_dim, out_dim, tokens, None, "%dx%d M=%d" % (in_dim, out_dim, tokens))
+    check(oracle, raw, Q4_K, x, in_dim, out_dim, tokens, res, "%dx%d M=%d add" % (in_dim, out_dim, tokens))
+
+
+def test_q4_k_matrix_core_kernel_activation_ranges(gpu, oracle):
+    """The matrix-core kernel feeds the activations as binary16 pairs scaled per token and super-block: values
+    far outside the binary16 range, zeros and mixed magnitudes must come out as from fp32 arithmetic."""
+    rng = np.random.default_rng(77)
+    in_dim, out_dim, tokens = 4096, 512, 4
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim).reshape(tokens, in_dim)
+    x[0] *= np.float32(1e-30)                       # far below the smallest binary16 subnormal
+    x[1] *= np.float32(1e30)                        # far above the largest binary16 number
+    x[2, :256] = 0.0                                # an all-zero super-block
+    x[2, 256:512] *= np.float32(1e-12)
+    x[2, 700] = np.float32(3e7)                     # one huge value among small ones
+    x[3] = np.where(rng.random(in_dim) < 0.5, x[3] * np.float32(1e-6), x[3] * np.float32(1e4)).astype(np.float32)
+    x = np.ascontiguousarray(x.reshape(-1))
+    got, want, frac = check(oracle, raw, Q4_K, x, in_dim, out_dim, tokens, None, "activation ranges")
+    # relative to each token's own output scale
+    g, w_ = got.reshape(tokens, out_dim).astype(np.float64), want.reshape(tokens, out_dim)
+    for m in range(tokens):
+        assert np.max(np.abs(g[m] - w_[m])) <= 2e-5 * np.max(np.abs(w_[m])), m

@@ -55,11 +55,13 @@ def test_active_token_prefix_and_per_token_path(gpu, oracle, weights):
         runner.run_sequence()
         runner.read_outputs()
         grouped = runner.outputs["k"].copy()
-        # token-local path: one launch per token gives the same bits for the active prefix
+        # token-local path: one launch per token gives the same values for the active prefix (another kernel
+        # than the three-token launch, so up to the order of the fp32 additions)
         for tok in range(3):
             runner._run_token(tok)
         runner.read_outputs()
-        assert np.array_equal(runner.outputs["k"][:3 * 1024], grouped[:3 * 1024])
+        single = runner.outputs["k"][:3 * 1024]
+        assert np.max(np.abs(single - grouped[:3 * 1024])) <= 2e-5 * np.max(np.abs(single))
         with pytest.raises(ValueError, match="active_tokens must be <= tokens"):
             runner.active_tokens = 7
         runner.reset_active_tokens()
