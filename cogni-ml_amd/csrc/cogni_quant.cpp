@@ -320,15 +320,12 @@ int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, u
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: workspace has " + std::to_string(workspace_bytes) + " bytes, needs " + std::to_string(need));
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 191) / 192;
   {
-    const uint64_t pieces = (uint64_t)need / 16;
-    uint64_t g = (pieces + 255) / 256;
-    uint32_t grid = (uint32_t)(g < 16384 ? g : 16384);
     void* params[] = {&x, &workspace, &tokens, &in_dim};
-    int rc = launch("pack_x_f16_q4k", grid, 256, 0, params, stream);
+    int rc = launch("pack_x_f16_q4k", mtiles * 4 * (in_dim / 256), 256, 0, params, stream);
     if (rc != 0) return rc;
   }
   void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};
-  return launch("q4_k_gemm_f16", mtiles * ntiles, 256, 0, params, stream);
+  return launch("q4_k_gemm_f16", 8 * ((mtiles * ntiles + 7) / 8), 256, 0, params, stream);
 }
 
 int cogni_set_gemm_threshold(int32_t tokens) {

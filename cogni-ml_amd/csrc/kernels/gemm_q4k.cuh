@@ -5,9 +5,9 @@
 // the rate of 16x16x32 (about 32 vs 2 x 32 clocks for the same 32768 flops per SIMD), hence the tile shape.
 //
 // Two kernels:
-//   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, any grid
+//   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 4 * in_dim/256
 //   q4_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
-//                   block 256, grid ceil(m/128) * ceil(out_dim/192), no dynamic LDS (128 KiB static)
+//                   block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), no dynamic LDS (128 KiB static)
 //
 // Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows, so 512 x 12288 gives 256
 // workgroups, one per CU. K is walked one 256-value super-block at a time = 16 MFMA k-steps of 16.
@@ -35,6 +35,7 @@
 
 #define GEMM_BM 128
 #define GEMM_BN 192
+#define GEMM_XCDS 8
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
@@ -51,31 +52,40 @@ __device__ __forceinline__ u32 gemm_k_element(u32 ks, u32 kg, u32 e) {
   return 64 * g + 32 * (op >> 1) + 16 * h + 8 * (op & 1) + perm;
 }
 
+// One workgroup packs 32 tokens x one super-block (256 k): the fp32 rows are read 1 KiB at a time (a wavefront
+// per row), converted, transposed through LDS into the [k-step][k-group][token][8 halves] image and written out
+// as 32 runs of 512 contiguous bytes. Grid: ceil(m/128) * 4 * (in_dim/256) workgroups, x fastest.
+#define PACK_TOK 32
 extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q4k(const float* __restrict__ x, uint4* __restrict__ xp,
                                                                   u32 m, u32 in_dim) {
+  // [32 (k-step, k-group)][32 tokens] uint4, each (k-step, k-group) row padded by one uint4 so that the
+  // transposing 8-byte writes of a wavefront (same token, 32 different rows) spread over the banks
+  __shared__ uint2 img[32 * (PACK_TOK + 1) * 2];
   const u32 nkb = in_dim >> 8;
-  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM;
-  const u64 total = (u64)mtiles * nkb * 4096;   // 16-byte pieces
-  const u64 step = (u64)gridDim.x * blockDim.x;
-  for (u64 idx = (u64)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += step) {
-    const u32 tok = idx & 127, kg = (idx >> 7) & 1, ks = (idx >> 8) & 15;
-    const u64 tile = idx >> 12;
-    const u32 kb = (u32)(tile % nkb), mt = (u32)(tile / nkb);
-    const u32 row = mt * GEMM_BM + tok;
-    uint4 o = make_uint4(0u, 0u, 0u, 0u);
-    if (row < m) {
-      const float* src = x + (size_t)row * in_dim + kb * 256 + gemm_k_element(ks, kg, 0);   // e = 0 is the base
-      float4 a, b;
-      __builtin_memcpy(&a, src, 16);
-      __builtin_memcpy(&b, src + 4, 16);
-      const __half2 p0 = __floats2half2_rn(a.x, a.z), p1 = __floats2half2_rn(a.y, a.w);
-      const __half2 p2 = __floats2half2_rn(b.x, b.z), p3 = __floats2half2_rn(b.y, b.w);
-      o.x = *reinterpret_cast<const u32*>(&p0);
-      o.y = *reinterpret_cast<const u32*>(&p1);
-      o.z = *reinterpret_cast<const u32*>(&p2);
-      o.w = *reinterpret_cast<const u32*>(&p3);
-    }
-    xp[idx] = o;
+  const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const u32 kb = blockIdx.x % nkb, tq = (blockIdx.x / nkb) & 3, mt = blockIdx.x / (4 * nkb);
+  // lane -> 4 consecutive k = 4 lane .. 4 lane + 3 of the super-block; their place in the image (inverse of
+  // gemm_k_element): group g = k / 64, high-nibble half, 16-byte half h, upper-8-bytes bit, slot 0 or 4
+  const u32 k0 = 4 * lane, g = k0 >> 6, hi = (k0 >> 5) & 1, h = (k0 >> 4) & 1, up = (k0 >> 3) & 1, slot4 = (k0 >> 2) & 1;
+  const u32 ks = 8 * (g & 1) + 4 * h + 2 * hi + up, kg = g >> 1;
+  const u32 cell = (ks * 2 + kg) * (PACK_TOK + 1);
+#pragma unroll
+  for (int p = 0; p < PACK_TOK / 4; p++) {
+    const u32 tl = 4 * p + wave;
+    const u32 row = mt * GEMM_BM + tq * PACK_TOK + tl;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (row < m) __builtin_memcpy(&v, x + (size_t)row * in_dim + kb * 256 + k0, 16);
+    const __half2 p0 = __floats2half2_rn(v.x, v.z), p1 = __floats2half2_rn(v.y, v.w);   // slot order 0,2,1,3
+    uint2 o;
+    o.x = *reinterpret_cast<const u32*>(&p0);
+    o.y = *reinterpret_cast<const u32*>(&p1);
+    img[(cell + tl) * 2 + slot4] = o;
+  }
+  __syncthreads();
+  uint4* dst = xp + ((size_t)mt * nkb + kb) * 4096 + tq * PACK_TOK;
+  for (u32 i = tid; i < 32 * PACK_TOK; i += 256) {
+    const u32 c = i / PACK_TOK, tl = i % PACK_TOK;
+    dst[c * 128 + tl] = *reinterpret_cast<const uint4*>(&img[(c * (PACK_TOK + 1) + tl) * 2]);
   }
 }
 
@@ -108,8 +118,16 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 j = lane & 31, kg = lane >> 5;
   const u32 g = 2 * kg + kh;
   const u32 nkb = in_dim >> 8;
-  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM;
-  const u32 mt = blockIdx.x % mtiles, nt = blockIdx.x / mtiles;
+  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_BN - 1) / GEMM_BN;
+  // Workgroup -> tile, XCD-aware. Workgroups go to the 8 XCDs round-robin (id % 8) and each XCD has its own
+  // L2, so the tiles are numbered token-tile-major and XCD x takes the contiguous run [x*per, (x+1)*per):
+  // the workgroups that share an L2 then share one or two x tiles (1 MiB each at in_dim 4096), which stay
+  // resident while the weights stream through. Numbered the other way round every L2 sees every x tile,
+  // and at M = 512 the x tiles alone (4 MiB) fill it. The grid is 8 * per; the surplus workgroups leave.
+  const u32 per = (mtiles * ntiles + GEMM_XCDS - 1) / GEMM_XCDS;
+  const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
+  if (vt >= mtiles * ntiles) return;
+  const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
   const u32 n0 = nt * GEMM_BN + nh * 96;             // first weight row of this wavefront
   const size_t row_bytes = (size_t)nkb * 144;
   const u32 sh = 16u * (g & 1);
@@ -142,17 +160,18 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   };
 
   // Stage super-block 0 of x and the first weights. The main loop below takes super-blocks in pairs with
-  // fixed buffer roles (buffer 0 then buffer 1) and no branch in its body; with an odd number of
-  // super-blocks the first one is taken alone out of buffer 1.
+  // fixed roles (x buffer 0 then 1, weight registers A then B) and no branch or register copy in its body;
+  // with an odd number of super-blocks the first one is taken alone out of buffer 1 / registers B.
   const bool odd = nkb & 1;
-  GemmRaw cur[3];
-  load_raw(cur, 0);
+  GemmRaw rawA[3], rawB[3];
   if (odd) {
+    load_raw(rawB, 0);
 #pragma unroll
     for (int i = 0; i < 16; i++)
       __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf1 + 256 * i + wave * 64),
                                        16, 0, 0);
   } else {
+    load_raw(rawA, 0);
 #pragma unroll
     for (int i = 0; i < 16; i++)
       __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
@@ -160,22 +179,10 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   }
   __syncthreads();
 
-  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt) {
-    const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
-    // The next x tile goes global -> LDS without passing through registers (global_load_lds_dwordx4:
-    // lane l of a wavefront lands at LDS base + 16*l), into the buffer that was last read in the previous
-    // iteration, which ended with a barrier. Loads complete in issue order, so these (L2 hits) go ahead of
-    // the raw weights of the next super-block (HBM).
-    const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
-#pragma unroll
-    for (int i = 0; i < 16; i++)
-      __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64),
-                                       16, 0, 0);
-    GemmRaw nxt[3];
-    load_raw(nxt, kn);
-    __builtin_amdgcn_sched_barrier(0);   // keep the prefetches up here
-
-    // (scale, -min) of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles) as duplicated half2
+  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt, const GemmRaw (&cur)[3], GemmRaw (&nxt)[3]) {
+    // (scale, -min) of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles) as duplicated half2. First thing
+    // in the iteration: the only loads in flight here are this super-block's weights, requested one
+    // iteration ago, so the wait in front of this costs nothing and does not cover the prefetches below.
     u32 S[3][4];
 #pragma unroll
     for (int c = 0; c < 3; c++) {
@@ -189,6 +196,9 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       S[c][2] = h2_dup(d * ubyte_f<1>(scp));
       S[c][3] = h2_dup(-(dm * ubyte_f<1>(mp)));
     }
+    const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
+    const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
+    const uint8_t* knbase = wbase + (size_t)kn * 144; // uniform
 
     const uint4* arow = xcur + (16 * kh + kg) * 128 + j;   // k-steps 8*kh .. 8*kh+7; 32 lanes read 512 contiguous bytes
     auto build_b = [&](half8_t (&B)[3], int t) {
@@ -220,6 +230,23 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
     for (int t = 0; t < 8; t++) {
       const int p = t & 1;
+      // Prefetches for the next super-block, a few per k-step rather than all up front: a wavefront issues
+      // in order and the memory pipeline takes a vector memory instruction only every so many clocks, so
+      // 25 of them in a row stall the (only) wavefront of the SIMD with nothing to overlap. The raw weights
+      // (HBM, longest latency) go first, then the next x tile global -> LDS without passing through
+      // registers (global_load_lds_dwordx4: lane l of a wavefront lands at LDS base + 16*l) into the buffer
+      // that was last read in the previous iteration, which ended with a barrier.
+      if (t < 3) {
+        nxt[t].hdr = ld16(knbase + rowoff[t]);
+        nxt[t].qa = ld16(knbase + (rowoff[t] + 16 + 32 * g));
+        nxt[t].qb = ld16(knbase + (rowoff[t] + 32 + 32 * g));
+      }
+      if (t < 6) {
+#pragma unroll
+        for (int i = (t < 3 ? 2 * t : 3 * t - 3); i < (t < 3 ? 2 * t + 2 : (t < 5 ? 3 * t : 16)); i++)
+          __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64),
+                                           16, 0, 0);
+      }
       if (t < 7) {
 #pragma unroll
         for (int r = 0; r < 4; r++) A[p ^ 1][r] = arow[(t + 1) * 256 + r * 32];
@@ -231,49 +258,77 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
         for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Ar, B[p][c], acc[r][c], 0, 0, 0);
       }
-      // scheduling window = one k-step: its MFMAs interleave with the operand preparation of the next
-      // step, but the preparation of later steps is not pulled forward (it would only occupy registers)
+      // Scheduling window = one k-step. Left alone the scheduler emits the twelve MFMAs back to back and the
+      // operand preparation of the next step behind them, so the matrix pipe and the vector ALU take turns;
+      // the group barriers below ask for the interleaving instead: the loads first, then one MFMA followed
+      // by four vector instructions, twelve times (an MFMA occupies the matrix pipe for 32 clocks, four
+      // vector instructions issue in 16).
+      __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);   // VMEM reads (weights, LDS-direct x) of this step
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
+#pragma unroll
+      for (int i = 0; i < 12; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // four VALU
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    __syncthreads();   // waits for the LDS-direct loads of this wavefront, then for everybody's
-#pragma unroll
-    for (int c = 0; c < 3; c++) cur[c] = nxt[c];
+    // End of the iteration: everything this wavefront requested has to be there (the x tile for everybody,
+    // the weights for its own next iteration), then everybody meets.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
   };
-  if (odd) iteration(0, gemm_xbuf1, gemm_xbuf0);
+  if (odd) iteration(0, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
   for (u32 kb = odd; kb < nkb; kb += 2) {
-    iteration(kb, gemm_xbuf0, gemm_xbuf1);
-    iteration(kb + 1, gemm_xbuf1, gemm_xbuf0);
+    iteration(kb, gemm_xbuf0, gemm_xbuf1, rawA, rawB);
+    iteration(kb + 1, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
   }
+  __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
-  // add the two k halves: kh = 1 wavefronts hand their accumulators to their kh = 0 partners through LDS
-  // (48 KiB each, [r][c][v][lane]; the x buffers are free after the final barrier above)
-  float* xch = reinterpret_cast<float*>(nh ? gemm_xbuf1 : gemm_xbuf0);
-  if (kh == 1) {
+  // Epilogue, in two halves of 64 tokens (the tiles r = 2 hf, 2 hf + 1): every wavefront writes its partial
+  // sums to LDS as [k half][token][weight row] (row stride 200 floats: the two k-groups of a wavefront land in
+  // disjoint banks), then all 256 threads add the two k halves and the bias and store 16 bytes at a time,
+  // 48 consecutive threads per 768-byte output row segment. 2 x 64 x 200 x 4 B = 100 KiB of the 128 KiB.
+  float* part0 = reinterpret_cast<float*>(gemm_xbuf0);   // k half 0: 64 x 200 floats = 51200 B <= 64 KiB
+  float* part1 = reinterpret_cast<float*>(gemm_xbuf1);   // k half 1
+  float* mine = kh ? part1 : part0;
+  const bool full_n = nt * GEMM_BN + GEMM_BN <= out_dim;
 #pragma unroll
-    for (int r = 0; r < 4; r++)
+  for (int hf = 0; hf < 2; hf++) {
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++) {
+      const int r = 2 * hf + rr;
 #pragma unroll
       for (int c = 0; c < 3; c++)
 #pragma unroll
-        for (int v = 0; v < 16; v++) xch[((r * 3 + c) * 16 + v) * 64 + lane] = acc[r][c][v];
-  }
-  __syncthreads();
-  if (kh == 1) return;
-
-  // D layout of a 32x32 tile: register v of lane (j, kg) is row 8*(v/4) + 4*kg + v%4 (token), column j (weight row)
-#pragma unroll
-  for (int c = 0; c < 3; c++) {
-    const u32 n = n0 + 32 * c + j;
-    if (n < out_dim) {
-      const float b = bias ? bias[n] : 0.0f;
-#pragma unroll
-      for (int r = 0; r < 4; r++) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const u32 row = mt * GEMM_BM + 32 * r + 8 * (v >> 2) + 4 * kg + (v & 3);
-          if (row < m) out[(size_t)row * out_dim + n] = acc[r][c][v] + xch[((r * 3 + c) * 16 + v) * 64 + lane] + b;
+        for (int v = 0; v < 16; v++)
+          mine[(32 * rr + 8 * (v >> 2) + 4 * kg + (v & 3)) * 200 + nh * 96 + 32 * c + j] = acc[r][c][v];
+    }
+    __syncthreads();
+    const u32 row0 = mt * GEMM_BM + 64 * hf;
+    for (u32 idx = tid; idx < 64 * 48; idx += 256) {
+      const u32 tl = idx / 48, q4 = idx - tl * 48;
+      const u32 row = row0 + tl, n = nt * GEMM_BN + 4 * q4;
+      if (row < m && n < out_dim) {
+        const float4 p0 = *reinterpret_cast<const float4*>(part0 + tl * 200 + 4 * q4);
+        const float4 p1 = *reinterpret_cast<const float4*>(part1 + tl * 200 + 4 * q4);
+        float4 o = make_float4(p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w);
+        float* dst = out + (size_t)row * out_dim + n;
+        if (full_n || n + 4 <= out_dim) {
+          if (bias) {
+            o.x += bias[n]; o.y += bias[n + 1]; o.z += bias[n + 2]; o.w += bias[n + 3];
+          }
+          if ((out_dim & 3u) == 0) {
+            *reinterpret_cast<float4*>(dst) = o;
+          } else {
+            dst[0] = o.x; dst[1] = o.y; dst[2] = o.z; dst[3] = o.w;
+          }
+        } else {
+          const float ov[4] = {o.x, o.y, o.z, o.w};
+          for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (bias ? bias[n + e] : 0.0f);
         }
-        __builtin_amdgcn_sched_barrier(0);   // one tile at a time: keeps the LDS reads from piling up in registers
       }
     }
+    if (hf == 0) __syncthreads();
   }
 }

@@ -118,7 +118,8 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
  * device memory of at least cogni_gemm_workspace_bytes(...) bytes (x repacked as fp16); nothing is allocated.
  * Kernels: pack_x_f16_q4k (x, workspace, tokens, in_dim) then
  *          q4_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,
- *          grid ceil(tokens/128)*ceil(out_dim/192), no dynamic shared memory. */
+ *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/192)/8), no dynamic shared memory.
+ * (pack_x_f16_q4k: block 256, grid ceil(tokens/128)*4*(in_dim/256).) */
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
                    uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream);
