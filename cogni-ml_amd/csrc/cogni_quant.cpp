@@ -273,10 +273,15 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: zero dimension");
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
-  // tokens per launch: groups of up to 4 where the matrix-core kernel takes the shape (two passes over the
-  // weights for 5..8 tokens are still far cheaper than one pass on the vector ALU), else up to 8
-  const uint32_t cap = gemv_mfma_supported(w_type, GEMV_MFMA_MAX_TOKENS, in_dim) ? (uint32_t)GEMV_MFMA_MAX_TOKENS
-                                                                                : (uint32_t)COGNI_MAX_GEMV_TOKENS;
+  // tokens per launch: groups of up to 4 where the matrix-core kernel takes the shape (several passes over
+  // the weights are still cheaper than one pass on the vector ALU, measured up to 8 tokens), else up to 8
+  uint32_t cap = COGNI_MAX_GEMV_TOKENS;
+  for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2; mt--) {
+    if (gemv_mfma_supported(w_type, mt, in_dim)) {   // the most tokens whose activations fit its staging buffer
+      cap = (uint32_t)mt;
+      break;
+    }
+  }
   for (uint32_t t0 = 0; t0 < tokens; t0 += cap) {
     const uint32_t left = tokens - t0;
     const uint32_t m = left < cap ? left : cap;

@@ -18,7 +18,7 @@
 //
 // Weights never touch LDS. In MFMA terms a lane is (weight row j = lane % 32, k-group kg = lane / 32)
 // and supplies 8 k values per k-step. Lane (j, kg) of a kh wavefront owns the 64-value group
-// g = 2*kg + kh of its row's super-block: the 32 bytes qs[32g, 32g+32) as two 16-byte loads, one
+// g = 2*kh + kg of its row's super-block: the 32 bytes qs[32g, 32g+32) as two 16-byte loads, one
 // (scale, min) pair decode. Eight consecutive bytes give two k-steps: their low nibbles (sub-block 2g)
 // and their high nibbles (sub-block 2g+1). A masked dword (q & 0x000F000F) | 0x64006400 is the half2
 // (1024 + n0, 1024 + n4); subtracting 1024 and one packed fma give fp16(d*sc*n - dmin*m) for two
@@ -44,10 +44,11 @@ typedef const __attribute__((address_space(1))) void gbl_void;
 
 // Element (0..255) of a super-block that k-slot (ks, kg, e) of the MFMA stands for. ks = 8*kh + 4*h + op:
 // kh = k half (which wavefront), h = 16-byte half of the lane's group, op & 1 = upper 8 bytes of that
-// half, op >> 1 = high nibbles. The group is g = 2*kg + kh.
+// half, op >> 1 = high nibbles. The group is g = 2*kh + kg: the two k-groups of a wavefront read 64 adjacent
+// bytes of a row, so a wavefront touches one or two cache lines per row rather than two or three.
 __device__ __forceinline__ u32 gemm_k_element(u32 ks, u32 kg, u32 e) {
   const u32 kh = ks >> 3, h = (ks >> 2) & 1, op = ks & 3;
-  const u32 g = 2 * kg + kh;
+  const u32 g = 2 * kh + kg;
   const u32 perm = ((e & 1) << 1) | ((e >> 1) & 1) | (e & 4);   // 0,2,1,3,4,6,5,7
   return 64 * g + 32 * (op >> 1) + 16 * h + 8 * (op & 1) + perm;
 }
@@ -67,7 +68,7 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q4k(const float* __
   // lane -> 4 consecutive k = 4 lane .. 4 lane + 3 of the super-block; their place in the image (inverse of
   // gemm_k_element): group g = k / 64, high-nibble half, 16-byte half h, upper-8-bytes bit, slot 0 or 4
   const u32 k0 = 4 * lane, g = k0 >> 6, hi = (k0 >> 5) & 1, h = (k0 >> 4) & 1, up = (k0 >> 3) & 1, slot4 = (k0 >> 2) & 1;
-  const u32 ks = 8 * (g & 1) + 4 * h + 2 * hi + up, kg = g >> 1;
+  const u32 ks = 8 * (g >> 1) + 4 * h + 2 * hi + up, kg = g & 1;
   const u32 cell = (ks * 2 + kg) * (PACK_TOK + 1);
 #pragma unroll
   for (int p = 0; p < PACK_TOK / 4; p++) {
@@ -116,7 +117,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const u32 nh = wave & 1, kh = wave >> 1;
   const u32 j = lane & 31, kg = lane >> 5;
-  const u32 g = 2 * kg + kh;
+  const u32 g = 2 * kh + kg;
   const u32 nkb = in_dim >> 8;
   const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_BN - 1) / GEMM_BN;
   // Workgroup -> tile, XCD-aware. Workgroups go to the 8 XCDs round-robin (id % 8) and each XCD has its own
@@ -261,14 +262,20 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       // Scheduling window = one k-step. Left alone the scheduler emits the twelve MFMAs back to back and the
       // operand preparation of the next step behind them, so the matrix pipe and the vector ALU take turns;
       // the group barriers below ask for the interleaving instead: the loads first, then one MFMA followed
-      // by four vector instructions, twelve times (an MFMA occupies the matrix pipe for 32 clocks, four
-      // vector instructions issue in 16).
+      // by five vector instructions, twelve times (an MFMA occupies the matrix pipe for 32 clocks, five
+      // vector instructions issue in 20 to 35).
+      if (t < 7) {
+        // keep the operands built above inside this window (otherwise they sink next to their first use,
+        // behind the window's MFMAs)
+#pragma unroll
+        for (int c = 0; c < 3; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
+      }
       __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);   // VMEM reads (weights, LDS-direct x) of this step
       __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
 #pragma unroll
       for (int i = 0; i < 12; i++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);   // four VALU
+        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // five VALU
       }
       __builtin_amdgcn_sched_barrier(0);
     }

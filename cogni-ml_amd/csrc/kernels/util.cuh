@@ -12,8 +12,9 @@ extern "C" __global__ __launch_bounds__(256) void copy_bytes_16(const uint4* __r
   for (u64 i = tid; i < n; i += step) dst[i] = src[i];
 }
 
-// (src, out, n_bytes): every thread XORs the 16-byte words it reads; one dword per workgroup is
-// written to out[blockIdx.x] so the loads cannot be dropped. block = 256, any grid.
+// (src, out, n_bytes): every thread XORs the 16-byte words it reads; the result is stored only if it has one
+// particular value, which keeps the loads alive and the kernel free of any epilogue. block = 256, any grid
+// (about 8 workgroups per compute unit reads a 28 MB buffer fastest).
 extern "C" __global__ __launch_bounds__(256) void read_bytes_16(const uint4* __restrict__ src,
                                                                  u32* __restrict__ out, u64 n_bytes) {
   const u64 n = n_bytes >> 4;
@@ -23,14 +24,7 @@ extern "C" __global__ __launch_bounds__(256) void read_bytes_16(const uint4* __r
     const uint4 v = src[i];
     a ^= v.x ^ v.y ^ v.z ^ v.w;
   }
-  __shared__ u32 red[256];
-  red[threadIdx.x] = a;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    u32 t = 0;
-    for (int i = 0; i < 256; i++) t ^= red[i];
-    out[blockIdx.x] = t;
-  }
+  if (a == 0x12345678u) out[tid & 1023] = a;
 }
 
 // (src f32, dst f16, n): round-to-nearest-even; n multiple of 4 is the fast path. block = 256, any grid.
