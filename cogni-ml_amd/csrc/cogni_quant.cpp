@@ -275,7 +275,9 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
   // tokens per launch: groups of up to 4 where the matrix-core kernel takes the shape (several passes over
   // the weights are still cheaper than one pass on the vector ALU, measured up to 8 tokens), else up to 8
-  uint32_t cap = COGNI_MAX_GEMV_TOKENS;
+  // (the vector-ALU kernels of the K-quants hold two tokens in registers and take a third in a second pass over
+  // the staged weights at little cost, a fourth costs as much as the first two: groups of 3 measure fastest)
+  uint32_t cap = k_quant(w_type) ? 3u : (uint32_t)COGNI_MAX_GEMV_TOKENS;
   for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2; mt--) {
     if (gemv_mfma_supported(w_type, mt, in_dim)) {   // the most tokens whose activations fit its staging buffer
       cap = (uint32_t)mt;

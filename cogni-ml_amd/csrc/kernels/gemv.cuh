@@ -532,7 +532,6 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     step(stA, s);
     if (two) step(stB, s + 1);
   }
-
 #pragma unroll
   for (int r = 0; r < R; r++) {
 #pragma unroll

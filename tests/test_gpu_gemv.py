@@ -78,7 +78,7 @@ def test_single_output_row_and_many_tokens(gpu, oracle):
     check(oracle, raw, Q4_K, synth.make_activations(rng, 1, 512), 512, 1, 1)
     raw = synth.make_weights(rng, Q6_K, 40, 512)
     res = rng.standard_normal(19 * 40).astype(np.float32)
-    check(oracle, raw, Q6_K, synth.make_activations(rng, 19, 512), 512, 40, 19, res, "19 tokens = 8 + 8 + 3")
+    check(oracle, raw, Q6_K, synth.make_activations(rng, 19, 512), 512, 40, 19, res, "19 tokens in several launches")
 
 
 CONFIGS = [
