@@ -292,6 +292,26 @@ def main():
             c.close()
 
     if args.mode == "cases":
+        # the gate | up pair of one layer against the same x in one launch (q4_k_dual_gemv_f32)
+        a = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES)
+        b = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES)
+        out_b = hip.DeviceBuffer(4 * 12288)
+
+        def dual(i, st):
+            quant.gemv_dual_dev(a.w[i % a.copies].ptr, b.w[i % b.copies].ptr, Q4_K, a.x.ptr, a.out.ptr, out_b.ptr, 4096, 12288,
+                                1, st.handle)
+        dsteps = max(20, min(args.steps, 1000))
+        dms, _ = time_steps(hip, stream, dual, dsteps, min(args.warmup, dsteps))
+        dbytes = 2 * a.w_bytes + 4 * 4096 + 2 * 4 * 12288
+        dg = dbytes / (dms / dsteps * 1e-3) / 1e9
+        extra["q4_k gate|up pair, one launch"] = {"gbps": round(dg, 1), "ms": round(dms / dsteps, 5), "frac_hbm": round(dg / HBM_PEAK_GBPS, 4)}
+        log("case=q4_k gate|up pair in one launch\ntype=Q4_K\nshape=2 x 4096x12288\ntokens=1\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\ngbps_hbm=%.1f\n" % (
+            2 * a.w_bytes, dsteps, dms / dsteps, dg))
+        a.close()
+        b.close()
+        out_b.close()
+
+    if args.mode == "cases":
         # config 5: the mixed-quant projection stack, resident, back to back in one stream
         from cogni_ml_amd.projection_stack import QwenProjectionStackRunner, Weights
         wts = Weights.synthetic(rng)

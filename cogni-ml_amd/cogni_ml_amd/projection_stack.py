@@ -84,9 +84,21 @@ class QwenProjectionStackRunner:
 
     def _launch(self, tok0, count):
         stream = hip.current_stream_handle()
-        for name, src, t, out_dim, in_dim, raw in self.weights.entries:
+        ents = self.weights.entries
+        i = 0
+        while i < len(ents):
+            name, src, t, out_dim, in_dim, raw = ents[i]
+            nxt = ents[i + 1] if i + 1 < len(ents) else None
+            if nxt is not None and nxt[1:5] == (src, t, out_dim, in_dim):
+                # two projections of one shape on the same input (k | v, gate | up) share one launch
+                quant.gemv_dual_dev(self._w[name].ptr, self._w[nxt[0]].ptr, t, self._act[src].ptr + 4 * tok0 * in_dim,
+                                    self._act[name].ptr + 4 * tok0 * out_dim, self._act[nxt[0]].ptr + 4 * tok0 * out_dim,
+                                    in_dim, out_dim, count, stream)
+                i += 2
+                continue
             quant.gemv_dev(self._w[name].ptr, t, self._act[src].ptr + 4 * tok0 * in_dim,
                            self._act[name].ptr + 4 * tok0 * out_dim, in_dim, out_dim, count, 0, stream)
+            i += 1
 
     def _run_token(self, tok):
         self._launch(tok, 1)

@@ -73,6 +73,13 @@ def gemv_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens=1, residual_
                                     ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+def gemv_dual_dev(w_a_ptr, w_b_ptr, w_type, x_ptr, out_a_ptr, out_b_ptr, in_dim, out_dim, tokens=1, stream=None):
+    """Two matrices of one shape against the same activations (gate | up, k | v)."""
+    _check(hip.lib().cogni_gemv_dual_dev(ctypes.c_uint64(w_a_ptr), ctypes.c_uint64(w_b_ptr), ctypes.c_uint32(int(w_type)),
+                                         ctypes.c_uint64(x_ptr), ctypes.c_uint64(out_a_ptr), ctypes.c_uint64(out_b_ptr),
+                                         ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
 def gemm_workspace_bytes(w_type, in_dim, tokens):
     f = hip.lib().cogni_gemm_workspace_bytes
     f.restype = ctypes.c_size_t

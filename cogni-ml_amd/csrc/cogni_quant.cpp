@@ -66,11 +66,12 @@ int get_fn(const char* name, hipFunction_t* out) {
   return 0;
 }
 
-int launch(const char* name, uint32_t grid, uint32_t block, uint32_t shmem, void** params, void* stream) {
+int launch(const char* name, uint32_t grid, uint32_t block, uint32_t shmem, void** params, void* stream,
+           uint32_t grid_y = 1) {
   hipFunction_t fn = nullptr;
   int rc = get_fn(name, &fn);
   if (rc != 0) return rc;
-  HIP_TRY(hipModuleLaunchKernel(fn, grid, 1, 1, block, 1, 1, shmem, (hipStream_t)stream, params, nullptr),
+  HIP_TRY(hipModuleLaunchKernel(fn, grid, grid_y, 1, block, 1, 1, shmem, (hipStream_t)stream, params, nullptr),
           std::string("hipModuleLaunchKernel(") + name + ")");
   return 0;
 }
@@ -304,6 +305,28 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
     if (rc != 0) return rc;
   }
   return 0;
+}
+
+int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uint64_t x, uint64_t out_a, uint64_t out_b,
+                        uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (!gemv_type(w_type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for fused matmul: ") + type_name(w_type));
+  if (!w_raw_a || !w_raw_b || !x || !out_a || !out_b)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dual_dev: null device pointer");
+  if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dual_dev: zero dimension");
+  if (w_type == COGNI_TYPE_Q4_K && tokens == 1 && (in_dim % 256) == 0) {
+    uint32_t grid = 0, block = 0, shmem = 0;
+    int rc = cogni_gemv_launch_dims(w_type, 1, in_dim, out_dim, &grid, &block, &shmem);
+    if (rc != 0) return rc;
+    const uint32_t rows = (uint32_t)gemv_rows_per_block(w_type, 1);
+    grid = (2 * out_dim + rows - 1) / rows;
+    void* params[] = {&w_raw_a, &w_raw_b, &x, &out_a, &out_b, &in_dim, &out_dim};
+    return launch("q4_k_dual_gemv_f32", grid, block, shmem, params, stream);
+  }
+  // other types, several tokens: the pair as two launches of the kernels cogni_gemv_dev picks
+  int rc = cogni_gemv_dev(w_raw_a, w_type, x, 0, out_a, in_dim, out_dim, tokens, stream);
+  if (rc != 0) return rc;
+  return cogni_gemv_dev(w_raw_b, w_type, x, 0, out_b, in_dim, out_dim, tokens, stream);
 }
 
 int g_gemm_threshold = -1;   // -1: not resolved yet

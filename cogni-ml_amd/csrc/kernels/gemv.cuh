@@ -356,10 +356,15 @@ struct FmtQ80 {
 };
 
 // ---------------------------------------------------------------------------------------------
-template <class F, int M, bool ADD>
+// DUAL: two matrices of the same shape share the activations in one launch; output row r of the launch is
+// row r of w / out for r < out_dim and row r - out_dim of w_b / out_b above (the reference's
+// q4_k_dual_gemv_warp4_f32, src/ml/cuda/kernels/q4k_dual_gemv_probe.ptx:5-52, used for the gate | up and
+// similar projection pairs, src/ml/cuda/qwen_recurrent_layer_runner.cr:519-520).
+template <class F, int M, bool ADD, bool DUAL = false>
 __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                           const float* __restrict__ residual, float* __restrict__ out,
-                                          u32 in_dim, u32 out_dim) {
+                                          u32 in_dim, u32 out_dim, const uint8_t* __restrict__ w_b = nullptr,
+                                          float* __restrict__ out_b = nullptr) {
   constexpr int R = F::rows(M);
   constexpr int MG = M < F::MG_MAX ? M : F::MG_MAX;   // tokens held in registers at a time
   constexpr int NG = (M + MG - 1) / MG;
@@ -378,9 +383,13 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   const size_t row_bytes = F::row_bytes(nb);
   const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
 
+  const u32 total_rows = DUAL ? 2 * out_dim : out_dim;
   const uint8_t* rowp[R];
 #pragma unroll
-  for (int r = 0; r < R; r++) rowp[r] = w + (size_t)min(row0 + r, out_dim - 1) * row_bytes;
+  for (int r = 0; r < R; r++) {
+    const u32 row = min(row0 + r, total_rows - 1);
+    rowp[r] = (DUAL && row >= out_dim) ? w_b + (size_t)(row - out_dim) * row_bytes : w + (size_t)row * row_bytes;
+  }
 
   float acc[R][M];
 #pragma unroll
@@ -538,10 +547,14 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     for (int m = 0; m < M; m++) {
       float v = wave_sum(acc[r][m]);
       const u32 row = row0 + r;
-      if (lane == 0 && row < out_dim) {
-        const size_t o = (size_t)m * out_dim + row;
-        if (ADD) v += residual[o];
-        out[o] = v;
+      if (lane == 0 && row < total_rows) {
+        if (DUAL && row >= out_dim) {
+          out_b[(size_t)m * out_dim + (row - out_dim)] = v;
+        } else {
+          const size_t o = (size_t)m * out_dim + row;
+          if (ADD) v += residual[o];
+          out[o] = v;
+        }
       }
     }
   }
@@ -586,3 +599,13 @@ GEMV_FAMILY(q4_k, FmtQ4K)
 GEMV_FAMILY(q5_k, FmtQ5K)
 GEMV_FAMILY(q6_k, FmtQ6K)
 GEMV_FAMILY(q8_0, FmtQ80)
+
+// (w_raw_a, w_raw_b, x, out_a, out_b, in_dim, out_dim): one token per grid.y slice (x + y * in_dim, out_* + y * out_dim),
+// grid.x = ceil(2 * out_dim / rows per workgroup), same block and dynamic shared memory as q4_k_gemv_f32.
+// The reference has this pair as q4_k_dual_gemv_warp4_f32 and ..._batched (q4k_dual_gemv_probe.ptx:5, 233).
+extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(1) void q4_k_dual_gemv_f32(
+    const uint8_t* w_a, const uint8_t* w_b, const float* x, float* out_a, float* out_b, u32 in_dim, u32 out_dim) {
+  const size_t tok = blockIdx.y;
+  gemv_core<FmtQ4K, 1, false, true>(w_a, x + tok * in_dim, nullptr, out_a + tok * out_dim, in_dim, out_dim, w_b,
+                                    out_b + tok * out_dim);
+}

@@ -2,8 +2,10 @@
 // A workgroup is 4 wavefronts; each wavefront owns GEMV_ROWS_*(tokens) consecutive output rows.
 #pragma once
 
-#define GEMV_BLOCK 256
+#ifndef GEMV_WAVES
 #define GEMV_WAVES 4
+#endif
+#define GEMV_BLOCK (64 * GEMV_WAVES)
 
 #define GEMV_ROWS_Q4K(M) ((M) <= 2 ? 4 : 2)
 #define GEMV_ROWS_Q5K(M) 2

@@ -112,6 +112,17 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
                    uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 
+/* Two matrices of one shape against the same activations (the gate | up, k | v pairs):
+ *   out_a[m*out_dim + o] = sum_j x[m*in_dim + j] * deq(W_a[o][j]),  out_b likewise with W_b.
+ * One token of a Q4_K pair is one launch of "q4_k_dual_gemv_f32" (w_raw_a, w_raw_b, x, out_a, out_b, in_dim, out_dim),
+ * the parameter list of the reference's q4_k_dual_gemv_warp4_f32 (src/ml/cuda/kernels/q4k_dual_gemv_probe.ptx:5-13,
+ * used by src/ml/cuda/qwen_recurrent_layer_runner.cr:519-520): output row r of the launch is row r of W_a for
+ * r < out_dim and row r - out_dim of W_b above; block and dynamic shared memory as cogni_gemv_launch_dims gives for
+ * one token, grid_x = ceil(2*out_dim / rows per workgroup), grid_y = tokens (one token per slice, x + y*in_dim,
+ * out_* + y*out_dim, the reference's ..._batched entry). Every other case is issued as two cogni_gemv_dev calls. */
+int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uint64_t x, uint64_t out_a, uint64_t out_b,
+                        uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
+
 /* Prefill GEMM for `tokens` > 8 (Q4_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
  * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
  * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:

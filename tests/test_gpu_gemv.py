@@ -204,3 +204,29 @@ def test_q4_k_matrix_core_kernel_activation_ranges(gpu, oracle):
     g, w_ = got.reshape(tokens, out_dim).astype(np.float64), want.reshape(tokens, out_dim)
     for m in range(tokens):
         assert np.max(np.abs(g[m] - w_[m])) <= 2e-5 * np.max(np.abs(w_[m])), m
+
+
+@pytest.mark.parametrize("type_id,in_dim,out_dim,tokens", [(Q4_K, 4096, 12288, 1), (Q4_K, 512, 37, 1), (Q4_K, 1024, 1024, 3),
+                                                            (Q6_K, 512, 40, 1), (Q4_K, 4096, 1024, 1)])
+def test_dual_gemv_shares_activations(gpu, oracle, type_id, in_dim, out_dim, tokens):
+    """Two matrices of one shape against the same x (gate | up, k | v): one launch for one token of a Q4_K pair,
+    including a row count that puts the a | b boundary inside a wavefront's rows."""
+    rng = np.random.default_rng(in_dim + 3 * out_dim + tokens)
+    raw_a = synth.make_weights(rng, type_id, out_dim, in_dim)
+    raw_b = synth.make_weights(rng, type_id, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    wa, wb, xd = DevArray(raw_a), DevArray(raw_b), DevArray(x)
+    oa, ob = DevArray(nbytes=4 * tokens * out_dim), DevArray(nbytes=4 * tokens * out_dim)
+    quant.gemv_dual_dev(wa.ptr, wb.ptr, type_id, xd.ptr, oa.ptr, ob.ptr, in_dim, out_dim, tokens)
+    zero = np.zeros(out_dim, dtype=np.float32)
+    for raw, o in ((raw_a, oa), (raw_b, ob)):
+        got = o.read(np.float32, tokens * out_dim)
+        want = oracle.matmul_add(x, tokens, in_dim, raw, type_id, out_dim, zero, threads=8).astype(np.float64)
+        dense = np.abs(oracle.dequantize(raw, type_id, out_dim * in_dim)).reshape(out_dim, in_dim)
+        tol = gemv_tolerance(x, dense, tokens, in_dim).reshape(-1)
+        assert np.all(np.abs(got.astype(np.float64) - want) <= tol)
+    if tokens == 1 and type_id == Q4_K:   # the pair in one launch gives the bits of the single-matrix kernel
+        assert np.array_equal(oa.read(np.float32, out_dim), run_gemv(raw_a, type_id, x, in_dim, out_dim, 1))
+        assert np.array_equal(ob.read(np.float32, out_dim), run_gemv(raw_b, type_id, x, in_dim, out_dim, 1))
+    for d in (wa, wb, xd, oa, ob):
+        d.close()
