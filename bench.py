@@ -312,6 +312,28 @@ def main():
         out_b.close()
 
     if args.mode == "cases":
+        # FFN sequence of one layer: gate | up | SwiGLU in one launch, then Q6_K down with the residual add
+        from cogni_ml_amd.ffn_sequence import FFNSequenceRunner
+        graw = [synth.make_weights(rng, Q4_K, 12288, 4096) for _ in range(2)] + [synth.make_weights(rng, Q6_K, 4096, 12288)]
+        for tokens in (1, 4):
+            fx = rng.uniform(-1.0, 1.0, tokens * 4096).astype(np.float32)
+            ffn = FFNSequenceRunner(graw[0], graw[1], graw[2], 4096, 12288, tokens, fx, fx.copy())
+            ffn.upload_weights()
+            ffn.reset_sequence()
+
+            def fseq(i, st, ffn=ffn):
+                with hip.with_stream(st):
+                    ffn.run_sequence()
+            reps = max(20, min(args.steps // 4, 300))
+            fms, _ = time_steps(hip, stream, fseq, reps, 10)
+            fg = ffn.bytes_per_sequence() / (fms / reps * 1e-3) / 1e9
+            extra["ffn sequence M=%d" % tokens] = {"gbps": round(fg, 1), "ms": round(fms / reps, 5), "frac_hbm": round(fg / HBM_PEAK_GBPS, 4)}
+            log("case=ffn sequence (gate|up Q4_K -> SwiGLU -> down Q6_K + residual)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\n"
+                "gbps=%.1f\nnote=weights %.0f MB stay in the 256 MB last-level cache between repetitions\n" % (
+                    tokens, sum(r.size for r in graw), reps, fms / reps, fg, sum(r.size for r in graw) / 1e6))
+            ffn.close()
+
+    if args.mode == "cases":
         # config 5: the mixed-quant projection stack, resident, back to back in one stream
         from cogni_ml_amd.projection_stack import QwenProjectionStackRunner, Weights
         wts = Weights.synthetic(rng)

@@ -1,0 +1,105 @@
+"""Resident FFN sequence on one HIP stream: Q4_K gate and up GEMVs -> SwiGLU -> Q6_K down GEMV (+ residual).
+
+The HIP counterpart of the reference's FFN sequence probe (bin/cuda_ffn_sequence_probe.cr:3, 254-266 for the
+CPU form, 314-440 for the launches): weights and activations stay on the device, the lifecycle goes through
+ResidentSequenceRunner. Where the reference launches gate, up, the activation and down as four kernels per token,
+one token here is two launches (gate | up | SwiGLU fused, then down with the residual add); several tokens go
+through the weight-stationary kernels (gate | up pair, swiglu_f32, down).
+"""
+import numpy as np
+
+from . import hip, quant
+from .types import TensorType
+
+
+class FFNSequenceRunner:
+    def __init__(self, gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, residual=None, down_type=TensorType.Q6_K):
+        if not tokens > 0:
+            raise ValueError("tokens must be positive")
+        if len(xs) != tokens * hidden:
+            raise ValueError("xs size mismatch")
+        if residual is not None and len(residual) != tokens * hidden:
+            raise ValueError("residual size mismatch")
+        self.hidden, self.ffn_dim, self.tokens, self.down_type = hidden, ffn_dim, tokens, down_type
+        self._raw = {"gate": gate_raw, "up": up_raw, "down": down_raw}
+        self._xs = np.ascontiguousarray(xs, dtype=np.float32)
+        self._residual = None if residual is None else np.ascontiguousarray(residual, dtype=np.float32)
+        self._buffers = []
+        self._w = {k: self._alloc(v.size) for k, v in self._raw.items()}
+        self._x = self._alloc(4 * tokens * hidden)
+        self._res = self._alloc(4 * tokens * hidden) if residual is not None else None
+        self._gate = self._alloc(4 * tokens * ffn_dim)      # only used when several tokens run together
+        self._up = self._alloc(4 * tokens * ffn_dim)
+        self._act = self._alloc(4 * tokens * ffn_dim)
+        self._out = self._alloc(4 * tokens * hidden)
+        self.combined = self.out = None
+        self._runner = hip.ResidentSequenceRunner(tokens, self._upload_weights, self._reset_sequence, self._run_token,
+                                                  self._read_outputs, self._run_sequence)
+
+    def _alloc(self, nbytes):
+        b = hip.DeviceBuffer(nbytes)
+        self._buffers.append(b)
+        return b
+
+    def _upload_weights(self):
+        for k, raw in self._raw.items():
+            hip.copy_htod(self._w[k].ptr, raw, raw.size, "%s weights" % k)
+
+    def _reset_sequence(self):
+        hip.copy_htod(self._x.ptr, self._xs, self._xs.nbytes, "sequence input")
+        if self._res is not None:
+            hip.copy_htod(self._res.ptr, self._residual, self._residual.nbytes, "residual")
+
+    def _launch(self, tok0, count):
+        st = hip.current_stream_handle()
+        h, f = self.hidden, self.ffn_dim
+        x, act = self._x.ptr + 4 * tok0 * h, self._act.ptr + 4 * tok0 * f
+        if count == 1:
+            quant.gemv_dual_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, x, act, h, f, 1, st)
+        else:
+            g, u = self._gate.ptr + 4 * tok0 * f, self._up.ptr + 4 * tok0 * f
+            quant.gemv_dual_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, x, g, u, h, f, count, st)
+            quant.swiglu_dev(g, u, act, count * f, st)
+        res = self._res.ptr + 4 * tok0 * h if self._res is not None else 0
+        quant.gemv_dev(self._w["down"].ptr, self.down_type, act, self._out.ptr + 4 * tok0 * h, f, h, count, res, st)
+
+    def _run_token(self, tok):
+        self._launch(tok, 1)
+
+    def _run_sequence(self, active_tokens):
+        for tok0 in range(0, active_tokens, quant.MAX_GEMV_TOKENS):
+            self._launch(tok0, min(quant.MAX_GEMV_TOKENS, active_tokens - tok0))
+
+    def _read_outputs(self):
+        hip.synchronize("hipDeviceSynchronize(read_outputs)")
+        self.combined = np.empty(self.tokens * self.ffn_dim, dtype=np.float32)
+        self.out = np.empty(self.tokens * self.hidden, dtype=np.float32)
+        hip.copy_dtoh(self.combined, self._act.ptr, self.combined.nbytes, "combined")
+        hip.copy_dtoh(self.out, self._out.ptr, self.out.nbytes, "out")
+
+    # lifecycle
+    def upload_weights(self):
+        self._runner.upload_weights()
+
+    def reset_sequence(self):
+        self._runner.reset_sequence()
+
+    def run_sequence(self):
+        self._runner.run_sequence()
+
+    def run_repeated(self, reps):
+        return self._runner.run_repeated(reps)
+
+    def read_outputs(self):
+        self._runner.read_outputs()
+
+    def bytes_per_sequence(self):
+        """Algorithmic bytes: the three matrices once per group of up to 8 tokens, x and residual in, out out."""
+        groups = -(-self.tokens // quant.MAX_GEMV_TOKENS)
+        vec = 4 * self.tokens * self.hidden * (3 if self._res is not None else 2)
+        return groups * sum(r.size for r in self._raw.values()) + vec
+
+    def close(self):
+        for b in self._buffers:
+            b.close()
+        self._buffers = []

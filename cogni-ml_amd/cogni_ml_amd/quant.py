@@ -80,6 +80,19 @@ def gemv_dual_dev(w_a_ptr, w_b_ptr, w_type, x_ptr, out_a_ptr, out_b_ptr, in_dim,
                                          ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+def swiglu_dev(gate_ptr, up_ptr, out_ptr, n, stream=None):
+    _check(hip.lib().cogni_swiglu_dev(ctypes.c_uint64(gate_ptr), ctypes.c_uint64(up_ptr), ctypes.c_uint64(out_ptr),
+                                      ctypes.c_uint32(n), stream))
+
+
+def gemv_dual_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens=1, stream=None):
+    """out = silu(x W_gate^T) * (x W_up^T) in one launch (Q4_K)."""
+    _check(hip.lib().cogni_gemv_dual_swiglu_dev(ctypes.c_uint64(w_gate_ptr), ctypes.c_uint64(w_up_ptr),
+                                                ctypes.c_uint32(int(w_type)), ctypes.c_uint64(x_ptr), ctypes.c_uint64(out_ptr),
+                                                ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens),
+                                                stream))
+
+
 def gemm_workspace_bytes(w_type, in_dim, tokens):
     f = hip.lib().cogni_gemm_workspace_bytes
     f.restype = ctypes.c_size_t

@@ -329,6 +329,31 @@ int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uin
   return cogni_gemv_dev(w_raw_b, w_type, x, 0, out_b, in_dim, out_dim, tokens, stream);
 }
 
+int cogni_swiglu_dev(uint64_t gate, uint64_t up, uint64_t out, uint32_t n, void* stream) {
+  if (!gate || !up || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_swiglu_dev: null device pointer");
+  if (n == 0) return 0;
+  void* params[] = {&gate, &up, &out, &n};
+  return launch("swiglu_f32", (n + 255) / 256, 256, 0, params, stream);
+}
+
+int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t x, uint64_t out, uint32_t in_dim,
+                               uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (w_type != COGNI_TYPE_Q4_K)
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the fused gate/up SwiGLU: ") + type_name(w_type));
+  if (!w_gate || !w_up || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dual_swiglu_dev: null device pointer");
+  if (in_dim == 0 || out_dim == 0 || tokens == 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dual_swiglu_dev: zero dimension");
+  if ((in_dim % 256) != 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "Q4_K GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  uint32_t grid = 0, block = 0, shmem = 0;
+  int rc = cogni_gemv_launch_dims(w_type, 1, in_dim, out_dim, &grid, &block, &shmem);
+  if (rc != 0) return rc;
+  const uint32_t rows = (uint32_t)gemv_rows_per_block(w_type, 1) / 2;   // gate rows per workgroup (as many of up)
+  grid = (out_dim + rows - 1) / rows;
+  void* params[] = {&w_gate, &w_up, &x, &out, &in_dim, &out_dim};
+  return launch("q4_k_dual_gemv_swiglu_f32", grid, block, shmem, params, stream, tokens);
+}
+
 int g_gemm_threshold = -1;   // -1: not resolved yet
 
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {

@@ -356,11 +356,20 @@ struct FmtQ80 {
 };
 
 // ---------------------------------------------------------------------------------------------
+// silu(g) * u in fp32: g / (1 + exp(-g)), then times u (bin/cuda_ffn_sequence_probe.cr:189-191)
+__device__ __forceinline__ float swiglu_one(float g, float u) {
+  const float s = g / (1.0f + expf(-g));
+  return s * u;
+}
+
 // DUAL: two matrices of the same shape share the activations in one launch; output row r of the launch is
 // row r of w / out for r < out_dim and row r - out_dim of w_b / out_b above (the reference's
 // q4_k_dual_gemv_warp4_f32, src/ml/cuda/kernels/q4k_dual_gemv_probe.ptx:5-52, used for the gate | up and
 // similar projection pairs, src/ml/cuda/qwen_recurrent_layer_runner.cr:519-520).
-template <class F, int M, bool ADD, bool DUAL = false>
+// SWIGLU (with DUAL, M = 1): a wavefront takes R/2 rows of w (gate) and the same R/2 rows of w_b (up) and stores
+// silu(gate) * up into out - the reference's gate/up GEMVs followed by its swiglu_f32 kernel
+// (bin/cuda_ffn_sequence_probe.cr:46-84) in one launch.
+template <class F, int M, bool ADD, bool DUAL = false, bool SWIGLU = false>
 __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                           const float* __restrict__ residual, float* __restrict__ out,
                                           u32 in_dim, u32 out_dim, const uint8_t* __restrict__ w_b = nullptr,
@@ -383,12 +392,18 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   const size_t row_bytes = F::row_bytes(nb);
   const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
 
+  static_assert(!SWIGLU || (DUAL && M == 1 && !ADD && R % 2 == 0), "SWIGLU is a one-token mode of the matrix pair");
   const u32 total_rows = DUAL ? 2 * out_dim : out_dim;
   const uint8_t* rowp[R];
 #pragma unroll
   for (int r = 0; r < R; r++) {
-    const u32 row = min(row0 + r, total_rows - 1);
-    rowp[r] = (DUAL && row >= out_dim) ? w_b + (size_t)(row - out_dim) * row_bytes : w + (size_t)row * row_bytes;
+    if (SWIGLU) {   // slots 0 .. R/2-1: gate rows, slots R/2 .. R-1: the same rows of up
+      const u32 row = min(row0 / 2 + (u32)(r % (R / 2)), out_dim - 1);
+      rowp[r] = (r < R / 2 ? w : w_b) + (size_t)row * row_bytes;
+    } else {
+      const u32 row = min(row0 + r, total_rows - 1);
+      rowp[r] = (DUAL && row >= out_dim) ? w_b + (size_t)(row - out_dim) * row_bytes : w + (size_t)row * row_bytes;
+    }
   }
 
   float acc[R][M];
@@ -541,6 +556,17 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     step(stA, s);
     if (two) step(stB, s + 1);
   }
+  if constexpr (SWIGLU) {
+    float v[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) v[r] = wave_sum(acc[r][0]);
+#pragma unroll
+    for (int r = 0; r < R / 2; r++) {
+      const u32 row = row0 / 2 + r;
+      if (lane == 0 && row < out_dim) out[row] = swiglu_one(v[r], v[r + R / 2]);
+    }
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < R; r++) {
 #pragma unroll
@@ -608,4 +634,20 @@ extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(1) void q4_k_dual_g
   const size_t tok = blockIdx.y;
   gemv_core<FmtQ4K, 1, false, true>(w_a, x + tok * in_dim, nullptr, out_a + tok * out_dim, in_dim, out_dim, w_b,
                                     out_b + tok * out_dim);
+}
+
+// (w_gate, w_up, x, out, in_dim, out_dim): out[o] = silu(gate[o]) * up[o] for one token per grid.y slice; block and
+// dynamic shared memory as q4_k_gemv_f32, grid.x = ceil(out_dim / (rows per workgroup / 2)).
+extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(1) void q4_k_dual_gemv_swiglu_f32(
+    const uint8_t* w_gate, const uint8_t* w_up, const float* x, float* out, u32 in_dim, u32 out_dim) {
+  const size_t tok = blockIdx.y;
+  gemv_core<FmtQ4K, 1, false, true, true>(w_gate, x + tok * in_dim, nullptr, out + tok * out_dim, in_dim, out_dim, w_up,
+                                          nullptr);
+}
+
+// (gate, up, out, n): out[i] = silu(gate[i]) * up[i], the reference's swiglu_f32 (bin/cuda_ffn_sequence_probe.cr:46-84).
+// block = 256, grid = ceil(n / 256).
+extern "C" __global__ __launch_bounds__(256) void swiglu_f32(const float* gate, const float* up, float* out, u32 n) {
+  const u32 i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = swiglu_one(gate[i], up[i]);
 }

@@ -123,6 +123,20 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
 int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uint64_t x, uint64_t out_a, uint64_t out_b,
                         uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 
+/* out[i] = silu(gate[i]) * up[i], silu(g) = g / (1 + exp(-g)) in fp32: kernel "swiglu_f32" (gate, up, out, n:u32),
+ * block 256, grid ceil(n/256) - the reference's swiglu_f32 (bin/cuda_ffn_sequence_probe.cr:46-84, CPU form :189-191). */
+int cogni_swiglu_dev(uint64_t gate, uint64_t up, uint64_t out, uint32_t n, void* stream);
+
+/* The gate and up projections and the SwiGLU in one launch (Q4_K):
+ *   out[m*out_dim + o] = silu(sum_j x[m][j] deq(W_gate[o][j])) * sum_j x[m][j] deq(W_up[o][j])
+ * i.e. the reference's gate/up GEMVs followed by swiglu_f32 (bin/cuda_ffn_sequence_probe.cr: FFN sequence) without
+ * the intermediate vectors. Kernel "q4_k_dual_gemv_swiglu_f32" (w_gate, w_up, x, out, in_dim, out_dim): block and
+ * dynamic shared memory as for one token of cogni_gemv_launch_dims, grid_x = ceil(out_dim / (rows per workgroup / 2)),
+ * grid_y = tokens (one token per slice). Other types return COGNI_ERR_UNSUPPORTED_TYPE: compose
+ * cogni_gemv_dual_dev and cogni_swiglu_dev. */
+int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t x, uint64_t out, uint32_t in_dim,
+                               uint32_t out_dim, uint32_t tokens, void* stream);
+
 /* Prefill GEMM for `tokens` > 8 (Q4_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
  * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
  * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:

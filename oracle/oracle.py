@@ -52,6 +52,8 @@ def lib():
         for name in ("oracle_block_bytes", "oracle_block_elements"):
             getattr(L, name).restype = ctypes.c_int
             getattr(L, name).argtypes = [ctypes.c_uint32]
+        L.oracle_swiglu.restype = None
+        L.oracle_swiglu.argtypes = [f32p, f32p, ctypes.c_void_p, ctypes.c_int64]
         L.oracle_data_bytes.restype = ctypes.c_int64
         L.oracle_data_bytes.argtypes = [ctypes.c_uint32, ctypes.c_int64]
         _lib = L
@@ -125,3 +127,13 @@ def matmul_add(x, rows, in_dim, w_raw, w_type, out_dim, bias, threads=1):
     if rc != 0:
         raise ValueError("Unsupported quant type for fused matmul: %s" % w_type)
     return res
+
+
+def swiglu(gate, up):
+    """silu(gate) * up in float32, as the reference's FFN probe checks it (bin/cuda_ffn_sequence_probe.cr:189-191)."""
+    ga, gp = _f32(gate)
+    ua, up_p = _f32(up)
+    assert ga.size == ua.size
+    out = np.empty(ga.size, dtype=np.float32)
+    lib().oracle_swiglu(gp, up_p, out.ctypes.data, ctypes.c_int64(ga.size))
+    return out

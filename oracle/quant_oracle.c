@@ -533,3 +533,17 @@ int oracle_matmul_add(const float *x, int rows, int in_dim, const uint8_t *w_raw
                       int out_dim, const float *bias, float *result) {
   return oracle_matmul_add_range(x, rows, in_dim, w_raw, w_type, out_dim, bias, result, 0, out_dim);
 }
+
+/* The CPU check of the reference's SwiGLU probe (bin/cuda_ffn_sequence_probe.cr:189-191 and its use on
+ * gate/up): silu(g) = g / (1 + exp(-g)) in Float32 (Math.exp on a Float32 is the single-precision libm exp),
+ * then silu(g) * u in Float32. Pinned by the closed forms silu(0) = 0, silu(x) - silu(-x) = x and a float64
+ * evaluation (tests/test_oracle_matmul.py). */
+void oracle_swiglu(const float *gate, const float *up, float *out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) {
+    const float g = gate[i];
+    const float e = expf(-g);
+    const float den = 1.0f + e;
+    const float s = g / den;
+    out[i] = s * up[i];
+  }
+}

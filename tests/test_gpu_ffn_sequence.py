@@ -1,0 +1,48 @@
+"""The resident FFN sequence (Q4_K gate/up -> SwiGLU -> Q6_K down, optional residual add) against the CPU form the
+reference's probe checks it with (bin/cuda_ffn_sequence_probe.cr:254-266): per token, gate and up through
+QuantMatmul.matmul_add, silu(gate) * up in float32, down through matmul_add with the residual row as bias."""
+import numpy as np
+import pytest
+
+from cogni_ml_amd import hip, synth
+from cogni_ml_amd.ffn_sequence import FFNSequenceRunner
+from gpu_common import gpu  # noqa: F401
+from helpers import cosine
+
+pytestmark = pytest.mark.gpu
+Q4_K, Q6_K = 12, 14
+
+
+@pytest.mark.parametrize("hidden,ffn_dim,tokens,residual_add", [(4096, 12288, 1, True), (4096, 12288, 4, True),
+                                                               (512, 768, 1, False), (512, 768, 3, True), (1024, 256, 9, True)])
+def test_ffn_sequence_matches_cpu_form(gpu, oracle, hidden, ffn_dim, tokens, residual_add):
+    rng = np.random.default_rng(hidden + ffn_dim + tokens)
+    gate_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
+    up_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
+    down_raw = synth.make_weights(rng, Q6_K, hidden, ffn_dim)
+    xs = rng.uniform(-1.0, 1.0, tokens * hidden).astype(np.float32)            # the probe's input distribution
+    residual = rng.uniform(-1.0, 1.0, tokens * hidden).astype(np.float32) if residual_add else None
+    runner = FFNSequenceRunner(gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, residual)
+    stream = hip.HIPStream()
+    try:
+        runner.upload_weights()
+        runner.reset_sequence()
+        with hip.with_stream(stream):
+            assert runner.run_repeated(2) == 2 * tokens
+        stream.synchronize()
+        runner.read_outputs()
+        zero_f, zero_h = np.zeros(ffn_dim, dtype=np.float32), np.zeros(hidden, dtype=np.float32)
+        for tok in range(tokens):
+            x = xs[tok * hidden:(tok + 1) * hidden]
+            gate = oracle.matmul_add(x, 1, hidden, gate_raw, Q4_K, ffn_dim, zero_f, threads=8)
+            up = oracle.matmul_add(x, 1, hidden, up_raw, Q4_K, ffn_dim, zero_f, threads=8)
+            combined = oracle.swiglu(gate, up)
+            bias = residual[tok * hidden:(tok + 1) * hidden] if residual_add else zero_h
+            want = oracle.matmul_add(combined, 1, ffn_dim, down_raw, Q6_K, hidden, bias, threads=8)
+            got_c = runner.combined[tok * ffn_dim:(tok + 1) * ffn_dim]
+            got = runner.out[tok * hidden:(tok + 1) * hidden]
+            assert np.max(np.abs(got_c - combined)) <= 1e-4 * np.max(np.abs(combined)), "combined, token %d" % tok
+            assert cosine(got, want) >= 0.99999 and np.max(np.abs(got - want)) <= 1e-4 * np.max(np.abs(want)), "out, token %d" % tok
+    finally:
+        runner.close()
+        stream.close()

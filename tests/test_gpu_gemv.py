@@ -230,3 +230,42 @@ def test_dual_gemv_shares_activations(gpu, oracle, type_id, in_dim, out_dim, tok
         assert np.array_equal(ob.read(np.float32, out_dim), run_gemv(raw_b, type_id, x, in_dim, out_dim, 1))
     for d in (wa, wb, xd, oa, ob):
         d.close()
+
+
+def test_swiglu_kernel_and_fused_gate_up(gpu, oracle):
+    """swiglu_f32 against the oracle's float32 form, and the fused gate/up + SwiGLU launch against the
+    two-step composition (same bits: same GEMV arithmetic, same device function) and the oracle."""
+    rng = np.random.default_rng(4242)
+    g = (rng.standard_normal(5000) * 4).astype(np.float32)
+    g[:6] = [0.0, -0.0, 100.0, -100.0, 1e-30, -20.0]
+    u = rng.standard_normal(5000).astype(np.float32)
+    gd, ud, od = DevArray(g), DevArray(u), DevArray(nbytes=g.nbytes)
+    quant.swiglu_dev(gd.ptr, ud.ptr, od.ptr, g.size)
+    got, want = od.read(np.float32, g.size), oracle.swiglu(g, u)
+    assert np.all(np.abs(got - want) <= 4e-7 * np.abs(want) + 1e-37)          # a few ulp: the two exp differ in the last bit
+    assert got[0] == 0.0 and got[3] == 0.0                                   # silu(0) = 0, silu(-100) * u underflows to -0 / 0
+    for in_dim, out_dim, tokens in ((4096, 12288, 1), (512, 37, 1), (1024, 130, 3)):
+        raw_g = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+        raw_u = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+        x = synth.make_activations(rng, tokens, in_dim)
+        wg, wu, xd = DevArray(raw_g), DevArray(raw_u), DevArray(x)
+        n = tokens * out_dim
+        og, ou, o2, of = (DevArray(nbytes=4 * n) for _ in range(4))
+        for t in range(tokens):   # two-step composition, one token per launch as the fused kernel works
+            quant.gemv_dual_dev(wg.ptr, wu.ptr, Q4_K, xd.ptr + 4 * t * in_dim, og.ptr + 4 * t * out_dim, ou.ptr + 4 * t * out_dim,
+                                in_dim, out_dim, 1)
+        quant.swiglu_dev(og.ptr, ou.ptr, o2.ptr, n)
+        quant.gemv_dual_swiglu_dev(wg.ptr, wu.ptr, Q4_K, xd.ptr, of.ptr, in_dim, out_dim, tokens)
+        fused, two_step = of.read(np.float32, n), o2.read(np.float32, n)
+        assert np.array_equal(fused, two_step)
+        zero = np.zeros(out_dim, dtype=np.float32)
+        ref = oracle.swiglu(oracle.matmul_add(x, tokens, in_dim, raw_g, Q4_K, out_dim, zero, threads=8),
+                            oracle.matmul_add(x, tokens, in_dim, raw_u, Q4_K, out_dim, zero, threads=8))
+        assert cosine(fused, ref) >= 0.999999
+        assert np.max(np.abs(fused - ref)) <= 1e-4 * np.max(np.abs(ref))
+        for d in (wg, wu, xd, og, ou, o2, of):
+            d.close()
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for the fused gate/up SwiGLU: Q6_K"):
+        quant.gemv_dual_swiglu_dev(1, 1, Q6_K, 1, 1, 256, 16, 1)
+    for d in (gd, ud, od):
+        d.close()

@@ -179,3 +179,19 @@ def test_geometry_table(oracle):
     assert oracle.data_bytes(Q5_K, 4096 * 4096) == 11534336
     assert oracle.data_bytes(F16, 10) == 20 and oracle.data_bytes(IQ4_NL, 40) == 36
     assert oracle.block_bytes(99) == -1
+
+
+def test_swiglu_closed_forms_and_float64():
+    """silu(0) = 0; silu(x) - silu(-x) = x; silu(x) -> x for large x, -> 0 for very negative x; against float64."""
+    from oracle import oracle
+    x = np.array([0.0, 1.0, -1.0, 3.5, -3.5, 50.0, -50.0, 1e-4, -1e-4], dtype=np.float32)
+    ones = np.ones_like(x)
+    s = oracle.swiglu(x, ones)
+    assert s[0] == 0.0
+    assert np.allclose(s[1] - s[2], 1.0, atol=1e-7) and np.allclose(s[3] - s[4], 3.5, atol=1e-6)
+    assert s[5] == np.float32(50.0) and abs(s[6]) < 1e-19
+    rng = np.random.default_rng(5)
+    g, u = (rng.standard_normal(4096) * 5).astype(np.float32), rng.standard_normal(4096).astype(np.float32)
+    ref = g.astype(np.float64) / (1.0 + np.exp(-g.astype(np.float64))) * u.astype(np.float64)
+    assert np.max(np.abs(oracle.swiglu(g, u) - ref)) <= 3e-7 * np.max(np.abs(ref))
+    assert np.array_equal(oracle.swiglu(g, 2 * u), 2 * oracle.swiglu(g, u))      # exact: a power of two in the last product
