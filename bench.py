@@ -315,9 +315,12 @@ def main():
         # FFN sequence of one layer: gate | up | SwiGLU in one launch, then Q6_K down with the residual add
         from cogni_ml_amd.ffn_sequence import FFNSequenceRunner
         graw = [synth.make_weights(rng, Q4_K, 12288, 4096) for _ in range(2)] + [synth.make_weights(rng, Q6_K, 4096, 12288)]
-        for tokens in (1, 4):
+        for tokens, block in ((1, False), (4, False), (1, True)):
             fx = rng.uniform(-1.0, 1.0, tokens * 4096).astype(np.float32)
-            ffn = FFNSequenceRunner(graw[0], graw[1], graw[2], 4096, 12288, tokens, fx, fx.copy())
+            if block:   # the FFN half of a decoder layer: add + RMSNorm ahead of the projections
+                ffn = FFNSequenceRunner(graw[0], graw[1], graw[2], 4096, 12288, tokens, fx, norm=np.ones(4096, dtype=np.float32), add=fx.copy())
+            else:
+                ffn = FFNSequenceRunner(graw[0], graw[1], graw[2], 4096, 12288, tokens, fx, fx.copy())
             ffn.upload_weights()
             ffn.reset_sequence()
 
@@ -327,7 +330,7 @@ def main():
             reps = max(20, min(args.steps // 4, 300))
             fms, _ = time_steps(hip, stream, fseq, reps, 10)
             fg = ffn.bytes_per_sequence() / (fms / reps * 1e-3) / 1e9
-            extra["ffn sequence M=%d" % tokens] = {"gbps": round(fg, 1), "ms": round(fms / reps, 5), "frac_hbm": round(fg / HBM_PEAK_GBPS, 4)}
+            extra["%s M=%d" % ("add+rmsnorm+ffn" if block else "ffn sequence", tokens)] = {"gbps": round(fg, 1), "ms": round(fms / reps, 5), "frac_hbm": round(fg / HBM_PEAK_GBPS, 4)}
             log("case=ffn sequence (gate|up Q4_K -> SwiGLU -> down Q6_K + residual)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\n"
                 "gbps=%.1f\nnote=weights %.0f MB stay in the 256 MB last-level cache between repetitions\n" % (
                     tokens, sum(r.size for r in graw), reps, fms / reps, fg, sum(r.size for r in graw) / 1e6))

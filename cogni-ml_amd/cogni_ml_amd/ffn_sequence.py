@@ -5,6 +5,9 @@ CPU form, 314-440 for the launches): weights and activations stay on the device,
 ResidentSequenceRunner. Where the reference launches gate, up, the activation and down as four kernels per token,
 one token here is two launches (gate | up | SwiGLU fused, then down with the residual add); several tokens go
 through the weight-stationary kernels (gate | up pair, swiglu_f32, down).
+
+With `norm` and `add` the sequence is the whole FFN half of a decoder layer (src/ml/gguf/qwen35_cpu.cr:1705-1725):
+r = x + add (the attention output joining the residual stream), h = rmsnorm(r, norm), out = r + down(silu(gate h) * up h).
 """
 import numpy as np
 
@@ -13,13 +16,18 @@ from .types import TensorType
 
 
 class FFNSequenceRunner:
-    def __init__(self, gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, residual=None, down_type=TensorType.Q6_K):
+    def __init__(self, gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, residual=None, down_type=TensorType.Q6_K,
+                 norm=None, add=None, eps=1.0e-6):
         if not tokens > 0:
             raise ValueError("tokens must be positive")
         if len(xs) != tokens * hidden:
             raise ValueError("xs size mismatch")
         if residual is not None and len(residual) != tokens * hidden:
             raise ValueError("residual size mismatch")
+        if (norm is None) != (add is None):
+            raise ValueError("norm and add go together")
+        if norm is not None and (residual is not None or len(norm) != hidden or len(add) != tokens * hidden):
+            raise ValueError("norm/add size mismatch, or a residual given besides them")
         self.hidden, self.ffn_dim, self.tokens, self.down_type = hidden, ffn_dim, tokens, down_type
         self._raw = {"gate": gate_raw, "up": up_raw, "down": down_raw}
         self._xs = np.ascontiguousarray(xs, dtype=np.float32)
@@ -27,7 +35,13 @@ class FFNSequenceRunner:
         self._buffers = []
         self._w = {k: self._alloc(v.size) for k, v in self._raw.items()}
         self._x = self._alloc(4 * tokens * hidden)
-        self._res = self._alloc(4 * tokens * hidden) if residual is not None else None
+        self._res = self._alloc(4 * tokens * hidden) if residual is not None or norm is not None else None
+        self._eps = eps
+        self._norm_w = None if norm is None else np.ascontiguousarray(norm, dtype=np.float32)
+        self._add_h = None if add is None else np.ascontiguousarray(add, dtype=np.float32)
+        self._norm = self._alloc(4 * hidden) if norm is not None else None
+        self._add = self._alloc(4 * tokens * hidden) if norm is not None else None
+        self._normed = self._alloc(4 * tokens * hidden) if norm is not None else None
         self._gate = self._alloc(4 * tokens * ffn_dim)      # only used when several tokens run together
         self._up = self._alloc(4 * tokens * ffn_dim)
         self._act = self._alloc(4 * tokens * ffn_dim)
@@ -44,16 +58,25 @@ class FFNSequenceRunner:
     def _upload_weights(self):
         for k, raw in self._raw.items():
             hip.copy_htod(self._w[k].ptr, raw, raw.size, "%s weights" % k)
+        if self._norm is not None:
+            hip.copy_htod(self._norm.ptr, self._norm_w, self._norm_w.nbytes, "norm weights")
 
     def _reset_sequence(self):
         hip.copy_htod(self._x.ptr, self._xs, self._xs.nbytes, "sequence input")
-        if self._res is not None:
+        if self._residual is not None:
             hip.copy_htod(self._res.ptr, self._residual, self._residual.nbytes, "residual")
+        if self._add is not None:
+            hip.copy_htod(self._add.ptr, self._add_h, self._add_h.nbytes, "add")
 
     def _launch(self, tok0, count):
         st = hip.current_stream_handle()
         h, f = self.hidden, self.ffn_dim
         x, act = self._x.ptr + 4 * tok0 * h, self._act.ptr + 4 * tok0 * f
+        if self._norm is not None:
+            normed = self._normed.ptr + 4 * tok0 * h
+            quant.add_rmsnorm_dev(x, self._add.ptr + 4 * tok0 * h, self._norm.ptr, self._res.ptr + 4 * tok0 * h, normed, h,
+                                  count, self._eps, st)
+            x = normed
         if count == 1:
             quant.gemv_dual_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, x, act, h, f, 1, st)
         else:
@@ -96,7 +119,7 @@ class FFNSequenceRunner:
     def bytes_per_sequence(self):
         """Algorithmic bytes: the three matrices once per group of up to 8 tokens, x and residual in, out out."""
         groups = -(-self.tokens // quant.MAX_GEMV_TOKENS)
-        vec = 4 * self.tokens * self.hidden * (3 if self._res is not None else 2)
+        vec = 4 * self.tokens * self.hidden * (4 if self._norm is not None else 3 if self._res is not None else 2)
         return groups * sum(r.size for r in self._raw.values()) + vec
 
     def close(self):

@@ -93,6 +93,18 @@ def gemv_dual_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, x_ptr, out_ptr, in_dim, o
                                                 stream))
 
 
+def rmsnorm_dev(x_ptr, norm_ptr, out_ptr, dim, tokens=1, eps=1.0e-6, stream=None):
+    _check(hip.lib().cogni_rmsnorm_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(out_ptr),
+                                       ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
+
+def add_rmsnorm_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_ptr, dim, tokens=1, eps=1.0e-6, stream=None):
+    """residual_out = x + add; normed_out = rmsnorm(residual_out)."""
+    _check(hip.lib().cogni_add_rmsnorm_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(add_ptr), ctypes.c_uint64(norm_ptr),
+                                           ctypes.c_uint64(residual_out_ptr), ctypes.c_uint64(normed_out_ptr),
+                                           ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
+
 def gemm_workspace_bytes(w_type, in_dim, tokens):
     f = hip.lib().cogni_gemm_workspace_bytes
     f.restype = ctypes.c_size_t

@@ -354,6 +354,24 @@ int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, 
   return launch("q4_k_dual_gemv_swiglu_f32", grid, block, shmem, params, stream, tokens);
 }
 
+int cogni_rmsnorm_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t dim, uint32_t tokens, float eps, void* stream) {
+  if (!x || !norm || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_dev: null device pointer");
+  if (dim == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_dev: zero dimension");
+  if (tokens == 0) return 0;
+  void* params[] = {&x, &norm, &out, &dim, &eps};
+  return launch("rmsnorm_f32", tokens, 256, 0, params, stream);
+}
+
+int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t dim,
+                          uint32_t tokens, float eps, void* stream) {
+  if (!x || !add || !norm || !residual_out || !normed_out)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_add_rmsnorm_dev: null device pointer");
+  if (dim == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_add_rmsnorm_dev: zero dimension");
+  if (tokens == 0) return 0;
+  void* params[] = {&x, &add, &norm, &residual_out, &normed_out, &dim, &eps};
+  return launch("add_rmsnorm_f32", tokens, 256, 0, params, stream);
+}
+
 int g_gemm_threshold = -1;   // -1: not resolved yet
 
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {

@@ -5,6 +5,7 @@
 #include "kernels/gemv.cuh"
 #include "kernels/gemv_mfma.cuh"
 #include "kernels/gemm_q4k.cuh"
+#include "kernels/norm.cuh"
 #include "kernels/util.cuh"
 
 GEMV_MFMA_ENTRY(q4_k_gemv_mfma_f32_tbatch2, 2)

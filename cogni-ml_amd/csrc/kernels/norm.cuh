@@ -1,0 +1,80 @@
+// RMSNorm over fp32 activation rows, one workgroup per token: the kernels that sit between the projections of a
+// decoder layer in the reference's runners (src/ml/cuda/kernels/deltanet_step_probe.ptx:744 rmsnorm_vec_parallel_probe,
+// :906 add_rmsnorm_vec_parallel_probe, :1157 and :1324 their batched forms; CPU form src/ml/gguf/qwen35_cpu.cr:484-490).
+//   inv = 1 / sqrt(sum(x^2) / dim + eps);  out[i] = (x[i] * inv) * norm[i]
+// The add form first forms r = x + add, stores r (the residual stream) and normalises r.
+#pragma once
+#include "common.cuh"
+
+#define NORM_BLOCK 256
+
+template <bool ADD>
+__device__ __forceinline__ void rmsnorm_core(const float* x, const float* __restrict__ add,
+                                             const float* __restrict__ norm, float* residual_out,
+                                             float* __restrict__ out, u32 dim, float eps) {
+  __shared__ float part[NORM_BLOCK / WAVE];
+  const u64 base = (u64)blockIdx.x * dim;
+  const float* xt = x + base;
+  const float* at = ADD ? add + base : nullptr;
+  float* rt = ADD ? residual_out + base : nullptr;
+  float* ot = out + base;
+  const float* st = ADD ? rt : xt;   // second pass: the sum this thread stored (residual_out may be x itself)
+  const u32 tid = threadIdx.x;
+  const bool vec = (dim & 3u) == 0;   // rows then start 16-byte aligned when the buffers do
+  float ss = 0.0f;
+  if (vec) {
+    for (u32 i = tid * 4; i < dim; i += NORM_BLOCK * 4) {
+      float4 v = *reinterpret_cast<const float4*>(xt + i);
+      if (ADD) {
+        const float4 a = *reinterpret_cast<const float4*>(at + i);
+        v.x += a.x, v.y += a.y, v.z += a.z, v.w += a.w;
+        *reinterpret_cast<float4*>(rt + i) = v;
+      }
+      ss += v.x * v.x;
+      ss += v.y * v.y;
+      ss += v.z * v.z;
+      ss += v.w * v.w;
+    }
+  } else {
+    for (u32 i = tid; i < dim; i += NORM_BLOCK) {
+      float v = xt[i];
+      if (ADD) {
+        v += at[i];
+        rt[i] = v;
+      }
+      ss += v * v;
+    }
+  }
+  ss = wave_sum(ss);
+  if ((tid & (WAVE - 1)) == 0) part[tid / WAVE] = ss;
+  __syncthreads();
+  const float total = (part[0] + part[1]) + (part[2] + part[3]);
+  const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+  if (vec) {
+    for (u32 i = tid * 4; i < dim; i += NORM_BLOCK * 4) {
+      const float4 v = *reinterpret_cast<const float4*>(st + i);
+      const float4 w = *reinterpret_cast<const float4*>(norm + i);
+      float4 o;
+      o.x = (v.x * inv) * w.x, o.y = (v.y * inv) * w.y, o.z = (v.z * inv) * w.z, o.w = (v.w * inv) * w.w;
+      *reinterpret_cast<float4*>(ot + i) = o;
+    }
+  } else {
+    for (u32 i = tid; i < dim; i += NORM_BLOCK) {
+      ot[i] = (st[i] * inv) * norm[i];
+    }
+  }
+}
+
+// (x, norm, out, dim, eps): grid.x = tokens (rows at stride dim), block 256.
+extern "C" __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_f32(const float* x, const float* norm, float* out, u32 dim,
+                                                                     float eps) {
+  rmsnorm_core<false>(x, nullptr, norm, nullptr, out, dim, eps);
+}
+
+// (x, add, norm, residual_out, normed_out, dim, eps): residual_out = x + add, normed_out = rmsnorm(residual_out).
+// residual_out may be x itself (every element is read and written by the same thread); grid.x = tokens, block 256.
+extern "C" __global__ __launch_bounds__(NORM_BLOCK) void add_rmsnorm_f32(const float* x, const float* add, const float* norm,
+                                                                         float* residual_out, float* normed_out, u32 dim,
+                                                                         float eps) {
+  rmsnorm_core<true>(x, add, norm, residual_out, normed_out, dim, eps);
+}

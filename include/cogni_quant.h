@@ -137,6 +137,19 @@ int cogni_swiglu_dev(uint64_t gate, uint64_t up, uint64_t out, uint32_t n, void*
 int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t x, uint64_t out, uint32_t in_dim,
                                uint32_t out_dim, uint32_t tokens, void* stream);
 
+/* RMSNorm of `tokens` rows of `dim` floats: inv = 1 / sqrt(sum(x^2) / dim + eps), out[i] = (x[i] * inv) * norm[i], all
+ * in fp32. Kernel "rmsnorm_f32" (x, norm, out, dim:u32, eps:f32), block 256, grid = tokens - the reference's
+ * rmsnorm_vec_parallel_probe and its batched form (src/ml/cuda/kernels/deltanet_step_probe.ptx:744, :1157; CPU form
+ * src/ml/gguf/qwen35_cpu.cr:484-490, which sums the squares in Float64). */
+int cogni_rmsnorm_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t dim, uint32_t tokens, float eps, void* stream);
+
+/* residual_out = x + add, normed_out = rmsnorm(residual_out): the step between attention and the FFN of a decoder layer
+ * (src/ml/gguf/qwen35_cpu.cr:1705-1708). Kernel "add_rmsnorm_f32" (x, add, norm, residual_out, normed_out, dim:u32,
+ * eps:f32), block 256, grid = tokens - the reference's add_rmsnorm_vec_parallel_probe and its batched form
+ * (src/ml/cuda/kernels/deltanet_step_probe.ptx:906, :1324). residual_out may alias x. */
+int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t dim,
+                          uint32_t tokens, float eps, void* stream);
+
 /* Prefill GEMM for `tokens` > 8 (Q4_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
  * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
  * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:

@@ -54,6 +54,8 @@ def lib():
             getattr(L, name).argtypes = [ctypes.c_uint32]
         L.oracle_swiglu.restype = None
         L.oracle_swiglu.argtypes = [f32p, f32p, ctypes.c_void_p, ctypes.c_int64]
+        L.oracle_rms_norm.restype = None
+        L.oracle_rms_norm.argtypes = [f32p, f32p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_float]
         L.oracle_data_bytes.restype = ctypes.c_int64
         L.oracle_data_bytes.argtypes = [ctypes.c_uint32, ctypes.c_int64]
         _lib = L
@@ -136,4 +138,14 @@ def swiglu(gate, up):
     assert ga.size == ua.size
     out = np.empty(ga.size, dtype=np.float32)
     lib().oracle_swiglu(gp, up_p, out.ctypes.data, ctypes.c_int64(ga.size))
+    return out
+
+
+def rms_norm(x, w, eps=1.0e-6):
+    """RMSNorm of one vector (src/ml/gguf/qwen35_cpu.cr:484-490): float64 sum of squares, float32 scaling."""
+    xa, xp = _f32(x)
+    wa, wp = _f32(w)
+    assert xa.size == wa.size
+    out = np.empty(xa.size, dtype=np.float32)
+    lib().oracle_rms_norm(xp, wp, out.ctypes.data, ctypes.c_int64(xa.size), ctypes.c_float(eps))
     return out

@@ -547,3 +547,17 @@ void oracle_swiglu(const float *gate, const float *up, float *out, int64_t n) {
     out[i] = s * up[i];
   }
 }
+
+/* RMSNorm of one dim-length vector as src/ml/gguf/qwen35_cpu.cr:484-490: the sum of squares in Float64 over
+ * x widened element by element, inv_rms = (1 / sqrt(ss / dim + eps)) rounded to Float32, then x[j] * inv_rms * w[j]
+ * left to right in Float32. Pinned by closed forms (constant vectors, unit weights: mean square of the output is
+ * ms / (ms + eps)), scale invariance at eps = 0 and a float64 numpy evaluation (tests/test_oracle_matmul.py). */
+void oracle_rms_norm(const float *x, const float *w, float *out, int64_t dim, float eps) {
+  double ss = 0.0;
+  for (int64_t j = 0; j < dim; j++) ss += (double)x[j] * (double)x[j];
+  const float inv_rms = (float)(1.0 / sqrt(ss / (double)dim + (double)eps));
+  for (int64_t j = 0; j < dim; j++) {
+    const float t = x[j] * inv_rms;
+    out[j] = t * w[j];
+  }
+}

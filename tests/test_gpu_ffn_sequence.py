@@ -46,3 +46,35 @@ def test_ffn_sequence_matches_cpu_form(gpu, oracle, hidden, ffn_dim, tokens, res
     finally:
         runner.close()
         stream.close()
+
+
+@pytest.mark.parametrize("tokens", [1, 3])
+def test_ffn_half_of_a_layer(gpu, oracle, tokens):
+    """r = x + attn_out; h = rmsnorm(r); out = r + down(silu(gate h) * up h) - src/ml/gguf/qwen35_cpu.cr:1705-1725."""
+    hidden, ffn_dim = 1024, 1536
+    rng = np.random.default_rng(77 + tokens)
+    gate_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
+    up_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
+    down_raw = synth.make_weights(rng, Q6_K, hidden, ffn_dim)
+    xs = rng.standard_normal(tokens * hidden).astype(np.float32)
+    attn = rng.standard_normal(tokens * hidden).astype(np.float32)
+    norm = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    runner = FFNSequenceRunner(gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, norm=norm, add=attn, eps=1e-6)
+    try:
+        runner.upload_weights()
+        runner.reset_sequence()
+        runner.run_sequence()
+        runner.read_outputs()
+        zero_f = np.zeros(ffn_dim, dtype=np.float32)
+        for tok in range(tokens):
+            r = xs[tok * hidden:(tok + 1) * hidden] + attn[tok * hidden:(tok + 1) * hidden]
+            h = oracle.rms_norm(r, norm, 1e-6)
+            gate = oracle.matmul_add(h, 1, hidden, gate_raw, Q4_K, ffn_dim, zero_f, threads=8)
+            up = oracle.matmul_add(h, 1, hidden, up_raw, Q4_K, ffn_dim, zero_f, threads=8)
+            want = oracle.matmul_add(oracle.swiglu(gate, up), 1, ffn_dim, down_raw, Q6_K, hidden, r, threads=8)
+            got = runner.out[tok * hidden:(tok + 1) * hidden]
+            assert cosine(got, want) >= 0.99999 and np.max(np.abs(got - want)) <= 1e-4 * np.max(np.abs(want)), "token %d" % tok
+        with pytest.raises(ValueError, match="norm and add go together"):
+            FFNSequenceRunner(gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, norm=norm)
+    finally:
+        runner.close()

@@ -195,3 +195,24 @@ def test_swiglu_closed_forms_and_float64():
     ref = g.astype(np.float64) / (1.0 + np.exp(-g.astype(np.float64))) * u.astype(np.float64)
     assert np.max(np.abs(oracle.swiglu(g, u) - ref)) <= 3e-7 * np.max(np.abs(ref))
     assert np.array_equal(oracle.swiglu(g, 2 * u), 2 * oracle.swiglu(g, u))      # exact: a power of two in the last product
+
+
+def test_rms_norm_closed_forms_and_float64():
+    """Constant vector c with unit weights -> c / sqrt(c^2 + eps); mean square of the output = ms / (ms + eps);
+    invariance under scaling of x at eps = 0; weights enter linearly; against float64."""
+    from oracle import oracle
+    dim = 1024
+    ones = np.ones(dim, dtype=np.float32)
+    for c, eps in ((2.0, 1e-6), (-0.5, 1e-2), (1e-3, 1e-6)):
+        out = oracle.rms_norm(np.full(dim, c, dtype=np.float32), ones, eps)
+        assert np.allclose(out, c / np.sqrt(c * c + eps), rtol=2e-7, atol=0)
+    rng = np.random.default_rng(6)
+    x, w = rng.standard_normal(dim).astype(np.float32) * 3, rng.standard_normal(dim).astype(np.float32)
+    ms = float(np.mean(x.astype(np.float64) ** 2))
+    out = oracle.rms_norm(x, ones, 0.25)
+    assert abs(float(np.mean(out.astype(np.float64) ** 2)) - ms / (ms + 0.25)) <= 1e-6
+    assert np.array_equal(oracle.rms_norm(4 * x, w, 0.0), oracle.rms_norm(x, w, 0.0))     # power-of-two scale: exact
+    assert np.array_equal(oracle.rms_norm(x, 2 * w, 1e-6), 2 * oracle.rms_norm(x, w, 1e-6))
+    ref = x.astype(np.float64) / np.sqrt(ms + 1e-6) * w.astype(np.float64)
+    assert np.max(np.abs(oracle.rms_norm(x, w, 1e-6) - ref)) <= 3e-7 * np.max(np.abs(ref))
+    assert np.array_equal(oracle.rms_norm(np.zeros(8, dtype=np.float32), np.ones(8, dtype=np.float32), 1e-6), np.zeros(8, dtype=np.float32))
