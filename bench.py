@@ -292,6 +292,26 @@ def main():
             c.close()
 
     if args.mode == "cases":
+        # output head without the logits: RMSNorm -> Q6_K vocabulary projection with arg-max -> top-1 reduce (510 MB)
+        from cogni_ml_amd.output_head import QwenOutputHeadRunner, Weights as HeadWeights
+        hw = HeadWeights(np.ones(4096, dtype=np.float32), synth.make_weights(rng, Q6_K, 151936, 4096), Q6_K, 4096, 151936)
+        for tokens in (1, 3):
+            ohead = QwenOutputHeadRunner.from_weights(hw, tokens, synth.make_activations(rng, tokens, 4096).reshape(-1), 1e-6)
+            ohead.upload_weights()
+            ohead.reset_sequence()
+
+            def hseq(i, st, ohead=ohead):
+                with hip.with_stream(st):
+                    ohead.run_sequence()
+            reps = 20
+            hms, _ = time_steps(hip, stream, hseq, reps, 3)
+            hg = ohead.bytes_per_sequence() / (hms / reps * 1e-3) / 1e9
+            extra["q6_k output head top-1 M=%d" % tokens] = {"gbps": round(hg, 1), "ms": round(hms / reps, 5), "frac_hbm": round(hg / HBM_PEAK_GBPS, 4)}
+            log("case=output head top-1 (rmsnorm -> q6_k gemv top1 partial -> reduce)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\ngbps_hbm=%.1f\n" % (
+                tokens, hw.output_raw.size, reps, hms / reps, hg))
+            ohead.close()
+
+    if args.mode == "cases":
         # the gate | up pair of one layer against the same x in one launch (q4_k_dual_gemv_f32)
         a = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES)
         b = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES)

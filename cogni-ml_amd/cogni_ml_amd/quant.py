@@ -93,6 +93,21 @@ def gemv_dual_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, x_ptr, out_ptr, in_dim, o
                                                 stream))
 
 
+def gemv_top1_partials(w_type, out_dim):
+    f = hip.lib().cogni_gemv_top1_partials
+    f.restype = ctypes.c_uint32
+    return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(out_dim))
+
+
+def gemv_top1_dev(w_ptr, w_type, x_ptr, partial_ids_ptr, partial_values_ptr, top1_ids_ptr, top1_values_ptr, in_dim, out_dim,
+                  tokens=1, stream=None):
+    """Index and value of the largest element of W x per token; partial_* hold tokens * gemv_top1_partials() elements."""
+    _check(hip.lib().cogni_gemv_top1_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(x_ptr),
+                                         ctypes.c_uint64(partial_ids_ptr), ctypes.c_uint64(partial_values_ptr),
+                                         ctypes.c_uint64(top1_ids_ptr), ctypes.c_uint64(top1_values_ptr),
+                                         ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
 def rmsnorm_dev(x_ptr, norm_ptr, out_ptr, dim, tokens=1, eps=1.0e-6, stream=None):
     _check(hip.lib().cogni_rmsnorm_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(out_ptr),
                                        ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))

@@ -354,6 +354,51 @@ int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, 
   return launch("q4_k_dual_gemv_swiglu_f32", grid, block, shmem, params, stream, tokens);
 }
 
+// ---- output head: GEMV with the arg-max over the rows ---------------------------------------------------
+static uint32_t top1_token_cap(uint32_t type) { return (type == COGNI_TYPE_Q4_K || type == COGNI_TYPE_Q6_K) ? 3u : 1u; }
+
+uint32_t cogni_gemv_top1_partials(uint32_t w_type, uint32_t out_dim) {
+  if (!gemv_type(w_type) || out_dim == 0) return 0;
+  uint32_t most = 0;
+  for (uint32_t m = 1; m <= top1_token_cap(w_type); m++) {
+    const uint32_t rows = (uint32_t)gemv_rows_per_block(w_type, (int)m);
+    const uint32_t grid = (out_dim + rows - 1) / rows;
+    if (grid > most) most = grid;
+  }
+  return most;
+}
+
+int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t partial_ids, uint64_t partial_values,
+                        uint64_t top1_ids, uint64_t top1_values, uint32_t in_dim, uint32_t out_dim, uint32_t tokens,
+                        void* stream) {
+  if (!gemv_type(w_type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for fused matmul: ") + type_name(w_type));
+  if (!w_raw || !x || !partial_ids || !partial_values || !top1_ids || !top1_values)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_top1_dev: null device pointer");
+  if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_top1_dev: zero dimension");
+  if (k_quant(w_type) && (in_dim % 256) != 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  const uint32_t cap = top1_token_cap(w_type), stride = cogni_gemv_top1_partials(w_type, out_dim);
+  for (uint32_t t0 = 0; t0 < tokens; t0 += cap) {
+    const uint32_t m = tokens - t0 < cap ? tokens - t0 : cap;
+    uint32_t grid = 0, block = 0, shmem = 0;
+    int rc = cogni_gemv_launch_dims(w_type, m, in_dim, out_dim, &grid, &block, &shmem);
+    if (rc != 0) return rc;
+    std::string name = std::string(type_prefix(w_type)) + "_gemv_top1_partial_f32";
+    if (m > 1) name += "_tbatch" + std::to_string(m);
+    // the group's partial results: [token in group][workgroup], inside the group's share of the caller's buffers
+    uint64_t xm = x + (uint64_t)t0 * in_dim * 4, pi = partial_ids + (uint64_t)t0 * stride * 4, pv = partial_values + (uint64_t)t0 * stride * 4;
+    uint64_t oi = top1_ids + (uint64_t)t0 * 4, ov = top1_values + (uint64_t)t0 * 4;
+    void* params[] = {&w_raw, &xm, &pi, &pv, &in_dim, &out_dim};
+    rc = launch(name.c_str(), grid, block, shmem, params, stream);
+    if (rc != 0) return rc;
+    void* rparams[] = {&pi, &pv, &oi, &ov, &grid};
+    rc = launch("top1_reduce_f32", m, 1024, 0, rparams, stream);
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+
 int cogni_rmsnorm_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t dim, uint32_t tokens, float eps, void* stream) {
   if (!x || !norm || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_dev: null device pointer");
   if (dim == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_dev: zero dimension");

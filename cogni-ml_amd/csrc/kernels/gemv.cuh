@@ -369,11 +369,14 @@ __device__ __forceinline__ float swiglu_one(float g, float u) {
 // SWIGLU (with DUAL, M = 1): a wavefront takes R/2 rows of w (gate) and the same R/2 rows of w_b (up) and stores
 // silu(gate) * up into out - the reference's gate/up GEMVs followed by its swiglu_f32 kernel
 // (bin/cuda_ffn_sequence_probe.cr:46-84) in one launch.
-template <class F, int M, bool ADD, bool DUAL = false, bool SWIGLU = false>
+// TOP1: instead of the row values the workgroup stores, per token, the largest of its rows and that row's index
+// (out[m * gridDim.x + blockIdx.x], top_ids[same]); of equal values the lowest row wins. The reference's
+// q6_k_gemv_top1_partial_f32 (src/ml/cuda/kernels/q6k_gemv_probe.ptx:1331-1580) for the output head.
+template <class F, int M, bool ADD, bool DUAL = false, bool SWIGLU = false, bool TOP1 = false>
 __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                           const float* __restrict__ residual, float* __restrict__ out,
                                           u32 in_dim, u32 out_dim, const uint8_t* __restrict__ w_b = nullptr,
-                                          float* __restrict__ out_b = nullptr) {
+                                          float* __restrict__ out_b = nullptr, u32* __restrict__ top_ids = nullptr) {
   constexpr int R = F::rows(M);
   constexpr int MG = M < F::MG_MAX ? M : F::MG_MAX;   // tokens held in registers at a time
   constexpr int NG = (M + MG - 1) / MG;
@@ -393,6 +396,7 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
 
   static_assert(!SWIGLU || (DUAL && M == 1 && !ADD && R % 2 == 0), "SWIGLU is a one-token mode of the matrix pair");
+  static_assert(!TOP1 || (!DUAL && !ADD), "TOP1 is a mode of the plain GEMV");
   const u32 total_rows = DUAL ? 2 * out_dim : out_dim;
   const uint8_t* rowp[R];
 #pragma unroll
@@ -567,6 +571,32 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     }
     return;
   }
+  if constexpr (TOP1) {
+    __shared__ float top_v[M][GEMV_WAVES];
+    __shared__ u32 top_i[M][GEMV_WAVES];
+#pragma unroll
+    for (int m = 0; m < M; m++) {
+      float best = -__builtin_inff();
+      u32 best_id = 0;
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const float v = wave_sum(acc[r][m]);
+        if (row0 + r < out_dim && v > best) best = v, best_id = row0 + r;
+      }
+      if (lane == 0) top_v[m][wave] = best, top_i[m][wave] = best_id;
+    }
+    __syncthreads();
+    if (tid < M) {
+      float best = top_v[tid][0];
+      u32 best_id = top_i[tid][0];
+#pragma unroll
+      for (int wv = 1; wv < GEMV_WAVES; wv++)
+        if (top_v[tid][wv] > best) best = top_v[tid][wv], best_id = top_i[tid][wv];
+      out[(size_t)tid * gridDim.x + blockIdx.x] = best;
+      top_ids[(size_t)tid * gridDim.x + blockIdx.x] = best_id;
+    }
+    return;
+  }
 #pragma unroll
   for (int r = 0; r < R; r++) {
 #pragma unroll
@@ -619,12 +649,63 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch7, FMT, 7) \
   GEMV_ADD_ENTRY(PFX##_gemv_add_f32_tbatch8, FMT, 8)
 
+// (w_raw, x, partial_ids, partial_values, in_dim, out_dim): the reference's parameter order
+// (src/ml/cuda/kernels/q6k_gemv_probe.ptx:1331-1338); same grid, block and dynamic shared memory as the GEMV of the
+// same type and token count, partial_*[token * grid + workgroup].
+#define GEMV_TOP1_ENTRY(NAME, FMT, M)                                                                            \
+  extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(M) void NAME(const uint8_t* w, const float* x, u32* partial_ids, \
+                                                                 float* partial_values, u32 in_dim, u32 out_dim) { \
+    gemv_core<FMT, M, false, false, false, true>(w, x, nullptr, partial_values, in_dim, out_dim, nullptr, nullptr, \
+                                                 partial_ids);                                                   \
+  }
+
 typedef FmtK45<false> FmtQ4K;
 typedef FmtK45<true> FmtQ5K;
 GEMV_FAMILY(q4_k, FmtQ4K)
 GEMV_FAMILY(q5_k, FmtQ5K)
 GEMV_FAMILY(q6_k, FmtQ6K)
 GEMV_FAMILY(q8_0, FmtQ80)
+GEMV_TOP1_ENTRY(q4_k_gemv_top1_partial_f32, FmtQ4K, 1)
+GEMV_TOP1_ENTRY(q4_k_gemv_top1_partial_f32_tbatch2, FmtQ4K, 2)
+GEMV_TOP1_ENTRY(q4_k_gemv_top1_partial_f32_tbatch3, FmtQ4K, 3)
+GEMV_TOP1_ENTRY(q5_k_gemv_top1_partial_f32, FmtQ5K, 1)
+GEMV_TOP1_ENTRY(q6_k_gemv_top1_partial_f32, FmtQ6K, 1)
+GEMV_TOP1_ENTRY(q6_k_gemv_top1_partial_f32_tbatch2, FmtQ6K, 2)
+GEMV_TOP1_ENTRY(q6_k_gemv_top1_partial_f32_tbatch3, FmtQ6K, 3)
+GEMV_TOP1_ENTRY(q8_0_gemv_top1_partial_f32, FmtQ80, 1)
+
+// (partial_ids, partial_values, out_ids, out_values, count): the largest of `count` partial values and its id, per
+// token (grid.x = tokens; partial_* + token * count, out_* + token). Of equal values the lowest id wins, which is
+// what the reference's CPU scan gives (bin/cuda_mixed_stack_probe.cr:1485-1497); its device reduce is
+// output_top1_values_reduce_probe (src/ml/cuda/qwen_output_head_runner.cr:530-612). block = 1024.
+#define TOP1_REDUCE_BLOCK 1024
+__device__ __forceinline__ void top1_take(float& best, u32& best_id, float v, u32 id) {
+  if (v > best || (v == best && id < best_id)) best = v, best_id = id;
+}
+extern "C" __global__ __launch_bounds__(TOP1_REDUCE_BLOCK) void top1_reduce_f32(const u32* partial_ids,
+                                                                                const float* partial_values, u32* out_ids,
+                                                                                float* out_values, u32 count) {
+  __shared__ float sv[TOP1_REDUCE_BLOCK / WAVE];
+  __shared__ u32 si[TOP1_REDUCE_BLOCK / WAVE];
+  const u32* ids = partial_ids + (size_t)blockIdx.x * count;
+  const float* vals = partial_values + (size_t)blockIdx.x * count;
+  float best = -__builtin_inff();
+  u32 best_id = 0xFFFFFFFFu;
+  for (u32 i = threadIdx.x; i < count; i += TOP1_REDUCE_BLOCK) top1_take(best, best_id, vals[i], ids[i]);
+#pragma unroll
+  for (int d = 1; d < WAVE; d <<= 1) {
+    const float ov = __shfl_xor(best, d, WAVE);
+    const u32 oi = (u32)__shfl_xor((int)best_id, d, WAVE);
+    top1_take(best, best_id, ov, oi);
+  }
+  if ((threadIdx.x & (WAVE - 1)) == 0) sv[threadIdx.x / WAVE] = best, si[threadIdx.x / WAVE] = best_id;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int wv = 1; wv < TOP1_REDUCE_BLOCK / WAVE; wv++) top1_take(best, best_id, sv[wv], si[wv]);
+    out_ids[blockIdx.x] = best_id == 0xFFFFFFFFu ? 0u : best_id;   // nothing above -inf: id 0, as the CPU scan
+    out_values[blockIdx.x] = best;
+  }
+}
 
 // (w_raw_a, w_raw_b, x, out_a, out_b, in_dim, out_dim): one token per grid.y slice (x + y * in_dim, out_* + y * out_dim),
 // grid.x = ceil(2 * out_dim / rows per workgroup), same block and dynamic shared memory as q4_k_gemv_f32.

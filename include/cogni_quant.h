@@ -150,6 +150,20 @@ int cogni_rmsnorm_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t dim, uin
 int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t dim,
                           uint32_t tokens, float eps, void* stream);
 
+/* Output head without the logits: for each token the index of the largest element of W x and that value
+ * (top1_ids: u32[tokens], top1_values: f32[tokens]); of equal values the lowest index wins, as in the reference's CPU scan
+ * (bin/cuda_mixed_stack_probe.cr:1485-1497). Two launches per group of up to 3 tokens (Q4_K, Q6_K; one token for the other
+ * types): kernel "<prefix>_gemv_top1_partial_f32[_tbatchM]" (w_raw, x, partial_ids, partial_values, in_dim, out_dim) -
+ * the reference's q6_k_gemv_top1_partial_f32 (src/ml/cuda/kernels/q6k_gemv_probe.ptx:1331), with the grid, block and
+ * shared memory of the GEMV of that type and token count and one (id, value) per workgroup and token - then
+ * "top1_reduce_f32" (partial_ids, partial_values, out_ids, out_values, count:u32), block 1024, grid = tokens of the group -
+ * the reference's output_top1_values_reduce_probe (src/ml/cuda/qwen_output_head_runner.cr:530, launched :939-940).
+ * partial_ids / partial_values are caller-owned scratch of tokens * cogni_gemv_top1_partials(w_type, out_dim) elements. */
+uint32_t cogni_gemv_top1_partials(uint32_t w_type, uint32_t out_dim);
+int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t partial_ids, uint64_t partial_values,
+                        uint64_t top1_ids, uint64_t top1_values, uint32_t in_dim, uint32_t out_dim, uint32_t tokens,
+                        void* stream);
+
 /* Prefill GEMM for `tokens` > 8 (Q4_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
  * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
  * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:

@@ -1,0 +1,104 @@
+"""GEMV fused with the arg-max over the rows, and the resident output head (RMSNorm -> vocabulary projection -> top-1),
+against the CPU form of the reference's probe (bin/cuda_mixed_stack_probe.cr:1479-1497): rms_norm, matmul_add with a zero
+bias, then a scan that keeps the first of equal maxima."""
+import numpy as np
+import pytest
+
+from cogni_ml_amd import hip, quant, synth
+from cogni_ml_amd.output_head import QwenOutputHeadRunner, Weights
+from gpu_common import DevArray, gpu  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+
+
+def first_max(v):
+    return int(np.argmax(v))        # numpy returns the first of equal maxima, as the reference's scan
+
+
+def run_top1(raw, t, x, in_dim, out_dim, tokens):
+    stride = quant.gemv_top1_partials(t, out_dim)
+    wd, xd = DevArray(raw), DevArray(x)
+    pi, pv = DevArray(nbytes=4 * tokens * stride), DevArray(nbytes=4 * tokens * stride)
+    oi, ov, lo = DevArray(nbytes=4 * tokens), DevArray(nbytes=4 * tokens), DevArray(nbytes=4 * tokens * out_dim)
+    try:
+        quant.gemv_top1_dev(wd.ptr, t, xd.ptr, pi.ptr, pv.ptr, oi.ptr, ov.ptr, in_dim, out_dim, tokens)
+        quant.gemv_dev(wd.ptr, t, xd.ptr, lo.ptr, in_dim, out_dim, tokens)
+        return oi.read(np.uint32, tokens), ov.read(np.float32, tokens), lo.read(np.float32, tokens * out_dim).reshape(tokens, out_dim)
+    finally:
+        for d in (wd, xd, pi, pv, oi, ov, lo):
+            d.close()
+
+
+@pytest.mark.parametrize("t,in_dim,out_dim,tokens", [(Q6_K, 4096, 32003, 1), (Q6_K, 1024, 5000, 5), (Q6_K, 256, 7, 2),
+                                                     (Q4_K, 1024, 4099, 1), (Q4_K, 512, 777, 7), (Q5_K, 512, 1001, 2),
+                                                     (Q8_0, 1024, 3584, 3), (Q6_K, 256, 1, 1)])
+def test_top1_matches_oracle_scan(gpu, oracle, t, in_dim, out_dim, tokens):
+    rng = np.random.default_rng(out_dim + tokens)
+    raw = synth.make_weights(rng, t, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    ids, vals, logits = run_top1(raw, t, x, in_dim, out_dim, tokens)
+    want = oracle.matmul_add(x, tokens, in_dim, raw, t, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).reshape(tokens, out_dim)
+    for tok in range(tokens):
+        # the device's own logits decide ties and near-ties exactly; the oracle's winner must be within the GEMV tolerance
+        assert ids[tok] == first_max(logits[tok]) or np.isclose(vals[tok], logits[tok].max(), rtol=2e-5, atol=0)
+        top = float(want[tok].max())
+        assert abs(float(vals[tok]) - top) <= 1e-4 * max(abs(top), float(np.abs(want[tok]).max()))
+        assert want[tok][ids[tok]] >= top - 1e-4 * float(np.abs(want[tok]).max())
+
+
+def test_top1_ties_take_the_lowest_row(gpu):
+    """Rows with identical bytes give identical sums: the lowest row index must win, across wavefronts, workgroups and
+    the strided final reduce."""
+    rng = np.random.default_rng(1)
+    in_dim, out_dim = 512, 6000
+    base = synth.make_weights(rng, Q6_K, out_dim, in_dim).reshape(out_dim, -1)
+    x = synth.make_activations(rng, 2, in_dim)
+    _, _, logits = run_top1(np.ascontiguousarray(base).reshape(-1), Q6_K, x, in_dim, out_dim, 2)
+    best = int(np.argmax(logits[0]))
+    for dup in ([5, 2048 + 3, 5999], [4097, 1031], [best]):
+        rows = base.copy()
+        for r in dup:
+            rows[r] = base[best]           # same bytes as the winning row
+        ids, vals, lg = run_top1(np.ascontiguousarray(rows).reshape(-1), Q6_K, x, in_dim, out_dim, 2)
+        assert ids[0] == min(dup + [best]) and vals[0] == lg[0].max()
+        assert ids[1] == first_max(lg[1])
+    # one row repeated everywhere: every partial result ties
+    rows = np.repeat(base[:1], out_dim, axis=0)
+    ids, _, _ = run_top1(np.ascontiguousarray(rows).reshape(-1), Q6_K, x, in_dim, out_dim, 2)
+    assert list(ids) == [0, 0]
+
+
+def test_output_head_runner(gpu, oracle):
+    hidden, vocab, tokens = 1024, 20011, 4
+    rng = np.random.default_rng(3)
+    w = Weights((1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32), synth.make_weights(rng, Q6_K, vocab, hidden),
+                Q6_K, hidden, vocab)
+    xs = (rng.standard_normal(tokens * hidden) * 3).astype(np.float32)
+    runner = QwenOutputHeadRunner.from_weights(w, tokens, xs, 1e-6, read_logits=True)
+    stream = hip.HIPStream()
+    try:
+        runner.upload_weights()
+        runner.reset_sequence()
+        with hip.with_stream(stream):
+            assert runner.run_repeated(2) == 2 * tokens
+        stream.synchronize()
+        runner.read_outputs()
+        for tok in range(tokens):
+            normed = oracle.rms_norm(xs[tok * hidden:(tok + 1) * hidden], w.norm, 1e-6)
+            logits = oracle.matmul_add(normed, 1, hidden, w.output_raw, Q6_K, vocab, np.zeros(vocab, dtype=np.float32), threads=8)
+            assert runner.top1_ids[tok] == first_max(logits)
+            assert abs(runner.top1_values[tok] - logits.max()) <= 1e-4 * np.abs(logits).max()
+            dev = runner.logits[tok * vocab:(tok + 1) * vocab]
+            assert runner.top1_ids[tok] == first_max(dev) and runner.top1_values[tok] == dev.max()
+        # token-local path gives the same ids
+        grouped = runner.top1_ids.copy()
+        for tok in range(tokens):
+            runner._run_token(tok)
+        runner.read_outputs()
+        assert np.array_equal(runner.top1_ids, grouped)
+        with pytest.raises(ValueError, match="xs size mismatch"):
+            runner.replace_sequence_input(xs[:-1])
+    finally:
+        runner.close()
+        stream.close()
