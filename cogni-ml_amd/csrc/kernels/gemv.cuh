@@ -27,6 +27,7 @@
 // honoured, so a code costs one mask per pair plus one fused multiply-add; the power of two is folded
 // into the block scale.
 #pragma once
+#include <type_traits>
 #include "common.cuh"
 #include "gemv_config.h"
 
@@ -72,6 +73,7 @@ struct FmtK45 {
   static constexpr int NSUM = 2;
   static constexpr int MG_MAX = 2;
   static constexpr int SPI = 1;   // sets per iteration: a column set is 4096 values
+  static constexpr unsigned TYPE = Q5 ? 13 : 12;
   static constexpr int rows(int m) { return Q5 ? GEMV_ROWS_Q5K(m) : GEMV_ROWS_Q4K(m); }
 
   struct Lane {
@@ -100,6 +102,14 @@ struct FmtK45 {
   }
   static __device__ __forceinline__ float4 load_x(const float* xrow, u32 e, u32 in_dim) {
     return e < in_dim ? ldx4(xrow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  // Place of 16-byte piece p (0..1023) of a column set in the directly staged LDS image: the natural order with the
+  // low four bits of the index XORed by a function of the higher ones. A lane reads the 16 consecutive pieces
+  // 16 l .. 16 l + 15, so without this the 16 lanes served together would all hit the same four banks; with it
+  // they hit 16 different groups of four. An involution: it also gives the piece that belongs at place p.
+  static __device__ __forceinline__ u32 swz(u32 p) {
+    const u32 grp = p >> 4;
+    return p ^ (((grp & 3u) << 2) | ((grp >> 2) & 3u));
   }
 
   template <int R>
@@ -190,6 +200,7 @@ struct FmtQ6K {
   static constexpr int NSUM = 4;
   static constexpr int MG_MAX = 2;
   static constexpr int SPI = 1;
+  static constexpr unsigned TYPE = 14;
   static constexpr int rows(int m) { return GEMV_ROWS_Q6K(m); }
 
   struct Lane {
@@ -211,6 +222,9 @@ struct FmtQ6K {
   static __device__ __forceinline__ float4 load_x(const float* xrow, u32 e, u32 in_dim) {
     return e < in_dim ? ldx4(xrow + e) : make_float4(0.f, 0.f, 0.f, 0.f);
   }
+  // As FmtK45::swz for this lane mapping: piece index = jb * 64 + n * 32 + (i >> 2) * 8 + v * 4 + (i & 3), so the
+  // 16 lanes served together differ in jb & 3, n and v; v already selects bit 2, n goes to bit 3, jb & 3 to bits 0-1.
+  static __device__ __forceinline__ u32 swz(u32 p) { return p ^ ((((p >> 5) & 1u) << 3) | ((p >> 6) & 3u)); }
 
   template <int R>
   static __device__ __forceinline__ void load(Stage<R>& st, const uint8_t* const (&rowp)[R], const Lane& ln,
@@ -292,6 +306,7 @@ struct FmtQ80 {
   static constexpr int NSUM = 1;
   static constexpr int MG_MAX = 4;
   static constexpr int SPI = 2;   // sets per iteration: a column set is 1024 values
+  static constexpr unsigned TYPE = 8;
   static constexpr int rows(int m) { return GEMV_ROWS_Q80(m); }
 
   struct Lane {
@@ -303,6 +318,7 @@ struct FmtQ80 {
     uint4 qs[R];
     u32 d[R];
   };
+  static __device__ __forceinline__ u32 swz(u32 p) { return p; }   // (no direct staging for this format)
 
   static __device__ __forceinline__ u32 nblocks(u32 in_dim) { return (in_dim + 31) >> 5; }
   static __device__ __forceinline__ size_t row_bytes(u32 nb) { return (size_t)nb * BB; }
@@ -387,11 +403,13 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const typename F::Lane ln(lane);
-  const u32 nb = F::nblocks(in_dim);
+  u32 nb = F::nblocks(in_dim);
   const u32 ncs = (nb + F::BPS - 1) / F::BPS;
+  // K-quants with one token group: the activations go global -> LDS directly (no registers), sums from registers
+  constexpr bool DIRECT = gemv_direct_x(F::TYPE, NG);
   // column sets staged in LDS at a time (the host sizes the dynamic LDS with the same formula);
   // with several token groups each set is staged per group
-  const u32 CH = NG > 1 ? 1u : (u32)gemv_chunk_sets(MG * SET_F4, ncs);
+  const u32 CH = NG > 1 ? 1u : (u32)(DIRECT ? gemv_chunk_sets_direct(MG * SET_F4, ncs) : gemv_chunk_sets(MG * SET_F4, ncs));
   const size_t row_bytes = F::row_bytes(nb);
   const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
 
@@ -467,6 +485,55 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     __syncthreads();
   };
 
+  // Direct staging of column sets [s0, s0+CH): the LDS image of a (token, set) is its 16 KiB in natural order up to
+  // F::swz. It is copied in 1 KiB units dealt round-robin to the wavefronts, each one global_load_lds_dwordx4
+  // (lane l lands at unit base + 16 l) over 1 KiB of contiguous global memory. Sets past the end of the row are
+  // replaced by the row's last float4: the lanes that would use them are masked out of the sums by `valid`.
+  auto stage_direct = [&](u32 s0) {
+    const u32 units = (u32)(MG * 16) * CH;
+    for (u32 u = wave; u < units; u += GEMV_WAVES) {
+      const u32 uu = u & 15u, cm = u >> 4;
+      const u32 cset = min(s0 + cm % CH, ncs - 1), m = cm / CH;
+      const u32 e = min((cset * 1024u + F::swz(uu * 64u + lane)) * 4u, in_dim - 4);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(x + (size_t)m * in_dim + e),
+                                       (__attribute__((address_space(3))) void*)(xs + (size_t)u * 64), 16, 0, 0);
+    }
+    // everything that loads weights below takes its block count from here, so it cannot move above the copies
+    asm volatile("" : "+s"(nb));
+  };
+  const u32 lane_piece = F::swz(F::x_elem(0, lane, 0) >> 2);   // place of the lane's first piece in the image
+  // The copies of this wavefront have landed once nothing it requested is outstanding. (Waiting for "all but the
+  // weight loads issued since" would let the arithmetic start a little earlier, but the compiler is free to move
+  // those loads below the wait, and then the count would be wrong.)
+  auto stage_direct_wait = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  auto read_x = [&](u32 s, float4 (&xr)[MG][NF4], float (&sx)[MG][NSUM]) {
+#pragma unroll
+    for (int mm = 0; mm < MG; mm++) {
+      const u32 cm = mm * CH + (s % CH);
+#pragma unroll
+      for (int i = 0; i < NF4; i++) {
+        // direct image: the lane's pieces differ from its first in bits the swizzle neither reads nor writes
+        if constexpr (DIRECT) xr[mm][i] = xs[cm * 1024 + (lane_piece ^ (F::x_elem(0, 0, i) >> 2))];
+        else xr[mm][i] = xs[(cm * NF4 + i) * 64 + lane];
+      }
+#pragma unroll
+      for (int k = 0; k < NSUM; k++) {
+        if constexpr (DIRECT) {
+          float a = 0.0f;
+#pragma unroll
+          for (int i = 0; i < NF4 / NSUM; i++) a += hsum4(xr[mm][k * (NF4 / NSUM) + i]);
+          sx[mm][k] = a;
+        } else {
+          sx[mm][k] = xsum[(cm * NSUM + k) * 64 + lane];
+        }
+      }
+    }
+  };
+
   auto step = [&](const typename F::template Stage<R>& st, u32 s) {
     const bool valid = s * F::BPS + ln.jb < nb;
 #pragma unroll
@@ -478,14 +545,7 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
       }
       float4 xr[MG][NF4];
       float sx[MG][NSUM];
-#pragma unroll
-      for (int mm = 0; mm < MG; mm++) {
-        const u32 cm = mm * CH + (s % CH);
-#pragma unroll
-        for (int i = 0; i < NF4; i++) xr[mm][i] = xs[(cm * NF4 + i) * 64 + lane];
-#pragma unroll
-        for (int k = 0; k < NSUM; k++) sx[mm][k] = xsum[(cm * NSUM + k) * 64 + lane];
-      }
+      read_x(s, xr, sx);
 #pragma unroll
       for (int r = 0; r < R; r++) {
         float c[MG];
@@ -509,28 +569,29 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     constexpr int PF = R >= 4 ? 2 : 1;
     typename F::template Stage<R> st;
     float4 buf[FU];
-    stage_begin(0, 0, buf);
+    if constexpr (DIRECT) stage_direct(0);
+    else stage_begin(0, 0, buf);
 #pragma unroll
     for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nb);
-    stage_end(0, 0, buf);
+    if constexpr (DIRECT) stage_direct_wait();
+    else stage_end(0, 0, buf);
     // one column set; `last` (a compile-time tag) says that no column set follows, so the prefetches that
     // would wrap into the next set are left out and the number of loads in flight stays a constant
     auto column_set = [&](u32 s, auto last) {
       if (s > 0 && (s % CH) == 0) {
-        stage_begin(s, 0, buf);
-        stage_end(s, 0, buf);
+        if constexpr (DIRECT) {
+          __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
+          stage_direct(s);
+          stage_direct_wait();
+        } else {
+          stage_begin(s, 0, buf);
+          stage_end(s, 0, buf);
+        }
       }
       const bool valid = s * F::BPS + ln.jb < nb;
       float4 xr[MG][NF4];
       float sx[MG][NSUM];
-#pragma unroll
-      for (int mm = 0; mm < MG; mm++) {
-        const u32 cm = mm * CH + (s % CH);
-#pragma unroll
-        for (int i = 0; i < NF4; i++) xr[mm][i] = xs[(cm * NF4 + i) * 64 + lane];
-#pragma unroll
-        for (int k = 0; k < NSUM; k++) sx[mm][k] = xsum[(cm * NSUM + k) * 64 + lane];
-      }
+      read_x(s, xr, sx);
 #pragma unroll
       for (int r = 0; r < R; r++) {
         const int rr = (r + PF) % R;
@@ -551,12 +612,23 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   for (u32 s = 0; s < ncs; s += F::SPI) {
     const bool restage = NG == 1 && (s % CH) == 0;   // CH is a multiple of SPI or covers the whole row
     float4 buf[FU];
-    if (restage) stage_begin(s, 0, buf);
+    if constexpr (DIRECT) {
+      if (restage) {
+        if (s > 0) __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
+        stage_direct(s);
+      }
+    } else if (restage) {
+      stage_begin(s, 0, buf);
+    }
     typename F::template Stage<R> stA, stB;
     F::template load<R>(stA, rowp, ln, s, nb);
     const bool two = F::SPI == 2 && s + 1 < ncs;
     if (two) F::template load<R>(stB, rowp, ln, s + 1, nb);
-    if (restage) stage_end(s, 0, buf);
+    if constexpr (DIRECT) {
+      if (restage) stage_direct_wait();
+    } else if (restage) {
+      stage_end(s, 0, buf);
+    }
     step(stA, s);
     if (two) step(stB, s + 1);
   }

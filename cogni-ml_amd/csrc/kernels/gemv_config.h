@@ -43,6 +43,21 @@ static inline GEMV_HD int gemv_chunk_sets(int per_set_f4, unsigned ncs) {
   return ch;
 }
 
+// K-quant kernels whose tokens all fit the registers at once (one token group) copy the activations global -> LDS
+// without passing through registers and form the per-lane sums from the registers they are read into: no sums in LDS.
+static inline GEMV_HD int gemv_chunk_sets_direct(int per_set_f4, unsigned ncs) {
+  int ch = GEMV_LDS_BYTES / 16 / per_set_f4;
+  if (ch < 1) ch = 1;
+  if ((unsigned)ch >= ncs) return (int)ncs;
+  return ch;
+}
+#ifndef GEMV_DIRECT_X
+#define GEMV_DIRECT_X 1
+#endif
+static constexpr inline GEMV_HD bool gemv_direct_x(unsigned type, int token_groups) {
+  return GEMV_DIRECT_X && (type == 12 || type == 13 || type == 14) && token_groups == 1;
+}
+
 // column-set geometry per type: blocks per set, float4 of x per lane and set, tokens per register group
 // (nsum = scale groups per lane whose activation sums are kept in LDS)
 static inline void gemv_set_geometry(unsigned type, int* bps, int* nf4, int* nsum, int* mg_max, int* block_elems) {
@@ -62,6 +77,7 @@ static inline unsigned gemv_lds_bytes(unsigned type, int tokens, unsigned in_dim
   const unsigned nb = (in_dim + (unsigned)be - 1) / (unsigned)be;
   const unsigned ncs = (nb + (unsigned)bps - 1) / (unsigned)bps;
   const int per_set_f4 = mg * nf4 * 64;
+  if (gemv_direct_x(type, ng)) return (unsigned)(per_set_f4 * gemv_chunk_sets_direct(per_set_f4, ncs)) * 16u;
   const int ch = ng > 1 ? 1 : gemv_chunk_sets(per_set_f4, ncs);
   return (unsigned)(per_set_f4 * ch) * 16u + (unsigned)(mg * nsum * 64 * ch) * 4u;
 }

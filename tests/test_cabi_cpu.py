@@ -69,10 +69,13 @@ def test_gemv_launch_dims():
             grid, block, lds = quant.gemv_launch_dims(t, m, 4096, 12288)
             assert block == 256 and 12288 % grid == 0 and 4 <= 12288 // grid <= 32
             assert 0 < lds <= 49152 and lds % 256 == 0
-    # M = 1: the whole activation vector is staged once when it fits, plus two per-lane sums per 4096-value column set
-    assert quant.gemv_launch_dims(12, 1, 4096, 12288)[2] == 4096 * 4 + 512
-    assert quant.gemv_launch_dims(12, 1, 8192, 4096)[2] == 8192 * 4 + 1024
+    # K-quants, M = 1: the whole activation vector is staged once when it fits (up to 12288 values)
+    assert quant.gemv_launch_dims(12, 1, 4096, 12288)[2] == 4096 * 4
+    assert quant.gemv_launch_dims(12, 1, 8192, 4096)[2] == 8192 * 4
+    assert quant.gemv_launch_dims(14, 1, 12288, 4096)[2] == 12288 * 4
     assert quant.gemv_launch_dims(12, 1, 65536, 4096)[2] <= 49152
+    # Q8_0 keeps per-lane sums beside the staged activations: one per 1024-value column set and lane
+    assert quant.gemv_launch_dims(8, 1, 1024, 3584)[2] == 1024 * 4 + 256
     g1 = quant.gemv_launch_dims(12, 1, 256, 17)[0]
     assert g1 == -(-17 // (12288 // quant.gemv_launch_dims(12, 1, 4096, 12288)[0]))
     with pytest.raises(quant.QuantError):

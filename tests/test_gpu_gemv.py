@@ -269,3 +269,28 @@ def test_swiglu_kernel_and_fused_gate_up(gpu, oracle):
         quant.gemv_dual_swiglu_dev(1, 1, Q6_K, 1, 1, 256, 16, 1)
     for d in (gd, ud, od):
         d.close()
+
+
+@pytest.mark.parametrize("type_id,in_dim,out_dim", [(Q4_K, 4096, 64), (Q6_K, 12288, 40), (Q5_K, 1024, 33), (Q4_K, 16384, 24)])
+@pytest.mark.parametrize("tokens", [1, 2])
+def test_activations_at_any_float_alignment(gpu, oracle, type_id, in_dim, out_dim, tokens):
+    """The activations are copied to LDS 16 bytes per lane; the pointer a caller passes is only float-aligned
+    (one token of a longer buffer, an offset into a workspace). in_dim 16384 is staged in two chunks."""
+    rng = np.random.default_rng(in_dim + tokens)
+    raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    wd, od = DevArray(raw), DevArray(nbytes=4 * tokens * out_dim)
+    want = oracle.matmul_add(x, tokens, in_dim, raw, type_id, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8)
+    dense = np.abs(oracle.dequantize(raw, type_id, out_dim * in_dim)).reshape(out_dim, in_dim)
+    tol = gemv_tolerance(x, dense, tokens, in_dim).reshape(-1)
+    try:
+        for shift in (1, 2, 3):                       # floats
+            padded = np.concatenate([np.zeros(shift, dtype=np.float32), x.reshape(-1)])
+            xd = DevArray(padded)
+            quant.gemv_dev(wd.ptr, type_id, xd.ptr + 4 * shift, od.ptr, in_dim, out_dim, tokens)
+            got = od.read(np.float32, tokens * out_dim)
+            assert np.all(np.abs(got - want) <= tol), "shift %d" % shift
+            xd.close()
+    finally:
+        wd.close()
+        od.close()
