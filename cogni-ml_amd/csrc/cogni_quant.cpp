@@ -184,7 +184,7 @@ int cogni_gemv_launch_dims(uint32_t type, uint32_t tokens, uint32_t in_dim, uint
   const int rows = (tokens >= 1 && tokens <= COGNI_MAX_GEMV_TOKENS) ? gemv_rows_per_block(type, (int)tokens) : 0;
   if (!grid_x || !block_x || !shared_mem_bytes || out_dim == 0 || in_dim == 0 || rows == 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_launch_dims: bad argument");
-  *grid_x = (out_dim + (uint32_t)rows - 1) / (uint32_t)rows;
+  *grid_x = gemv_grid(type, (int)tokens, out_dim);
   *block_x = GEMV_BLOCK;
   *shared_mem_bytes = gemv_lds_bytes(type, (int)tokens, in_dim);
   return 0;
@@ -361,8 +361,7 @@ uint32_t cogni_gemv_top1_partials(uint32_t w_type, uint32_t out_dim) {
   if (!gemv_type(w_type) || out_dim == 0) return 0;
   uint32_t most = 0;
   for (uint32_t m = 1; m <= top1_token_cap(w_type); m++) {
-    const uint32_t rows = (uint32_t)gemv_rows_per_block(w_type, (int)m);
-    const uint32_t grid = (out_dim + rows - 1) / rows;
+    const uint32_t grid = gemv_grid(w_type, (int)m, out_dim);
     if (grid > most) most = grid;
   }
   return most;

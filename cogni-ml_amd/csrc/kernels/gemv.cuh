@@ -403,7 +403,8 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const typename F::Lane ln(lane);
-  u32 nb = F::nblocks(in_dim);
+  const u32 nb = F::nblocks(in_dim);
+  u32 nbv = nb;   // the copy the weight loads take their bounds from (see stage_direct)
   const u32 ncs = (nb + F::BPS - 1) / F::BPS;
   // K-quants with one token group: the activations go global -> LDS directly (no registers), sums from registers
   constexpr bool DIRECT = gemv_direct_x(F::TYPE, NG);
@@ -411,22 +412,29 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   // with several token groups each set is staged per group
   const u32 CH = NG > 1 ? 1u : (u32)(DIRECT ? gemv_chunk_sets_direct(MG * SET_F4, ncs) : gemv_chunk_sets(MG * SET_F4, ncs));
   const size_t row_bytes = F::row_bytes(nb);
-  const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
-
   static_assert(!SWIGLU || (DUAL && M == 1 && !ADD && R % 2 == 0), "SWIGLU is a one-token mode of the matrix pair");
   static_assert(!TOP1 || (!DUAL && !ADD), "TOP1 is a mode of the plain GEMV");
   const u32 total_rows = DUAL ? 2 * out_dim : out_dim;
+  // A workgroup takes the row groups blockIdx.x, blockIdx.x + gridDim.x, ... (GEMV_WAVES * R rows each; with SWIGLU
+  // half as many rows of each matrix); a grid of one workgroup per group is the plain case.
+  const u32 group_rows = SWIGLU ? GEMV_WAVES * R / 2 : GEMV_WAVES * R;
+  const u32 ngroups = ((SWIGLU ? out_dim : total_rows) + group_rows - 1) / group_rows;
+  u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
   const uint8_t* rowp[R];
+  auto set_group = [&](u32 grp) {
+    row0 = (grp * GEMV_WAVES + wave) * R;
 #pragma unroll
-  for (int r = 0; r < R; r++) {
-    if (SWIGLU) {   // slots 0 .. R/2-1: gate rows, slots R/2 .. R-1: the same rows of up
-      const u32 row = min(row0 / 2 + (u32)(r % (R / 2)), out_dim - 1);
-      rowp[r] = (r < R / 2 ? w : w_b) + (size_t)row * row_bytes;
-    } else {
-      const u32 row = min(row0 + r, total_rows - 1);
-      rowp[r] = (DUAL && row >= out_dim) ? w_b + (size_t)(row - out_dim) * row_bytes : w + (size_t)row * row_bytes;
+    for (int r = 0; r < R; r++) {
+      if (SWIGLU) {   // slots 0 .. R/2-1: gate rows, slots R/2 .. R-1: the same rows of up
+        const u32 row = min(row0 / 2 + (u32)(r % (R / 2)), out_dim - 1);
+        rowp[r] = (r < R / 2 ? w : w_b) + (size_t)row * row_bytes;
+      } else {
+        const u32 row = min(row0 + r, total_rows - 1);
+        rowp[r] = (DUAL && row >= out_dim) ? w_b + (size_t)(row - out_dim) * row_bytes : w + (size_t)row * row_bytes;
+      }
     }
-  }
+  };
+  set_group(blockIdx.x);
 
   float acc[R][M];
 #pragma unroll
@@ -499,7 +507,7 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
                                        (__attribute__((address_space(3))) void*)(xs + (size_t)u * 64), 16, 0, 0);
     }
     // everything that loads weights below takes its block count from here, so it cannot move above the copies
-    asm volatile("" : "+s"(nb));
+    asm volatile("" : "+v"(nbv));
   };
   const u32 lane_piece = F::swz(F::x_elem(0, lane, 0) >> 2);   // place of the lane's first piece in the image
   // The copies of this wavefront have landed once nothing it requested is outstanding. (Waiting for "all but the
@@ -557,36 +565,93 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     }
   };
 
+  // end of a row group: the lanes' partial sums become row values, which are stored (or, with TOP1, compared)
+  float top_best[M];
+  u32 top_best_id[M];
+#pragma unroll
+  for (int m = 0; m < M; m++) top_best[m] = -__builtin_inff(), top_best_id[m] = 0;
+  auto finish = [&](u32 row0) {
+    if constexpr (SWIGLU) {
+      float v[R];
+#pragma unroll
+      for (int r = 0; r < R; r++) v[r] = wave_sum(acc[r][0]);
+#pragma unroll
+      for (int r = 0; r < R / 2; r++) {
+        const u32 row = row0 / 2 + r;
+        if (lane == 0 && row < out_dim) out[row] = swiglu_one(v[r], v[r + R / 2]);
+      }
+    } else if constexpr (TOP1) {
+#pragma unroll
+      for (int m = 0; m < M; m++) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          const float v = wave_sum(acc[r][m]);
+          if (row0 + r < out_dim && v > top_best[m]) top_best[m] = v, top_best_id[m] = row0 + r;   // rows ascend
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int m = 0; m < M; m++) {
+          float v = wave_sum(acc[r][m]);
+          const u32 row = row0 + r;
+          if (lane == 0 && row < total_rows) {
+            if (DUAL && row >= out_dim) {
+              out_b[(size_t)m * out_dim + (row - out_dim)] = v;
+            } else {
+              const size_t o = (size_t)m * out_dim + row;
+              if (ADD) v += residual[o];
+              out[o] = v;
+            }
+          }
+        }
+      }
+    }
+  };
+  // TOP1: the wavefronts' winners meet in LDS; within a wavefront and from wavefront to wavefront the rows ascend,
+  // so "greater than" keeps the lowest row among equal values
+  auto top1_store = [&]() {
+    __shared__ float top_v[M][GEMV_WAVES];
+    __shared__ u32 top_i[M][GEMV_WAVES];
+    if (lane == 0) {
+#pragma unroll
+      for (int m = 0; m < M; m++) top_v[m][wave] = top_best[m], top_i[m][wave] = top_best_id[m];
+    }
+    __syncthreads();
+    if (tid < M) {
+      float best = top_v[tid][0];
+      u32 best_id = top_i[tid][0];
+#pragma unroll
+      for (int wv = 1; wv < GEMV_WAVES; wv++)
+        if (top_v[tid][wv] > best || (top_v[tid][wv] == best && top_i[tid][wv] < best_id)) best = top_v[tid][wv], best_id = top_i[tid][wv];
+      out[(size_t)tid * gridDim.x + blockIdx.x] = best;
+      top_ids[(size_t)tid * gridDim.x + blockIdx.x] = best_id;
+    }
+  };
+
   // (one token only: with two the registers no longer allow it; and only while the grid is a few
   // workgroups per compute unit - a long grid keeps the memory pipeline full by itself and is better off
   // with every load queued at once)
-  if (M == 1 && NG == 1 && F::SPI == 1 && GEMV_PIPELINED && gridDim.x <= GEMV_PIPELINE_MAX_GRID) {
+  constexpr bool PIPE = M == 1 && NG == 1 && F::SPI == 1 && GEMV_PIPELINED && DIRECT;
+  bool pipelined = false;
+  if constexpr (PIPE) pipelined = gridDim.x <= GEMV_PIPELINE_MAX_GRID;
+  if constexpr (PIPE) if (pipelined) {
     // Rolling pipeline over (column set, row): PF rows are in flight while one is consumed. A compute unit
     // accepts only so many loads at a time and serves its oldest wavefronts first, so a wavefront that
     // queues all its loads up front sits in the issue of them, and the ones served last still have all
     // their arithmetic to do when the last byte arrives. Here the arithmetic of a row starts as soon as
     // that row is there, and what is left after the last byte is one row's worth.
-    constexpr int PF = R >= 4 ? 2 : 1;
+    constexpr int PF = R >= 3 ? 2 : 1;
     typename F::template Stage<R> st;
-    float4 buf[FU];
-    if constexpr (DIRECT) stage_direct(0);
-    else stage_begin(0, 0, buf);
-#pragma unroll
-    for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nb);
-    if constexpr (DIRECT) stage_direct_wait();
-    else stage_end(0, 0, buf);
+    stage_direct(0);
     // one column set; `last` (a compile-time tag) says that no column set follows, so the prefetches that
     // would wrap into the next set are left out and the number of loads in flight stays a constant
     auto column_set = [&](u32 s, auto last) {
       if (s > 0 && (s % CH) == 0) {
-        if constexpr (DIRECT) {
-          __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
-          stage_direct(s);
-          stage_direct_wait();
-        } else {
-          stage_begin(s, 0, buf);
-          stage_end(s, 0, buf);
-        }
+        __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
+        stage_direct(s);
+        stage_direct_wait();
       }
       const bool valid = s * F::BPS + ln.jb < nb;
       float4 xr[MG][NF4];
@@ -595,8 +660,8 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
 #pragma unroll
       for (int r = 0; r < R; r++) {
         const int rr = (r + PF) % R;
-        if (r + PF < R) F::template load_row<R>(st, rr, rowp[rr], ln, s, nb);
-        else if constexpr (!decltype(last)::value) F::template load_row<R>(st, rr, rowp[rr], ln, s + 1, nb);
+        if (r + PF < R) F::template load_row<R>(st, rr, rowp[rr], ln, s, nbv);
+        else if constexpr (!decltype(last)::value) F::template load_row<R>(st, rr, rowp[rr], ln, s + 1, nbv);
         __builtin_amdgcn_sched_barrier(0);
         float c[MG];
         F::template compute<R, MG>(st, r, ln, xr, sx, c);
@@ -605,10 +670,31 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    for (u32 s = 0; s + 1 < ncs; s++) column_set(s, gemv_false{});
-    column_set(ncs - 1, gemv_true{});
-  } else
+    for (u32 grp = blockIdx.x;;) {
+      // the first rows of the group are requested, then (first group, or a row longer than one chunk) the staged
+      // activations are waited for
+#pragma unroll
+      for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nbv);
+      if (grp == blockIdx.x || ncs > CH) stage_direct_wait();
+      for (u32 s = 0; s + 1 < ncs; s++) column_set(s, gemv_false{});
+      column_set(ncs - 1, gemv_true{});
+      grp += gridDim.x;
+      if (grp >= ngroups) break;
+      // next row group of this workgroup; the activations stay where they are unless the row is longer than a chunk
+      finish(row0);
+#pragma unroll
+      for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
+      set_group(grp);
+      if (ncs > CH) {
+        __builtin_amdgcn_s_barrier();   // every wavefront has read the last chunk into registers
+        stage_direct(0);
+      }
+    }
+  }
   // Column sets are taken F::SPI at a time: all their weight loads are issued before the first is consumed.
+  if (!pipelined)
   for (u32 s = 0; s < ncs; s += F::SPI) {
     const bool restage = NG == 1 && (s % CH) == 0;   // CH is a multiple of SPI or covers the whole row
     float4 buf[FU];
@@ -621,9 +707,9 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
       stage_begin(s, 0, buf);
     }
     typename F::template Stage<R> stA, stB;
-    F::template load<R>(stA, rowp, ln, s, nb);
+    F::template load<R>(stA, rowp, ln, s, nbv);
     const bool two = F::SPI == 2 && s + 1 < ncs;
-    if (two) F::template load<R>(stB, rowp, ln, s + 1, nb);
+    if (two) F::template load<R>(stB, rowp, ln, s + 1, nbv);
     if constexpr (DIRECT) {
       if (restage) stage_direct_wait();
     } else if (restage) {
@@ -632,60 +718,8 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     step(stA, s);
     if (two) step(stB, s + 1);
   }
-  if constexpr (SWIGLU) {
-    float v[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) v[r] = wave_sum(acc[r][0]);
-#pragma unroll
-    for (int r = 0; r < R / 2; r++) {
-      const u32 row = row0 / 2 + r;
-      if (lane == 0 && row < out_dim) out[row] = swiglu_one(v[r], v[r + R / 2]);
-    }
-    return;
-  }
-  if constexpr (TOP1) {
-    __shared__ float top_v[M][GEMV_WAVES];
-    __shared__ u32 top_i[M][GEMV_WAVES];
-#pragma unroll
-    for (int m = 0; m < M; m++) {
-      float best = -__builtin_inff();
-      u32 best_id = 0;
-#pragma unroll
-      for (int r = 0; r < R; r++) {
-        const float v = wave_sum(acc[r][m]);
-        if (row0 + r < out_dim && v > best) best = v, best_id = row0 + r;
-      }
-      if (lane == 0) top_v[m][wave] = best, top_i[m][wave] = best_id;
-    }
-    __syncthreads();
-    if (tid < M) {
-      float best = top_v[tid][0];
-      u32 best_id = top_i[tid][0];
-#pragma unroll
-      for (int wv = 1; wv < GEMV_WAVES; wv++)
-        if (top_v[tid][wv] > best) best = top_v[tid][wv], best_id = top_i[tid][wv];
-      out[(size_t)tid * gridDim.x + blockIdx.x] = best;
-      top_ids[(size_t)tid * gridDim.x + blockIdx.x] = best_id;
-    }
-    return;
-  }
-#pragma unroll
-  for (int r = 0; r < R; r++) {
-#pragma unroll
-    for (int m = 0; m < M; m++) {
-      float v = wave_sum(acc[r][m]);
-      const u32 row = row0 + r;
-      if (lane == 0 && row < total_rows) {
-        if (DUAL && row >= out_dim) {
-          out_b[(size_t)m * out_dim + (row - out_dim)] = v;
-        } else {
-          const size_t o = (size_t)m * out_dim + row;
-          if (ADD) v += residual[o];
-          out[o] = v;
-        }
-      }
-    }
-  }
+  finish(row0);
+  if constexpr (TOP1) top1_store();
 }
 
 // ---- entry points ---------------------------------------------------------------------------

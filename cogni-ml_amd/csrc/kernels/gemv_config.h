@@ -9,7 +9,9 @@
 
 #define GEMV_ROWS_Q4K(M) ((M) <= 2 ? 4 : 2)
 #define GEMV_ROWS_Q5K(M) 2
+#ifndef GEMV_ROWS_Q6K
 #define GEMV_ROWS_Q6K(M) 2
+#endif
 #define GEMV_ROWS_Q80(M) 4
 
 // rows of the weight matrix one workgroup produces
@@ -56,6 +58,18 @@ static inline GEMV_HD int gemv_chunk_sets_direct(int per_set_f4, unsigned ncs) {
 #endif
 static constexpr inline GEMV_HD bool gemv_direct_x(unsigned type, int token_groups) {
   return GEMV_DIRECT_X && (type == 12 || type == 13 || type == 14) && token_groups == 1;
+}
+
+// One token of a K-quant matrix: the kernel walks row groups blockIdx.x, blockIdx.x + gridDim.x, ... with the
+// activations staged once, so a long matrix is launched as the workgroups that are resident together (3 per
+// compute unit at 3 wavefronts per SIMD, 256 compute units), each with the same number of groups up to one.
+#define GEMV_RESIDENT_WGS 768u
+static inline unsigned gemv_grid(unsigned type, int tokens, unsigned out_dim) {
+  const unsigned rows = (unsigned)gemv_rows_per_block(type, tokens);
+  const unsigned groups = (out_dim + rows - 1) / rows;
+  if (tokens != 1 || !gemv_direct_x(type, 1) || groups <= GEMV_RESIDENT_WGS) return groups;
+  const unsigned per_wg = (groups + GEMV_RESIDENT_WGS - 1) / GEMV_RESIDENT_WGS;
+  return (groups + per_wg - 1) / per_wg;
 }
 
 // column-set geometry per type: blocks per set, float4 of x per lane and set, tokens per register group

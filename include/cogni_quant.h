@@ -71,7 +71,9 @@ int cogni_quant_code_object(const void** image, size_t* size);
  * Returns NULL for an unsupported combination. No GPU needed. */
 const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add);
 /* Launch geometry of the GEMV kernel for (type, tokens) at this shape: block_x = 256 threads, grid_x =
- * ceil(out_dim / rows_per_block) where rows_per_block depends on the type and token count, all other
+ * ceil(out_dim / rows_per_block) where rows_per_block depends on the type and token count - except that one token
+ * of a K-quant matrix with more than 768 such row groups is launched as at most 768 workgroups, each walking
+ * several groups (the kernels accept any grid_x up to the number of row groups) - all other
  * grid/block extents 1, and shared_mem_bytes of dynamic shared memory (the staged activations), which
  * goes into the shared_mem_bytes argument of the launch (driver.cr:278-286). (The reference's kernels
  * use grid ceil(out_dim/4) x block 128 and no dynamic shared memory, bin/cuda_q4k_gemv_probe.cr:225-230.)

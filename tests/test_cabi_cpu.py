@@ -76,6 +76,12 @@ def test_gemv_launch_dims():
     assert quant.gemv_launch_dims(12, 1, 65536, 4096)[2] <= 49152
     # Q8_0 keeps per-lane sums beside the staged activations: one per 1024-value column set and lane
     assert quant.gemv_launch_dims(8, 1, 1024, 3584)[2] == 1024 * 4 + 256
+    # one token of a long K-quant matrix: at most 768 workgroups that share the row groups evenly
+    g_head = quant.gemv_launch_dims(14, 1, 4096, 151936)[0]
+    groups = -(-151936 // 8)
+    assert g_head <= 768 and -(-groups // g_head) * (g_head - 1) < groups
+    assert quant.gemv_launch_dims(14, 2, 4096, 151936)[0] == groups and quant.gemv_launch_dims(8, 1, 4096, 151936)[0] == 151936 // 16
+    assert quant.gemv_top1_partials(14, 151936) == groups
     g1 = quant.gemv_launch_dims(12, 1, 256, 17)[0]
     assert g1 == -(-17 // (12288 // quant.gemv_launch_dims(12, 1, 4096, 12288)[0]))
     with pytest.raises(quant.QuantError):

@@ -294,3 +294,41 @@ def test_activations_at_any_float_alignment(gpu, oracle, type_id, in_dim, out_di
     finally:
         wd.close()
         od.close()
+
+
+@pytest.mark.parametrize("type_id,in_dim,out_dim", [(Q4_K, 256, 16 * 768 * 2 + 5), (Q6_K, 1024, 8 * 768 * 3 + 3),
+                                                    (Q5_K, 512, 8 * 768 + 1), (Q4_K, 16384, 16 * 768 + 17)])
+@pytest.mark.parametrize("add", [False, True])
+def test_long_matrices_walk_row_groups(gpu, oracle, type_id, in_dim, out_dim, add):
+    """One token of a K-quant matrix with more row groups than resident workgroups: every workgroup takes several
+    groups. Rows are independent, so the result must equal, bit for bit, what the same kernel gives on slices of
+    the matrix short enough for one group per workgroup; a few rows are also checked against the oracle.
+    in_dim 16384 does not fit the staging buffer at once: the activations are staged again for every group."""
+    rng = np.random.default_rng(out_dim)
+    raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+    x = synth.make_activations(rng, 1, in_dim)
+    res = rng.standard_normal(out_dim).astype(np.float32) if add else None
+    row_bytes = raw.size // out_dim
+    wd, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * out_dim)
+    rd = DevArray(res) if add else None
+    try:
+        grid = quant.gemv_launch_dims(type_id, 1, in_dim, out_dim)[0]
+        assert grid <= 768
+        quant.gemv_dev(wd.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, 1, rd.ptr if add else 0)
+        full = od.read(np.float32, out_dim)
+        piece = 4096                                   # at most 512 row groups
+        parts = np.empty(out_dim, dtype=np.float32)
+        for r0 in range(0, out_dim, piece):
+            n = min(piece, out_dim - r0)
+            quant.gemv_dev(wd.ptr + r0 * row_bytes, type_id, xd.ptr, od.ptr, in_dim, n, 1, rd.ptr + 4 * r0 if add else 0)
+            parts[r0:r0 + n] = od.read(np.float32, n)
+        assert np.array_equal(full, parts)
+        rows = np.unique(np.concatenate([np.arange(3), rng.integers(0, out_dim, 24), np.arange(out_dim - 3, out_dim)]))
+        for r in rows:
+            bias = np.array([res[r] if add else 0.0], dtype=np.float32)
+            want = oracle.matmul_add(x, 1, in_dim, raw[r * row_bytes:(r + 1) * row_bytes], type_id, 1, bias)[0]
+            w_abs = np.abs(oracle.dequantize(raw[r * row_bytes:(r + 1) * row_bytes], type_id, in_dim)).max()
+            assert abs(full[r] - want) <= 1e-4 * np.linalg.norm(x) * w_abs, "row %d" % r
+    finally:
+        for d in (wd, xd, od) + ((rd,) if add else ()):
+            d.close()

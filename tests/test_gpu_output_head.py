@@ -51,12 +51,12 @@ def test_top1_ties_take_the_lowest_row(gpu):
     """Rows with identical bytes give identical sums: the lowest row index must win, across wavefronts, workgroups and
     the strided final reduce."""
     rng = np.random.default_rng(1)
-    in_dim, out_dim = 512, 6000
+    in_dim, out_dim = 512, 20000          # 2500 row groups: every workgroup takes three or four of them
     base = synth.make_weights(rng, Q6_K, out_dim, in_dim).reshape(out_dim, -1)
     x = synth.make_activations(rng, 2, in_dim)
     _, _, logits = run_top1(np.ascontiguousarray(base).reshape(-1), Q6_K, x, in_dim, out_dim, 2)
     best = int(np.argmax(logits[0]))
-    for dup in ([5, 2048 + 3, 5999], [4097, 1031], [best]):
+    for dup in ([5, 2048 + 3, 5999], [4097, 1031], [19999, 12000], [best]):
         rows = base.copy()
         for r in dup:
             rows[r] = base[best]           # same bytes as the winning row
