@@ -49,10 +49,6 @@ __device__ __forceinline__ float mix2(u32 t, float a, float b, float acc) {
 
 struct gemv_true { static constexpr bool value = true; };
 struct gemv_false { static constexpr bool value = false; };
-#ifndef GEMV_PIPELINED
-#define GEMV_PIPELINED 1
-#endif
-#define GEMV_PIPELINE_MAX_GRID 4096u
 #define TWO_P24 16777216.0f
 #define TWO_P20 1048576.0f
 
@@ -404,7 +400,6 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const typename F::Lane ln(lane);
   const u32 nb = F::nblocks(in_dim);
-  u32 nbv = nb;   // the copy the weight loads take their bounds from (see stage_direct)
   const u32 ncs = (nb + F::BPS - 1) / F::BPS;
   // K-quants with one token group: the activations go global -> LDS directly (no registers), sums from registers
   constexpr bool DIRECT = gemv_direct_x(F::TYPE, NG);
@@ -493,39 +488,66 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     __syncthreads();
   };
 
-  // Direct staging of column sets [s0, s0+CH): the LDS image of a (token, set) is its 16 KiB in natural order up to
-  // F::swz. It is copied in 1 KiB units dealt round-robin to the wavefronts, each one global_load_lds_dwordx4
-  // (lane l lands at unit base + 16 l) over 1 KiB of contiguous global memory. Sets past the end of the row are
-  // replaced by the row's last float4: the lanes that would use them are masked out of the sums by `valid`.
-  auto stage_direct = [&](u32 s0) {
-    const u32 units = (u32)(MG * 16) * CH;
-    for (u32 u = wave; u < units; u += GEMV_WAVES) {
-      const u32 uu = u & 15u, cm = u >> 4;
-      const u32 cset = min(s0 + cm % CH, ncs - 1), m = cm / CH;
-      const u32 e = min((cset * 1024u + F::swz(uu * 64u + lane)) * 4u, in_dim - 4);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(x + (size_t)m * in_dim + e),
-                                       (__attribute__((address_space(3))) void*)(xs + (size_t)u * 64), 16, 0, 0);
+  // Staging of the chunk of column sets that starts at s0 for the kernels with one token group (DIRECT): the LDS image
+  // of a (token, set) is its 16 KiB in natural order up to F::swz, 1024 float4 = 4 per thread, read from global memory
+  // 1 KiB per wavefront and instruction. Every float4 of the chunk is requested before anything else happens (up to 12
+  // per thread, in registers that are free this early), `between` then requests the first weight rows, and the values
+  // are stored to LDS: the wait in front of the stores is a register dependency, so the compiler counts the younger
+  // loads and the weight rows stay in flight across the barrier. Sets past the end of the row are replaced by the
+  // row's last float4; the lanes that would use them are masked out of the sums by `valid`.
+  constexpr int CHC = gemv_chunk_sets_direct(MG * SET_F4, 2);   // sets per chunk of a row longer than one set
+  auto stage_rounds = [&](u32 s0, auto rounds, auto&& between) {
+    constexpr int NR = decltype(rounds)::value, PER_TOKEN = NR / MG;
+    float4 buf[NR * 4];
+#pragma unroll
+    for (int q = 0; q < NR; q++) {
+      const u32 cset = min(s0 + (u32)(q % PER_TOKEN), ncs - 1);
+      const float* xrow = x + (size_t)(q / PER_TOKEN) * in_dim;
+#pragma unroll
+      for (int k = 0; k < 4; k++)
+        buf[q * 4 + k] = ldx4(xrow + min((cset * 1024u + F::swz(k * GEMV_BLOCK + tid)) * 4u, in_dim - 4));
     }
-    // everything that loads weights below takes its block count from here, so it cannot move above the copies
-    asm volatile("" : "+v"(nbv));
-  };
-  const u32 lane_piece = F::swz(F::x_elem(0, lane, 0) >> 2);   // place of the lane's first piece in the image
-  // The copies of this wavefront have landed once nothing it requested is outstanding. (Waiting for "all but the
-  // weight loads issued since" would let the arithmetic start a little earlier, but the compiler is free to move
-  // those loads below the wait, and then the count would be wrong.)
-  auto stage_direct_wait = [&]() {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    between();
+#pragma unroll
+    for (int q = 0; q < NR; q++)
+#pragma unroll
+      for (int k = 0; k < 4; k++) xs[q * 1024 + k * GEMV_BLOCK + tid] = buf[q * 4 + k];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
+  auto stage_chunk = [&](u32 s0, auto&& between) {
+    if (ncs == 1) stage_rounds(s0, std::integral_constant<int, MG>{}, between);
+    else stage_rounds(s0, std::integral_constant<int, MG * CHC>{}, between);
+  };
+  // The same chunk one (token, set) at a time, for the places where many registers are live: the later chunks of a
+  // row that is longer than one chunk.
+  auto stage_chunk_serial = [&](u32 s0) {
+    for (u32 q = 0; q < (u32)MG * CH; q++) {
+      const u32 cset = min(s0 + q % CH, ncs - 1);
+      const float* xrow = x + (size_t)(q / CH) * in_dim;
+#pragma unroll 1
+      for (u32 k = 0; k < 4; k++)   // (one float4 at a time: this runs with most registers taken)
+        xs[q * 1024 + k * GEMV_BLOCK + tid] = ldx4(xrow + min((cset * 1024u + F::swz(k * GEMV_BLOCK + tid)) * 4u, in_dim - 4));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  const u32 lane_byte = F::swz(F::x_elem(0, lane, 0) >> 2) << 4;   // byte offset of the lane's first piece in the image
   auto read_x = [&](u32 s, float4 (&xr)[MG][NF4], float (&sx)[MG][NSUM]) {
+    // (one XOR per address, formed here every time: left to itself the compiler keeps the 16 addresses in registers
+    // for the whole kernel, which the pipeline below cannot spare)
+    u32 lb = lane_byte;
+    asm volatile("" : "+v"(lb));
+    const char* xsb = reinterpret_cast<const char*>(xs);
 #pragma unroll
     for (int mm = 0; mm < MG; mm++) {
       const u32 cm = mm * CH + (s % CH);
 #pragma unroll
       for (int i = 0; i < NF4; i++) {
         // direct image: the lane's pieces differ from its first in bits the swizzle neither reads nor writes
-        if constexpr (DIRECT) xr[mm][i] = xs[cm * 1024 + (lane_piece ^ (F::x_elem(0, 0, i) >> 2))];
+        if constexpr (DIRECT) xr[mm][i] = *reinterpret_cast<const float4*>(xsb + ((lb + cm * 16384u) ^ ((F::x_elem(0, 0, i) >> 2) << 4)));
         else xr[mm][i] = xs[(cm * NF4 + i) * 64 + lane];
       }
 #pragma unroll
@@ -630,13 +652,9 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     }
   };
 
-  // (one token only: with two the registers no longer allow it; and only while the grid is a few
-  // workgroups per compute unit - a long grid keeps the memory pipeline full by itself and is better off
-  // with every load queued at once)
-  constexpr bool PIPE = M == 1 && NG == 1 && F::SPI == 1 && GEMV_PIPELINED && DIRECT;
-  bool pipelined = false;
-  if constexpr (PIPE) pipelined = gridDim.x <= GEMV_PIPELINE_MAX_GRID;
-  if constexpr (PIPE) if (pipelined) {
+  // (one token only: with two the registers no longer allow it)
+  constexpr bool PIPE = M == 1 && NG == 1 && F::SPI == 1 && DIRECT;
+  if constexpr (PIPE) {
     // Rolling pipeline over (column set, row): PF rows are in flight while one is consumed. A compute unit
     // accepts only so many loads at a time and serves its oldest wavefronts first, so a wavefront that
     // queues all its loads up front sits in the issue of them, and the ones served last still have all
@@ -644,14 +662,16 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     // that row is there, and what is left after the last byte is one row's worth.
     constexpr int PF = R >= 3 ? 2 : 1;
     typename F::template Stage<R> st;
-    stage_direct(0);
+    stage_chunk(0, [&]() {
+#pragma unroll
+      for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nb);
+    });
     // one column set; `last` (a compile-time tag) says that no column set follows, so the prefetches that
     // would wrap into the next set are left out and the number of loads in flight stays a constant
     auto column_set = [&](u32 s, auto last) {
       if (s > 0 && (s % CH) == 0) {
         __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
-        stage_direct(s);
-        stage_direct_wait();
+        stage_chunk_serial(s);
       }
       const bool valid = s * F::BPS + ln.jb < nb;
       float4 xr[MG][NF4];
@@ -660,8 +680,8 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
 #pragma unroll
       for (int r = 0; r < R; r++) {
         const int rr = (r + PF) % R;
-        if (r + PF < R) F::template load_row<R>(st, rr, rowp[rr], ln, s, nbv);
-        else if constexpr (!decltype(last)::value) F::template load_row<R>(st, rr, rowp[rr], ln, s + 1, nbv);
+        if (r + PF < R) F::template load_row<R>(st, rr, rowp[rr], ln, s, nb);
+        else if constexpr (!decltype(last)::value) F::template load_row<R>(st, rr, rowp[rr], ln, s + 1, nb);
         __builtin_amdgcn_sched_barrier(0);
         float c[MG];
         F::template compute<R, MG>(st, r, ln, xr, sx, c);
@@ -670,50 +690,51 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
         __builtin_amdgcn_sched_barrier(0);
       }
     };
+    // The row groups of this workgroup. The first rows of the first group are in flight already (requested above,
+    // between the request for the activations and their way into LDS); a later group requests them at the top of the
+    // loop, after staging its first chunk of activations again if the row is longer than one chunk (otherwise the
+    // activations stay where they are).
     for (u32 grp = blockIdx.x;;) {
-      // the first rows of the group are requested, then (first group, or a row longer than one chunk) the staged
-      // activations are waited for
+      if (grp != blockIdx.x) {
+        if (ncs > CH) {
+          __builtin_amdgcn_s_barrier();   // every wavefront has read the last chunk into registers
+          stage_chunk_serial(0);
+        }
 #pragma unroll
-      for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nbv);
-      if (grp == blockIdx.x || ncs > CH) stage_direct_wait();
+        for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nb);
+      }
       for (u32 s = 0; s + 1 < ncs; s++) column_set(s, gemv_false{});
       column_set(ncs - 1, gemv_true{});
       grp += gridDim.x;
       if (grp >= ngroups) break;
-      // next row group of this workgroup; the activations stay where they are unless the row is longer than a chunk
       finish(row0);
 #pragma unroll
       for (int r = 0; r < R; r++)
 #pragma unroll
         for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
       set_group(grp);
-      if (ncs > CH) {
-        __builtin_amdgcn_s_barrier();   // every wavefront has read the last chunk into registers
-        stage_direct(0);
-      }
     }
   }
   // Column sets are taken F::SPI at a time: all their weight loads are issued before the first is consumed.
-  if (!pipelined)
+  if constexpr (!PIPE)
   for (u32 s = 0; s < ncs; s += F::SPI) {
     const bool restage = NG == 1 && (s % CH) == 0;   // CH is a multiple of SPI or covers the whole row
-    float4 buf[FU];
+    typename F::template Stage<R> stA, stB;
+    const bool two = F::SPI == 2 && s + 1 < ncs;
     if constexpr (DIRECT) {
+      auto rows = [&]() { F::template load<R>(stA, rowp, ln, s, nb); };   // (SPI is 1 for these formats)
       if (restage) {
         if (s > 0) __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
-        stage_direct(s);
+        stage_chunk(s, rows);
+      } else {
+        rows();
       }
-    } else if (restage) {
-      stage_begin(s, 0, buf);
-    }
-    typename F::template Stage<R> stA, stB;
-    F::template load<R>(stA, rowp, ln, s, nbv);
-    const bool two = F::SPI == 2 && s + 1 < ncs;
-    if (two) F::template load<R>(stB, rowp, ln, s + 1, nbv);
-    if constexpr (DIRECT) {
-      if (restage) stage_direct_wait();
-    } else if (restage) {
-      stage_end(s, 0, buf);
+    } else {
+      float4 buf[FU];
+      if (restage) stage_begin(s, 0, buf);
+      F::template load<R>(stA, rowp, ln, s, nb);
+      if (two) F::template load<R>(stB, rowp, ln, s + 1, nb);
+      if (restage) stage_end(s, 0, buf);
     }
     step(stA, s);
     if (two) step(stB, s + 1);

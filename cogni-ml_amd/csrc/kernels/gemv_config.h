@@ -45,19 +45,17 @@ static inline GEMV_HD int gemv_chunk_sets(int per_set_f4, unsigned ncs) {
   return ch;
 }
 
-// K-quant kernels whose tokens all fit the registers at once (one token group) copy the activations global -> LDS
-// without passing through registers and form the per-lane sums from the registers they are read into: no sums in LDS.
-static inline GEMV_HD int gemv_chunk_sets_direct(int per_set_f4, unsigned ncs) {
+// K-quant kernels whose tokens all fit the registers at once (one token group) keep the activations in LDS in natural
+// order (16 KiB per token and column set) and form the per-lane sums from the registers they are read into: no sums
+// in LDS. A row of one column set is staged as just that; longer rows in chunks of as many sets as fit the budget
+// (3 for one token, 1 for two), whole chunks even where the row ends inside one.
+static constexpr inline GEMV_HD int gemv_chunk_sets_direct(int per_set_f4, unsigned ncs) {
   int ch = GEMV_LDS_BYTES / 16 / per_set_f4;
   if (ch < 1) ch = 1;
-  if ((unsigned)ch >= ncs) return (int)ncs;
-  return ch;
+  return ncs <= 1 ? 1 : ch;
 }
-#ifndef GEMV_DIRECT_X
-#define GEMV_DIRECT_X 1
-#endif
 static constexpr inline GEMV_HD bool gemv_direct_x(unsigned type, int token_groups) {
-  return GEMV_DIRECT_X && (type == 12 || type == 13 || type == 14) && token_groups == 1;
+  return (type == 12 || type == 13 || type == 14) && token_groups == 1;
 }
 
 // One token of a K-quant matrix: the kernel walks row groups blockIdx.x, blockIdx.x + gridDim.x, ... with the

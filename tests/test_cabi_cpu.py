@@ -69,9 +69,9 @@ def test_gemv_launch_dims():
             grid, block, lds = quant.gemv_launch_dims(t, m, 4096, 12288)
             assert block == 256 and 12288 % grid == 0 and 4 <= 12288 // grid <= 32
             assert 0 < lds <= 49152 and lds % 256 == 0
-    # K-quants, M = 1: the whole activation vector is staged once when it fits (up to 12288 values)
+    # K-quants, M = 1: a row of one 4096-value column set is staged as that; a longer one in chunks of three sets
     assert quant.gemv_launch_dims(12, 1, 4096, 12288)[2] == 4096 * 4
-    assert quant.gemv_launch_dims(12, 1, 8192, 4096)[2] == 8192 * 4
+    assert quant.gemv_launch_dims(12, 1, 8192, 4096)[2] == 12288 * 4
     assert quant.gemv_launch_dims(14, 1, 12288, 4096)[2] == 12288 * 4
     assert quant.gemv_launch_dims(12, 1, 65536, 4096)[2] <= 49152
     # Q8_0 keeps per-lane sums beside the staged activations: one per 1024-value column set and lane
