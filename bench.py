@@ -85,19 +85,16 @@ class GemvCase:
             b.close()
 
 
-def graph_ok(wanted):
-    return bool(wanted)
-
-
 def time_steps(hip, stream, launch, steps, warmup, graph=True):
     """Run `warmup` untimed and exactly `steps` timed launches on `stream`; returns ms for the timed region.
     The timed launches are captured into one HIP graph so host launch latency does not gate the GPU."""
     for i in range(warmup):
         launch(i, stream)
     stream.synchronize()
+    graph_wanted = bool(graph)
     graph, exe = None, None
     try:
-        if not graph_ok(graph_wanted := graph):
+        if not graph_wanted:
             raise RuntimeError("direct launches requested")
         stream.begin_capture(1)
         for i in range(steps):

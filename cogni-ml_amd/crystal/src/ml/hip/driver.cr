@@ -54,6 +54,21 @@ lib LibCogniHIP
   fun cogni_dequantize_dev(w_raw : UInt64, w_type : UInt32, n_elements : UInt64, out : UInt64, stream : Void*) : Int32
   fun cogni_gemv_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, residual : UInt64, out : UInt64,
                      in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemv_plan(type : UInt32, tokens : UInt32, add : Int32, in_dim : UInt32, out_dim : UInt32, kernel : UInt8**,
+                      grid_x : UInt32*, block_x : UInt32*, shared_mem_bytes : UInt32*) : Int32
+  fun cogni_gemv_dual_dev(w_raw_a : UInt64, w_raw_b : UInt64, w_type : UInt32, x : UInt64, out_a : UInt64, out_b : UInt64,
+                          in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_swiglu_dev(gate : UInt64, up : UInt64, out : UInt64, n : UInt32, stream : Void*) : Int32
+  fun cogni_gemv_dual_swiglu_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, x : UInt64, out : UInt64,
+                                 in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_rmsnorm_dev(x : UInt64, norm : UInt64, out : UInt64, dim : UInt32, tokens : UInt32, eps : Float32,
+                        stream : Void*) : Int32
+  fun cogni_add_rmsnorm_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,
+                            dim : UInt32, tokens : UInt32, eps : Float32, stream : Void*) : Int32
+  fun cogni_gemv_top1_partials(w_type : UInt32, out_dim : UInt32) : UInt32
+  fun cogni_gemv_top1_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, partial_ids : UInt64, partial_values : UInt64,
+                          top1_ids : UInt64, top1_values : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
+                          stream : Void*) : Int32
   fun cogni_gemm_workspace_bytes(w_type : UInt32, in_dim : UInt32, tokens : UInt32) : LibC::SizeT
   fun cogni_gemm_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, bias : UInt64, out : UInt64,
                      in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
