@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 matrix peak, published
 # HBM bytes one q4_k_gemv_f32 launch moves at 12288x4096, M=1: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # (13974.0 and 48.0 per dispatch), scaled by what a 512 MiB copy kernel reads on the same counters (2.0, 1.0)
-MEASURED_TRAFFIC_BYTES = int((13974.0 * 2.0 + 48.0 * 1.0) * 1024)
+MEASURED_TRAFFIC_BYTES = int((13967.0 * 2.0 + 48.0 * 1.0) * 1024)
 LLC_BYTES = 256 << 20           # last-level (Infinity) cache
 Q4_K, Q5_K, Q6_K, Q8_0 = 12, 13, 14, 8
 TYPE_NAME = {Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", Q8_0: "Q8_0"}

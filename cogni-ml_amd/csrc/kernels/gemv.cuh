@@ -6,18 +6,21 @@
 //   *_gemv_add_f32        (w_raw, x, residual, out, in_dim, out_dim)           (q4k_gemv_probe.ptx:1572-1578)
 //   *_gemv_f32_tbatchM    same, M tokens: x rows at stride in_dim, out/residual rows at stride out_dim
 //   *_gemv_add_f32_tbatchM
-// Launch: block = 256 threads (4 wavefronts), grid = ceil(out_dim / rows_per_block), dynamic shared
-// memory = gemv_lds_bytes(type, tokens, in_dim), both from gemv_config.h. w_raw is row-major [out_dim][in_dim/QK][block_bytes];
+// Launch: block = 256 threads (4 wavefronts), grid = any number of workgroups up to ceil(out_dim / rows_per_block)
+// (a workgroup walks the row groups blockIdx.x, blockIdx.x + gridDim.x, ...; gemv_grid in gemv_config.h gives the
+// grid the library uses), dynamic shared memory = gemv_lds_bytes(type, tokens, in_dim), also from gemv_config.h.
+// w_raw is row-major [out_dim][in_dim/QK][block_bytes];
 // in_dim must be a multiple of 256 for the K-quants (Q8_0 takes any in_dim). Accumulation is fp32.
 //
 // Work split. A wavefront owns R consecutive output rows and walks them in "column sets": the span
 // of blocks the 64 lanes cover side by side (Q4_K/Q5_K/Q6_K: 4 lanes per 256-value super-block ->
-// 16 blocks; Q8_0: 2 lanes per 32-value block -> 32 blocks), all loads 16 bytes per lane. A lane always sits at the same position inside a block, so the activations it needs
-// for a column set are fixed: the workgroup stages x into LDS already in lane order
-// ([float4 index][lane]: conflict-free 16-byte reads), each lane pulls its share into registers and
-// reuses it for all R rows. Every weight byte is loaded exactly once, 16 bytes per lane; the loads of
-// column set s+2 are issued while set s is being consumed (two register stages), so a row of up to
-// two column sets is requested in full before the first byte is used.
+// 16 blocks; Q8_0: 2 lanes per 32-value block -> 32 blocks), all loads 16 bytes per lane. A lane always sits at
+// the same position inside a block, so the activations it needs for a column set are fixed: the workgroup stages
+// x into LDS once (K-quants with one or two tokens: in natural order with a bank swizzle, see stage_rounds;
+// otherwise already in lane order, [float4 index][lane]), each lane pulls its share into registers and reuses it
+// for all R rows. Every weight byte is loaded exactly once, 16 bytes per lane. One token of a K-quant matrix takes
+// its rows through a rolling pipeline (a row or two in flight while one is consumed); the other kernels request
+// the R rows of a column set together.
 //
 // Arithmetic. Per 32-value sub-block sum_j x_j*(d*sc*q_j - dmin*m) = d*sc*sum(q_j x_j) - dmin*m*sum(x_j);
 // sum(x_j) is per lane and computed once per column set. The integer codes are not converted to
