@@ -7,7 +7,7 @@
 // Two kernels:
 //   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 4 * in_dim/256
 //   q4_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
-//                   block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), no dynamic LDS (128 KiB static)
+//                   block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), no dynamic LDS (156 KiB static)
 //
 // Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows, so 512 x 12288 gives 256
 // workgroups, one per CU. K is walked one 256-value super-block at a time = 16 MFMA k-steps of 16.
@@ -16,9 +16,11 @@
 // every super-block; the two k halves are added through LDS once, at the end. Every weight is
 // dequantized by exactly one wavefront and reused for 128 tokens.
 //
-// Weights never touch LDS. In MFMA terms a lane is (weight row j = lane % 32, k-group kg = lane / 32)
+// The weights pass through LDS as raw bytes only (27 KiB per super-block, copied global -> LDS 16 bytes per lane
+// along the rows and picked up once per super-block by the lanes that decode them); they are never stored
+// dequantized. In MFMA terms a lane is (weight row j = lane % 32, k-group kg = lane / 32)
 // and supplies 8 k values per k-step. Lane (j, kg) of a kh wavefront owns the 64-value group
-// g = 2*kh + kg of its row's super-block: the 32 bytes qs[32g, 32g+32) as two 16-byte loads, one
+// g = 2*kh + kg of its row's super-block: the 32 bytes qs[32g, 32g+32) as two 16-byte LDS reads, one
 // (scale, min) pair decode. Eight consecutive bytes give two k-steps: their low nibbles (sub-block 2g)
 // and their high nibbles (sub-block 2g+1). A masked dword (q & 0x000F000F) | 0x64006400 is the half2
 // (1024 + n0, 1024 + n4); subtracting 1024 and one packed fma give fp16(d*sc*n - dmin*m) for two
@@ -27,9 +29,10 @@
 // [k-step][k-group][token][8 halves] of each (128-token tile, super-block), so staging x is a straight
 // 64 KiB copy (global_load_lds_dwordx4, no registers) and an A operand is one conflict-free ds_read_b128.
 //
-// The only LDS traffic in the loop is the activations: 4 KiB read per wavefront and k-step for 12
-// MFMAs. The x tile of the next super-block is copied while the current one is consumed (two 64 KiB
-// buffers) and the raw weight bytes of the next super-block are prefetched into registers.
+// LDS traffic in the loop: the activations, 4 KiB read per wavefront and k-step for 12 MFMAs, and the raw weights,
+// 9 x 16 bytes per lane and super-block. The x tile of the next super-block is copied while the current one is
+// consumed (two 64 KiB buffers); the raw weight bytes of the next super-block are copied into the one 28 KiB
+// buffer as soon as every wavefront has taken the current ones into registers.
 #pragma once
 #include "common.cuh"
 
@@ -104,6 +107,10 @@ __device__ __forceinline__ u32 h2_fma_off(u32 t, u32 off, u32 scale, u32 negmin)
 // the operand reads out of the other (otherwise every read would first wait for all loads in flight).
 __shared__ uint4 gemm_xbuf0[4096];   // [16 k-steps][2 k-groups][128 tokens] uint4
 __shared__ uint4 gemm_xbuf1[4096];
+// Raw bytes of one super-block of the workgroup's 192 weight rows, [row][144 B] = 1728 pieces of 16 bytes. Copied
+// global -> LDS 16 bytes per lane with consecutive lanes on consecutive pieces of a row (a 64-lane copy touches 7 or 8
+// rows = 14 to 16 cache lines; the same bytes fetched straight into the MFMA lane layout, one row per lane, touch 64).
+__shared__ uint4 gemm_wbuf[28 * 64];   // 27 copies of 64 pieces, and a 28th that keeps the four wavefronts in step
 
 struct GemmRaw {   // raw bytes of one group of one super-block of one weight row, as a lane sees them
   uint4 hdr, qa, qb;
@@ -129,17 +136,27 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
   if (vt >= mtiles * ntiles) return;
   const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
-  const u32 n0 = nt * GEMM_BN + nh * 96;             // first weight row of this wavefront
   const size_t row_bytes = (size_t)nkb * 144;
   const u32 sh = 16u * (g & 1);
   const bool upper = g >= 2;
 
-  // uniform base of the wavefront's rows + a 32-bit per-lane offset (96 rows are far below 4 GiB)
-  const u32 base_row = min(n0, out_dim - 1);
-  const uint8_t* wbase = w + (size_t)base_row * row_bytes;
-  u32 rowoff[3];
+  // Weight copies: piece p = 64 i + lane of the tile's super-block, i = wave, wave + 4, ... (27 copies of 64 pieces per
+  // workgroup and super-block; every wavefront issues 7, the 28th repeats the last piece into spare LDS so that no
+  // copy is conditional). Piece p is bytes [16 (p % 9), +16) of row p / 9.
+  const u32 tile_row0 = min(nt * GEMM_BN, out_dim - 1);
+  const uint8_t* wbase = w + (size_t)tile_row0 * row_bytes;   // uniform
+  u32 woff[7];
 #pragma unroll
-  for (int c = 0; c < 3; c++) rowoff[c] = (min(n0 + 32 * c + j, out_dim - 1) - base_row) * (u32)row_bytes;
+  for (int i = 0; i < 7; i++) {
+    const u32 p = min((4u * i + wave) * 64u + lane, (u32)GEMM_BN * 9u - 1u);
+    const u32 r = p / 9u, part = p - 9u * r;
+    woff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part;
+  }
+  // where this lane finds the raw bytes of its three rows in gemm_wbuf (in uint4 units): header, then the 32 bytes of
+  // its group
+  u32 wrow[3];
+#pragma unroll
+  for (int c = 0; c < 3; c++) wrow[c] = (nh * 96 + 32 * c + j) * 9;
   const uint4* xtile = xp + (size_t)mt * nkb * 4096;
 
   float16_t acc[4][3];
@@ -150,29 +167,23 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
-  auto load_raw = [&](GemmRaw (&raw)[3], u32 kb) {
-    const uint8_t* kbase = wbase + (size_t)kb * 144;   // uniform
-#pragma unroll
-    for (int c = 0; c < 3; c++) {
-      raw[c].hdr = ld16(kbase + rowoff[c]);
-      raw[c].qa = ld16(kbase + (rowoff[c] + 16 + 32 * g));
-      raw[c].qb = ld16(kbase + (rowoff[c] + 32 + 32 * g));
-    }
+  auto copy_w = [&](u32 kb, int i) {   // copy i of this wavefront for super-block kb
+    __builtin_amdgcn_global_load_lds((gbl_void*)(wbase + (size_t)kb * 144 + woff[i]),
+                                     (lds_void*)(gemm_wbuf + (4 * i + wave) * 64), 16, 0, 0);
   };
 
-  // Stage super-block 0 of x and the first weights. The main loop below takes super-blocks in pairs with
-  // fixed roles (x buffer 0 then 1, weight registers A then B) and no branch or register copy in its body;
-  // with an odd number of super-blocks the first one is taken alone out of buffer 1 / registers B.
+  // Stage super-block 0 of x and of the weights. The main loop below takes super-blocks in pairs with fixed x buffers
+  // (0 then 1) and no branch in its body; with an odd number of super-blocks the first one is taken alone out of
+  // buffer 1.
   const bool odd = nkb & 1;
-  GemmRaw rawA[3], rawB[3];
+#pragma unroll
+  for (int i = 0; i < 7; i++) copy_w(0, i);
   if (odd) {
-    load_raw(rawB, 0);
 #pragma unroll
     for (int i = 0; i < 16; i++)
       __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf1 + 256 * i + wave * 64),
                                        16, 0, 0);
   } else {
-    load_raw(rawA, 0);
 #pragma unroll
     for (int i = 0; i < 16; i++)
       __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
@@ -180,11 +191,23 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   }
   __syncthreads();
 
-  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt, const GemmRaw (&cur)[3], GemmRaw (&nxt)[3]) {
-    // (scale, -min) of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles) as duplicated half2. First thing
-    // in the iteration: the only loads in flight here are this super-block's weights, requested one
-    // iteration ago, so the wait in front of this costs nothing and does not cover the prefetches below.
-    u32 S[3][4];
+  // State that lives across super-blocks: the raw bytes and the decoded (scale, -min) pairs of the current one, and
+  // the two operand sets of the k-step pipeline.
+  GemmRaw cur[3];
+  u32 S[3][4];
+  uint4 A[2][4];
+  half8_t B[2][3];
+  // The raw bytes of a super-block, out of gemm_wbuf into the registers of the lanes that decode them.
+  auto take_raw = [&]() {
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      cur[c].hdr = gemm_wbuf[wrow[c]];
+      cur[c].qa = gemm_wbuf[wrow[c] + 1 + 2 * g];
+      cur[c].qb = gemm_wbuf[wrow[c] + 2 + 2 * g];
+    }
+  };
+  // (scale, -min) of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles) as duplicated half2
+  auto decode_scales = [&]() {
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const float d = h2f(cur[c].hdr.x), dm = h2f(cur[c].hdr.x >> 16);
@@ -197,61 +220,76 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       S[c][2] = h2_dup(d * ubyte_f<1>(scp));
       S[c][3] = h2_dup(-(dm * ubyte_f<1>(mp)));
     }
+  };
+  auto build_b = [&](half8_t (&Bd)[3], int t) {
+    const int h = t >> 2, op = t & 3, hi = op >> 1;
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      const uint4 Q = h ? cur[c].qb : cur[c].qa;
+      const u32 qa = (op & 1) ? Q.z : Q.x, qb = (op & 1) ? Q.w : Q.y;
+      const u32 mask = hi ? 0x00F000F0u : 0x000F000Fu;
+      const u32 magic = hi ? 0x54005400u : 0x64006400u;     // 64 + n (n sits 4 bits up) : 1024 + n
+      const u32 off = hi ? 0xD400D400u : 0xE400E400u;       // half2(-64) : half2(-1024)
+      const u32 sc = S[c][2 * hi], nm = S[c][2 * hi + 1];
+      uint4 bw;
+      bw.x = h2_fma_off((qa & mask) | magic, off, sc, nm);
+      bw.y = h2_fma_off(((qa >> 8) & mask) | magic, off, sc, nm);
+      bw.z = h2_fma_off((qb & mask) | magic, off, sc, nm);
+      bw.w = h2_fma_off(((qb >> 8) & mask) | magic, off, sc, nm);
+      Bd[c] = *reinterpret_cast<const half8_t*>(&bw);
+    }
+  };
+  // A operands of k-step t of the wavefront (k-steps 8*kh .. 8*kh+7 of the tile; 32 lanes read 512 contiguous bytes)
+  auto read_a = [&](uint4 (&Ad)[4], const uint4* xbuf, int t) {
+    const uint4* arow = xbuf + (16 * kh + kg) * 128 + j;
+#pragma unroll
+    for (int r = 0; r < 4; r++) Ad[r] = arow[t * 256 + r * 32];
+  };
+
+  // Operands of k-step 0 of the first super-block; after that every super-block prepares the first k-step of the
+  // next one in the shadow of its own last k-step.
+  take_raw();
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();   // gemm_wbuf is free for the copies of the next super-block
+  asm volatile("" ::: "memory");
+  decode_scales();
+  read_a(A[0], odd ? gemm_xbuf1 : gemm_xbuf0, 0);
+  build_b(B[0], 0);
+
+  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt) {
     const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
     const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
-    const uint8_t* knbase = wbase + (size_t)kn * 144; // uniform
-
-    const uint4* arow = xcur + (16 * kh + kg) * 128 + j;   // k-steps 8*kh .. 8*kh+7; 32 lanes read 512 contiguous bytes
-    auto build_b = [&](half8_t (&B)[3], int t) {
-      const int h = t >> 2, op = t & 3, hi = op >> 1;
-#pragma unroll
-      for (int c = 0; c < 3; c++) {
-        const uint4 Q = h ? cur[c].qb : cur[c].qa;
-        const u32 qa = (op & 1) ? Q.z : Q.x, qb = (op & 1) ? Q.w : Q.y;
-        const u32 mask = hi ? 0x00F000F0u : 0x000F000Fu;
-        const u32 magic = hi ? 0x54005400u : 0x64006400u;     // 64 + n (n sits 4 bits up) : 1024 + n
-        const u32 off = hi ? 0xD400D400u : 0xE400E400u;       // half2(-64) : half2(-1024)
-        const u32 sc = S[c][2 * hi], nm = S[c][2 * hi + 1];
-        uint4 bw;
-        bw.x = h2_fma_off((qa & mask) | magic, off, sc, nm);
-        bw.y = h2_fma_off(((qa >> 8) & mask) | magic, off, sc, nm);
-        bw.z = h2_fma_off((qb & mask) | magic, off, sc, nm);
-        bw.w = h2_fma_off(((qb >> 8) & mask) | magic, off, sc, nm);
-        B[c] = *reinterpret_cast<const half8_t*>(&bw);
-      }
+    auto copy_x = [&](int i) {
+      __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64), 16, 0, 0);
     };
-
     // software pipeline over the wavefront's eight k-steps: while the MFMAs of step t run, the A operands
     // of step t+1 are read from LDS and its B operands are built
-    uint4 A[2][4];
-    half8_t B[2][3];
-#pragma unroll
-    for (int r = 0; r < 4; r++) A[0][r] = arow[r * 32];
-    build_b(B[0], 0);
 #pragma unroll
     for (int t = 0; t < 8; t++) {
       const int p = t & 1;
-      // Prefetches for the next super-block, a few per k-step rather than all up front: a wavefront issues
-      // in order and the memory pipeline takes a vector memory instruction only every so many clocks, so
-      // 25 of them in a row stall the (only) wavefront of the SIMD with nothing to overlap. The raw weights
-      // (HBM, longest latency) go first, then the next x tile global -> LDS without passing through
-      // registers (global_load_lds_dwordx4: lane l of a wavefront lands at LDS base + 16*l) into the buffer
-      // that was last read in the previous iteration, which ended with a barrier.
+      // Copies for the next super-block, a few per k-step rather than all up front: a wavefront issues in order and
+      // a vector memory instruction costs it some 50 clocks, so 23 of them in a row stall the (only) wavefront of the
+      // SIMD with nothing to overlap. All of them are out by k-step 5; they are waited for behind k-step 6.
       if (t < 3) {
-        nxt[t].hdr = ld16(knbase + rowoff[t]);
-        nxt[t].qa = ld16(knbase + (rowoff[t] + 16 + 32 * g));
-        nxt[t].qb = ld16(knbase + (rowoff[t] + 32 + 32 * g));
+        copy_w(kn, 2 * t);
+        copy_w(kn, 2 * t + 1);
       }
+      if (t == 3) copy_w(kn, 6);
       if (t < 6) {
 #pragma unroll
-        for (int i = (t < 3 ? 2 * t : 3 * t - 3); i < (t < 3 ? 2 * t + 2 : (t < 5 ? 3 * t : 16)); i++)
-          __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64),
-                                           16, 0, 0);
+        for (int i = (t < 2 ? 2 * t : 3 * t - 2); i < (t < 2 ? 2 * t + 2 : 3 * t + 1); i++) copy_x(i);
       }
       if (t < 7) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) A[p ^ 1][r] = arow[(t + 1) * 256 + r * 32];
+        read_a(A[p ^ 1], xcur, t + 1);
         build_b(B[p ^ 1], t + 1);
+      } else {
+        // last k-step: the next super-block is in LDS (wait and barrier behind k-step 6); its raw bytes, scales and
+        // the operands of its first k-step are prepared while this step's MFMAs run (the current raw bytes and
+        // scales are no longer needed: the operands of this step were built in the previous one)
+        take_raw();
+        read_a(A[0], xnxt, 0);
+        decode_scales();
+        build_b(B[0], 0);
       }
 #pragma unroll
       for (int r = 0; r < 4; r++) {
@@ -262,33 +300,48 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       // Scheduling window = one k-step. Left alone the scheduler emits the twelve MFMAs back to back and the
       // operand preparation of the next step behind them, so the matrix pipe and the vector ALU take turns;
       // the group barriers below ask for the interleaving instead: the loads first, then one MFMA followed
-      // by five vector instructions, twelve times (an MFMA occupies the matrix pipe for 32 clocks, five
+      // by a few vector instructions, twelve times (an MFMA occupies the matrix pipe for 32 clocks, five
       // vector instructions issue in 20 to 35).
+      // keep the operands built above inside this window (otherwise they sink next to their first use,
+      // behind the window's MFMAs)
+#pragma unroll
+      for (int c = 0; c < 3; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
       if (t < 7) {
-        // keep the operands built above inside this window (otherwise they sink next to their first use,
-        // behind the window's MFMAs)
+        __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);   // VMEM reads (LDS-direct copies) of this step
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
 #pragma unroll
-        for (int c = 0; c < 3; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
-      }
-      __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);   // VMEM reads (weights, LDS-direct x) of this step
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
+        for (int i = 0; i < 12; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // five VALU
+        }
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x100, 13, 0);  // LDS reads: raw bytes and first A operands of the next super-block
 #pragma unroll
-      for (int i = 0; i < 12; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // five VALU
+        for (int i = 0; i < 3; i++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // three MFMAs while they arrive
+#pragma unroll
+        for (int i = 0; i < 9; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
+      if (t == 6) {
+        // everything this wavefront requested for the next super-block has to be there, then everybody meets
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    // End of the iteration: everything this wavefront requested has to be there (the x tile for everybody,
-    // the weights for its own next iteration), then everybody meets.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // End of the iteration: every wavefront has taken the next raw bytes out of gemm_wbuf and is done reading xcur;
+    // both are free for the copies of the super-block after next.
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
-  if (odd) iteration(0, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
+  if (odd) iteration(0, gemm_xbuf1, gemm_xbuf0);
   for (u32 kb = odd; kb < nkb; kb += 2) {
-    iteration(kb, gemm_xbuf0, gemm_xbuf1, rawA, rawB);
-    iteration(kb + 1, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
+    iteration(kb, gemm_xbuf0, gemm_xbuf1);
+    iteration(kb + 1, gemm_xbuf1, gemm_xbuf0);
   }
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
