@@ -275,19 +275,24 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
   // tokens per launch: groups of up to 4 where the matrix-core kernel takes the shape (several passes over
-  // the weights are still cheaper than one pass on the vector ALU, measured up to 8 tokens), else up to 8
-  // (the vector-ALU kernels of the K-quants hold two tokens in registers and take a third in a second pass over
-  // the staged weights at little cost, a fourth costs as much as the first two: groups of 3 measure fastest)
-  uint32_t cap = k_quant(w_type) ? 3u : (uint32_t)COGNI_MAX_GEMV_TOKENS;
+  // the weights are still cheaper than one pass on the vector ALU, measured up to 8 tokens); Q8_0 up to 8; the
+  // vector-ALU kernels of the K-quants hold two tokens in registers (a third costs a second pass over the staged
+  // weights, a fourth as much as the first two: Q6_K 4096x12288 takes 10.6 / 14.9 / 23.6 / 43.0 us for 1 / 2 / 3 / 4
+  // tokens), so they go in pairs, with one group of three when the count is odd
+  uint32_t cap = k_quant(w_type) ? 2u : (uint32_t)COGNI_MAX_GEMV_TOKENS;
+  bool pairs = k_quant(w_type);
   for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2; mt--) {
     if (gemv_mfma_supported(w_type, mt, in_dim)) {   // the most tokens whose activations fit its staging buffer
       cap = (uint32_t)mt;
+      pairs = false;
       break;
     }
   }
-  for (uint32_t t0 = 0; t0 < tokens; t0 += cap) {
+  uint32_t m = 0;
+  for (uint32_t t0 = 0; t0 < tokens; t0 += m) {
     const uint32_t left = tokens - t0;
-    const uint32_t m = left < cap ? left : cap;
+    m = left < cap ? left : cap;
+    if (pairs && left >= 3 && (left & 1u)) m = 3;
     uint32_t grid = 0, block = 0, shmem = 0;
     const char* kernel = nullptr;
     int rc = cogni_gemv_plan(w_type, m, residual != 0, in_dim, out_dim, &kernel, &grid, &block, &shmem);

@@ -107,8 +107,8 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 /* Decode GEMV, weights read once for all tokens:
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
  * fp32 accumulation. tokens >= 1; they are issued as consecutive launches of the token count that measures
- * fastest for the type and shape: up to 4 where cogni_gemv_plan picks the matrix-core kernel, else 3 for the
- * K-quants and 8 for Q8_0. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
+ * fastest for the type and shape: up to 4 where cogni_gemv_plan picks the matrix-core kernel, else pairs for the
+ * K-quants (one group of three when the count is odd) and up to 8 for Q8_0. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
  * same, bin/cuda_q4k_gemv_probe.cr:125); Q8_0 accepts any in_dim >= 1 (its last block is clipped,
  * quant_matmul.cr:241,259). Types: Q8_0, Q4_K, Q5_K, Q6_K. */
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
