@@ -93,6 +93,13 @@ def gemv_dual_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, x_ptr, out_ptr, in_dim, o
                                                 stream))
 
 
+def embed_dev(w_ptr, w_type, token_ids_ptr, output_ptr, history_ptr, token_index, hidden_dim, vocab_size, stream=None):
+    """output = dequantized embedding row token_ids[0]; history[token_index] = token_ids[0] (Q4_K, Q6_K)."""
+    _check(hip.lib().cogni_embed_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(token_ids_ptr),
+                                     ctypes.c_uint64(output_ptr), ctypes.c_uint64(history_ptr), ctypes.c_uint32(token_index),
+                                     ctypes.c_uint32(hidden_dim), ctypes.c_uint32(vocab_size), stream))
+
+
 def gemv_top1_partials(w_type, out_dim):
     f = hip.lib().cogni_gemv_top1_partials
     f.restype = ctypes.c_uint32

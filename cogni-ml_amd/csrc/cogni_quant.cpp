@@ -359,6 +359,18 @@ int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, 
   return launch("q4_k_dual_gemv_swiglu_f32", grid, block, shmem, params, stream, tokens);
 }
 
+int cogni_embed_dev(uint64_t w_raw, uint32_t w_type, uint64_t token_ids, uint64_t output, uint64_t history,
+                    uint32_t token_index, uint32_t hidden_dim, uint32_t vocab_size, void* stream) {
+  if (w_type != COGNI_TYPE_Q4_K && w_type != COGNI_TYPE_Q6_K)
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("GPU token embedding requires Q4_K or Q6_K token embeddings, got ") + type_name(w_type));
+  if (!w_raw || !token_ids || !output || !history) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_embed_dev: null device pointer");
+  if (hidden_dim == 0 || (hidden_dim % 256) != 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "embedding dim " + std::to_string(hidden_dim) + " must be divisible by 256");
+  const std::string name = std::string("embed_") + type_prefix(w_type) + "_f32_from_token_id";
+  void* params[] = {&w_raw, &token_ids, &output, &history, &token_index, &hidden_dim, &vocab_size};
+  return launch(name.c_str(), (hidden_dim + 1023) / 1024, 256, 0, params, stream);
+}
+
 // ---- output head: GEMV with the arg-max over the rows ---------------------------------------------------
 static uint32_t top1_token_cap(uint32_t type) { return (type == COGNI_TYPE_Q4_K || type == COGNI_TYPE_Q6_K) ? 3u : 1u; }
 

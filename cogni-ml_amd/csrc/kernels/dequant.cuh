@@ -23,28 +23,31 @@ __device__ __forceinline__ void zero_tail(float* out, u64 from, u64 n) {
   for (u64 e = from + tid; e < n; e += step) out[e] = 0.0f;
 }
 
+// Elements 4 lane .. 4 lane + 3 of the 256-element super-block at bp.
+__device__ __forceinline__ float4 deq4_q4_k(const uint8_t* bp, int lane) {
+  const int g = lane >> 4, li = lane & 15, hi = li >> 3;
+  const uint4 hdr = ld16(bp);
+  u32 q = ld4(bp + 16 + 32 * g + 4 * (li & 7));
+  u32 sc, m;
+  get_scale_min_k4(2 * g + hi, hdr.y, hdr.z, hdr.w, sc, m);
+  const float d = h2f_canonical(hdr.x), dmin = h2f_canonical(hdr.x >> 16);
+  const float d1 = d * (float)sc;
+  const float m1 = dmin * (float)m;
+  q = (hi ? (q >> 4) : q) & 0x0F0F0F0Fu;
+  float4 y;
+  y.x = d1 * ubyte_f<0>(q) - m1;
+  y.y = d1 * ubyte_f<1>(q) - m1;
+  y.z = d1 * ubyte_f<2>(q) - m1;
+  y.w = d1 * ubyte_f<3>(q) - m1;
+  return y;
+}
+
 extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q4_k_f32(const uint8_t* __restrict__ w,
                                                                               float* __restrict__ out, u64 n) {
   const u64 nb = n >> 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int g = lane >> 4, li = lane & 15, hi = li >> 3;
-  for (u64 b = (u64)blockIdx.x * DEQ_WAVES + wave; b < nb; b += (u64)gridDim.x * DEQ_WAVES) {
-    const uint8_t* bp = w + b * 144;
-    const uint4 hdr = ld16(bp);
-    u32 q = ld4(bp + 16 + 32 * g + 4 * (li & 7));
-    u32 sc, m;
-    get_scale_min_k4(2 * g + hi, hdr.y, hdr.z, hdr.w, sc, m);
-    const float d = h2f_canonical(hdr.x), dmin = h2f_canonical(hdr.x >> 16);
-    const float d1 = d * (float)sc;
-    const float m1 = dmin * (float)m;
-    q = (hi ? (q >> 4) : q) & 0x0F0F0F0Fu;
-    float4 y;
-    y.x = d1 * ubyte_f<0>(q) - m1;
-    y.y = d1 * ubyte_f<1>(q) - m1;
-    y.z = d1 * ubyte_f<2>(q) - m1;
-    y.w = d1 * ubyte_f<3>(q) - m1;
-    *reinterpret_cast<float4*>(out + b * 256 + 4 * lane) = y;
-  }
+  for (u64 b = (u64)blockIdx.x * DEQ_WAVES + wave; b < nb; b += (u64)gridDim.x * DEQ_WAVES)
+    *reinterpret_cast<float4*>(out + b * 256 + 4 * lane) = deq4_q4_k(w + b * 144, lane);
   zero_tail(out, nb << 8, n);
 }
 
@@ -75,29 +78,54 @@ extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q5_k_f32(cons
   zero_tail(out, nb << 8, n);
 }
 
+__device__ __forceinline__ float4 deq4_q6_k(const uint8_t* bp, int lane) {   // bp is 2-byte aligned only
+  const int half = lane >> 5, k = (lane & 31) >> 3, l0 = 4 * (lane & 7);
+  u32 ql = ld4(bp + 64 * half + 32 * (k & 1) + l0);
+  const u32 qh = ld4(bp + 128 + 32 * half + l0);
+  const int sc = (int)(signed char)bp[192 + 8 * half + 2 * k + (l0 >> 4)];
+  const float d = h2f_canonical(ld2(bp + 208));
+  const float ds = d * (float)sc;
+  ql = ((k < 2) ? ql : (ql >> 4)) & 0x0F0F0F0Fu;
+  const u32 q = ql | (((qh >> (2 * k)) & 0x03030303u) << 4);
+  float4 y;
+  y.x = ds * (float)((int)((q >> 0) & 0xFFu) - 32);
+  y.y = ds * (float)((int)((q >> 8) & 0xFFu) - 32);
+  y.z = ds * (float)((int)((q >> 16) & 0xFFu) - 32);
+  y.w = ds * (float)((int)((q >> 24) & 0xFFu) - 32);
+  return y;
+}
+
 extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q6_k_f32(const uint8_t* __restrict__ w,
                                                                               float* __restrict__ out, u64 n) {
   const u64 nb = n >> 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int half = lane >> 5, k = (lane & 31) >> 3, l0 = 4 * (lane & 7);
-  for (u64 b = (u64)blockIdx.x * DEQ_WAVES + wave; b < nb; b += (u64)gridDim.x * DEQ_WAVES) {
-    const uint8_t* bp = w + b * 210;  // 2-byte aligned only
-    u32 ql = ld4(bp + 64 * half + 32 * (k & 1) + l0);
-    const u32 qh = ld4(bp + 128 + 32 * half + l0);
-    const int sc = (int)(signed char)bp[192 + 8 * half + 2 * k + (l0 >> 4)];
-    const float d = h2f_canonical(ld2(bp + 208));
-    const float ds = d * (float)sc;
-    ql = ((k < 2) ? ql : (ql >> 4)) & 0x0F0F0F0Fu;
-    const u32 q = ql | (((qh >> (2 * k)) & 0x03030303u) << 4);
-    float4 y;
-    y.x = ds * (float)((int)((q >> 0) & 0xFFu) - 32);
-    y.y = ds * (float)((int)((q >> 8) & 0xFFu) - 32);
-    y.z = ds * (float)((int)((q >> 16) & 0xFFu) - 32);
-    y.w = ds * (float)((int)((q >> 24) & 0xFFu) - 32);
-    *reinterpret_cast<float4*>(out + b * 256 + 4 * lane) = y;
-  }
+  for (u64 b = (u64)blockIdx.x * DEQ_WAVES + wave; b < nb; b += (u64)gridDim.x * DEQ_WAVES)
+    *reinterpret_cast<float4*>(out + b * 256 + 4 * lane) = deq4_q6_k(w + b * 210, lane);
   zero_tail(out, nb << 8, n);
 }
+
+// One row of a Q4_K / Q6_K embedding matrix, picked by a token id that lives on the device - the reference's
+// embed_q4k_f32_from_token_id_cuda (src/ml/cuda/kernels/embed_q4k_probe.ptx:5-13; host side
+// bin/cuda_mixed_stack_probe.cr:900-947), same parameters:
+//   (w_raw, token_ids:u32*, output:f32*, history:u32*, token_index:u32, hidden_dim:u32, vocab_size:u32)
+// output[0..hidden_dim) = dequantized row token_ids[0] (zeros if the id is not below vocab_size), and
+// history[token_index] = token_ids[0]. hidden_dim is a multiple of 256; block 256, grid ceil(hidden_dim / 1024)
+// (a wavefront per super-block; the reference uses a thread per element, grid hidden_dim / 256).
+#define EMBED_KERNEL(NAME, DEQ4, BB)                                                                              \
+  extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void NAME(const uint8_t* w, const u32* token_ids, float* output, \
+                                                               u32* history, u32 token_index, u32 hidden_dim,     \
+                                                               u32 vocab_size) {                                  \
+    const u32 id = token_ids[0];                                                                                  \
+    if (blockIdx.x == 0 && threadIdx.x == 0) history[token_index] = id;                                           \
+    const int lane = threadIdx.x & 63;                                                                            \
+    const u32 b = blockIdx.x * DEQ_WAVES + (threadIdx.x >> 6), nb = hidden_dim >> 8;                              \
+    if (b >= nb) return;                                                                                          \
+    float4 y = make_float4(0.f, 0.f, 0.f, 0.f);                                                                   \
+    if (id < vocab_size) y = DEQ4(w + ((size_t)id * nb + b) * BB, lane);                                          \
+    *reinterpret_cast<float4*>(output + b * 256 + 4 * lane) = y;                                                  \
+  }
+EMBED_KERNEL(embed_q4_k_f32_from_token_id, deq4_q4_k, 144)
+EMBED_KERNEL(embed_q6_k_f32_from_token_id, deq4_q6_k, 210)
 
 // Q8_0 and IQ4_NL: 32-element blocks, ceil(n/32) of them, the last one clipped to n.
 extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q8_0_f32(const uint8_t* __restrict__ w,

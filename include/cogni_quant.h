@@ -152,6 +152,15 @@ int cogni_rmsnorm_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t dim, uin
 int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t dim,
                           uint32_t tokens, float eps, void* stream);
 
+/* One row of a Q4_K or Q6_K embedding matrix chosen by a token id that lives on the device: output[0..hidden_dim) =
+ * dequantized row token_ids[0] (zeros if the id is not below vocab_size) and history[token_index] = token_ids[0].
+ * Kernel "embed_<prefix>_f32_from_token_id" (w_raw, token_ids:u32*, output, history:u32*, token_index:u32,
+ * hidden_dim:u32, vocab_size:u32), block 256, grid ceil(hidden_dim / 1024) - the reference's
+ * embed_q4k_f32_from_token_id_cuda (src/ml/cuda/kernels/embed_q4k_probe.ptx:5-13, launched from
+ * bin/cuda_mixed_stack_probe.cr:935-941 with grid hidden_dim / 256). hidden_dim must be a multiple of 256. */
+int cogni_embed_dev(uint64_t w_raw, uint32_t w_type, uint64_t token_ids, uint64_t output, uint64_t history,
+                    uint32_t token_index, uint32_t hidden_dim, uint32_t vocab_size, void* stream);
+
 /* Output head without the logits: for each token the index of the largest element of W x and that value
  * (top1_ids: u32[tokens], top1_values: f32[tokens]); of equal values the lowest index wins, as in the reference's CPU scan
  * (bin/cuda_mixed_stack_probe.cr:1485-1497). Two launches per group of up to 3 tokens (Q4_K, Q6_K; one token for the other

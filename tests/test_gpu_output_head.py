@@ -102,3 +102,30 @@ def test_output_head_runner(gpu, oracle):
     finally:
         runner.close()
         stream.close()
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+def test_embedding_row_from_a_device_token_id(gpu, oracle, t):
+    """The reference's token embedder (bin/cuda_mixed_stack_probe.cr:900-947): row token_ids[0] of the embedding matrix,
+    bit-exact with the bulk dequantize; the id goes into the history; an id outside the vocabulary gives zeros."""
+    hidden, vocab = 1024, 300
+    rng = np.random.default_rng(int(t))
+    raw = synth.make_weights(rng, t, vocab, hidden)
+    table = oracle.dequantize(raw, t, vocab * hidden).reshape(vocab, hidden)
+    wd, idd = DevArray(raw), DevArray(np.zeros(1, dtype=np.uint32))
+    od, hd = DevArray(nbytes=4 * hidden), DevArray(np.full(8, 0xFFFFFFFF, dtype=np.uint32))
+    try:
+        for pos, tok in enumerate((0, 299, 17, 300, 4000000000)):
+            hip.copy_htod(idd.ptr, np.array([tok], dtype=np.uint32), 4, "token id")
+            quant.embed_dev(wd.ptr, t, idd.ptr, od.ptr, hd.ptr, pos, hidden, vocab)
+            got = od.read(np.float32, hidden)
+            want = table[tok] if tok < vocab else np.zeros(hidden, dtype=np.float32)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "token %d" % tok
+        assert list(hd.read(np.uint32, 8)) == [0, 299, 17, 300, 4000000000, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF]
+        with pytest.raises(quant.QuantError, match="requires Q4_K or Q6_K token embeddings, got Q8_0"):
+            quant.embed_dev(wd.ptr, Q8_0, idd.ptr, od.ptr, hd.ptr, 0, hidden, vocab)
+        with pytest.raises(quant.QuantError, match="embedding dim 1000 must be divisible by 256"):
+            quant.embed_dev(wd.ptr, t, idd.ptr, od.ptr, hd.ptr, 0, 1000, vocab)
+    finally:
+        for d in (wd, idd, od, hd):
+            d.close()
