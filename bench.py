@@ -127,11 +127,11 @@ def time_steps(hip, stream, launch, steps, warmup, graph=True):
     return ms, exe is not None
 
 
-def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, warmup, graph=True):
-    """Q4_K prefill GEMM (x repack + MFMA kernel) at `tokens`; returns (ms per call, TFLOP/s)."""
+def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, warmup, graph=True, Q4_K=Q4_K):
+    """Prefill GEMM (x repack + MFMA kernel) at `tokens`, Q4_K unless another type is given; returns (ms per call, TFLOP/s)."""
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
-    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens)
+    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens, out_dim)
     bufs = [hip.DeviceBuffer(n) for n in (raw.nbytes, x.nbytes, 4 * tokens * out_dim, wsb)]
     hip.copy_htod(bufs[0].ptr, raw, raw.nbytes, "w")
     hip.copy_htod(bufs[1].ptr, x, x.nbytes, "x")
@@ -269,6 +269,13 @@ def main():
         gemm["M=%d" % tokens] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
         log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
             tokens, gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
+
+    if args.mode == "cases":
+        gsteps = max(10, min(200, args.steps // 10))
+        per, tf = bench_gemm(hip, quant, synth, rng, stream, 512, 4096, 12288, gsteps, 5, Q4_K=Q6_K)
+        gemm["q6_k down 4096x12288 M=512"] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        log("case=q6_k_gemm prefill\ntype=Q6_K\nshape=12288x4096\ntokens=512\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
+            gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
 
     extra = {}
     if args.mode == "cases":

@@ -127,10 +127,16 @@ def add_rmsnorm_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_ptr, 
                                            ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
 
 
-def gemm_workspace_bytes(w_type, in_dim, tokens):
-    f = hip.lib().cogni_gemm_workspace_bytes
+def gemm_workspace_bytes(w_type, in_dim, tokens, out_dim=None):
+    """Bytes of caller-owned scratch for gemm_dev: the packed activations, and with `out_dim` given also the planes of
+    a k-split launch (few tiles), which gemm_dev uses when the workspace has room for them."""
+    if out_dim is None:
+        f = hip.lib().cogni_gemm_workspace_bytes
+        f.restype = ctypes.c_size_t
+        return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens))
+    f = hip.lib().cogni_gemm_workspace_bytes_split
     f.restype = ctypes.c_size_t
-    return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens))
+    return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens))
 
 
 def gemm_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_ptr, workspace_bytes, bias_ptr=0,

@@ -72,6 +72,7 @@ lib LibCogniHIP
                           top1_ids : UInt64, top1_values : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
                           stream : Void*) : Int32
   fun cogni_gemm_workspace_bytes(w_type : UInt32, in_dim : UInt32, tokens : UInt32) : LibC::SizeT
+  fun cogni_gemm_workspace_bytes_split(w_type : UInt32, in_dim : UInt32, out_dim : UInt32, tokens : UInt32) : LibC::SizeT
   fun cogni_gemm_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, bias : UInt64, out : UInt64,
                      in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
                      workspace : UInt64, workspace_bytes : LibC::SizeT, stream : Void*) : Int32

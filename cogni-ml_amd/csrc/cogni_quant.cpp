@@ -435,31 +435,69 @@ int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t resi
 
 int g_gemm_threshold = -1;   // -1: not resolved yet
 
+static bool gemm_type(uint32_t t) { return t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q6_K; }
+
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {
-  if (w_type != COGNI_TYPE_Q4_K || in_dim == 0 || tokens == 0) return 0;
+  if (!gemm_type(w_type) || in_dim == 0 || tokens == 0) return 0;
   const size_t mtiles = ((size_t)tokens + 127) / 128;
   return mtiles * 128 * (size_t)in_dim * 2;
 }
 
+// k splits of the prefill GEMM: a launch of fewer than half as many 128 x 192 tiles as there are compute units (256)
+// leaves most of them idle, so the super-blocks of a row are divided among up to 8 workgroups per tile, each with at
+// least two super-blocks; the partial sums go through the workspace.
+static uint32_t gemm_splits(uint32_t in_dim, uint32_t out_dim, uint32_t tokens) {
+  const uint32_t tiles = ((tokens + 127) / 128) * ((out_dim + 191) / 192), nkb = in_dim / 256;
+  uint32_t s = 256u / tiles;
+  if (s > 8) s = 8;
+  if (s > nkb / 2) s = nkb / 2;
+  return s < 2 ? 1 : s;
+}
+
+size_t cogni_gemm_workspace_bytes_split(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens) {
+  const size_t pack = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
+  if (pack == 0 || out_dim == 0 || (in_dim % 256) != 0) return pack;
+  const uint32_t s = gemm_splits(in_dim, out_dim, tokens);
+  return s == 1 ? pack : pack + (size_t)s * tokens * out_dim * sizeof(float);
+}
+
 int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
                    uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream) {
-  if (w_type != COGNI_TYPE_Q4_K)
+  if (!gemm_type(w_type))
     return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the prefill GEMM: ") + type_name(w_type));
   if (!w_raw || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: null device pointer");
   if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: zero dimension");
   if ((in_dim % 256) != 0)
-    return fail(COGNI_ERR_INVALID_ARGUMENT, "Q4_K GEMM requires in_dim multiple of 256, got " + std::to_string(in_dim));
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMM requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  if ((uint64_t)tokens * out_dim > 0xFFFFFFFFull)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: tokens * out_dim exceeds 2^32 - 1");
   const size_t need = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
   if (!workspace || workspace_bytes < need)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: workspace has " + std::to_string(workspace_bytes) + " bytes, needs " + std::to_string(need));
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 191) / 192;
   {
     void* params[] = {&x, &workspace, &tokens, &in_dim};
-    int rc = launch("pack_x_f16_q4k", mtiles * 4 * (in_dim / 256), 256, 0, params, stream);
+    int rc = launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_f16_q6k" : "pack_x_f16_q4k", mtiles * 4 * (in_dim / 256), 256, 0, params, stream);
     if (rc != 0) return rc;
   }
-  void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};
-  return launch("q4_k_gemm_f16", 8 * ((mtiles * ntiles + 7) / 8), 256, 0, params, stream);
+  // a workspace that holds the packed activations only: one workgroup per tile walks the whole row
+  uint32_t splits = gemm_splits(in_dim, out_dim, tokens);
+  if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) splits = 1;
+  const char* kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : "q4_k_gemm_f16";
+  const uint32_t grid = 8 * ((mtiles * ntiles + 7) / 8);
+  if (splits == 1) {
+    void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};
+    return launch(kernel, grid, 256, 0, params, stream);
+  }
+  uint64_t planes = workspace + need, none = 0;
+  uint32_t total = tokens * out_dim;
+  {
+    void* params[] = {&w_raw, &workspace, &none, &planes, &in_dim, &out_dim, &tokens};
+    int rc = launch(kernel, grid, 256, 0, params, stream, splits);
+    if (rc != 0) return rc;
+  }
+  void* params[] = {&planes, &bias, &out, &total, &out_dim, &splits};
+  return launch("gemm_sum_splits_f32", (total + 1023) / 1024, 256, 0, params, stream);
 }
 
 int cogni_set_gemm_threshold(int32_t tokens) {
@@ -481,7 +519,7 @@ int32_t cogni_get_gemm_threshold(void) {
 
 int cogni_matmul_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
                      uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream) {
-  if (w_type == COGNI_TYPE_Q4_K && tokens > (uint32_t)cogni_get_gemm_threshold())
+  if (gemm_type(w_type) && tokens > (uint32_t)cogni_get_gemm_threshold())
     return cogni_gemm_dev(w_raw, w_type, x, bias, out, in_dim, out_dim, tokens, workspace, workspace_bytes, stream);
   if (bias && tokens != 1)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_matmul_dev: a [out_dim] bias is only accepted with one token or on the GEMM path; "
@@ -564,7 +602,7 @@ int cogni_weight_matmul(const cogni_quant_weight* qw, const float* x, int32_t ro
   HIP_TRY(hipMalloc(&dx.p, xin), "hipMalloc(x)");
   HIP_TRY(hipMalloc(&dout.p, xout), "hipMalloc(result)");
   HIP_TRY(hipMemcpyHtoD(dx.p, const_cast<float*>(x), xin), "hipMemcpyHtoD(x)");
-  const bool gemm_path = qw->type == COGNI_TYPE_Q4_K && rows > cogni_get_gemm_threshold();
+  const bool gemm_path = gemm_type(qw->type) && rows > cogni_get_gemm_threshold();
   if (bias && !gemm_path) {  // bias[o] is added to every row: stage it as a [rows][out_dim] residual
     std::vector<float> tiled((size_t)rows * qw->out_dim);
     for (int32_t r = 0; r < rows; r++) std::memcpy(&tiled[(size_t)r * qw->out_dim], bias, (size_t)qw->out_dim * 4);
@@ -574,7 +612,7 @@ int cogni_weight_matmul(const cogni_quant_weight* qw, const float* x, int32_t ro
   int rc;
   if (gemm_path) {
     DeviceMem dws, dbias;
-    const size_t wsb = cogni_gemm_workspace_bytes(qw->type, (uint32_t)qw->in_dim, (uint32_t)rows);
+    const size_t wsb = cogni_gemm_workspace_bytes_split(qw->type, (uint32_t)qw->in_dim, (uint32_t)qw->out_dim, (uint32_t)rows);
     HIP_TRY(hipMalloc(&dws.p, wsb), "hipMalloc(gemm workspace)");
     if (bias) {
       HIP_TRY(hipMalloc(&dbias.p, (size_t)qw->out_dim * 4), "hipMalloc(bias)");

@@ -5,6 +5,7 @@
 #include "kernels/gemv.cuh"
 #include "kernels/gemv_mfma.cuh"
 #include "kernels/gemm_q4k.cuh"
+#include "kernels/gemm_q6k.cuh"
 #include "kernels/norm.cuh"
 #include "kernels/util.cuh"
 

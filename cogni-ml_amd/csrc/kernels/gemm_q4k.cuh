@@ -60,8 +60,9 @@ __device__ __forceinline__ u32 gemm_k_element(u32 ks, u32 kg, u32 e) {
 // per row), converted, transposed through LDS into the [k-step][k-group][token][8 halves] image and written out
 // as 32 runs of 512 contiguous bytes. Grid: ceil(m/128) * 4 * (in_dim/256) workgroups, x fastest.
 #define PACK_TOK 32
-extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q4k(const float* __restrict__ x, uint4* __restrict__ xp,
-                                                                  u32 m, u32 in_dim) {
+// Q6: the element order of the Q6_K kernel (gemm_q6k.cuh) instead of the Q4_K one.
+template <bool Q6>
+__device__ __forceinline__ void pack_x_core(const float* __restrict__ x, uint4* __restrict__ xp, u32 m, u32 in_dim) {
   // [32 (k-step, k-group)][32 tokens] uint4, each (k-step, k-group) row padded by one uint4 so that the
   // transposing 8-byte writes of a wavefront (same token, 32 different rows) spread over the banks
   __shared__ uint2 img[32 * (PACK_TOK + 1) * 2];
@@ -69,9 +70,19 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q4k(const float* __
   const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const u32 kb = blockIdx.x % nkb, tq = (blockIdx.x / nkb) & 3, mt = blockIdx.x / (4 * nkb);
   // lane -> 4 consecutive k = 4 lane .. 4 lane + 3 of the super-block; their place in the image (inverse of
-  // gemm_k_element): group g = k / 64, high-nibble half, 16-byte half h, upper-8-bytes bit, slot 0 or 4
-  const u32 k0 = 4 * lane, g = k0 >> 6, hi = (k0 >> 5) & 1, h = (k0 >> 4) & 1, up = (k0 >> 3) & 1, slot4 = (k0 >> 2) & 1;
-  const u32 ks = 8 * (g >> 1) + 4 * h + 2 * hi + up, kg = g & 1;
+  // gemm_k_element): Q4_K: group g = k / 64, high-nibble half, 16-byte half h, upper-8-bytes bit, slot 0 or 4;
+  // Q6_K: 128-half n, quadrant qd, 16-run u, upper-8 bit, slot 0 or 4 (gemm_k_element_q6k)
+  const u32 k0 = 4 * lane, slot4 = (k0 >> 2) & 1;
+  u32 ks, kg;
+  if (Q6) {
+    const u32 n = k0 >> 7, qd = (k0 >> 5) & 3, u = (k0 >> 4) & 1, h8 = (k0 >> 3) & 1;
+    ks = 8 * n + 2 * qd + h8;
+    kg = u;
+  } else {
+    const u32 g = k0 >> 6, hi = (k0 >> 5) & 1, h = (k0 >> 4) & 1, up = (k0 >> 3) & 1;
+    ks = 8 * (g >> 1) + 4 * h + 2 * hi + up;
+    kg = g & 1;
+  }
   const u32 cell = (ks * 2 + kg) * (PACK_TOK + 1);
 #pragma unroll
   for (int p = 0; p < PACK_TOK / 4; p++) {
@@ -91,6 +102,9 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q4k(const float* __
     const u32 c = i / PACK_TOK, tl = i % PACK_TOK;
     dst[c * 128 + tl] = *reinterpret_cast<const uint4*>(&img[(c * (PACK_TOK + 1) + tl) * 2]);
   }
+}
+extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q4k(const float* x, uint4* xp, u32 m, u32 in_dim) {
+  pack_x_core<false>(x, xp, m, in_dim);
 }
 
 __device__ __forceinline__ u32 h2_dup(float v) {
@@ -112,6 +126,56 @@ __shared__ uint4 gemm_xbuf1[4096];
 // rows = 14 to 16 cache lines; the same bytes fetched straight into the MFMA lane layout, one row per lane, touch 64).
 __shared__ uint4 gemm_wbuf[28 * 64];   // 27 copies of 64 pieces, and a 28th that keeps the four wavefronts in step
 
+// Epilogue shared by the GEMM kernels, in two halves of 64 tokens (the tiles r = 2 hf, 2 hf + 1): every wavefront
+// writes its partial sums to LDS as [k half][token][weight row] (row stride 200 floats: the two k-groups of a
+// wavefront land in disjoint banks), then all 256 threads add the two k halves and the bias and store 16 bytes at a
+// time, 48 consecutive threads per 768-byte output row segment. 2 x 64 x 200 x 4 B = 100 KiB of the two x buffers.
+__device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
+                                              u32 mt, u32 nt, u32 nh, u32 kh, u32 j, u32 kg, u32 tid) {
+  float* part0 = reinterpret_cast<float*>(gemm_xbuf0);   // k half 0: 64 x 200 floats = 51200 B <= 64 KiB
+  float* part1 = reinterpret_cast<float*>(gemm_xbuf1);   // k half 1
+  float* mine = kh ? part1 : part0;
+  const bool full_n = nt * GEMM_BN + GEMM_BN <= out_dim;
+#pragma unroll
+  for (int hf = 0; hf < 2; hf++) {
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++) {
+      const int r = 2 * hf + rr;
+#pragma unroll
+      for (int c = 0; c < 3; c++)
+#pragma unroll
+        for (int v = 0; v < 16; v++)
+          mine[(32 * rr + 8 * (v >> 2) + 4 * kg + (v & 3)) * 200 + nh * 96 + 32 * c + j] = acc[r][c][v];
+    }
+    __syncthreads();
+    const u32 row0 = mt * GEMM_BM + 64 * hf;
+    for (u32 idx = tid; idx < 64 * 48; idx += 256) {
+      const u32 tl = idx / 48, q4 = idx - tl * 48;
+      const u32 row = row0 + tl, n = nt * GEMM_BN + 4 * q4;
+      if (row < m && n < out_dim) {
+        const float4 p0 = *reinterpret_cast<const float4*>(part0 + tl * 200 + 4 * q4);
+        const float4 p1 = *reinterpret_cast<const float4*>(part1 + tl * 200 + 4 * q4);
+        float4 o = make_float4(p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w);
+        float* dst = out + (size_t)row * out_dim + n;
+        if (full_n || n + 4 <= out_dim) {
+          if (bias) {
+            o.x += bias[n]; o.y += bias[n + 1]; o.z += bias[n + 2]; o.w += bias[n + 3];
+          }
+          if ((out_dim & 3u) == 0) {
+            *reinterpret_cast<float4*>(dst) = o;
+          } else {
+            dst[0] = o.x; dst[1] = o.y; dst[2] = o.z; dst[3] = o.w;
+          }
+        } else {
+          const float ov[4] = {o.x, o.y, o.z, o.w};
+          for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (bias ? bias[n + e] : 0.0f);
+        }
+      }
+    }
+    if (hf == 0) __syncthreads();
+  }
+}
+
 struct GemmRaw {   // raw bytes of one group of one super-block of one weight row, as a lane sees them
   uint4 hdr, qa, qb;
 };
@@ -125,7 +189,11 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 nh = wave & 1, kh = wave >> 1;
   const u32 j = lane & 31, kg = lane >> 5;
   const u32 g = 2 * kh + kg;
-  const u32 nkb = in_dim >> 8;
+  // k split: workgroups of blockIdx.y = s take super-blocks [kb0, kb0 + nkb) of the nkb_all a row has and write their
+  // sums to the s-th [m][out_dim] plane behind `out` (the host passes the partial planes and no bias, then sums them)
+  const u32 nkb_all = in_dim >> 8;
+  const u32 kb0 = blockIdx.y * nkb_all / gridDim.y, nkb = (blockIdx.y + 1) * nkb_all / gridDim.y - kb0;
+  out += (size_t)blockIdx.y * m * out_dim;
   const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_BN - 1) / GEMM_BN;
   // Workgroup -> tile, XCD-aware. Workgroups go to the 8 XCDs round-robin (id % 8) and each XCD has its own
   // L2, so the tiles are numbered token-tile-major and XCD x takes the contiguous run [x*per, (x+1)*per):
@@ -136,7 +204,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
   if (vt >= mtiles * ntiles) return;
   const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
-  const size_t row_bytes = (size_t)nkb * 144;
+  const size_t row_bytes = (size_t)nkb_all * 144;
   const u32 sh = 16u * (g & 1);
   const bool upper = g >= 2;
 
@@ -144,7 +212,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   // workgroup and super-block; every wavefront issues 7, the 28th repeats the last piece into spare LDS so that no
   // copy is conditional). Piece p is bytes [16 (p % 9), +16) of row p / 9.
   const u32 tile_row0 = min(nt * GEMM_BN, out_dim - 1);
-  const uint8_t* wbase = w + (size_t)tile_row0 * row_bytes;   // uniform
+  const uint8_t* wbase = w + (size_t)tile_row0 * row_bytes + (size_t)kb0 * 144;   // uniform
   u32 woff[7];
 #pragma unroll
   for (int i = 0; i < 7; i++) {
@@ -157,7 +225,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   u32 wrow[3];
 #pragma unroll
   for (int c = 0; c < 3; c++) wrow[c] = (nh * 96 + 32 * c + j) * 9;
-  const uint4* xtile = xp + (size_t)mt * nkb * 4096;
+  const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
   float16_t acc[4][3];
 #pragma unroll
@@ -345,50 +413,30 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   }
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
-  // Epilogue, in two halves of 64 tokens (the tiles r = 2 hf, 2 hf + 1): every wavefront writes its partial
-  // sums to LDS as [k half][token][weight row] (row stride 200 floats: the two k-groups of a wavefront land in
-  // disjoint banks), then all 256 threads add the two k halves and the bias and store 16 bytes at a time,
-  // 48 consecutive threads per 768-byte output row segment. 2 x 64 x 200 x 4 B = 100 KiB of the 128 KiB.
-  float* part0 = reinterpret_cast<float*>(gemm_xbuf0);   // k half 0: 64 x 200 floats = 51200 B <= 64 KiB
-  float* part1 = reinterpret_cast<float*>(gemm_xbuf1);   // k half 1
-  float* mine = kh ? part1 : part0;
-  const bool full_n = nt * GEMM_BN + GEMM_BN <= out_dim;
-#pragma unroll
-  for (int hf = 0; hf < 2; hf++) {
-#pragma unroll
-    for (int rr = 0; rr < 2; rr++) {
-      const int r = 2 * hf + rr;
-#pragma unroll
-      for (int c = 0; c < 3; c++)
-#pragma unroll
-        for (int v = 0; v < 16; v++)
-          mine[(32 * rr + 8 * (v >> 2) + 4 * kg + (v & 3)) * 200 + nh * 96 + 32 * c + j] = acc[r][c][v];
+  gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid);
+}
+
+// Sum of the k-split planes: out[i] = (bias ? bias[i % out_dim] : 0) + partials[0][i] + partials[1][i] + ... in that order
+// (the result does not depend on which workgroup finished first). block 256, grid ceil(total / 1024); 4 elements per lane.
+extern "C" __global__ __launch_bounds__(256) void gemm_sum_splits_f32(const float* __restrict__ partials, const float* __restrict__ bias,
+                                                                       float* __restrict__ out, u32 total, u32 out_dim, u32 splits) {
+  const u32 i = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= total) return;
+  if (i + 4 <= total && (total & 3u) == 0) {
+    float4 a = *reinterpret_cast<const float4*>(partials + i);
+    for (u32 s = 1; s < splits; s++) {
+      const float4 b = *reinterpret_cast<const float4*>(partials + (size_t)s * total + i);
+      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
     }
-    __syncthreads();
-    const u32 row0 = mt * GEMM_BM + 64 * hf;
-    for (u32 idx = tid; idx < 64 * 48; idx += 256) {
-      const u32 tl = idx / 48, q4 = idx - tl * 48;
-      const u32 row = row0 + tl, n = nt * GEMM_BN + 4 * q4;
-      if (row < m && n < out_dim) {
-        const float4 p0 = *reinterpret_cast<const float4*>(part0 + tl * 200 + 4 * q4);
-        const float4 p1 = *reinterpret_cast<const float4*>(part1 + tl * 200 + 4 * q4);
-        float4 o = make_float4(p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w);
-        float* dst = out + (size_t)row * out_dim + n;
-        if (full_n || n + 4 <= out_dim) {
-          if (bias) {
-            o.x += bias[n]; o.y += bias[n + 1]; o.z += bias[n + 2]; o.w += bias[n + 3];
-          }
-          if ((out_dim & 3u) == 0) {
-            *reinterpret_cast<float4*>(dst) = o;
-          } else {
-            dst[0] = o.x; dst[1] = o.y; dst[2] = o.z; dst[3] = o.w;
-          }
-        } else {
-          const float ov[4] = {o.x, o.y, o.z, o.w};
-          for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (bias ? bias[n + e] : 0.0f);
-        }
-      }
+    if (bias) {
+      a.x += bias[i % out_dim]; a.y += bias[(i + 1) % out_dim]; a.z += bias[(i + 2) % out_dim]; a.w += bias[(i + 3) % out_dim];
     }
-    if (hf == 0) __syncthreads();
+    *reinterpret_cast<float4*>(out + i) = a;
+  } else {
+    for (u32 e = i; e < total && e < i + 4; e++) {
+      float a = partials[e];
+      for (u32 s = 1; s < splits; s++) a += partials[(size_t)s * total + e];
+      out[e] = a + (bias ? bias[e % out_dim] : 0.0f);
+    }
   }
 }

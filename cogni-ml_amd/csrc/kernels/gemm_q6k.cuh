@@ -1,0 +1,207 @@
+// Prefill GEMM over raw Q6_K weights: out[m][n] = (bias[n] +) sum_k x[m][k] * deq(W[n][k]), M >= 9.
+// Same tiling, operand layouts, x workspace format and epilogue as the Q4_K kernel (gemm_q4k.cuh): 128 tokens x 192
+// rows per workgroup, 4 wavefronts = 2 row halves x 2 k-step halves, v_mfma_f32_32x32x16_f16 with fp32 accumulation,
+// x as fp16 in LDS (two 64 KiB buffers filled by global_load_lds_dwordx4). What differs is the weight side:
+//
+//   pack_x_f16_q6k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 4 * in_dim/256
+//   q6_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
+//                   block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), no dynamic LDS (128 KiB static)
+//
+// A Q6_K super-block (210 bytes, 2-byte aligned: ql[128], qh[64], scales:i8[16], d:f16; src/ml/gguf/dequant.cr:197-236)
+// is walked in the reference as two halves n of 128 values, each l in [0, 32) giving four values l, l+32, l+64, l+96
+// ("quadrants") from the low / high nibbles of ql[l], ql[l+32] and two bits of qh[l]. Lane (j, kg) of a kh wavefront
+// owns the 64-value group (n = kh, u = kg): l in [16u, 16u+16) of half n, i.e. the three 16-byte pieces
+// ql[64n + 16u ..], ql[64n + 32 + 16u ..], qh[32n + 16u ..], the eight scale bytes of the half and d. They are read
+// straight from global memory into registers, one super-block ahead (the raw bytes cannot go through LDS the way the
+// Q4_K ones do: the rows are only 2-byte aligned and 192 of them are 40 KiB). k-step t of the wavefront is quadrant
+// t / 2, bytes 8 (t % 2) .. +8 of the pieces: 8 values with one scale. A code is put together in the low bits of a
+// half, (ql nibble) | (qh bits << 4) | 0x6400 = 1024 + q as binary16; subtracting 1056 gives q - 32 exactly and one
+// packed multiply gives fp16((q - 32) * (d * sc)). The 8 values come in byte order 0,2,1,3,4,6,5,7;
+// pack_x_f16_q6k writes x accordingly (gemm_k_element_q6k).
+#pragma once
+#include "gemm_q4k.cuh"
+
+// Element (0..255) of a super-block that k-slot (ks, kg, e) of the MFMA stands for: ks = 8 n + 2 qd + h8.
+__device__ __forceinline__ u32 gemm_k_element_q6k(u32 ks, u32 kg, u32 e) {
+  const u32 n = ks >> 3, qd = (ks >> 1) & 3, h8 = ks & 1;
+  const u32 perm = ((e & 1) << 1) | ((e >> 1) & 1) | (e & 4);   // 0,2,1,3,4,6,5,7
+  return 128 * n + 32 * qd + 16 * kg + 8 * h8 + perm;
+}
+
+extern "C" __global__ __launch_bounds__(256) void pack_x_f16_q6k(const float* x, uint4* xp, u32 m, u32 in_dim) {
+  pack_x_core<true>(x, xp, m, in_dim);
+}
+
+struct GemmRaw6 {   // raw bytes of one group of one super-block of one weight row, as a lane sees them
+  uint4 qa, qb, qh;
+  uint2 sc;
+  u32 d;
+};
+
+__device__ __forceinline__ u32 h2_sub_mul(u32 t, u32 off, u32 scale) {
+  const __half2 q = __hadd2(*reinterpret_cast<const __half2*>(&t), *reinterpret_cast<const __half2*>(&off));
+  const __half2 w = __hmul2(q, *reinterpret_cast<const __half2*>(&scale));
+  return *reinterpret_cast<const u32*>(&w);
+}
+
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
+  const u32 tid = threadIdx.x, lane = tid & 63;
+  const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const u32 nh = wave & 1, kh = wave >> 1;
+  const u32 j = lane & 31, kg = lane >> 5;
+  // k split as in q4_k_gemm_f16: super-blocks [kb0, kb0 + nkb) into plane blockIdx.y behind `out`
+  const u32 nkb_all = in_dim >> 8;
+  const u32 kb0 = blockIdx.y * nkb_all / gridDim.y, nkb = (blockIdx.y + 1) * nkb_all / gridDim.y - kb0;
+  out += (size_t)blockIdx.y * m * out_dim;
+  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_BN - 1) / GEMM_BN;
+  // workgroup -> tile as in q4_k_gemm_f16: XCD x takes a contiguous run of token-tile-major tiles
+  const u32 per = (mtiles * ntiles + GEMM_XCDS - 1) / GEMM_XCDS;
+  const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
+  if (vt >= mtiles * ntiles) return;
+  const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
+  const u32 n0 = nt * GEMM_BN + nh * 96;             // first weight row of this wavefront
+  const size_t row_bytes = (size_t)nkb_all * 210;
+
+  // uniform base of the wavefront's rows + a 32-bit per-lane offset (96 rows are far below 4 GiB), already at the
+  // lane's pieces: ql at 64 kh + 16 kg, qh at 128 + 32 kh + 16 kg, scales at 192 + 8 kh
+  const u32 base_row = min(n0, out_dim - 1);
+  const uint8_t* wbase = w + (size_t)base_row * row_bytes + (size_t)kb0 * 210;
+  u32 rowoff[3];
+#pragma unroll
+  for (int c = 0; c < 3; c++) rowoff[c] = (min(n0 + 32 * c + j, out_dim - 1) - base_row) * (u32)row_bytes;
+  const u32 o_ql = 64 * kh + 16 * kg, o_qh = 128 + 32 * kh + 16 * kg, o_sc = 192 + 8 * kh;
+  const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
+
+  float16_t acc[4][3];
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
+
+  auto load_row = [&](GemmRaw6& raw, const uint8_t* kbase, int c) {
+    raw.qa = ld16(kbase + (rowoff[c] + o_ql));
+    raw.qb = ld16(kbase + (rowoff[c] + o_ql + 32));
+    raw.qh = ld16(kbase + (rowoff[c] + o_qh));
+    raw.sc = ld8(kbase + (rowoff[c] + o_sc));
+    raw.d = ld2(kbase + (rowoff[c] + 208));
+  };
+
+  // Stage super-block 0 of x and the first weights. The main loop takes super-blocks in pairs with fixed roles (x
+  // buffer 0 then 1, weight registers A then B); with an odd number of super-blocks the first one is taken alone
+  // out of buffer 1 / registers B.
+  const bool odd = nkb & 1;
+  GemmRaw6 rawA[3], rawB[3];
+  if (odd) {
+#pragma unroll
+    for (int c = 0; c < 3; c++) load_row(rawB[c], wbase, c);
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf1 + 256 * i + wave * 64),
+                                       16, 0, 0);
+  } else {
+#pragma unroll
+    for (int c = 0; c < 3; c++) load_row(rawA[c], wbase, c);
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
+                                       16, 0, 0);
+  }
+  __syncthreads();
+
+  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt, const GemmRaw6 (&cur)[3], GemmRaw6 (&nxt)[3]) {
+    // d * sc of the four 16-value sub-blocks of the lane's group (scale bytes kg, kg + 2, kg + 4, kg + 6 of the
+    // half's eight), as duplicated half2
+    u32 S[3][4];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      const float d = h2f(cur[c].d);
+      const u32 lo = cur[c].sc.x >> (8 * kg), hi = cur[c].sc.y >> (8 * kg);
+      S[c][0] = h2_dup(d * (float)(int)(signed char)(lo & 0xFFu));
+      S[c][1] = h2_dup(d * (float)(int)(signed char)((lo >> 16) & 0xFFu));
+      S[c][2] = h2_dup(d * (float)(int)(signed char)(hi & 0xFFu));
+      S[c][3] = h2_dup(d * (float)(int)(signed char)((hi >> 16) & 0xFFu));
+    }
+    const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
+    const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
+    const uint8_t* knbase = wbase + (size_t)kn * 210; // uniform
+
+    const uint4* arow = xcur + (16 * kh + kg) * 128 + j;   // k-steps 8*kh .. 8*kh+7; 32 lanes read 512 contiguous bytes
+    auto build_b = [&](half8_t (&B)[3], int t) {
+      const int qd = t >> 1, h8 = t & 1, hi = qd >> 1;
+#pragma unroll
+      for (int c = 0; c < 3; c++) {
+        const uint4 Q = (qd & 1) ? cur[c].qb : cur[c].qa;
+        const u32 qa = h8 ? Q.z : Q.x, qb = h8 ? Q.w : Q.y;
+        const u32 ha = (h8 ? cur[c].qh.z : cur[c].qh.x) >> (2 * qd), hb = (h8 ? cur[c].qh.w : cur[c].qh.y) >> (2 * qd);
+        const u32 qsa = hi ? (qa >> 4) : qa, qsb = hi ? (qb >> 4) : qb;
+        const u32 off = 0xE420E420u;   // half2(-1056): 1024 + q - 1056 = q - 32
+        const u32 sc = S[c][qd];
+        uint4 bw;
+        bw.x = h2_sub_mul((qsa & 0x000F000Fu) | ((ha & 0x00030003u) << 4) | 0x64006400u, off, sc);
+        bw.y = h2_sub_mul(((qsa >> 8) & 0x000F000Fu) | (((ha >> 8) & 0x00030003u) << 4) | 0x64006400u, off, sc);
+        bw.z = h2_sub_mul((qsb & 0x000F000Fu) | ((hb & 0x00030003u) << 4) | 0x64006400u, off, sc);
+        bw.w = h2_sub_mul(((qsb >> 8) & 0x000F000Fu) | (((hb >> 8) & 0x00030003u) << 4) | 0x64006400u, off, sc);
+        B[c] = *reinterpret_cast<const half8_t*>(&bw);
+      }
+    };
+
+    // software pipeline over the wavefront's eight k-steps: while the MFMAs of step t run, the A operands
+    // of step t+1 are read from LDS and its B operands are built
+    uint4 A[2][4];
+    half8_t B[2][3];
+#pragma unroll
+    for (int r = 0; r < 4; r++) A[0][r] = arow[r * 32];
+    build_b(B[0], 0);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      const int p = t & 1;
+      // prefetches for the next super-block, a few per k-step: the raw weights of one row tile (5 loads) in each of
+      // the first three steps, the x tile global -> LDS spread over the first six
+      if (t < 3) load_row(nxt[t], knbase, t);
+      if (t < 6) {
+#pragma unroll
+        for (int i = (t < 3 ? 2 * t : 3 * t - 3); i < (t < 3 ? 2 * t + 2 : (t < 5 ? 3 * t : 16)); i++)
+          __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64),
+                                           16, 0, 0);
+      }
+      if (t < 7) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) A[p ^ 1][r] = arow[(t + 1) * 256 + r * 32];
+        build_b(B[p ^ 1], t + 1);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const half8_t Ar = *reinterpret_cast<const half8_t*>(&A[p][r]);
+#pragma unroll
+        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Ar, B[p][c], acc[r][c], 0, 0, 0);
+      }
+      if (t < 7) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
+      }
+      __builtin_amdgcn_sched_group_barrier(0x020, 10, 0);  // VMEM reads (weights, LDS-direct x) of this step
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
+#pragma unroll
+      for (int i = 0; i < 12; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);   // eight VALU (a Q6_K operand takes more than a Q4_K one)
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // End of the iteration: everything this wavefront requested has to be there (the x tile for everybody,
+    // the weights for its own next iteration), then everybody meets.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  if (odd) iteration(0, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
+  for (u32 kb = odd; kb < nkb; kb += 2) {
+    iteration(kb, gemm_xbuf0, gemm_xbuf1, rawA, rawB);
+    iteration(kb + 1, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
+  }
+  __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
+  gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid);
+}

@@ -1,4 +1,4 @@
-"""GPU prefill GEMM (Q4_K, fp16 MFMA path) vs the CPU oracle.
+"""GPU prefill GEMM (Q4_K and Q6_K, fp16 MFMA path) vs the CPU oracle.
 
 Tolerance (fp16-MFMA path): max|err| <= 2e-3 * max|ref| over the output, plus cos >= 0.9999 -- the
 reference's own convention for its Metal GEMM (spec/qwen35_metal_spec.cr:78,104 uses 0.05 * max|cpu|).
@@ -9,18 +9,18 @@ import pytest
 
 from cogni_ml_amd import quant, synth
 from gpu_common import DevArray, gpu  # noqa: F401
-from helpers import Q4_K, Q6_K, cosine
+from helpers import Q4_K, Q5_K, Q6_K, cosine
 
 pytestmark = pytest.mark.gpu
 
 
-def run_gemm(raw, x, in_dim, out_dim, tokens, bias=None, router=False):
+def run_gemm(raw, x, in_dim, out_dim, tokens, bias=None, router=False, t=Q4_K, split=True):
     w, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim)
-    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens)
+    wsb = quant.gemm_workspace_bytes(t, in_dim, tokens, out_dim if split else None)
     ws = DevArray(nbytes=wsb)
     bd = DevArray(bias) if bias is not None else None
     fn = quant.matmul_dev if router else quant.gemm_dev
-    fn(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens, ws.ptr, wsb, bd.ptr if bd else 0)
+    fn(w.ptr, t, xd.ptr, od.ptr, in_dim, out_dim, tokens, ws.ptr, wsb, bd.ptr if bd else 0)
     out = od.read(np.float32, tokens * out_dim)
     for a in (w, xd, od, ws, bd):
         if a:
@@ -28,15 +28,15 @@ def run_gemm(raw, x, in_dim, out_dim, tokens, bias=None, router=False):
     return out
 
 
-def check(oracle, raw, x, in_dim, out_dim, tokens, bias=None, what="", router=False, sample_tokens=None):
-    got = run_gemm(raw, x, in_dim, out_dim, tokens, bias, router).reshape(tokens, out_dim)
+def check(oracle, raw, x, in_dim, out_dim, tokens, bias=None, what="", router=False, sample_tokens=None, t=Q4_K):
+    got = run_gemm(raw, x, in_dim, out_dim, tokens, bias, router, t).reshape(tokens, out_dim)
     b = bias if bias is not None else np.zeros(out_dim, dtype=np.float32)
     rows = np.arange(tokens) if sample_tokens is None else np.asarray(sample_tokens)
     xs = x.reshape(tokens, in_dim)[rows]
-    want = oracle.matmul_add(xs.reshape(-1), len(rows), in_dim, raw, Q4_K, out_dim, b, threads=16).reshape(len(rows), out_dim)
+    want = oracle.matmul_add(xs.reshape(-1), len(rows), in_dim, raw, t, out_dim, b, threads=16).reshape(len(rows), out_dim)
     err = np.max(np.abs(got[rows].astype(np.float64) - want))
     ref_max = np.max(np.abs(want))
-    dense_max = np.max(np.abs(oracle.dequantize(raw, Q4_K, out_dim * in_dim)))
+    dense_max = np.max(np.abs(oracle.dequantize(raw, t, out_dim * in_dim)))
     fp32_style = err / (np.max(np.linalg.norm(xs, axis=1)) * dense_max)
     print("%s: max|err|/max|ref| = %.3e, max|err|/(||x|| max|w|) = %.3e" % (what, err / ref_max, fp32_style))
     assert cosine(got[rows].reshape(-1), want.reshape(-1)) >= 0.9999, what
@@ -44,25 +44,49 @@ def check(oracle, raw, x, in_dim, out_dim, tokens, bias=None, what="", router=Fa
     return got
 
 
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
 @pytest.mark.parametrize("tokens,out_dim,in_dim", [(9, 192, 256), (16, 48, 512), (64, 200, 1024), (128, 192, 256),
                                                      (130, 400, 768), (257, 31, 256)])
-def test_small_shapes_and_tails(gpu, oracle, tokens, out_dim, in_dim):
+def test_small_shapes_and_tails(gpu, oracle, tokens, out_dim, in_dim, t):
     rng = np.random.default_rng(tokens * 1000 + out_dim)
-    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    raw = synth.make_weights(rng, t, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
-    check(oracle, raw, x, in_dim, out_dim, tokens, None, "M=%d N=%d K=%d" % (tokens, out_dim, in_dim))
+    check(oracle, raw, x, in_dim, out_dim, tokens, None, "type %d M=%d N=%d K=%d" % (t, tokens, out_dim, in_dim), t=t)
 
 
-def test_bias_and_router(gpu, oracle):
+def test_q6_k_codes_and_scales_one_at_a_time(gpu, oracle):
+    """Q6_K blocks with a single non-zero scale and codes that count up: every (quadrant, 16-run, byte) of the operand
+    assembly lands on its own activation, so a swapped piece, a wrong shift or a wrong scale byte shows as a wrong value."""
+    in_dim, out_dim, tokens = 256, 32, 16
+    rng = np.random.default_rng(66)
+    x = synth.make_activations(rng, tokens, in_dim)
+    for which in range(16):
+        raw = np.zeros((out_dim, 210), dtype=np.uint8)
+        codes = (np.arange(256)[None, :] * 7 + np.arange(out_dim)[:, None] * 3) % 64          # 6-bit codes per element
+        for nn in range(2):
+            for l in range(32):
+                e = 128 * nn + l
+                raw[:, 64 * nn + l] = (codes[:, e] & 15) | ((codes[:, e + 64] & 15) << 4)
+                raw[:, 64 * nn + 32 + l] = (codes[:, e + 32] & 15) | ((codes[:, e + 96] & 15) << 4)
+                raw[:, 128 + 32 * nn + l] = ((codes[:, e] >> 4) | ((codes[:, e + 32] >> 4) << 2) |
+                                             ((codes[:, e + 64] >> 4) << 4) | ((codes[:, e + 96] >> 4) << 6))
+        raw[:, 192 + which] = np.uint8(5 + which)                                            # one live sub-block scale
+        raw[:, 208:210] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
+        check(oracle, raw.reshape(-1), x, in_dim, out_dim, tokens, None, "Q6_K scale %d" % which, t=Q6_K)
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+def test_bias_and_router(gpu, oracle, t):
+    Q4_K = t        # (the body below is written for one type; it runs for both)
     rng = np.random.default_rng(4)
     out_dim, in_dim = 384, 512
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
     bias = rng.standard_normal(out_dim).astype(np.float32)
     x = synth.make_activations(rng, 40, in_dim)
-    check(oracle, raw, x, in_dim, out_dim, 40, bias, "bias M=40", router=True)
+    check(oracle, raw, x, in_dim, out_dim, 40, bias, "bias M=40", router=True, t=t)
     # at or below the threshold the router takes the fp32 GEMV path: agreement with the oracle is ~1e-6
     assert quant.get_gemm_threshold() == 8
-    got = run_gemm(raw, x[:8 * in_dim], in_dim, out_dim, 8, None, router=True)
+    got = run_gemm(raw, x[:8 * in_dim], in_dim, out_dim, 8, None, router=True, t=t)
     want = oracle.matmul_add(x[:8 * in_dim], 8, in_dim, raw, Q4_K, out_dim, np.zeros(out_dim, dtype=np.float32))
     assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
     # host-level matmul_add with rows > 8 goes through the GEMM as well
@@ -77,10 +101,26 @@ def test_bias_and_router(gpu, oracle):
         quant.set_gemm_threshold(8)
 
 
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("tokens,out_dim,in_dim", [(64, 384, 4096), (20, 100, 1280), (200, 4096, 2048), (128, 1000, 1536)])
+def test_k_split_matches_unsplit(gpu, oracle, tokens, out_dim, in_dim, t):
+    """Few tiles: the k range is divided among workgroups (the workspace has room for the planes). Against the oracle,
+    against the unsplit launch, with a bias, and the same bits on a second run."""
+    rng = np.random.default_rng(tokens + out_dim + in_dim + t)
+    raw = synth.make_weights(rng, t, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    bias = rng.standard_normal(out_dim).astype(np.float32)
+    assert quant.gemm_workspace_bytes(t, in_dim, tokens, out_dim) > quant.gemm_workspace_bytes(t, in_dim, tokens)
+    got = check(oracle, raw, x, in_dim, out_dim, tokens, bias, "split M=%d N=%d K=%d" % (tokens, out_dim, in_dim), t=t)
+    one = run_gemm(raw, x, in_dim, out_dim, tokens, bias, t=t, split=False).reshape(tokens, out_dim)
+    assert np.max(np.abs(one - got)) <= 2e-5 * np.max(np.abs(got))
+    assert np.array_equal(run_gemm(raw, x, in_dim, out_dim, tokens, bias, t=t).reshape(tokens, out_dim), got)
+
+
 def test_argument_checks(gpu):
     w, x, o = DevArray(nbytes=4096), DevArray(nbytes=4096), DevArray(nbytes=4096)
     with pytest.raises(quant.QuantError, match="Unsupported quant type for the prefill GEMM") as e:
-        quant.gemm_dev(w.ptr, Q6_K, x.ptr, o.ptr, 256, 1, 16, w.ptr, 4096)
+        quant.gemm_dev(w.ptr, Q5_K, x.ptr, o.ptr, 256, 1, 16, w.ptr, 4096)
     assert e.value.code == -2
     with pytest.raises(quant.QuantError, match="workspace has 16 bytes, needs 65536"):
         quant.gemm_dev(w.ptr, Q4_K, x.ptr, o.ptr, 256, 1, 16, w.ptr, 16)
@@ -103,14 +143,29 @@ def test_configured_prefill_shapes(gpu, oracle, tokens):
     check(oracle, raw, x, in_dim, out_dim, tokens, None, "cfg4 M=%d" % tokens, sample_tokens=sample)
 
 
+def test_q6_k_down_projection_prefill(gpu, oracle):
+    """The Q6_K down projection of the mixed-quant layer (12288 -> 4096) at M = 512: a sample of tokens against the
+    oracle and every token against the same token in a smaller GEMM."""
+    rng = np.random.default_rng(6)
+    out_dim, in_dim, tokens = 4096, 12288, 512
+    raw = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    got = check(oracle, raw, x, in_dim, out_dim, tokens, None, "Q6_K down M=512", sample_tokens=[0, 1, 127, 128, 300, 511], t=Q6_K)
+    # the same tokens in a launch of their own, without the k split: equal up to the order of the fp32 sums
+    part = run_gemm(raw, x[400 * in_dim:], in_dim, out_dim, tokens - 400, t=Q6_K, split=False).reshape(-1, out_dim)
+    assert np.max(np.abs(part - got[400:])) <= 2e-5 * np.max(np.abs(got))
+    again = run_gemm(raw, x, in_dim, out_dim, tokens, t=Q6_K).reshape(tokens, out_dim)
+    assert np.array_equal(again, got)                      # the split sums its planes in a fixed order
+
+
 def test_m2048_row_identity(gpu, oracle):
     """M = 2048: a sample of tokens against the oracle, and every token against the same token run through a
-    smaller GEMM (the result for a token does not depend on which tile it sits in)."""
+    smaller unsplit GEMM (the result for a token does not depend on which tile it sits in)."""
     rng = np.random.default_rng(2048)
     out_dim, in_dim, tokens = 12288, 4096, 2048
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
     got = check(oracle, raw, x, in_dim, out_dim, tokens, None, "cfg4 M=2048",
                 sample_tokens=[0, 1, 127, 128, 1000, 1023, 1024, 2046, 2047])
-    part = run_gemm(raw, x[1900 * in_dim:], in_dim, out_dim, tokens - 1900).reshape(-1, out_dim)
+    part = run_gemm(raw, x[1900 * in_dim:], in_dim, out_dim, tokens - 1900, split=False).reshape(-1, out_dim)
     assert np.array_equal(part, got[1900:])
