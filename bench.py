@@ -276,6 +276,10 @@ def main():
         gemm["q6_k down 4096x12288 M=512"] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
         log("case=q6_k_gemm prefill\ntype=Q6_K\nshape=12288x4096\ntokens=512\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
             gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
+        per, tf = bench_gemm(hip, quant, synth, rng, stream, 512, 12288, 4096, gsteps, 5, Q4_K=Q5_K)
+        gemm["q5_k 12288x4096 M=512"] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
+        log("case=q5_k_gemm prefill\ntype=Q5_K\nshape=4096x12288\ntokens=512\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
+            gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
 
     extra = {}
     if args.mode == "cases":

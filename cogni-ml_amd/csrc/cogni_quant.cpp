@@ -435,7 +435,7 @@ int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t resi
 
 int g_gemm_threshold = -1;   // -1: not resolved yet
 
-static bool gemm_type(uint32_t t) { return t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q6_K; }
+static bool gemm_type(uint32_t t) { return t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q5_K || t == COGNI_TYPE_Q6_K; }
 
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {
   if (!gemm_type(w_type) || in_dim == 0 || tokens == 0) return 0;
@@ -483,7 +483,7 @@ int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, u
   // a workspace that holds the packed activations only: one workgroup per tile walks the whole row
   uint32_t splits = gemm_splits(in_dim, out_dim, tokens);
   if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) splits = 1;
-  const char* kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : "q4_k_gemm_f16";
+  const char* kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : w_type == COGNI_TYPE_Q5_K ? "q5_k_gemm_f16" : "q4_k_gemm_f16";
   const uint32_t grid = 8 * ((mtiles * ntiles + 7) / 8);
   if (splits == 1) {
     void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};

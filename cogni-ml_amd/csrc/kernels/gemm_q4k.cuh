@@ -1,13 +1,16 @@
-// Prefill GEMM over raw Q4_K weights: out[m][n] = (bias[n] +) sum_k x[m][k] * deq(W[n][k]), M >= 9.
+// Prefill GEMM over raw Q4_K (and, as the same template, Q5_K) weights: out[m][n] = (bias[n] +) sum_k x[m][k] * deq(W[n][k]), M >= 9.
 // fp16 operands, v_mfma_f32_32x32x16_f16, fp32 accumulation (the precision of the reference's Metal
 // prefill kernels, which round both x and the dequantized weights to half:
 // src/ml/gguf/kernels/gemm_q4k.metal:97-105,678-686). On gfx950 the 32x32x16 instruction sustains twice
 // the rate of 16x16x32 (about 32 vs 2 x 32 clocks for the same 32768 flops per SIMD), hence the tile shape.
 //
-// Two kernels:
+// Kernels:
 //   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 4 * in_dim/256
-//   q4_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
-//                   block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), no dynamic LDS (156 KiB static)
+//   q4_k_gemm_f16, q5_k_gemm_f16
+//                   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
+//                   block 256, grid (8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), k splits), no dynamic LDS
+//                   (156 / 160 KiB static); with k splits > 1 `out` is `splits` planes of [m][out_dim] and bias is null
+//   gemm_sum_splits_f32 (planes, bias|null, out, m*out_dim:u32, out_dim:u32, splits:u32)   block 256, grid ceil(m*out_dim/1024)
 //
 // Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows, so 512 x 12288 gives 256
 // workgroups, one per CU. K is walked one 256-value super-block at a time = 16 MFMA k-steps of 16.
@@ -125,6 +128,10 @@ __shared__ uint4 gemm_xbuf1[4096];
 // global -> LDS 16 bytes per lane with consecutive lanes on consecutive pieces of a row (a 64-lane copy touches 7 or 8
 // rows = 14 to 16 cache lines; the same bytes fetched straight into the MFMA lane layout, one row per lane, touch 64).
 __shared__ uint4 gemm_wbuf[28 * 64];   // 27 copies of 64 pieces, and a 28th that keeps the four wavefronts in step
+// Q5_K: the 160 bytes behind the 16-byte header of each row (qh[32], qs[128]) = 1920 pieces, 30 copies of 64 and two more
+// for the same reason; with the two x buffers this is all of the 160 KiB a workgroup can have. The header (d, dmin,
+// 12 scale bytes) goes from global memory straight to the lane that decodes it.
+__shared__ uint4 gemm_wbuf5[32 * 64];
 
 // Epilogue shared by the GEMM kernels, in two halves of 64 tokens (the tiles r = 2 hf, 2 hf + 1): every wavefront
 // writes its partial sums to LDS as [k half][token][weight row] (row stride 200 floats: the two k-groups of a
@@ -176,12 +183,25 @@ __device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][3], const floa
   }
 }
 
-struct GemmRaw {   // raw bytes of one group of one super-block of one weight row, as a lane sees them
+// raw bytes of one group of one super-block of one weight row, as a lane sees them
+template <bool Q5>
+struct GemmRawT {
   uint4 hdr, qa, qb;
 };
+template <>
+struct GemmRawT<true> {   // Q5_K: plus the 32 bytes of fifth bits (bit 2g + hi of qh[l] belongs to value 64g + 32hi + l)
+  uint4 hdr, qa, qb, qh0, qh1;
+};
 
-extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_f16(
-    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
+// Q5 = false: Q4_K (144-byte super-blocks, everything through gemm_wbuf); true: Q5_K (176 bytes; same nibbles, groups and
+// x order, one more bit per value).
+template <bool Q5>
+__device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim,
+                                              u32 out_dim, u32 m) {
+  constexpr u32 BS = Q5 ? 176 : 144;      // bytes of a super-block
+  constexpr u32 PPR = Q5 ? 10 : 9;        // 16-byte pieces of a row that go through LDS
+  constexpr int NCOPY = Q5 ? 8 : 7;       // copies of 64 pieces a wavefront issues per super-block
+  uint4* const wbuf = Q5 ? gemm_wbuf5 : gemm_wbuf;
   // (no __restrict__ on w / xp: loads the compiler knows to be invariant are rematerialised next to
   // their use, which would undo the prefetch distance set up below)
   const u32 tid = threadIdx.x, lane = tid & 63;
@@ -204,7 +224,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
   if (vt >= mtiles * ntiles) return;
   const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
-  const size_t row_bytes = (size_t)nkb_all * 144;
+  const size_t row_bytes = (size_t)nkb_all * BS;
   const u32 sh = 16u * (g & 1);
   const bool upper = g >= 2;
 
@@ -212,19 +232,23 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   // workgroup and super-block; every wavefront issues 7, the 28th repeats the last piece into spare LDS so that no
   // copy is conditional). Piece p is bytes [16 (p % 9), +16) of row p / 9.
   const u32 tile_row0 = min(nt * GEMM_BN, out_dim - 1);
-  const uint8_t* wbase = w + (size_t)tile_row0 * row_bytes + (size_t)kb0 * 144;   // uniform
-  u32 woff[7];
+  const uint8_t* wbase = w + (size_t)tile_row0 * row_bytes + (size_t)kb0 * BS;   // uniform
+  u32 woff[NCOPY];
 #pragma unroll
-  for (int i = 0; i < 7; i++) {
-    const u32 p = min((4u * i + wave) * 64u + lane, (u32)GEMM_BN * 9u - 1u);
-    const u32 r = p / 9u, part = p - 9u * r;
-    woff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part;
+  for (int i = 0; i < NCOPY; i++) {
+    const u32 p = min((4u * i + wave) * 64u + lane, (u32)GEMM_BN * PPR - 1u);
+    const u32 r = p / PPR, part = p - PPR * r;
+    woff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part + (Q5 ? 16u : 0u);
   }
   // where this lane finds the raw bytes of its three rows in gemm_wbuf (in uint4 units): header, then the 32 bytes of
   // its group
   u32 wrow[3];
 #pragma unroll
-  for (int c = 0; c < 3; c++) wrow[c] = (nh * 96 + 32 * c + j) * 9;
+  for (int c = 0; c < 3; c++) wrow[c] = (nh * 96 + 32 * c + j) * PPR;
+  // Q5_K: where this lane's three rows start relative to wbase (their headers are read from there)
+  u32 hoff[3];
+#pragma unroll
+  for (int c = 0; c < 3; c++) hoff[c] = (min(nt * GEMM_BN + nh * 96 + 32 * c + j, out_dim - 1) - tile_row0) * (u32)row_bytes;
   const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
   float16_t acc[4][3];
@@ -236,8 +260,12 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
   auto copy_w = [&](u32 kb, int i) {   // copy i of this wavefront for super-block kb
-    __builtin_amdgcn_global_load_lds((gbl_void*)(wbase + (size_t)kb * 144 + woff[i]),
-                                     (lds_void*)(gemm_wbuf + (4 * i + wave) * 64), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gbl_void*)(wbase + (size_t)kb * BS + woff[i]),
+                                     (lds_void*)(wbuf + (4 * i + wave) * 64), 16, 0, 0);
+  };
+  uint4 nhdr[3];   // Q5_K: headers of the super-block being copied
+  auto load_hdr = [&](u32 kb, int c) {
+    if constexpr (Q5) nhdr[c] = ld16(wbase + (size_t)kb * BS + hoff[c]);
   };
 
   // Stage super-block 0 of x and of the weights. The main loop below takes super-blocks in pairs with fixed x buffers
@@ -245,7 +273,9 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   // buffer 1.
   const bool odd = nkb & 1;
 #pragma unroll
-  for (int i = 0; i < 7; i++) copy_w(0, i);
+  for (int i = 0; i < NCOPY; i++) copy_w(0, i);
+#pragma unroll
+  for (int c = 0; c < 3; c++) load_hdr(0, c);
   if (odd) {
 #pragma unroll
     for (int i = 0; i < 16; i++)
@@ -261,7 +291,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 
   // State that lives across super-blocks: the raw bytes and the decoded (scale, -min) pairs of the current one, and
   // the two operand sets of the k-step pipeline.
-  GemmRaw cur[3];
+  GemmRawT<Q5> cur[3];
   u32 S[3][4];
   uint4 A[2][4];
   half8_t B[2][3];
@@ -269,9 +299,17 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   auto take_raw = [&]() {
 #pragma unroll
     for (int c = 0; c < 3; c++) {
-      cur[c].hdr = gemm_wbuf[wrow[c]];
-      cur[c].qa = gemm_wbuf[wrow[c] + 1 + 2 * g];
-      cur[c].qb = gemm_wbuf[wrow[c] + 2 + 2 * g];
+      if constexpr (Q5) {
+        cur[c].hdr = nhdr[c];
+        cur[c].qh0 = wbuf[wrow[c]];
+        cur[c].qh1 = wbuf[wrow[c] + 1];
+        cur[c].qa = wbuf[wrow[c] + 2 + 2 * g];
+        cur[c].qb = wbuf[wrow[c] + 3 + 2 * g];
+      } else {
+        cur[c].hdr = wbuf[wrow[c]];
+        cur[c].qa = wbuf[wrow[c] + 1 + 2 * g];
+        cur[c].qb = wbuf[wrow[c] + 2 + 2 * g];
+      }
     }
   };
   // (scale, -min) of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles) as duplicated half2
@@ -300,10 +338,22 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       const u32 off = hi ? 0xD400D400u : 0xE400E400u;       // half2(-64) : half2(-1024)
       const u32 sc = S[c][2 * hi], nm = S[c][2 * hi + 1];
       uint4 bw;
-      bw.x = h2_fma_off((qa & mask) | magic, off, sc, nm);
-      bw.y = h2_fma_off(((qa >> 8) & mask) | magic, off, sc, nm);
-      bw.z = h2_fma_off((qb & mask) | magic, off, sc, nm);
-      bw.w = h2_fma_off(((qb >> 8) & mask) | magic, off, sc, nm);
+      if constexpr (Q5) {
+        // the fifth bit is worth 16: bit 4 beside a low nibble (1024 + q, one unit per mantissa step), bit 8 beside a
+        // high nibble (64 + q with the nibble 4 bits up, 1/16 per step)
+        const uint4 QH = h ? cur[c].qh1 : cur[c].qh0;
+        const u32 ha = ((op & 1) ? QH.z : QH.x) >> (2 * g + hi), hb = ((op & 1) ? QH.w : QH.y) >> (2 * g + hi);
+        const int up = hi ? 8 : 4;
+        bw.x = h2_fma_off((qa & mask) | magic | ((ha & 0x00010001u) << up), off, sc, nm);
+        bw.y = h2_fma_off(((qa >> 8) & mask) | magic | (((ha >> 8) & 0x00010001u) << up), off, sc, nm);
+        bw.z = h2_fma_off((qb & mask) | magic | ((hb & 0x00010001u) << up), off, sc, nm);
+        bw.w = h2_fma_off(((qb >> 8) & mask) | magic | (((hb >> 8) & 0x00010001u) << up), off, sc, nm);
+      } else {
+        bw.x = h2_fma_off((qa & mask) | magic, off, sc, nm);
+        bw.y = h2_fma_off(((qa >> 8) & mask) | magic, off, sc, nm);
+        bw.z = h2_fma_off((qb & mask) | magic, off, sc, nm);
+        bw.w = h2_fma_off(((qb >> 8) & mask) | magic, off, sc, nm);
+      }
       Bd[c] = *reinterpret_cast<const half8_t*>(&bw);
     }
   };
@@ -341,8 +391,10 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       if (t < 3) {
         copy_w(kn, 2 * t);
         copy_w(kn, 2 * t + 1);
+        load_hdr(kn, t);
       }
       if (t == 3) copy_w(kn, 6);
+      if (Q5 && t == 4) copy_w(kn, 7);
       if (t < 6) {
 #pragma unroll
         for (int i = (t < 2 ? 2 * t : 3 * t - 2); i < (t < 2 ? 2 * t + 2 : 3 * t + 1); i++) copy_x(i);
@@ -379,11 +431,11 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
 #pragma unroll
         for (int i = 0; i < 12; i++) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);   // five VALU
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, Q5 ? 8 : 5, 0);   // five VALU (eight with the fifth bits)
         }
       } else {
-        __builtin_amdgcn_sched_group_barrier(0x100, 13, 0);  // LDS reads: raw bytes and first A operands of the next super-block
+        __builtin_amdgcn_sched_group_barrier(0x100, Q5 ? 16 : 13, 0);  // LDS reads: raw bytes and first A operands of the next super-block
 #pragma unroll
         for (int i = 0; i < 3; i++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // three MFMAs while they arrive
 #pragma unroll
@@ -414,6 +466,16 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
   gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid);
+}
+
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<false>(w, xp, bias, out, in_dim, out_dim, m);
+}
+// Q5_K: x is packed by pack_x_f16_q4k (the values of a super-block sit where the Q4_K ones do).
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q5_k_gemm_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<true>(w, xp, bias, out, in_dim, out_dim, m);
 }
 
 // Sum of the k-split planes: out[i] = (bias ? bias[i % out_dim] : 0) + partials[0][i] + partials[1][i] + ... in that order

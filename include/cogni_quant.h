@@ -175,14 +175,14 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
                         uint64_t top1_ids, uint64_t top1_values, uint32_t in_dim, uint32_t out_dim, uint32_t tokens,
                         void* stream);
 
-/* Prefill GEMM for `tokens` > 8 (Q4_K, Q6_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
+/* Prefill GEMM for `tokens` > 8 (Q4_K, Q5_K, Q6_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
  * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
  * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:
- * 97-105,678-686; Q6_K: gemm_q56k.metal, pipelines mm6 src/ml/gguf/qwen35_metal.cr:11035); expect about 5e-4 of
+ * 97-105,678-686; Q5_K and Q6_K: gemm_q56k.metal, pipelines mm5 / mm6 src/ml/gguf/qwen35_metal.cr:11035); expect about 5e-4 of
  * max|out| where the GEMV path gives 1e-6. `workspace` is caller-owned device memory of at least
  * cogni_gemm_workspace_bytes(...) bytes (x repacked as fp16, in the k order of the weight type); nothing is allocated.
- * Kernels: pack_x_f16_q4k | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
- *          q4_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,
+ * Kernels: pack_x_f16_q4k (Q4_K and Q5_K) | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
+ *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,
  *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/192)/8), no dynamic shared memory.
  * (pack_x_f16_*: block 256, grid ceil(tokens/128)*4*(in_dim/256).) Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);

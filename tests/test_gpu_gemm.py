@@ -1,4 +1,4 @@
-"""GPU prefill GEMM (Q4_K and Q6_K, fp16 MFMA path) vs the CPU oracle.
+"""GPU prefill GEMM (Q4_K, Q5_K and Q6_K, fp16 MFMA path) vs the CPU oracle.
 
 Tolerance (fp16-MFMA path): max|err| <= 2e-3 * max|ref| over the output, plus cos >= 0.9999 -- the
 reference's own convention for its Metal GEMM (spec/qwen35_metal_spec.cr:78,104 uses 0.05 * max|cpu|).
@@ -9,7 +9,7 @@ import pytest
 
 from cogni_ml_amd import quant, synth
 from gpu_common import DevArray, gpu  # noqa: F401
-from helpers import Q4_K, Q5_K, Q6_K, cosine
+from helpers import Q4_K, Q5_K, Q6_K, Q8_0, cosine
 
 pytestmark = pytest.mark.gpu
 
@@ -44,7 +44,7 @@ def check(oracle, raw, x, in_dim, out_dim, tokens, bias=None, what="", router=Fa
     return got
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("tokens,out_dim,in_dim", [(9, 192, 256), (16, 48, 512), (64, 200, 1024), (128, 192, 256),
                                                      (130, 400, 768), (257, 31, 256)])
 def test_small_shapes_and_tails(gpu, oracle, tokens, out_dim, in_dim, t):
@@ -75,7 +75,7 @@ def test_q6_k_codes_and_scales_one_at_a_time(gpu, oracle):
         check(oracle, raw.reshape(-1), x, in_dim, out_dim, tokens, None, "Q6_K scale %d" % which, t=Q6_K)
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
 def test_bias_and_router(gpu, oracle, t):
     Q4_K = t        # (the body below is written for one type; it runs for both)
     rng = np.random.default_rng(4)
@@ -101,7 +101,7 @@ def test_bias_and_router(gpu, oracle, t):
         quant.set_gemm_threshold(8)
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
 @pytest.mark.parametrize("tokens,out_dim,in_dim", [(64, 384, 4096), (20, 100, 1280), (200, 4096, 2048), (128, 1000, 1536)])
 def test_k_split_matches_unsplit(gpu, oracle, tokens, out_dim, in_dim, t):
     """Few tiles: the k range is divided among workgroups (the workspace has room for the planes). Against the oracle,
@@ -120,7 +120,7 @@ def test_k_split_matches_unsplit(gpu, oracle, tokens, out_dim, in_dim, t):
 def test_argument_checks(gpu):
     w, x, o = DevArray(nbytes=4096), DevArray(nbytes=4096), DevArray(nbytes=4096)
     with pytest.raises(quant.QuantError, match="Unsupported quant type for the prefill GEMM") as e:
-        quant.gemm_dev(w.ptr, Q5_K, x.ptr, o.ptr, 256, 1, 16, w.ptr, 4096)
+        quant.gemm_dev(w.ptr, Q8_0, x.ptr, o.ptr, 256, 1, 16, w.ptr, 4096)
     assert e.value.code == -2
     with pytest.raises(quant.QuantError, match="workspace has 16 bytes, needs 65536"):
         quant.gemm_dev(w.ptr, Q4_K, x.ptr, o.ptr, 256, 1, 16, w.ptr, 16)
@@ -141,6 +141,23 @@ def test_configured_prefill_shapes(gpu, oracle, tokens):
     x = synth.make_activations(rng, tokens, in_dim)
     sample = None if tokens <= 64 else np.concatenate([np.arange(0, 24), np.arange(250, 262), np.arange(tokens - 12, tokens)])
     check(oracle, raw, x, in_dim, out_dim, tokens, None, "cfg4 M=%d" % tokens, sample_tokens=sample)
+
+
+def test_q5_k_fifth_bits_one_position_at_a_time(gpu, oracle):
+    """Q5_K blocks whose nibbles are zero and whose fifth bits are set for one sub-block at a time, with distinct scales:
+    a bit taken from the wrong position of qh, or put beside the wrong nibble, moves weight to other activations."""
+    in_dim, out_dim, tokens = 256, 32, 16
+    rng = np.random.default_rng(55)
+    x = synth.make_activations(rng, tokens, in_dim)
+    for sub in range(8):
+        raw = np.zeros((out_dim, 176), dtype=np.uint8)
+        raw[:, 0:2] = np.frombuffer(np.float16(0.03).tobytes(), dtype=np.uint8)      # d; dmin = 0
+        raw[:, 4:8] = np.array([3, 5, 7, 9], dtype=np.uint8)                         # scales of sub-blocks 0..3
+        raw[:, 12:16] = np.array([11, 13, 15, 2], dtype=np.uint8)                    # low 4 bits: scales of sub-blocks 4..7
+        pattern = ((np.arange(32)[None, :] + np.arange(out_dim)[:, None]) % 3 != 0)  # which l carry the bit
+        raw[:, 16:48] = (pattern.astype(np.uint8) << sub)
+        raw[:, 48:176] = ((np.arange(128)[None, :] * 5 + np.arange(out_dim)[:, None]) % 16 * 17).astype(np.uint8)
+        check(oracle, raw.reshape(-1), x, in_dim, out_dim, tokens, None, "Q5_K fifth bits of sub-block %d" % sub, t=Q5_K)
 
 
 def test_q6_k_down_projection_prefill(gpu, oracle):
