@@ -11,9 +11,13 @@
 // is walked in the reference as two halves n of 128 values, each l in [0, 32) giving four values l, l+32, l+64, l+96
 // ("quadrants") from the low / high nibbles of ql[l], ql[l+32] and two bits of qh[l]. Lane (j, kg) of a kh wavefront
 // owns the 64-value group (n = kh, u = kg): l in [16u, 16u+16) of half n, i.e. the three 16-byte pieces
-// ql[64n + 16u ..], ql[64n + 32 + 16u ..], qh[32n + 16u ..], the eight scale bytes of the half and d. They are read
-// straight from global memory into registers, one super-block ahead (the raw bytes cannot go through LDS the way the
-// Q4_K ones do: the rows are only 2-byte aligned and 192 of them are 40 KiB). k-step t of the wavefront is quadrant
+// ql[64n + 16u ..], ql[64n + 32 + 16u ..], qh[32n + 16u ..], the eight scale bytes of the half and d. All 39 KiB of raw
+// bytes of 192 rows do not fit beside the two x buffers (160 KiB of LDS in all), so only ql does (128 of the 210 bytes:
+// gemm_wbuf6, loaded one super-block ahead with consecutive lanes on consecutive pieces of a row, stored to LDS behind
+// k-step 6 and picked up during k-step 7) and the 18 bytes of scales and d (gemm_wsc6, one row per thread); qh is read
+// from global memory straight into the registers of the lane that decodes it, also one super-block ahead. Rows are only 2-byte aligned, and a 16-byte load
+// from an odd multiple of 2 costs about twice an aligned one; the one-row-per-lane loads cost more again because a
+// wavefront instruction touches 32 rows. k-step t of the wavefront is quadrant
 // t / 2, bytes 8 (t % 2) .. +8 of the pieces: 8 values with one scale. A code is put together in the low bits of a
 // half, (ql nibble) | (qh bits << 4) | 0x6400 = 1024 + q as binary16; subtracting 1056 gives q - 32 exactly and one
 // packed multiply gives fp16((q - 32) * (d * sc)). The 8 values come in byte order 0,2,1,3,4,6,5,7;
@@ -44,6 +48,12 @@ __device__ __forceinline__ u32 h2_sub_mul(u32 t, u32 off, u32 scale) {
   return *reinterpret_cast<const u32*>(&w);
 }
 
+// ql of one super-block of the workgroup's 192 rows, [row][128 B + 16 B of padding]: staged by all lanes with consecutive
+// lanes on consecutive 16-byte pieces of a row (8 rows per wavefront instruction), picked up by the lanes that decode it.
+__shared__ uint4 gemm_wbuf6[GEMM_BN * 9];
+// the 16 scale bytes and d of the same rows, [row][6 dwords]: staged one row per thread by the first three wavefronts
+__shared__ u32 gemm_wsc6[GEMM_BN * 6];
+
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_f16(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
   const u32 tid = threadIdx.x, lane = tid & 63;
@@ -63,14 +73,14 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 n0 = nt * GEMM_BN + nh * 96;             // first weight row of this wavefront
   const size_t row_bytes = (size_t)nkb_all * 210;
 
-  // uniform base of the wavefront's rows + a 32-bit per-lane offset (96 rows are far below 4 GiB), already at the
-  // lane's pieces: ql at 64 kh + 16 kg, qh at 128 + 32 kh + 16 kg, scales at 192 + 8 kh
+  // uniform base of the wavefront's rows + a 32-bit per-lane offset (96 rows are far below 4 GiB) to the lane's
+  // piece of qh at 128 + 32 kh + 16 kg
   const u32 base_row = min(n0, out_dim - 1);
   const uint8_t* wbase = w + (size_t)base_row * row_bytes + (size_t)kb0 * 210;
   u32 rowoff[3];
 #pragma unroll
   for (int c = 0; c < 3; c++) rowoff[c] = (min(n0 + 32 * c + j, out_dim - 1) - base_row) * (u32)row_bytes;
-  const u32 o_ql = 64 * kh + 16 * kg, o_qh = 128 + 32 * kh + 16 * kg, o_sc = 192 + 8 * kh;
+  const u32 o_qh = 128 + 32 * kh + 16 * kg;
   const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
   float16_t acc[4][3];
@@ -81,12 +91,49 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
+  // staging of ql: piece p = 64 (4 i + wave) + lane, i < 6, is bytes [16 (p % 8), +16) of row p / 8 of the tile
+  const u32 tile_row0 = min(nt * GEMM_BN, out_dim - 1);
+  const uint8_t* tbase = w + (size_t)tile_row0 * row_bytes + (size_t)kb0 * 210;   // uniform
+  u32 soff[6], sdst[6];
+#pragma unroll
+  for (int i = 0; i < 6; i++) {
+    const u32 p = (4u * i + wave) * 64u + lane, r = p >> 3, part = p & 7u;
+    soff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part;
+    sdst[i] = r * 9u + part;
+  }
+  const u32 take0 = (nh * 96 + j) * 9 + 4 * kh + kg;   // the lane's first ql piece of its row c = 0; the second is 2 further
+  const u32 srow = (min(nt * GEMM_BN + min(tid, (u32)GEMM_BN - 1), out_dim - 1) - tile_row0) * (u32)row_bytes + 192u;
+  const u32 tsc = (nh * 96 + j) * 6;                   // the lane's row c = 0 in gemm_wsc6
+  uint4 stg[6], stg_sc;
+  u32 stg_d;
+  auto stage_load = [&](const uint8_t* kbase, int i) { stg[i] = ld16(kbase + soff[i]); };
+  auto stage_load_sc = [&](const uint8_t* kbase) {
+    if (wave < 3) {
+      stg_sc = ld16(kbase + srow);
+      stg_d = ld2(kbase + (srow + 16));
+    }
+  };
+  auto stage_store = [&]() {
+#pragma unroll
+    for (int i = 0; i < 6; i++) gemm_wbuf6[sdst[i]] = stg[i];
+    if (wave < 3) {
+      *reinterpret_cast<uint2*>(&gemm_wsc6[tid * 6]) = make_uint2(stg_sc.x, stg_sc.y);
+      *reinterpret_cast<uint2*>(&gemm_wsc6[tid * 6 + 2]) = make_uint2(stg_sc.z, stg_sc.w);
+      gemm_wsc6[tid * 6 + 4] = stg_d;
+    }
+  };
+  auto take_ql = [&](GemmRaw6 (&raw)[3]) {
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+      raw[c].qa = gemm_wbuf6[take0 + 288 * c];
+      raw[c].qb = gemm_wbuf6[take0 + 288 * c + 2];
+      raw[c].sc = *reinterpret_cast<const uint2*>(&gemm_wsc6[tsc + 192 * c + 2 * kh]);
+      raw[c].d = gemm_wsc6[tsc + 192 * c + 4];
+    }
+  };
+
   auto load_row = [&](GemmRaw6& raw, const uint8_t* kbase, int c) {
-    raw.qa = ld16(kbase + (rowoff[c] + o_ql));
-    raw.qb = ld16(kbase + (rowoff[c] + o_ql + 32));
     raw.qh = ld16(kbase + (rowoff[c] + o_qh));
-    raw.sc = ld8(kbase + (rowoff[c] + o_sc));
-    raw.d = ld2(kbase + (rowoff[c] + 208));
   };
 
   // Stage super-block 0 of x and the first weights. The main loop takes super-blocks in pairs with fixed roles (x
@@ -94,6 +141,9 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   // out of buffer 1 / registers B.
   const bool odd = nkb & 1;
   GemmRaw6 rawA[3], rawB[3];
+#pragma unroll
+  for (int i = 0; i < 6; i++) stage_load(tbase, i);
+  stage_load_sc(tbase);
   if (odd) {
 #pragma unroll
     for (int c = 0; c < 3; c++) load_row(rawB[c], wbase, c);
@@ -109,7 +159,12 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
                                        16, 0, 0);
   }
+  stage_store();
   __syncthreads();
+  if (odd) take_ql(rawB); else take_ql(rawA);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();   // gemm_wbuf6 is free for the next super-block
+  asm volatile("" ::: "memory");
 
   auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt, const GemmRaw6 (&cur)[3], GemmRaw6 (&nxt)[3]) {
     // d * sc of the four 16-value sub-blocks of the lane's group (scale bytes kg, kg + 2, kg + 4, kg + 6 of the
@@ -127,6 +182,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
     const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
     const uint8_t* knbase = wbase + (size_t)kn * 210; // uniform
+    const uint8_t* tnext = tbase + (size_t)kn * 210;  // uniform
 
     const uint4* arow = xcur + (16 * kh + kg) * 128 + j;   // k-steps 8*kh .. 8*kh+7; 32 lanes read 512 contiguous bytes
     auto build_b = [&](half8_t (&B)[3], int t) {
@@ -160,7 +216,14 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       const int p = t & 1;
       // prefetches for the next super-block, a few per k-step: the raw weights of one row tile (5 loads) in each of
       // the first three steps, the x tile global -> LDS spread over the first six
-      if (t < 3) load_row(nxt[t], knbase, t);
+      if (t < 3) {
+        stage_load(tnext, 2 * t);
+        stage_load(tnext, 2 * t + 1);
+        load_row(nxt[t], knbase, t);
+      }
+      if (t == 3) stage_load_sc(tnext);
+      if (t == 6) stage_store();
+      if (t == 7) take_ql(nxt);
       if (t < 6) {
 #pragma unroll
         for (int i = (t < 3 ? 2 * t : 3 * t - 3); i < (t < 3 ? 2 * t + 2 : (t < 5 ? 3 * t : 16)); i++)
@@ -190,10 +253,16 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
         __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);   // eight VALU (a Q6_K operand takes more than a Q4_K one)
       }
       __builtin_amdgcn_sched_barrier(0);
+      if (t == 6) {
+        // the staged ql of the next super-block is complete once every wavefront's stores have landed
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    // End of the iteration: everything this wavefront requested has to be there (the x tile for everybody,
-    // the weights for its own next iteration), then everybody meets.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // End of the iteration: everything this wavefront requested has to be there (the x tile for everybody, the
+    // weights for its own next iteration) and its reads of gemm_wbuf6 have to be done, then everybody meets.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   };
