@@ -146,12 +146,14 @@ def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, w
     return per, 2.0 * tokens * out_dim * in_dim / (per * 1e-3) / 1e12
 
 
-def cpu_baseline(oracle, case, budget_s=10.0):
-    """The CPU oracle (C restatement of QuantMatmul.matmul_add, 1 thread, f64 accumulation) on the same matrix."""
+def cpu_baseline(oracle, case, budget_s=10.0, threads=1):
+    """The CPU oracle (C restatement of QuantMatmul.matmul_add, f64 accumulation) on the same matrix: one thread, or
+    the output rows divided among `threads` host threads."""
     zero = np.zeros(case.out_dim, dtype=np.float32)
     reps, t0 = 0, time.perf_counter()
     while True:
-        ref = oracle.matmul_add(case.host_x, case.tokens, case.in_dim, case.host_w, case.w_type, case.out_dim, zero)
+        ref = oracle.matmul_add(case.host_x, case.tokens, case.in_dim, case.host_w, case.w_type, case.out_dim, zero,
+                                threads=threads)
         reps += 1
         el = time.perf_counter() - t0
         if el >= budget_s and reps >= 3 or reps >= 200:
@@ -247,6 +249,12 @@ def main():
                 np.sqrt((got.astype(np.float64) @ got.astype(np.float64)) * (ref.astype(np.float64) @ ref.astype(np.float64))))
     ok = cos >= 0.99999 and max_diff <= 1e-3
     cpu_gbps = head.bytes_per_step * cpu_reps / cpu_s / 1e9
+    # the same restatement with the rows divided among the host cores this job may use (16 on a one-GPU box)
+    mt_cores = max(1, min(16, os.cpu_count() or 1))
+    _, mt_reps, mt_s = cpu_baseline(oracle, head, min(3.0, args.cpu_seconds), threads=mt_cores)
+    mt_gbps = head.bytes_per_step * mt_reps / mt_s / 1e9
+    log("cpu_baseline: 1 thread %.4f GB/s (%d reps, %.1f s); %d threads %.4f GB/s (%d reps, %.1f s); gcc -O2 -ffp-contract=off, "
+        "stands in for the reference's Crystal QuantMatmul" % (cpu_gbps, cpu_reps, cpu_s, mt_cores, mt_gbps, mt_reps, mt_s))
 
     # ---- timed region ------------------------------------------------------------------------------------
     ms, graphed = time_steps(hip, stream, head.launch, args.steps, args.warmup)
@@ -417,6 +425,8 @@ def main():
             "sample": "%d x the same 12288x4096 Q4_K GEMV (M=1) through the C restatement of QuantMatmul.matmul_add, "
                       "1 thread, %.1f s" % (cpu_reps, cpu_s),
         },
+        "cpu_baseline_all_cores": {"value": round(mt_gbps, 4), "unit": "GB/s", "cores": mt_cores, "kind": "port",
+                                   "sample": "%d x the same GEMV, rows divided among %d threads, %.1f s" % (mt_reps, mt_cores, mt_s)},
     }
     if extra:
         result["cases"] = extra
