@@ -1,0 +1,75 @@
+"""Seeded sweep over random valid shapes: every decode entry point and the prefill GEMM against the CPU oracle.
+
+The shapes are drawn, not chosen: odd out_dim (partial row groups), in_dim of any whole number of blocks (partial column
+sets), every token count and weight type. Same tolerances as the per-kernel tests.
+"""
+import numpy as np
+import pytest
+
+from cogni_ml_amd import quant, synth
+from gpu_common import DevArray, gpu  # noqa: F401
+from helpers import BLOCK, Q4_K, Q5_K, Q6_K, Q8_0
+from test_gpu_gemm import check as check_gemm
+from test_gpu_gemv import check as check_gemv
+from test_gpu_output_head import run_top1
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_shape(rng, type_id, max_out, max_blocks):
+    be = BLOCK[type_id][1]
+    out_dim = int(rng.integers(1, max_out + 1))
+    in_dim = be * int(rng.integers(1, max_blocks * (256 // be) + 1))
+    return out_dim, in_dim
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_gemv_shapes(gpu, oracle, seed):
+    rng = np.random.default_rng(7000 + seed)
+    for case in range(10):
+        type_id = [Q8_0, Q4_K, Q5_K, Q6_K][int(rng.integers(0, 4))]
+        tokens = int(rng.integers(1, 9))
+        out_dim, in_dim = draw_shape(rng, type_id, 600, 20)
+        raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+        x = synth.make_activations(rng, tokens, in_dim)
+        res = rng.standard_normal(tokens * out_dim).astype(np.float32) if rng.integers(0, 2) else None
+        what = "seed %d case %d: type %d M=%d out=%d in=%d add=%s" % (seed, case, type_id, tokens, out_dim, in_dim, res is not None)
+        print(what, flush=True)
+        check_gemv(oracle, raw, type_id, x, in_dim, out_dim, tokens, res, what)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_random_top1_shapes(gpu, oracle, seed):
+    rng = np.random.default_rng(8000 + seed)
+    for case in range(6):
+        type_id = [Q8_0, Q4_K, Q5_K, Q6_K][int(rng.integers(0, 4))]
+        tokens = int(rng.integers(1, 8))
+        out_dim, in_dim = draw_shape(rng, type_id, 3000, 8)
+        raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+        x = synth.make_activations(rng, tokens, in_dim)
+        print("seed %d case %d: type %d M=%d out=%d in=%d" % (seed, case, type_id, tokens, out_dim, in_dim), flush=True)
+        ids, vals, logits = run_top1(raw, type_id, x, in_dim, out_dim, tokens)
+        want = oracle.matmul_add(x, tokens, in_dim, raw, type_id, out_dim, np.zeros(out_dim, dtype=np.float32),
+                                 threads=8).reshape(tokens, out_dim)
+        for tok in range(tokens):
+            # the winner is the first maximum of the device's own logits, up to the different summation order of the
+            # kernels that produce the two; against the oracle it is within the GEMV tolerance of the best row
+            assert ids[tok] == int(np.argmax(logits[tok])) or np.isclose(vals[tok], logits[tok].max(), rtol=2e-5, atol=0)
+            top, scale = float(want[tok].max()), float(np.abs(want[tok]).max())
+            assert abs(float(vals[tok]) - top) <= 1e-4 * scale
+            assert want[tok][ids[tok]] >= top - 1e-4 * scale
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_gemm_shapes(gpu, oracle, seed):
+    rng = np.random.default_rng(9000 + seed)
+    for case in range(5):
+        t = [Q4_K, Q5_K, Q6_K][int(rng.integers(0, 3))]
+        tokens = int(rng.integers(9, 400))
+        out_dim, in_dim = draw_shape(rng, t, 700, 12)
+        raw = synth.make_weights(rng, t, out_dim, in_dim)
+        x = synth.make_activations(rng, tokens, in_dim)
+        bias = rng.standard_normal(out_dim).astype(np.float32) if rng.integers(0, 2) else None
+        what = "seed %d case %d: type %d M=%d out=%d in=%d bias=%s" % (seed, case, t, tokens, out_dim, in_dim, bias is not None)
+        print(what, flush=True)
+        check_gemm(oracle, raw, x, in_dim, out_dim, tokens, bias, what, t=t)
