@@ -236,6 +236,27 @@ def main():
             ms, _ = time_steps(hip, stream, rd, args.steps, args.warmup)
             us = ms / args.steps * 1e3
             log("read_only grid=%d us=%.3f gbps=%.1f" % (grid, us, head.w_bytes / us / 1e3))
+        # a loop of nothing but fp16 MFMAs on every SIMD of the chip, one and two wavefronts per SIMD, short and long
+        # (the clock the chip sustains under that load is part of the answer)
+        ops = hip.DeviceBuffer(7 * 64 * 16)
+        vals = (rng.standard_normal(7 * 64 * 8) * 0.5).astype(np.float16)
+        hip.copy_htod(ops.ptr, vals, vals.nbytes, "mfma operands")
+        res = hip.DeviceBuffer(4 * 512 * 1024)
+        for name, block in (("mfma_f16_ceiling_w4", 256), ("mfma_f16_ceiling_w8", 512)):
+            fn = mod.function(name)
+            for wgs in (256, 1024):
+                for iters in (128, 1024):
+                    box = hip.KernelParams(ctypes.c_uint64(ops.ptr), ctypes.c_uint64(res.ptr), ctypes.c_uint32(iters))
+
+                    def mm(i, st, fn=fn, wgs=wgs, block=block, box=box):
+                        with hip.with_stream(st):
+                            hip.launch(fn, wgs, 1, 1, block, 1, 1, box, "mfma")
+                    reps = 20
+                    ms, _ = time_steps(hip, stream, mm, reps, 3)
+                    us = ms / reps * 1e3
+                    flops = 2.0 * 32 * 32 * 16 * 12 * iters * (block // 64) * wgs
+                    log("%s workgroups=%d iters=%d us=%.2f tflops=%.1f frac_of_published_peak=%.3f" % (
+                        name, wgs, iters, us, flops / us / 1e6, flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS))
         return
 
     # ---- parity spot check of the measured kernel against the oracle, and the CPU baseline ------------
