@@ -221,3 +221,19 @@ class QuantWeight:
         if self._handle:
             hip.lib().cogni_weight_destroy(self._handle)
             self._handle = None
+
+
+def matvec_many(qws, x):
+    """qmatvec_many(qws, x) (qwen35_cpu.cr:1419-1445): every weight against the same one-token x in one call; a list of
+    float32 arrays, one per weight, [] for no weights."""
+    qws = list(qws)
+    if not qws:
+        return []
+    xa = np.ascontiguousarray(x, dtype=np.float32)
+    if xa.size != qws[0].in_dim:
+        raise ValueError("matvec_many x size mismatch: expected %d, got %d" % (qws[0].in_dim, xa.size))
+    outs = [np.empty(q.out_dim, dtype=np.float32) for q in qws]
+    handles = (ctypes.c_void_p * len(qws))(*[q._handle for q in qws])
+    ptrs = (ctypes.c_void_p * len(qws))(*[o.ctypes.data for o in outs])
+    _check(hip.lib().cogni_weight_matvec_many(handles, ctypes.c_int32(len(qws)), ctypes.c_void_p(xa.ctypes.data), ptrs))
+    return outs

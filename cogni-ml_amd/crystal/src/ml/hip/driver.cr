@@ -82,6 +82,11 @@ lib LibCogniHIP
   fun cogni_dequantize(data : Void*, data_bytes : LibC::SizeT, type : UInt32, n_elements : Int64, out : Float32*) : Int32
   fun cogni_matmul_add(x : Float32*, rows : Int32, in_dim : Int32, w_raw : Void*, w_bytes : LibC::SizeT,
                        w_type : UInt32, out_dim : Int32, bias : Float32*, result : Float32*) : Int32
+  fun cogni_weight_create(qw : Void**, raw : Void*, raw_bytes : LibC::SizeT, type : UInt32, out_dim : Int32, in_dim : Int32) : Int32
+  fun cogni_weight_device_ptr(qw : Void*) : UInt64
+  fun cogni_weight_matmul(qw : Void*, x : Float32*, rows : Int32, bias : Float32*, result : Float32*) : Int32
+  fun cogni_weight_matvec_many(qws : Void**, count : Int32, x : Float32*, results : Float32**) : Int32
+  fun cogni_weight_destroy(qw : Void*) : Int32
   fun cogni_last_error : UInt8*
 end
 

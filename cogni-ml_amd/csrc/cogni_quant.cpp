@@ -633,6 +633,39 @@ int cogni_weight_matmul(const cogni_quant_weight* qw, const float* x, int32_t ro
   return 0;
 }
 
+int cogni_weight_matvec_many(const cogni_quant_weight* const* qws, int32_t count, const float* x, float* const* results) {
+  if (count < 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_matvec_many: count must not be negative");
+  if (count == 0) return 0;
+  if (!qws || !x || !results) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_matvec_many: null argument");
+  size_t total_out = 0;
+  for (int32_t i = 0; i < count; i++) {
+    if (!qws[i] || !results[i]) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_matvec_many: null weight or result");
+    if (qws[i]->in_dim != qws[0]->in_dim)
+      return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_matvec_many: weight " + std::to_string(i) + " has in_dim " +
+                                                  std::to_string(qws[i]->in_dim) + ", the first one " + std::to_string(qws[0]->in_dim));
+    total_out += (size_t)qws[i]->out_dim;
+  }
+  // one upload of x, every GEMV on the default stream, one wait, then the outputs (they share one allocation)
+  DeviceMem dx, dout;
+  HIP_TRY(hipMalloc(&dx.p, (size_t)qws[0]->in_dim * 4), "hipMalloc(x)");
+  HIP_TRY(hipMalloc(&dout.p, total_out * 4), "hipMalloc(results)");
+  HIP_TRY(hipMemcpyHtoD(dx.p, const_cast<float*>(x), (size_t)qws[0]->in_dim * 4), "hipMemcpyHtoD(x)");
+  size_t at = 0;
+  for (int32_t i = 0; i < count; i++) {
+    const int rc = cogni_gemv_dev((uint64_t)(uintptr_t)qws[i]->dev, qws[i]->type, dx.addr(), 0, dout.addr() + at * 4,
+                                  (uint32_t)qws[i]->in_dim, (uint32_t)qws[i]->out_dim, 1, nullptr);
+    if (rc != 0) return rc;
+    at += (size_t)qws[i]->out_dim;
+  }
+  HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize(matvec_many)");
+  at = 0;
+  for (int32_t i = 0; i < count; i++) {
+    HIP_TRY(hipMemcpyDtoH(results[i], static_cast<char*>(dout.p) + at * 4, (size_t)qws[i]->out_dim * 4), "hipMemcpyDtoH(result)");
+    at += (size_t)qws[i]->out_dim;
+  }
+  return 0;
+}
+
 int cogni_matmul_add(const float* x, int32_t rows, int32_t in_dim, const void* w_raw, size_t w_bytes, uint32_t w_type,
                      int32_t out_dim, const float* bias, float* result) {
   cogni_quant_weight* qw = nullptr;

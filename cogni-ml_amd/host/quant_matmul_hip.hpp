@@ -85,6 +85,21 @@ class QuantWeight {
     if (handle_) cogni_weight_destroy(handle_);
     handle_ = nullptr;
   }
+  // qmatvec_many(qws, x) (qwen35_cpu.cr:1419-1445): every weight against the same one-token x in one call
+  static std::vector<std::vector<float>> matvec_many(const std::vector<const QuantWeight*>& qws, const std::vector<float>& x) {
+    std::vector<std::vector<float>> results(qws.size());
+    if (qws.empty()) return results;
+    if (x.size() != (size_t)qws[0]->in_dim_) throw std::invalid_argument("matvec_many x size mismatch");
+    std::vector<const cogni_quant_weight*> handles(qws.size());
+    std::vector<float*> outs(qws.size());
+    for (size_t i = 0; i < qws.size(); i++) {
+      results[i].resize((size_t)qws[i]->out_dim_);
+      handles[i] = qws[i]->handle_;
+      outs[i] = results[i].data();
+    }
+    qcheck(cogni_weight_matvec_many(handles.data(), (int32_t)qws.size(), x.data(), outs.data()));
+    return results;
+  }
 
  private:
   const uint8_t* raw_;

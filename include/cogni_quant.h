@@ -230,6 +230,10 @@ uint64_t cogni_weight_device_ptr(const cogni_quant_weight* qw);
  * src/ml/gguf/qwen35_cpu.cr:1462-1468). */
 int cogni_weight_matmul(const cogni_quant_weight* qw, const float* x, int32_t rows, const float* bias,
                         float* result);
+/* qmatvec_many(qws, x) (src/ml/gguf/qwen35_cpu.cr:1419-1445, Qwen35Metal.matmul_many): `count` resident weights of one
+ * in_dim against the same x (one token) with one upload of x, one wait and results[i] receiving qws[i].out_dim floats.
+ * count == 0 does nothing (the reference returns an empty array). */
+int cogni_weight_matvec_many(const cogni_quant_weight* const* qws, int32_t count, const float* x, float* const* results);
 int cogni_weight_destroy(cogni_quant_weight* qw);
 
 /* Text of the last failure on the calling thread ("hipModuleLoadData failed with HIP error 209 (...)"). */

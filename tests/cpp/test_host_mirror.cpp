@@ -147,6 +147,11 @@ static int gpu_probe() {
   EXPECT(qw.device_ptr() != 0);
   std::vector<float> via_qw = qw.matmul(x, 1);
   EXPECT(std::memcmp(via_qw.data(), gpu.data(), 4 * out_dim) == 0);
+  // qmatvec_many: the same weight twice against one x, and no weights at all
+  std::vector<std::vector<float>> many = QuantWeight::matvec_many({&qw, &qw}, x);
+  EXPECT(many.size() == 2 && std::memcmp(many[0].data(), gpu.data(), 4 * out_dim) == 0 &&
+         std::memcmp(many[1].data(), gpu.data(), 4 * out_dim) == 0);
+  EXPECT(QuantWeight::matvec_many({}, x).empty());
   // bit-exact dequantize of the first rows
   std::vector<float> deq = Dequant::dequantize(w.data(), w.size(), TensorType::Q4_K, 8 * in_dim), ref(8 * in_dim);
   oracle_dequantize(w.data(), 12, 8 * in_dim, ref.data());

@@ -142,6 +142,28 @@ def test_matmul_add_host_signature_with_bias(gpu, oracle):
         qw.close()
 
 
+def test_matvec_many_shares_one_activation_vector(gpu, oracle):
+    """qmatvec_many (qwen35_cpu.cr:1419-1445): weights of different types and sizes against one x; each result equals the
+    single-weight call bit for bit; no weights -> no results; a weight of another in_dim is refused."""
+    rng = np.random.default_rng(1419)
+    in_dim = 1024
+    x = synth.make_activations(rng, 1, in_dim)
+    shapes = [(Q4_K, 512), (Q4_K, 128), (Q6_K, 128), (Q5_K, 300), (Q8_0, 77)]
+    qws = [quant.QuantWeight(synth.make_weights(rng, t, out_dim, in_dim), t, out_dim, in_dim) for t, out_dim in shapes]
+    outs = quant.matvec_many(qws, x)
+    assert [o.size for o in outs] == [out_dim for _, out_dim in shapes]
+    for qw, o in zip(qws, outs):
+        assert np.array_equal(o, qw.matmul(x, 1))
+        ref = oracle.matmul_add(x, 1, in_dim, qw.raw, int(qw.type), qw.out_dim, np.zeros(qw.out_dim, dtype=np.float32))
+        assert np.max(np.abs(o - ref)) <= 1e-5 * np.max(np.abs(ref))
+    assert quant.matvec_many([], x) == []
+    other = quant.QuantWeight(synth.make_weights(rng, Q4_K, 16, 512), Q4_K, 16, 512)
+    with pytest.raises(quant.QuantError, match="in_dim"):
+        quant.matvec_many([qws[0], other], x)
+    for qw in qws + [other]:
+        qw.close()
+
+
 def test_linearity_and_determinism_at_full_size(gpu):
     """Size-independent properties at the headline shape: same input -> same bits; f(2a) == 2 f(a) exactly;
     f(a) + f(b) ~= f(a + b)."""
