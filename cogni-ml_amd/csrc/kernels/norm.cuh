@@ -7,6 +7,7 @@
 #include "common.cuh"
 
 #define NORM_BLOCK 256
+#define NORM_KEEP 4   // float4 a thread keeps across the reduction on the short-row path
 
 template <bool ADD>
 __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __restrict__ add,
@@ -22,6 +23,44 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
   const u32 tid = threadIdx.x;
   const bool vec = (dim & 3u) == 0;   // rows then start 16-byte aligned when the buffers do
   float ss = 0.0f;
+  if (vec && dim <= NORM_BLOCK * 4 * NORM_KEEP) {
+    // rows of up to 4096 values: a thread's values and norm weights stay in registers across the reduction (no second
+    // read of what was just written, the weights are on their way before the barrier); same sums in the same order
+    float4 v[NORM_KEEP], w[NORM_KEEP];
+#pragma unroll
+    for (int k = 0; k < NORM_KEEP; k++) {
+      const u32 i = ((u32)k * NORM_BLOCK + tid) * 4;
+      v[k] = w[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < dim) {
+        v[k] = *reinterpret_cast<const float4*>(xt + i);
+        w[k] = *reinterpret_cast<const float4*>(norm + i);
+        if (ADD) {
+          const float4 a = *reinterpret_cast<const float4*>(at + i);
+          v[k].x += a.x, v[k].y += a.y, v[k].z += a.z, v[k].w += a.w;
+          *reinterpret_cast<float4*>(rt + i) = v[k];
+        }
+        ss += v[k].x * v[k].x;
+        ss += v[k].y * v[k].y;
+        ss += v[k].z * v[k].z;
+        ss += v[k].w * v[k].w;
+      }
+    }
+    ss = wave_sum(ss);
+    if ((tid & (WAVE - 1)) == 0) part[tid / WAVE] = ss;
+    __syncthreads();
+    const float total = (part[0] + part[1]) + (part[2] + part[3]);
+    const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+#pragma unroll
+    for (int k = 0; k < NORM_KEEP; k++) {
+      const u32 i = ((u32)k * NORM_BLOCK + tid) * 4;
+      if (i < dim) {
+        float4 o;
+        o.x = (v[k].x * inv) * w[k].x, o.y = (v[k].y * inv) * w[k].y, o.z = (v[k].z * inv) * w[k].z, o.w = (v[k].w * inv) * w[k].w;
+        *reinterpret_cast<float4*>(ot + i) = o;
+      }
+    }
+    return;
+  }
   if (vec) {
     for (u32 i = tid * 4; i < dim; i += NORM_BLOCK * 4) {
       float4 v = *reinterpret_cast<const float4*>(xt + i);
