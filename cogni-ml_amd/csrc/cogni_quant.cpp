@@ -292,7 +292,10 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   for (uint32_t t0 = 0; t0 < tokens; t0 += m) {
     const uint32_t left = tokens - t0;
     m = left < cap ? left : cap;
-    if (pairs && left >= 3 && (left & 1u)) m = 3;
+    // an odd count ends in a group of three, except on a matrix long enough for the pair kernel to walk its row groups
+    // (there a pair and a single token are faster: Q6_K 151936 x 4096 158 + 96 us against 283)
+    const bool walks = (uint64_t)gemv_grid(w_type, 2, out_dim) * (uint32_t)gemv_rows_per_block(w_type, 2) < out_dim;
+    if (pairs && left == 3 && !walks) m = 3;
     uint32_t grid = 0, block = 0, shmem = 0;
     const char* kernel = nullptr;
     int rc = cogni_gemv_plan(w_type, m, residual != 0, in_dim, out_dim, &kernel, &grid, &block, &shmem);
@@ -372,7 +375,10 @@ int cogni_embed_dev(uint64_t w_raw, uint32_t w_type, uint64_t token_ids, uint64_
 }
 
 // ---- output head: GEMV with the arg-max over the rows ---------------------------------------------------
-static uint32_t top1_token_cap(uint32_t type) { return (type == COGNI_TYPE_Q4_K || type == COGNI_TYPE_Q6_K) ? 3u : 1u; }
+// tokens per launch: two for the types that have the kernel (a pair shares one pass over the weights and, on a long
+// matrix, walks the row groups with the activations staged once; a third token would be a second token group with its
+// own staging: Q6_K 151936 x 4096 takes 100 / 168 / 310 us for 1 / 2 / 3 tokens)
+static uint32_t top1_token_cap(uint32_t type) { return (type == COGNI_TYPE_Q4_K || type == COGNI_TYPE_Q6_K) ? 2u : 1u; }
 
 uint32_t cogni_gemv_top1_partials(uint32_t w_type, uint32_t out_dim) {
   if (!gemv_type(w_type) || out_dim == 0) return 0;

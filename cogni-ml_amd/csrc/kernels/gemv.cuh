@@ -718,29 +718,45 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
       set_group(grp);
     }
   }
-  // Column sets are taken F::SPI at a time: all their weight loads are issued before the first is consumed.
-  if constexpr (!PIPE)
-  for (u32 s = 0; s < ncs; s += F::SPI) {
-    const bool restage = NG == 1 && (s % CH) == 0;   // CH is a multiple of SPI or covers the whole row
-    typename F::template Stage<R> stA, stB;
-    const bool two = F::SPI == 2 && s + 1 < ncs;
-    if constexpr (DIRECT) {
-      auto rows = [&]() { F::template load<R>(stA, rowp, ln, s, nb); };   // (SPI is 1 for these formats)
-      if (restage) {
-        if (s > 0) __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
-        stage_chunk(s, rows);
-      } else {
-        rows();
+  // Column sets are taken F::SPI at a time: all their weight loads are issued before the first is consumed. Directly
+  // staged activations of one token group (two tokens of a K-quant): the workgroup walks the row groups blockIdx.x,
+  // blockIdx.x + gridDim.x, ... and stages the activations again only if the row is longer than one chunk.
+  if constexpr (!PIPE) {
+    constexpr bool WALK = DIRECT && NG == 1;
+    for (u32 grp = blockIdx.x;;) {
+      const bool first = grp == blockIdx.x;
+      for (u32 s = 0; s < ncs; s += F::SPI) {
+        const bool restage = NG == 1 && (s % CH) == 0 && (first || ncs > CH);   // CH is a multiple of SPI or covers the whole row
+        typename F::template Stage<R> stA, stB;
+        const bool two = F::SPI == 2 && s + 1 < ncs;
+        if constexpr (DIRECT) {
+          auto rows = [&]() { F::template load<R>(stA, rowp, ln, s, nb); };   // (SPI is 1 for these formats)
+          if (restage) {
+            if (s > 0 || !first) __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
+            stage_chunk(s, rows);
+          } else {
+            rows();
+          }
+        } else {
+          float4 buf[FU];
+          if (restage) stage_begin(s, 0, buf);
+          F::template load<R>(stA, rowp, ln, s, nb);
+          if (two) F::template load<R>(stB, rowp, ln, s + 1, nb);
+          if (restage) stage_end(s, 0, buf);
+        }
+        step(stA, s);
+        if (two) step(stB, s + 1);
       }
-    } else {
-      float4 buf[FU];
-      if (restage) stage_begin(s, 0, buf);
-      F::template load<R>(stA, rowp, ln, s, nb);
-      if (two) F::template load<R>(stB, rowp, ln, s + 1, nb);
-      if (restage) stage_end(s, 0, buf);
+      if (!WALK) break;
+      grp += gridDim.x;
+      if (grp >= ngroups) break;
+      finish(row0);
+#pragma unroll
+      for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int m = 0; m < M; m++) acc[r][m] = 0.0f;
+      set_group(grp);
     }
-    step(stA, s);
-    if (two) step(stB, s + 1);
   }
   finish(row0);
   if constexpr (TOP1) top1_store();

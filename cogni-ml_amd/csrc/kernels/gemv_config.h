@@ -58,15 +58,18 @@ static constexpr inline GEMV_HD bool gemv_direct_x(unsigned type, int token_grou
   return (type == 12 || type == 13 || type == 14) && token_groups == 1;
 }
 
-// One token of a K-quant matrix: the kernel walks row groups blockIdx.x, blockIdx.x + gridDim.x, ... with the
-// activations staged once, so a long matrix is launched as the workgroups that are resident together (3 per
-// compute unit at 3 wavefronts per SIMD, 256 compute units), each with the same number of groups up to one.
+// One or two tokens of a K-quant matrix (one token group): the kernel walks row groups blockIdx.x, blockIdx.x +
+// gridDim.x, ... with the activations staged once, so a long matrix is launched as the workgroups that are resident
+// together (256 compute units x 3 per unit at 3 wavefronts per SIMD for one token, x 2 for two), each with the same
+// number of groups up to one.
 #define GEMV_RESIDENT_WGS 768u
+#define GEMV_RESIDENT_WGS_2 512u
 static inline unsigned gemv_grid(unsigned type, int tokens, unsigned out_dim) {
   const unsigned rows = (unsigned)gemv_rows_per_block(type, tokens);
   const unsigned groups = (out_dim + rows - 1) / rows;
-  if (tokens != 1 || !gemv_direct_x(type, 1) || groups <= GEMV_RESIDENT_WGS) return groups;
-  const unsigned per_wg = (groups + GEMV_RESIDENT_WGS - 1) / GEMV_RESIDENT_WGS;
+  const unsigned resident = tokens == 1 ? GEMV_RESIDENT_WGS : GEMV_RESIDENT_WGS_2;
+  if (tokens > 2 || !gemv_direct_x(type, 1) || groups <= resident) return groups;
+  const unsigned per_wg = (groups + resident - 1) / resident;
   return (groups + per_wg - 1) / per_wg;
 }
 

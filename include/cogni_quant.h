@@ -108,7 +108,7 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
  * fp32 accumulation. tokens >= 1; they are issued as consecutive launches of the token count that measures
  * fastest for the type and shape: up to 4 where cogni_gemv_plan picks the matrix-core kernel, else pairs for the
- * K-quants (one group of three when the count is odd) and up to 8 for Q8_0. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
+ * K-quants (one group of three when the count is odd and the matrix is short enough for one workgroup per row group) and up to 8 for Q8_0. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
  * same, bin/cuda_q4k_gemv_probe.cr:125); Q8_0 accepts any in_dim >= 1 (its last block is clipped,
  * quant_matmul.cr:241,259). Types: Q8_0, Q4_K, Q5_K, Q6_K. */
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
@@ -163,8 +163,8 @@ int cogni_embed_dev(uint64_t w_raw, uint32_t w_type, uint64_t token_ids, uint64_
 
 /* Output head without the logits: for each token the index of the largest element of W x and that value
  * (top1_ids: u32[tokens], top1_values: f32[tokens]); of equal values the lowest index wins, as in the reference's CPU scan
- * (bin/cuda_mixed_stack_probe.cr:1485-1497). Two launches per group of up to 3 tokens (Q4_K, Q6_K; one token for the other
- * types): kernel "<prefix>_gemv_top1_partial_f32[_tbatchM]" (w_raw, x, partial_ids, partial_values, in_dim, out_dim) -
+ * (bin/cuda_mixed_stack_probe.cr:1485-1497). Two launches per group of up to 2 tokens (Q4_K, Q6_K; one token for the other
+ * types; kernels for 3 tokens exist but a pair and a single token are faster): kernel "<prefix>_gemv_top1_partial_f32[_tbatchM]" (w_raw, x, partial_ids, partial_values, in_dim, out_dim) -
  * the reference's q6_k_gemv_top1_partial_f32 (src/ml/cuda/kernels/q6k_gemv_probe.ptx:1331), with the grid, block and
  * shared memory of the GEMV of that type and token count and one (id, value) per workgroup and token - then
  * "top1_reduce_f32" (partial_ids, partial_values, out_ids, out_values, count:u32), block 1024, grid = tokens of the group -

@@ -80,8 +80,12 @@ def test_gemv_launch_dims():
     g_head = quant.gemv_launch_dims(14, 1, 4096, 151936)[0]
     groups = -(-151936 // 8)
     assert g_head <= 768 and -(-groups // g_head) * (g_head - 1) < groups
-    assert quant.gemv_launch_dims(14, 2, 4096, 151936)[0] == groups and quant.gemv_launch_dims(8, 1, 4096, 151936)[0] == 151936 // 16
-    assert quant.gemv_top1_partials(14, 151936) == groups
+    # two tokens (one token group) walk the row groups too, 512 workgroups at most; three tokens and Q8_0 do not
+    g2 = quant.gemv_launch_dims(14, 2, 4096, 151936)[0]
+    assert g2 <= 512 and -(-groups // g2) * (g2 - 1) < groups
+    assert quant.gemv_launch_dims(14, 3, 4096, 151936)[0] == groups and quant.gemv_launch_dims(8, 1, 4096, 151936)[0] == 151936 // 16
+    # the top-1 scratch holds one entry per workgroup of the widest launch it is used with (one or two tokens)
+    assert quant.gemv_top1_partials(14, 151936) == max(g_head, g2)
     g1 = quant.gemv_launch_dims(12, 1, 256, 17)[0]
     assert g1 == -(-17 // (12288 // quant.gemv_launch_dims(12, 1, 4096, 12288)[0]))
     with pytest.raises(quant.QuantError):
