@@ -133,54 +133,82 @@ __shared__ uint4 gemm_wbuf[28 * 64];   // 27 copies of 64 pieces, and a 28th tha
 // 12 scale bytes) goes from global memory straight to the lane that decodes it.
 __shared__ uint4 gemm_wbuf5[32 * 64];
 
-// Epilogue shared by the GEMM kernels, in two halves of 64 tokens (the tiles r = 2 hf, 2 hf + 1): every wavefront
-// writes its partial sums to LDS as [k half][token][weight row] (row stride 200 floats: the two k-groups of a
-// wavefront land in disjoint banks), then all 256 threads add the two k halves and the bias and store 16 bytes at a
-// time, 48 consecutive threads per 768-byte output row segment. 2 x 64 x 200 x 4 B = 100 KiB of the two x buffers.
-__device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
-                                              u32 mt, u32 nt, u32 nh, u32 kh, u32 j, u32 kg, u32 tid) {
-  float* part0 = reinterpret_cast<float*>(gemm_xbuf0);   // k half 0: 64 x 200 floats = 51200 B <= 64 KiB
-  float* part1 = reinterpret_cast<float*>(gemm_xbuf1);   // k half 1
-  float* mine = kh ? part1 : part0;
-  const bool full_n = nt * GEMM_BN + GEMM_BN <= out_dim;
+// Epilogue shared by the GEMM kernels. The MFMAs are issued as (weights, x), so an accumulator tile is laid out with the
+// weight rows along the register index: acc[r][c][v] of lane (j, kg) belongs to token 32 r + j and weight row
+// nh * 96 + 32 c + 8 (v / 4) + 4 kg + v % 4 - four consecutive output floats per register quad, which leave as one
+// 16-byte store without passing through LDS. What does pass through LDS is the other k half: a kh wavefront finishes the
+// token tiles r = 2 kh, 2 kh + 1 and hands the other two to its partner (same nh) as 24 float4 per lane in the lane
+// layout both share (kh = 0 writes into x buffer 0, kh = 1 into x buffer 1: 2 x 24 KiB each). Sum first, bias second.
+template <int KH>
+__device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
+                                                   u32 mt, u32 nt, u32 nh, u32 j, u32 kg, u32 lane) {
+  float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * 24 * 64 + lane;
+  const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * 24 * 64 + lane;
 #pragma unroll
-  for (int hf = 0; hf < 2; hf++) {
+  for (int rr = 0; rr < 2; rr++)
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const float16_t& t = acc[2 * (1 - KH) + rr][c];
+        mine[((rr * 3 + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
+      }
+  __syncthreads();
+  const bool vec = (out_dim & 3u) == 0;
+  if (vec && !bias && mt * GEMM_BM + GEMM_BM <= m && nt * GEMM_BN + GEMM_BN <= out_dim) {
+    // a whole tile and nothing to add: one address per token row, the 12 stores of a row at constant offsets from it
 #pragma unroll
     for (int rr = 0; rr < 2; rr++) {
-      const int r = 2 * hf + rr;
+      float* base = out + (size_t)(mt * GEMM_BM + 32 * (2 * KH + rr) + j) * out_dim + (nt * GEMM_BN + nh * 96 + 4 * kg);
 #pragma unroll
       for (int c = 0; c < 3; c++)
 #pragma unroll
-        for (int v = 0; v < 16; v++)
-          mine[(32 * rr + 8 * (v >> 2) + 4 * kg + (v & 3)) * 200 + nh * 96 + 32 * c + j] = acc[r][c][v];
+        for (int g4 = 0; g4 < 4; g4++) {
+          const float16_t& t = acc[2 * KH + rr][c];
+          const float4 p = theirs[((rr * 3 + c) * 4 + g4) * 64];
+          *reinterpret_cast<float4*>(base + 32 * c + 8 * g4) =
+              KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
+                 : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
+        }
     }
-    __syncthreads();
-    const u32 row0 = mt * GEMM_BM + 64 * hf;
-    for (u32 idx = tid; idx < 64 * 48; idx += 256) {
-      const u32 tl = idx / 48, q4 = idx - tl * 48;
-      const u32 row = row0 + tl, n = nt * GEMM_BN + 4 * q4;
-      if (row < m && n < out_dim) {
-        const float4 p0 = *reinterpret_cast<const float4*>(part0 + tl * 200 + 4 * q4);
-        const float4 p1 = *reinterpret_cast<const float4*>(part1 + tl * 200 + 4 * q4);
-        float4 o = make_float4(p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w);
-        float* dst = out + (size_t)row * out_dim + n;
-        if (full_n || n + 4 <= out_dim) {
-          if (bias) {
-            o.x += bias[n]; o.y += bias[n + 1]; o.z += bias[n + 2]; o.w += bias[n + 3];
-          }
-          if ((out_dim & 3u) == 0) {
-            *reinterpret_cast<float4*>(dst) = o;
+    return;
+  }
+#pragma unroll
+  for (int rr = 0; rr < 2; rr++) {
+    const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const float16_t& t = acc[2 * KH + rr][c];
+        const float4 p = theirs[((rr * 3 + c) * 4 + g4) * 64];
+        // (k half 0) + (k half 1) whichever of the two this wavefront holds
+        float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
+                      : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
+        const u32 n = nt * GEMM_BN + nh * 96 + 32 * c + 8 * g4 + 4 * kg;
+        if (token < m && n < out_dim) {
+          float* dst = out + (size_t)token * out_dim + n;
+          if (n + 4 <= out_dim) {
+            if (bias) {
+              o.x += bias[n]; o.y += bias[n + 1]; o.z += bias[n + 2]; o.w += bias[n + 3];
+            }
+            if (vec) {
+              *reinterpret_cast<float4*>(dst) = o;
+            } else {
+              dst[0] = o.x; dst[1] = o.y; dst[2] = o.z; dst[3] = o.w;
+            }
           } else {
-            dst[0] = o.x; dst[1] = o.y; dst[2] = o.z; dst[3] = o.w;
+            const float ov[4] = {o.x, o.y, o.z, o.w};
+            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (bias ? bias[n + e] : 0.0f);
           }
-        } else {
-          const float ov[4] = {o.x, o.y, o.z, o.w};
-          for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (bias ? bias[n + e] : 0.0f);
         }
       }
-    }
-    if (hf == 0) __syncthreads();
   }
+}
+__device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
+                                              u32 mt, u32 nt, u32 nh, u32 kh, u32 j, u32 kg, u32 tid) {
+  if (kh == 0) gemm_epilogue_half<0>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63);
+  else gemm_epilogue_half<1>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63);
 }
 
 // raw bytes of one group of one super-block of one weight row, as a lane sees them
@@ -415,7 +443,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       for (int r = 0; r < 4; r++) {
         const half8_t Ar = *reinterpret_cast<const half8_t*>(&A[p][r]);
 #pragma unroll
-        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(Ar, B[p][c], acc[r][c], 0, 0, 0);
+        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[p][c], Ar, acc[r][c], 0, 0, 0);
       }
       // Scheduling window = one k-step. Left alone the scheduler emits the twelve MFMAs back to back and the
       // operand preparation of the next step behind them, so the matrix pipe and the vector ALU take turns;
