@@ -665,10 +665,12 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
     // that row is there, and what is left after the last byte is one row's worth.
     constexpr int PF = R >= 3 ? 2 : 1;
     typename F::template Stage<R> st;
-    stage_chunk(0, [&]() {
+    // The first rows are requested only once the activations are staged: a compute unit returns loads in order, and
+    // weight loads (HBM misses) issued ahead of the barrier hold up the activation loads (L2 hits) of the wavefronts
+    // that issue theirs a little later - measured 8.05-8.25 us with the rows requested before the barrier, 7.75 after.
+    stage_chunk(0, [&]() {});
 #pragma unroll
-      for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nb);
-    });
+    for (int r = 0; r < PF; r++) F::template load_row<R>(st, r, rowp[r], ln, 0, nb);
     // one column set; `last` (a compile-time tag) says that no column set follows, so the prefetches that
     // would wrap into the next set are left out and the number of loads in flight stays a constant
     auto column_set = [&](u32 s, auto last) {
