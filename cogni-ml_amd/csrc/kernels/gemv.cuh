@@ -735,7 +735,8 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
           auto rows = [&]() { F::template load<R>(stA, rowp, ln, s, nb); };   // (SPI is 1 for these formats)
           if (restage) {
             if (s > 0 || !first) __builtin_amdgcn_s_barrier();   // every wavefront has read the previous chunk into registers
-            stage_chunk(s, rows);
+            stage_chunk(s, [&]() {});   // (rows after the barrier, as in the one-token pipeline)
+            rows();
           } else {
             rows();
           }
