@@ -110,10 +110,16 @@ static inline GEMV_HD unsigned gemv_mfma_log2_kslices(unsigned nsb) {
   while (lg < 3 && (2u << lg) <= nsb) lg++;
   return lg;
 }
-// Shapes the matrix-core kernel takes: Q4_K, 1..4 tokens, in_dim a multiple of 256, all activations staged at once.
+// Rows too long for all their activations to be staged at once are staged a chunk at a time, which needs every
+// wavefront to be a k-slice of its own: in_dim a multiple of 2048.
+static inline GEMV_HD int gemv_mfma_chunked(int tokens, unsigned in_dim) {
+  return (unsigned)tokens * (in_dim >> 8) > (unsigned)GEMV_MFMA_MAX_UNITS(tokens) && (in_dim & 2047u) == 0;
+}
+// Shapes the matrix-core kernel takes: Q4_K, 1..4 tokens, in_dim a multiple of 256, all activations staged at once
+// or in_dim a multiple of 2048.
 static inline int gemv_mfma_supported(unsigned type, int tokens, unsigned in_dim) {
   if (type != 12 || tokens < 1 || tokens > GEMV_MFMA_MAX_TOKENS || in_dim == 0 || (in_dim & 255u)) return 0;
-  return (unsigned)tokens * (in_dim >> 8) <= (unsigned)GEMV_MFMA_MAX_UNITS(tokens);
+  return (unsigned)tokens * (in_dim >> 8) <= (unsigned)GEMV_MFMA_MAX_UNITS(tokens) || (in_dim & 2047u) == 0;
 }
 // 16-row tiles per row group and the grid: aim at one workgroup per compute unit (256 of them)
 static inline unsigned gemv_mfma_tiles(int tokens, unsigned in_dim, unsigned out_dim) {
@@ -132,6 +138,9 @@ static inline unsigned gemv_mfma_grid(int tokens, unsigned in_dim, unsigned out_
 }
 static inline unsigned gemv_mfma_lds_bytes(int tokens, unsigned in_dim) {
   const int mp = tokens <= 1 ? 1 : (tokens <= 2 ? 2 : 4);
+  // (token, super-block) units the activation image holds: all of them, or one chunk per wavefront
+  const unsigned per_wave = (unsigned)(GEMV_MFMA_MAX_UNITS(tokens) / GEMV_MFMA_WAVES / tokens * tokens);
+  const unsigned units = gemv_mfma_chunked(tokens, in_dim) ? GEMV_MFMA_WAVES * per_wave : (unsigned)tokens * (in_dim >> 8);
   return 64u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * 1024u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * (unsigned)mp * 64u +
-         (unsigned)tokens * (in_dim >> 8) * (4u + 32u + 1024u);
+         units * (4u + 32u + 1024u);
 }

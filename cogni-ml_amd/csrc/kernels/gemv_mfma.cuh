@@ -55,13 +55,19 @@ __device__ __forceinline__ void wave_lds_fence() {
 
 // T: 16-row tiles per wavefront, compile-time so that the number of weight loads in flight is a constant and
 // a wait for the (older) activation loads never has to drain them.
-template <int M, bool ADD, int T>
+//
+// CHUNK: rows whose activations do not fit the staging buffer at once. With in_dim a multiple of 2048 the eight
+// wavefronts are eight k-slices and each stages and reads the activations of its own super-blocks only, so a wavefront
+// stages them C super-blocks at a time into a region of its own (no workgroup barrier), with the next chunk's
+// activations requested while the current one is consumed.
+template <int M, bool ADD, int T, bool CHUNK = false>
 __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float* x, const float* residual,
                                                    float* out, u32 in_dim, u32 out_dim) {
   constexpr int MP = M <= 1 ? 1 : (M <= 2 ? 2 : 4);   // token slots in the column index
   constexpr int ND = MP;                              // accumulator tiles per 16 rows and super-block
   constexpr int BB = 144;
   constexpr int NPRE = GEMV_MFMA_MAX_UNITS(M) / GEMV_MFMA_WAVES;   // staging units (token, super-block) per wavefront
+  constexpr int C = NPRE / M;                                      // CHUNK: super-blocks of a k-slice staged at a time
   extern __shared__ uint4 mf_lds4[];
   char* lds = reinterpret_cast<char*>(mf_lds4);
 
@@ -79,8 +85,13 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   const u32 off_tb = 64 + (u32)wave * (GEMV_MFMA_TMAX * 1024);
   const u32 off_part = 64 + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * 1024;
   const u32 off_fs = off_part + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * MP * 64;
-  const u32 off_sx = off_fs + (u32)M * nsb * 4;
-  const u32 off_x = off_sx + (u32)M * nsb * 32;
+  const u32 units_lds = CHUNK ? (u32)(GEMV_MFMA_WAVES * C * M) : (u32)M * nsb;   // units the LDS image has room for
+  const u32 off_sx = off_fs + units_lds * 4;
+  const u32 off_x = off_sx + units_lds * 32;
+  // place of super-block sb in the activation image, and of (token, super-block) in fs / sx: by super-block, or
+  // (CHUNK) by wavefront and position in the chunk
+  auto xslot = [&](u32 sb) -> u32 { return CHUNK ? (u32)wave * C + ((sb >> 3) % (u32)C) : sb; };
+  auto uidx = [&](u32 m, u32 sb) -> u32 { return CHUNK ? xslot(sb) * M + m : m * nsb + sb; };
   if (tid < 16) reinterpret_cast<u32*>(lds)[tid] = 0u;
 
   // ---- lane roles -------------------------------------------------------------------------------
@@ -117,15 +128,30 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   // barrier): the compute unit's memory pipeline returns loads in order, and the staging below, with the
   // barrier behind it, must not wait for weight bytes.
   const u32 nunits = (u32)M * nsb;
-  float4 xv[NPRE];
-#pragma unroll
-  for (int i = 0; i < NPRE; i++) {
-    const u32 p = (u32)wave + (u32)i * GEMV_MFMA_WAVES;   // wave-uniform
-    if (p < nunits) {
-      const u32 m = p / nsb, sb = p - m * nsb;
-      __builtin_memcpy(&xv[i], x + (size_t)m * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  // unit i of this wavefront (wave-uniform): whole rows: unit wave + 8 i of the M * nsb; CHUNK: token i / C,
+  // super-block i0 + i % C of the wavefront's k-slice
+  auto unit_of = [&](int i, u32 i0, u32& m, u32& sb) -> bool {
+    if constexpr (CHUNK) {
+      const u32 j = (u32)(i % C);
+      m = (u32)(i / C);
+      sb = kslice + 8u * (i0 + j);
+      return i < C * M && i0 + j < (nsb >> 3);
+    } else {
+      const u32 p = (u32)wave + (u32)i * GEMV_MFMA_WAVES;
+      m = p / nsb;
+      sb = p - m * nsb;
+      return p < nunits;
     }
-  }
+  };
+  float4 xv[NPRE];
+  auto load_xv = [&](u32 i0) {
+#pragma unroll
+    for (int i = 0; i < NPRE; i++) {
+      u32 m, sb;
+      if (unit_of(i, i0, m, sb)) __builtin_memcpy(&xv[i], x + (size_t)m * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+    }
+  };
+  load_xv(0);
   __builtin_amdgcn_sched_barrier(0);
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
@@ -136,11 +162,11 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   for (int t = 0; t < T; t++) acc[t] = (mf_float4){0.f, 0.f, 0.f, 0.f};
 
   // ---- stage the activations: one wavefront per (token, super-block) -----------------------------------
+  auto stage_xv = [&](u32 i0) {
 #pragma unroll
   for (int i = 0; i < NPRE; i++) {
-    const u32 p = (u32)wave + (u32)i * GEMV_MFMA_WAVES;
-    if (p < nunits) {
-      const u32 m = p / nsb, sb = p - m * nsb;
+    u32 m, sb;
+    if (unit_of(i, i0, m, sb)) {
       const float4 v = xv[i];
       // power of two that brings the largest magnitude of the super-block to [2^12, 2^13)
       float am = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
@@ -165,7 +191,7 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
       // k-slot order inside a run of 8 weights is 0,2,1,3,4,6,5,7 (how the nibble masks deliver them)
       typedef _Float16 h4 __attribute__((ext_vector_type(4)));
       const h4 hv = {h0, h2, h1, h3}, lv = {l0, l2, l1, l3};
-      char* img = lds + off_x + ((size_t)(sb * M + m) * 2) * 512 + 8 * lane;
+      char* img = lds + off_x + ((size_t)(xslot(sb) * M + m) * 2) * 512 + 8 * lane;
       *reinterpret_cast<h4*>(img) = hv;
       *reinterpret_cast<h4*>(img + 512) = lv;
       // sums of the 8 sub-blocks (8 lanes each) for the min term, unscaled
@@ -173,10 +199,12 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
       sm += MF_DPP(sm, MF_DPP_QUAD_1032);
       sm += MF_DPP(sm, MF_DPP_QUAD_2301);
       sm += MF_DPP(sm, MF_DPP_ROW_HALF_MIRROR);
-      if ((lane & 7) == 0) reinterpret_cast<float*>(lds + off_sx)[(m * nsb + sb) * 8 + (lane >> 3)] = sm;
-      if (lane == 0) reinterpret_cast<float*>(lds + off_fs)[m * nsb + sb] = inv;
+      if ((lane & 7) == 0) reinterpret_cast<float*>(lds + off_sx)[uidx(m, sb) * 8 + (lane >> 3)] = sm;
+      if (lane == 0) reinterpret_cast<float*>(lds + off_fs)[uidx(m, sb)] = inv;
     }
   }
+  };
+  stage_xv(0);
   // With all eight wavefronts in one row group and in_dim a multiple of 2048 the units a wavefront staged
   // are exactly the super-blocks of its own k-slice (unit p sits on wavefront p % 8 and covers super-block
   // p % nsb), so nobody has to wait for anybody; only the zeroed LDS words need the workgroup.
@@ -197,7 +225,7 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     // hh = kg % 2, par = t % 2, half = t / 2. Live iff the column's slot is the one of sub-block
     // s = 4 j + 2 (kg / 2) + par.
     uint4 breg[8];
-    const u32 ximg = off_x + ((sb * M + tok) * 2 + hl) * 512;
+    const u32 ximg = off_x + ((xslot(sb) * M + tok) * 2 + hl) * 512;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
 #pragma unroll
@@ -219,10 +247,10 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
       sxl[d] = 0.f;
     }
     if (col_live) {
-      fsc = reinterpret_cast<const float*>(lds + off_fs)[tok * nsb + sb];
+      fsc = reinterpret_cast<const float*>(lds + off_fs)[uidx(tok, sb)];
       if (hl == 0) {
 #pragma unroll
-        for (int d = 0; d < ND; d++) sxl[d] = reinterpret_cast<const float*>(lds + off_sx)[(tok * nsb + sb) * 8 + sd[d]];
+        for (int d = 0; d < ND; d++) sxl[d] = reinterpret_cast<const float*>(lds + off_sx)[uidx(tok, sb) * 8 + sd[d]];
       }
     }
     float* tb = reinterpret_cast<float*>(lds + off_tb);
@@ -295,10 +323,26 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     wave_lds_fence();
   };
 
-  {
+  if constexpr (!CHUNK) {
     u32 sb = kslice;
     for (; sb + NWK < nsb; sb += NWK) process(stA, sb, sb + NWK, mf_true{});
     process(stA, sb, 0, mf_false{});
+  } else {
+    const u32 nslice = nsb >> 3;   // super-blocks of a k-slice: kslice, kslice + 8, ...
+    for (u32 i0 = 0;;) {
+      const bool more = i0 + C < nslice;
+      if (more) load_xv(i0 + C);   // behind the weights in flight, ahead of the ones process() requests
+      const u32 iend = min(i0 + (u32)C, nslice);
+      for (u32 i = i0; i < iend; i++) {
+        const u32 sb = kslice + 8u * i;
+        if (i + 1 < nslice) process(stA, sb, sb + 8u, mf_true{});
+        else process(stA, sb, 0, mf_false{});
+      }
+      if (!more) break;
+      i0 += C;
+      stage_xv(i0);   // (process ends with a wavefront fence: the old chunk has been read)
+      wave_lds_fence();
+    }
   }
 
   // ---- add up the columns of a token inside the wavefront, then the k-slices through LDS ------------
@@ -346,6 +390,12 @@ __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const f
   const u32 nwr = GEMV_MFMA_WAVES >> lg;
   const u32 ntiles = (out_dim + 15) >> 4;
   const u32 t = (ntiles + gridDim.x * nwr - 1) / (gridDim.x * nwr);
+  if (gemv_mfma_chunked(M, in_dim)) {
+    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true>(w, x, residual, out, in_dim, out_dim);
+    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true>(w, x, residual, out, in_dim, out_dim);
+    else q4k_gemv_mfma_core<M, ADD, 3, true>(w, x, residual, out, in_dim, out_dim);
+    return;
+  }
   if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1>(w, x, residual, out, in_dim, out_dim);
   else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2>(w, x, residual, out, in_dim, out_dim);
   else q4k_gemv_mfma_core<M, ADD, 3>(w, x, residual, out, in_dim, out_dim);

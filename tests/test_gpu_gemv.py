@@ -187,21 +187,24 @@ def test_linearity_and_determinism_at_full_size(gpu):
     assert np.array_equal(swapped[out_dim:], both[:out_dim]) and np.array_equal(swapped[:out_dim], both[out_dim:])
 
 
-MFMA_SHAPES = [(256, 17), (512, 100), (768, 33), (1024, 3584), (2048, 48), (2304, 250), (4096, 1024), (8192, 300)]
+MFMA_SHAPES = [(256, 17), (512, 100), (768, 33), (1024, 3584), (2048, 48), (2304, 250), (4096, 1024), (8192, 300),
+               (6144, 40), (12288, 530), (16384, 64), (26624, 33), (8448, 20)]
 
 
 @pytest.mark.parametrize("in_dim,out_dim", MFMA_SHAPES)
 @pytest.mark.parametrize("tokens", [2, 3, 4, 7])
 def test_q4_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
-    """2..4 tokens of a Q4_K matrix run on the matrix cores where the activations fit the staging buffer:
-    odd row counts, every k-slice split (1, 2, 3, 4, 8, 9, 16, 32 super-blocks), with and without residual."""
+    """2..4 tokens of a Q4_K matrix run on the matrix cores where the activations fit the staging buffer or the row is
+    a multiple of 2048 values (staged a chunk at a time: whole chunks, a half-filled last chunk at 6144 and 26624, several
+    row tiles per wavefront): odd row counts, every k-slice split (1, 2, 3, 4, 8, 9, 16, 32 super-blocks), with and
+    without residual. 8448 values (33 super-blocks) are neither: three and four tokens stay on the vector ALU."""
     rng = np.random.default_rng(in_dim * 131 + out_dim * 7 + tokens)
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
     res = rng.standard_normal(tokens * out_dim).astype(np.float32)
     m = min(tokens, 4)
     name = quant.gemv_plan(Q4_K, m, in_dim, out_dim)[0]
-    expect_mfma = m * (in_dim // 256) <= (64 if m >= 3 else 96)
+    expect_mfma = m * (in_dim // 256) <= (64 if m >= 3 else 96) or in_dim % 2048 == 0
     assert ("mfma" in name) == expect_mfma, name
     check(oracle, raw, Q4_K, x, in_dim, out_dim, tokens, None, "%dx%d M=%d" % (in_dim, out_dim, tokens))
     check(oracle, raw, Q4_K, x, in_dim, out_dim, tokens, res, "%dx%d M=%d add" % (in_dim, out_dim, tokens))
