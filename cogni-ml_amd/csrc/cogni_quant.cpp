@@ -253,13 +253,15 @@ int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, ui
   if (!kernel || !grid_x || !block_x || !shared_mem_bytes || !gemv_type(type) || tokens < 1 ||
       tokens > COGNI_MAX_GEMV_TOKENS || in_dim == 0 || out_dim == 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_plan: bad argument");
-  // two to four tokens of a Q4_K matrix go to the matrix-core kernel; one token is faster on the vector ALU
+  // two to four tokens of a Q4_K matrix and three or four of a Q6_K matrix go to the matrix-core kernels; one token
+  // is faster on the vector ALU
   if (tokens >= 2 && gemv_mfma_supported(type, (int)tokens, in_dim)) {
-    std::snprintf(buf, sizeof buf, "q4_k_gemv_mfma_%sf32_tbatch%u", add ? "add_" : "", tokens);
+    std::snprintf(buf, sizeof buf, "q%c_k_gemv_mfma_%sf32_tbatch%u", type == COGNI_TYPE_Q6_K ? '6' : '4', add ? "add_" : "",
+                  tokens);
     *kernel = buf;
     *grid_x = gemv_mfma_grid((int)tokens, in_dim, out_dim);
     *block_x = GEMV_MFMA_WAVES * 64;
-    *shared_mem_bytes = gemv_mfma_lds_bytes((int)tokens, in_dim);
+    *shared_mem_bytes = gemv_mfma_lds_bytes(type, (int)tokens, in_dim);
     return 0;
   }
   *kernel = cogni_gemv_kernel_name(type, tokens, add);

@@ -4,6 +4,7 @@
 #include "kernels/dequant.cuh"
 #include "kernels/gemv.cuh"
 #include "kernels/gemv_mfma.cuh"
+#include "kernels/gemv_mfma_q6k.cuh"
 #include "kernels/gemm_q4k.cuh"
 #include "kernels/gemm_q6k.cuh"
 #include "kernels/norm.cuh"
@@ -15,3 +16,7 @@ GEMV_MFMA_ENTRY(q4_k_gemv_mfma_f32_tbatch4, 4)
 GEMV_MFMA_ADD_ENTRY(q4_k_gemv_mfma_add_f32_tbatch2, 2)
 GEMV_MFMA_ADD_ENTRY(q4_k_gemv_mfma_add_f32_tbatch3, 3)
 GEMV_MFMA_ADD_ENTRY(q4_k_gemv_mfma_add_f32_tbatch4, 4)
+GEMV_MFMA_Q6K_ENTRY(q6_k_gemv_mfma_f32_tbatch3, 3)
+GEMV_MFMA_Q6K_ENTRY(q6_k_gemv_mfma_f32_tbatch4, 4)
+GEMV_MFMA_Q6K_ADD_ENTRY(q6_k_gemv_mfma_add_f32_tbatch3, 3)
+GEMV_MFMA_Q6K_ADD_ENTRY(q6_k_gemv_mfma_add_f32_tbatch4, 4)

@@ -115,10 +115,13 @@ static inline GEMV_HD unsigned gemv_mfma_log2_kslices(unsigned nsb) {
 static inline GEMV_HD int gemv_mfma_chunked(int tokens, unsigned in_dim) {
   return (unsigned)tokens * (in_dim >> 8) > (unsigned)GEMV_MFMA_MAX_UNITS(tokens) && (in_dim & 2047u) == 0;
 }
-// Shapes the matrix-core kernel takes: Q4_K, 1..4 tokens, in_dim a multiple of 256, all activations staged at once
-// or in_dim a multiple of 2048.
+// Shapes the matrix-core kernels take: Q4_K with 1..4 tokens, Q6_K with 3 or 4 (its columns are laid out for four
+// tokens, and two are as fast on the vector ALU); in_dim a multiple of 256, all activations staged at once or in_dim a
+// multiple of 2048.
 static inline int gemv_mfma_supported(unsigned type, int tokens, unsigned in_dim) {
-  if (type != 12 || tokens < 1 || tokens > GEMV_MFMA_MAX_TOKENS || in_dim == 0 || (in_dim & 255u)) return 0;
+  if ((type != 12 && type != 14) || tokens < (type == 14 ? 3 : 1) || tokens > GEMV_MFMA_MAX_TOKENS || in_dim == 0 ||
+      (in_dim & 255u))
+    return 0;
   return (unsigned)tokens * (in_dim >> 8) <= (unsigned)GEMV_MFMA_MAX_UNITS(tokens) || (in_dim & 2047u) == 0;
 }
 // 16-row tiles per row group and the grid: aim at one workgroup per compute unit (256 of them)
@@ -136,11 +139,12 @@ static inline unsigned gemv_mfma_grid(int tokens, unsigned in_dim, unsigned out_
   const unsigned ntiles = (out_dim + 15) / 16, per_wg = nwr * gemv_mfma_tiles(tokens, in_dim, out_dim);
   return (ntiles + per_wg - 1) / per_wg;
 }
-static inline unsigned gemv_mfma_lds_bytes(int tokens, unsigned in_dim) {
-  const int mp = tokens <= 1 ? 1 : (tokens <= 2 ? 2 : 4);
+static inline unsigned gemv_mfma_lds_bytes(unsigned type, int tokens, unsigned in_dim) {
+  const int mp = type == 14 ? 4 : (tokens <= 1 ? 1 : (tokens <= 2 ? 2 : 4));
+  const unsigned nsums = type == 14 ? 16u : 8u;   // sub-block sums of the activations kept per (token, super-block)
   // (token, super-block) units the activation image holds: all of them, or one chunk per wavefront
   const unsigned per_wave = (unsigned)(GEMV_MFMA_MAX_UNITS(tokens) / GEMV_MFMA_WAVES / tokens * tokens);
   const unsigned units = gemv_mfma_chunked(tokens, in_dim) ? GEMV_MFMA_WAVES * per_wave : (unsigned)tokens * (in_dim >> 8);
   return 64u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * 1024u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * (unsigned)mp * 64u +
-         units * (4u + 32u + 1024u);
+         units * (4u + 4u * nsums + 1024u);
 }

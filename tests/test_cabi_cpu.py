@@ -112,7 +112,14 @@ def test_gemv_plan_picks_the_kernel_for_the_shape():
     # other row lengths that do not fit, other types, more tokens: the vector-ALU kernels
     assert quant.gemv_plan(12, 4, 8448, 4096)[0] == "q4_k_gemv_f32_tbatch4"
     assert quant.gemv_plan(12, 2, 12288, 4096)[0] == "q4_k_gemv_mfma_f32_tbatch2"
-    assert quant.gemv_plan(14, 4, 4096, 4096)[0] == "q6_k_gemv_f32_tbatch4"
+    # Q6_K: three and four tokens on the matrix cores (16 sub-block sums per staged super-block), two on the vector ALU
+    name, grid, block, lds = quant.gemv_plan(14, 4, 4096, 4096)
+    assert (name, grid, block) == ("q6_k_gemv_mfma_f32_tbatch4", 256, 512)
+    assert lds == 64 + 8 * 3 * 1024 + 8 * 3 * 4 * 64 + 64 * (4 + 64 + 1024)
+    assert quant.gemv_plan(14, 3, 12288, 4096, add=True)[0] == "q6_k_gemv_mfma_add_f32_tbatch3"
+    assert quant.gemv_plan(14, 2, 4096, 4096)[0] == "q6_k_gemv_f32_tbatch2"
+    assert quant.gemv_plan(14, 4, 8448, 4096)[0] == "q6_k_gemv_f32_tbatch4"
+    assert quant.gemv_plan(13, 4, 4096, 4096)[0] == "q5_k_gemv_f32_tbatch4"
     assert quant.gemv_plan(12, 8, 4096, 4096)[0] == "q4_k_gemv_f32_tbatch8"
     with pytest.raises(quant.QuantError):
         quant.gemv_plan(12, 9, 4096, 4096)

@@ -210,6 +210,53 @@ def test_q4_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
     check(oracle, raw, Q4_K, x, in_dim, out_dim, tokens, res, "%dx%d M=%d add" % (in_dim, out_dim, tokens))
 
 
+@pytest.mark.parametrize("in_dim,out_dim", MFMA_SHAPES)
+@pytest.mark.parametrize("tokens", [3, 4, 7])
+def test_q6_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
+    """Three and four tokens of a Q6_K matrix run on the matrix cores under the same shape rule as Q4_K (7 tokens:
+    a group of four and one of three); two tokens stay on the vector ALU. With and without residual."""
+    rng = np.random.default_rng(in_dim * 137 + out_dim * 11 + tokens)
+    raw = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = rng.standard_normal(tokens * out_dim).astype(np.float32)
+    m = min(tokens, 4)
+    name = quant.gemv_plan(Q6_K, m, in_dim, out_dim)[0]
+    expect_mfma = m * (in_dim // 256) <= 64 or in_dim % 2048 == 0
+    assert name == ("q6_k_gemv_mfma_f32_tbatch%d" % m if expect_mfma else "q6_k_gemv_f32_tbatch%d" % m), name
+    assert quant.gemv_plan(Q6_K, 2, in_dim, out_dim)[0] == "q6_k_gemv_f32_tbatch2"
+    check(oracle, raw, Q6_K, x, in_dim, out_dim, tokens, None, "%dx%d M=%d" % (in_dim, out_dim, tokens))
+    check(oracle, raw, Q6_K, x, in_dim, out_dim, tokens, res, "%dx%d M=%d add" % (in_dim, out_dim, tokens))
+
+
+def test_q6_k_matrix_core_kernel_element_order_and_ranges(gpu, oracle):
+    """One-hot activations pick single weights out of every position of a super-block (a wrong quadrant, nibble or
+    scale index shows as a wrong value, not as a small error); then activations far outside the binary16 range."""
+    rng = np.random.default_rng(78)
+    in_dim, out_dim, tokens = 512, 48, 4
+    raw = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    dense = oracle.dequantize(raw, Q6_K, out_dim * in_dim).reshape(out_dim, in_dim)
+    for base in range(0, in_dim, tokens):
+        x = np.zeros((tokens, in_dim), dtype=np.float32)
+        for m in range(tokens):
+            x[m, base + m] = 1.0
+        got = run_gemv(raw, Q6_K, np.ascontiguousarray(x.reshape(-1)), in_dim, out_dim, tokens).reshape(tokens, out_dim)
+        for m in range(tokens):
+            assert np.allclose(got[m], dense[:, base + m], rtol=0, atol=1e-5 * np.max(np.abs(dense))), (base, m)
+    in_dim, out_dim = 4096, 512
+    raw = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim).reshape(tokens, in_dim)
+    x[0] *= np.float32(1e-30)
+    x[1] *= np.float32(1e30)
+    x[2, :256] = 0.0
+    x[2, 700] = np.float32(3e7)
+    x[3] = np.where(rng.random(in_dim) < 0.5, x[3] * np.float32(1e-6), x[3] * np.float32(1e4)).astype(np.float32)
+    x = np.ascontiguousarray(x.reshape(-1))
+    got, want, frac = check(oracle, raw, Q6_K, x, in_dim, out_dim, tokens, None, "activation ranges")
+    g, w_ = got.reshape(tokens, out_dim).astype(np.float64), want.reshape(tokens, out_dim)
+    for m in range(tokens):
+        assert np.max(np.abs(g[m] - w_[m])) <= 2e-5 * np.max(np.abs(w_[m])), m
+
+
 def test_q4_k_matrix_core_kernel_activation_ranges(gpu, oracle):
     """The matrix-core kernel feeds the activations as binary16 pairs scaled per token and super-block: values
     far outside the binary16 range, zeros and mixed magnitudes must come out as from fp32 arithmetic."""

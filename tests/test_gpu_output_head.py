@@ -90,7 +90,10 @@ def test_output_head_runner(gpu, oracle):
             assert runner.top1_ids[tok] == first_max(logits)
             assert abs(runner.top1_values[tok] - logits.max()) <= 1e-4 * np.abs(logits).max()
             dev = runner.logits[tok * vocab:(tok + 1) * vocab]
-            assert runner.top1_ids[tok] == first_max(dev) and runner.top1_values[tok] == dev.max()
+            # (the logits of a group of four tokens come from the matrix-core kernel, the top-1 from the vector-ALU
+            # one: the same sums in a different order)
+            slack = 2e-5 * np.abs(dev).max()
+            assert abs(runner.top1_values[tok] - dev.max()) <= slack and dev[runner.top1_ids[tok]] >= dev.max() - slack
         # token-local path gives the same ids
         grouped = runner.top1_ids.copy()
         for tok in range(tokens):
