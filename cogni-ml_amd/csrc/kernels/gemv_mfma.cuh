@@ -39,6 +39,7 @@ struct mf_true { static constexpr bool value = true; };
 struct mf_false { static constexpr bool value = false; };
 
 #define MF_DPP(v, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (v)), (ctrl), 0xF, 0xF, false))
+#define MF_DPP_U(v, ctrl) ((u32)__builtin_amdgcn_update_dpp(0, (int)(v), (ctrl), 0xF, 0xF, false))
 #define MF_DPP_QUAD_1032 0xB1
 #define MF_DPP_QUAD_2301 0x4E
 #define MF_DPP_ROW_ROR4 0x124
@@ -169,17 +170,16 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     if (unit_of(i, i0, m, sb)) {
       const float4 v = xv[i];
       // power of two that brings the largest magnitude of the super-block to [2^12, 2^13)
-      float am = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-      am = fmaxf(am, MF_DPP(am, MF_DPP_QUAD_1032));
-      am = fmaxf(am, MF_DPP(am, MF_DPP_QUAD_2301));
-      am = fmaxf(am, MF_DPP(am, MF_DPP_ROW_ROR4));
-      am = fmaxf(am, MF_DPP(am, MF_DPP_ROW_ROR8));
-      const int ai = __builtin_bit_cast(int, am);
-      const float am4 = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 0)),
-                                    __builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 16))),
-                              fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 32)),
-                                    __builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 48))));
-      const int e = (int)((__builtin_bit_cast(u32, am4) >> 23) & 0xFFu);
+      // (unsigned maximum of the bit patterns without sign: orders magnitudes like the floats, and its DPP steps are
+      // single instructions)
+      u32 ab = __builtin_bit_cast(u32, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+      ab = max(ab, MF_DPP_U(ab, MF_DPP_QUAD_1032));
+      ab = max(ab, MF_DPP_U(ab, MF_DPP_QUAD_2301));
+      ab = max(ab, MF_DPP_U(ab, MF_DPP_ROW_ROR4));
+      ab = max(ab, MF_DPP_U(ab, MF_DPP_ROW_ROR8));
+      const u32 ab4 = max(max((u32)__builtin_amdgcn_readlane((int)ab, 0), (u32)__builtin_amdgcn_readlane((int)ab, 16)),
+                          max((u32)__builtin_amdgcn_readlane((int)ab, 32), (u32)__builtin_amdgcn_readlane((int)ab, 48)));
+      const int e = (int)((ab4 >> 23) & 0xFFu);
       int sh = 139 - e;                      // scale = 2^sh
       sh = sh > 100 ? 100 : sh;              // zeros / tiny values: keep 2^-sh a normal number
       const float scale = __builtin_bit_cast(float, (u32)(127 + sh) << 23);
@@ -199,8 +199,9 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
       sm += MF_DPP(sm, MF_DPP_QUAD_1032);
       sm += MF_DPP(sm, MF_DPP_QUAD_2301);
       sm += MF_DPP(sm, MF_DPP_ROW_HALF_MIRROR);
-      if ((lane & 7) == 0) reinterpret_cast<float*>(lds + off_sx)[uidx(m, sb) * 8 + (lane >> 3)] = sm;
-      if (lane == 0) reinterpret_cast<float*>(lds + off_fs)[uidx(m, sb)] = inv;
+      // (every lane of a group holds the group's sum, every lane the scale: stored by all of them, no lane masks)
+      reinterpret_cast<float*>(lds + off_sx)[uidx(m, sb) * 8 + (lane >> 3)] = sm;
+      reinterpret_cast<float*>(lds + off_fs)[uidx(m, sb)] = inv;
     }
   }
   };

@@ -132,17 +132,16 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
       if (unit_of(i, i0, m, sb)) {
         const float4 v = xv[i];
         // power of two that brings the largest magnitude of the super-block to [2^12, 2^13)
-        float am = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        am = fmaxf(am, MF_DPP(am, MF_DPP_QUAD_1032));
-        am = fmaxf(am, MF_DPP(am, MF_DPP_QUAD_2301));
-        am = fmaxf(am, MF_DPP(am, MF_DPP_ROW_ROR4));
-        am = fmaxf(am, MF_DPP(am, MF_DPP_ROW_ROR8));
-        const int ai = __builtin_bit_cast(int, am);
-        const float am4 = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 0)),
-                                      __builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 16))),
-                                fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 32)),
-                                      __builtin_bit_cast(float, __builtin_amdgcn_readlane(ai, 48))));
-        const int e = (int)((__builtin_bit_cast(u32, am4) >> 23) & 0xFFu);
+        // (unsigned maximum of the bit patterns without sign: orders magnitudes like the floats, and its DPP steps are
+        // single instructions)
+        u32 ab = __builtin_bit_cast(u32, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        ab = max(ab, MF_DPP_U(ab, MF_DPP_QUAD_1032));
+        ab = max(ab, MF_DPP_U(ab, MF_DPP_QUAD_2301));
+        ab = max(ab, MF_DPP_U(ab, MF_DPP_ROW_ROR4));
+        ab = max(ab, MF_DPP_U(ab, MF_DPP_ROW_ROR8));
+        const u32 ab4 = max(max((u32)__builtin_amdgcn_readlane((int)ab, 0), (u32)__builtin_amdgcn_readlane((int)ab, 16)),
+                            max((u32)__builtin_amdgcn_readlane((int)ab, 32), (u32)__builtin_amdgcn_readlane((int)ab, 48)));
+        const int e = (int)((ab4 >> 23) & 0xFFu);
         int sh = 139 - e;                      // scale = 2^sh
         sh = sh > 100 ? 100 : sh;              // zeros / tiny values: keep 2^-sh a normal number
         const float scale = __builtin_bit_cast(float, (u32)(127 + sh) << 23);
@@ -161,8 +160,9 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
         float sm = (v.x + v.y) + (v.z + v.w);
         sm += MF_DPP(sm, MF_DPP_QUAD_1032);
         sm += MF_DPP(sm, MF_DPP_QUAD_2301);
-        if ((lane & 3) == 0) reinterpret_cast<float*>(lds + off_sx)[uidx(m, sb) * 16 + (lane >> 2)] = sm;
-        if (lane == 0) reinterpret_cast<float*>(lds + off_fs)[uidx(m, sb)] = inv;
+        // (every lane of a quad holds the quad's sum, every lane the scale: stored by all of them, no lane masks)
+        reinterpret_cast<float*>(lds + off_sx)[uidx(m, sb) * 16 + (lane >> 2)] = sm;
+        reinterpret_cast<float*>(lds + off_fs)[uidx(m, sb)] = inv;
       }
     }
   };
@@ -226,18 +226,22 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
       mf_float4 dacc[8];
 #pragma unroll
       for (int na = 0; na < 4; na++) {
+        // The two qh bits of a code go to bits 4, 5 of its 16-bit half (beside a low nibble) or 8, 9 (above a high
+        // nibble left in place). For bytes 0 and 2 of a dword that is one left shift by 4 - hshift, for bytes 1 and 3
+        // one right shift by 4 + hshift; the masks pick the quadrant's pair out of either.
         const uint2 q = st[t].ql[na];
-        const u32 ha = st[t].qh[na].x >> hshift, hb2 = st[t].qh[na].y >> hshift;
-        const u32 qa8 = q.x >> 8, qb8 = q.y >> 8, ha8 = ha >> 8, hb8 = hb2 >> 8;
+        const u32 hax = st[t].qh[na].x << (4 - hshift), hay = st[t].qh[na].x >> (4 + hshift);
+        const u32 hbx = st[t].qh[na].y << (4 - hshift), hby = st[t].qh[na].y >> (4 + hshift);
+        const u32 qa8 = q.x >> 8, qb8 = q.y >> 8;
         uint4 lo, hi;
-        lo.x = (q.x & 0x000F000Fu) | ((ha & 0x00030003u) << 4);
-        lo.y = (qa8 & 0x000F000Fu) | ((ha8 & 0x00030003u) << 4);
-        lo.z = (q.y & 0x000F000Fu) | ((hb2 & 0x00030003u) << 4);
-        lo.w = (qb8 & 0x000F000Fu) | ((hb8 & 0x00030003u) << 4);
-        hi.x = (q.x & 0x00F000F0u) | ((ha << 4) & 0x03000300u);
-        hi.y = (qa8 & 0x00F000F0u) | ((ha8 << 4) & 0x03000300u);
-        hi.z = (q.y & 0x00F000F0u) | ((hb2 << 4) & 0x03000300u);
-        hi.w = (qb8 & 0x00F000F0u) | ((hb8 << 4) & 0x03000300u);
+        lo.x = (q.x & 0x000F000Fu) | (hax & 0x00300030u);
+        lo.y = (qa8 & 0x000F000Fu) | (hay & 0x00300030u);
+        lo.z = (q.y & 0x000F000Fu) | (hbx & 0x00300030u);
+        lo.w = (qb8 & 0x000F000Fu) | (hby & 0x00300030u);
+        hi.x = (q.x & 0x00F000F0u) | (hax & 0x03000300u);
+        hi.y = (qa8 & 0x00F000F0u) | (hay & 0x03000300u);
+        hi.z = (q.y & 0x00F000F0u) | (hbx & 0x03000300u);
+        hi.w = (qb8 & 0x00F000F0u) | (hby & 0x03000300u);
         const mf_float4 zero = (mf_float4){0.f, 0.f, 0.f, 0.f};
         dacc[2 * na] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mf_half8, lo),
                                                               __builtin_bit_cast(mf_half8, breg[2 * na]), zero, 0, 0, 0);
@@ -263,14 +267,10 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
         const u32 s = 8 * n + 4 * lohi + 2 * slot + a;
         const float4 sv = *reinterpret_cast<const float4*>(tb + t * 256 + s * 16 + 4 * rg);
         const float f = lohi ? fsc20 : fsc24;
-        acc[t][0] = fmaf(f, sv.x * dacc[q][0], acc[t][0]);
-        acc[t][1] = fmaf(f, sv.y * dacc[q][1], acc[t][1]);
-        acc[t][2] = fmaf(f, sv.z * dacc[q][2], acc[t][2]);
-        acc[t][3] = fmaf(f, sv.w * dacc[q][3], acc[t][3]);
-        acc[t][0] = fmaf(sv.x, m32sx[q], acc[t][0]);
-        acc[t][1] = fmaf(sv.y, m32sx[q], acc[t][1]);
-        acc[t][2] = fmaf(sv.z, m32sx[q], acc[t][2]);
-        acc[t][3] = fmaf(sv.w, m32sx[q], acc[t][3]);
+        acc[t][0] = fmaf(sv.x, fmaf(f, dacc[q][0], m32sx[q]), acc[t][0]);   // d sc (2^-e sum(code x) - 32 sum(x))
+        acc[t][1] = fmaf(sv.y, fmaf(f, dacc[q][1], m32sx[q]), acc[t][1]);
+        acc[t][2] = fmaf(sv.z, fmaf(f, dacc[q][2], m32sx[q]), acc[t][2]);
+        acc[t][3] = fmaf(sv.w, fmaf(f, dacc[q][3], m32sx[q]), acc[t][3]);
       }
     }
     wave_lds_fence();
