@@ -88,9 +88,6 @@ class GemvCase:
 def time_steps(hip, stream, launch, steps, warmup, graph=True):
     """Run `warmup` untimed and exactly `steps` timed launches on `stream`; returns ms for the timed region.
     The timed launches are captured into one HIP graph so host launch latency does not gate the GPU."""
-    for i in range(warmup):
-        launch(i, stream)
-    stream.synchronize()
     graph_wanted = bool(graph)
     graph, exe = None, None
     try:
@@ -107,6 +104,10 @@ def time_steps(hip, stream, launch, steps, warmup, graph=True):
         if graph_wanted:
             log("graph capture failed (%s); timing direct launches" % e)
         graph, exe = None, None
+    # the warm-up runs once the graph is built, directly ahead of the timed region: capture and instantiation are
+    # host work during which the GPU would otherwise sit idle and drop its clocks
+    for i in range(warmup):
+        launch(i, stream)
     e0, e1 = hip.Event(), hip.Event()
     hip.synchronize()
     e0.record(stream)
