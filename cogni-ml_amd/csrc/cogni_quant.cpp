@@ -485,7 +485,7 @@ int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, u
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 191) / 192;
   {
     void* params[] = {&x, &workspace, &tokens, &in_dim};
-    int rc = launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_f16_q6k" : "pack_x_f16_q4k", mtiles * 4 * (in_dim / 256), 256, 0, params, stream);
+    int rc = launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_f16_q6k" : "pack_x_f16_q4k", mtiles * 16 * (in_dim / 256), 256, 0, params, stream);   // 8 tokens x one super-block per workgroup
     if (rc != 0) return rc;
   }
   // a workspace that holds the packed activations only: one workgroup per tile walks the whole row

@@ -5,7 +5,7 @@
 // the rate of 16x16x32 (about 32 vs 2 x 32 clocks for the same 32768 flops per SIMD), hence the tile shape.
 //
 // Kernels:
-//   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 4 * in_dim/256
+//   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 16 * in_dim/256
 //   q4_k_gemm_f16, q5_k_gemm_f16
 //                   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
 //                   block 256, grid (8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), k splits), no dynamic LDS
@@ -59,10 +59,13 @@ __device__ __forceinline__ u32 gemm_k_element(u32 ks, u32 kg, u32 e) {
   return 64 * g + 32 * (op >> 1) + 16 * h + 8 * (op & 1) + perm;
 }
 
-// One workgroup packs 32 tokens x one super-block (256 k): the fp32 rows are read 1 KiB at a time (a wavefront
+// One workgroup packs 8 tokens x one super-block (256 k): the fp32 rows are read 1 KiB at a time (a wavefront
 // per row), converted, transposed through LDS into the [k-step][k-group][token][8 halves] image and written out
-// as 32 runs of 512 contiguous bytes. Grid: ceil(m/128) * 4 * (in_dim/256) workgroups, x fastest.
-#define PACK_TOK 32
+// as 32 runs of 128 contiguous bytes. Grid: ceil(m/128) * 16 * (in_dim/256) workgroups, x fastest (1024 workgroups at
+// 512 tokens x 4096: with 32 tokens per workgroup there were 256, one per compute unit, and the kernel was all latency).
+#ifndef PACK_TOK
+#define PACK_TOK 8
+#endif
 // Q6: the element order of the Q6_K kernel (gemm_q6k.cuh) instead of the Q4_K one.
 template <bool Q6>
 __device__ __forceinline__ void pack_x_core(const float* __restrict__ x, uint4* __restrict__ xp, u32 m, u32 in_dim) {
@@ -71,7 +74,8 @@ __device__ __forceinline__ void pack_x_core(const float* __restrict__ x, uint4* 
   __shared__ uint2 img[32 * (PACK_TOK + 1) * 2];
   const u32 nkb = in_dim >> 8;
   const u32 tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const u32 kb = blockIdx.x % nkb, tq = (blockIdx.x / nkb) & 3, mt = blockIdx.x / (4 * nkb);
+  constexpr u32 NQ = GEMM_BM / PACK_TOK;
+  const u32 kb = blockIdx.x % nkb, tq = (blockIdx.x / nkb) % NQ, mt = blockIdx.x / (NQ * nkb);
   // lane -> 4 consecutive k = 4 lane .. 4 lane + 3 of the super-block; their place in the image (inverse of
   // gemm_k_element): Q4_K: group g = k / 64, high-nibble half, 16-byte half h, upper-8-bytes bit, slot 0 or 4;
   // Q6_K: 128-half n, quadrant qd, 16-run u, upper-8 bit, slot 0 or 4 (gemm_k_element_q6k)

@@ -3,7 +3,7 @@
 // rows per workgroup, 4 wavefronts = 2 row halves x 2 k-step halves, v_mfma_f32_32x32x16_f16 with fp32 accumulation,
 // x as fp16 in LDS (two 64 KiB buffers filled by global_load_lds_dwordx4). What differs is the weight side:
 //
-//   pack_x_f16_q6k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 4 * in_dim/256
+//   pack_x_f16_q6k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 16 * in_dim/256
 //   q6_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
 //                   block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), no dynamic LDS (128 KiB static)
 //

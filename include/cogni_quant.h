@@ -185,7 +185,7 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
  * Kernels: pack_x_f16_q4k (Q4_K and Q5_K) | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
  *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,
  *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/192)/8), no dynamic shared memory.
- * (pack_x_f16_*: block 256, grid ceil(tokens/128)*4*(in_dim/256).) Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
+ * (pack_x_f16_*: block 256, grid ceil(tokens/128)*16*(in_dim/256).) Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 /* The workspace size with which cogni_gemm_dev may also split the k range: a launch with fewer than 128 tiles of
  * 128 tokens x 192 rows (few tokens, or a short out_dim such as the 12288 -> 4096 down projection) would leave most
