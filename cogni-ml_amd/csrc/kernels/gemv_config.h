@@ -137,7 +137,11 @@ static inline unsigned gemv_mfma_tiles(int tokens, unsigned in_dim, unsigned out
 static inline unsigned gemv_mfma_grid(int tokens, unsigned in_dim, unsigned out_dim) {
   const unsigned nwr = GEMV_MFMA_WAVES >> gemv_mfma_log2_kslices(in_dim >> 8);
   const unsigned ntiles = (out_dim + 15) / 16, per_wg = nwr * gemv_mfma_tiles(tokens, in_dim, out_dim);
-  return (ntiles + per_wg - 1) / per_wg;
+  const unsigned groups = (ntiles + per_wg - 1) / per_wg;
+  // more row groups of the largest size than compute units: one workgroup per unit walks them with the activations
+  // staged once (not where the activations are staged in chunks)
+  if (groups > 256u && per_wg == nwr * (unsigned)GEMV_MFMA_TMAX && !gemv_mfma_chunked(tokens, in_dim)) return 256u;
+  return groups;
 }
 static inline unsigned gemv_mfma_lds_bytes(unsigned type, int tokens, unsigned in_dim) {
   const int mp = type == 14 ? 4 : (tokens <= 1 ? 1 : (tokens <= 2 ? 2 : 4));

@@ -79,7 +79,10 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   const u32 NWK = 1u << lg_nwk, NWR = GEMV_MFMA_WAVES >> lg_nwk;
   const u32 kslice = wave & (NWK - 1), rgrp = wave >> lg_nwk;
   const u32 ntiles = (out_dim + 15) >> 4;
-  const u32 tile0 = (blockIdx.x * NWR + rgrp) * T;
+  // A workgroup takes the row groups (NWR * T tiles each) blockIdx.x, blockIdx.x + gridDim.x, ... with the activations
+  // staged once: a matrix with more groups than compute units (an output head) is launched as one workgroup per unit.
+  const u32 ngroups = (ntiles + NWR * T - 1) / (NWR * T);
+  u32 grp = blockIdx.x;
 
   // LDS map (gemv_mfma_lds_bytes): zero[64] | handover[waves][TMAX][2][8][16] f32 | partial[waves][TMAX][MP][16] f32
   //                                | fs[M][nsb] f32 | sx[M][nsb][8] f32 | ximg[nsb][M][2][256] f16
@@ -108,11 +111,15 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   // weight rows of this lane, one per tile
   const size_t row_bytes = (size_t)nsb * BB;
   const uint8_t* rowp[T];
+  auto set_rows = [&](u32 g) {
+    const u32 tile0 = (g * NWR + rgrp) * T;
 #pragma unroll
-  for (int t = 0; t < T; t++) {
-    const u32 tile = min(tile0 + (u32)t, ntiles - 1);
-    rowp[t] = w + (size_t)min(tile * 16 + ar, out_dim - 1) * row_bytes;
-  }
+    for (int t = 0; t < T; t++) {
+      const u32 tile = min(tile0 + (u32)t, ntiles - 1);
+      rowp[t] = w + (size_t)min(tile * 16 + ar, out_dim - 1) * row_bytes;
+    }
+  };
+  set_rows(grp);
 
   struct Stage { uint4 hdr, q0, q1; };
   Stage stA[T];
@@ -159,8 +166,6 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   load_sb(stA, kslice);
 
   mf_float4 acc[T];
-#pragma unroll
-  for (int t = 0; t < T; t++) acc[t] = (mf_float4){0.f, 0.f, 0.f, 0.f};
 
   // ---- stage the activations: one wavefront per (token, super-block) -----------------------------------
   auto stage_xv = [&](u32 i0) {
@@ -324,6 +329,9 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     wave_lds_fence();
   };
 
+  for (;;) {
+#pragma unroll
+  for (int t = 0; t < T; t++) acc[t] = (mf_float4){0.f, 0.f, 0.f, 0.f};
   if constexpr (!CHUNK) {
     u32 sb = kslice;
     for (; sb + NWK < nsb; sb += NWK) process(stA, sb, sb + NWK, mf_true{});
@@ -346,6 +354,13 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     }
   }
 
+  // the first super-block of the next row group is requested ahead of the reduction (the stage is free)
+  const u32 next = grp + gridDim.x;
+  const bool walk = !CHUNK && next < ngroups;   // (rows staged in chunks: one group per workgroup)
+  if (walk) {
+    set_rows(next);
+    load_sb(stA, kslice);
+  }
   // ---- add up the columns of a token inside the wavefront, then the k-slices through LDS ------------
 #pragma unroll
   for (int t = 0; t < T; t++) {
@@ -371,12 +386,16 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     const u32 r = o & 15, m = (o >> 4) % M, tt = (o / (16 * M)) % T, rgp = o / (16 * M * T);
     float v = 0.f;
     for (u32 k = 0; k < NWK; k++) v += part[(((rgp << lg_nwk) + k) * GEMV_MFMA_TMAX + tt) * MP * 16 + m * 16 + r];
-    const u32 row = ((blockIdx.x * NWR + rgp) * T + tt) * 16 + r;
+    const u32 row = ((grp * NWR + rgp) * T + tt) * 16 + r;
     if (row < out_dim) {
       const size_t oi = (size_t)m * out_dim + row;
       if (ADD) v += residual[oi];
       out[oi] = v;
     }
+  }
+  if (!walk) break;
+  grp = next;
+  __syncthreads();   // every partial sum has been read
   }
 }
 

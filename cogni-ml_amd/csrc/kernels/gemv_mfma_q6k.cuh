@@ -40,7 +40,10 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
   const u32 NWK = 1u << lg_nwk, NWR = GEMV_MFMA_WAVES >> lg_nwk;
   const u32 kslice = wave & (NWK - 1), rgrp = wave >> lg_nwk;
   const u32 ntiles = (out_dim + 15) >> 4;
-  const u32 tile0 = (blockIdx.x * NWR + rgrp) * T;
+  // A workgroup takes the row groups (NWR * T tiles each) blockIdx.x, blockIdx.x + gridDim.x, ... with the activations
+  // staged once: a matrix with more groups than compute units (an output head) is launched as one workgroup per unit.
+  const u32 ngroups = (ntiles + NWR * T - 1) / (NWR * T);
+  u32 grp = blockIdx.x;
 
   // LDS map (gemv_mfma_lds_bytes): zero[64] | handover[waves][TMAX][16 sub-blocks][16 rows] f32
   //                                | partial[waves][TMAX][MP][16] f32 | fs[units] f32 | sx[units][16] f32
@@ -67,11 +70,15 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
 
   const size_t row_bytes = (size_t)nsb * BB;
   const uint8_t* rowp[T];
+  auto set_rows = [&](u32 g) {
+    const u32 tile0 = (g * NWR + rgrp) * T;
 #pragma unroll
-  for (int t = 0; t < T; t++) {
-    const u32 tile = min(tile0 + (u32)t, ntiles - 1);
-    rowp[t] = w + (size_t)min(tile * 16 + ar, out_dim - 1) * row_bytes;
-  }
+    for (int t = 0; t < T; t++) {
+      const u32 tile = min(tile0 + (u32)t, ntiles - 1);
+      rowp[t] = w + (size_t)min(tile * 16 + ar, out_dim - 1) * row_bytes;
+    }
+  };
+  set_rows(grp);
 
   // per tile and super-block: four 8-byte pieces of ql and of qh (half n, l range a), the lane's four scale bytes, d
   struct Stage { uint2 ql[4], qh[4]; u32 sc, d; };
@@ -121,8 +128,6 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
   load_sb(stA, kslice);
 
   mf_float4 acc[T];
-#pragma unroll
-  for (int t = 0; t < T; t++) acc[t] = (mf_float4){0.f, 0.f, 0.f, 0.f};
 
   // ---- stage the activations: one wavefront per (token, super-block) -----------------------------------
   auto stage_xv = [&](u32 i0) {
@@ -222,8 +227,20 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
     wave_lds_fence();
 #pragma unroll
     for (int t = 0; t < T; t++) {
-      // (b) the 8 MFMAs of the tile, each into its own accumulator tile
-      mf_float4 dacc[8];
+      // (b) the 8 MFMAs of the tile, each into its own accumulator tile; (c) a pair is folded into the row sums while
+      // the next pair is in the matrix cores (two pairs of accumulator tiles live, not four): rows 4 rg .. 4 rg + 3 of
+      // the column's sub-block s = 8 n + 4 lohi + 2 slot + a
+      auto fold = [&](int q, const mf_float4& dq) {
+        const u32 n = q >> 2, a = (q >> 1) & 1, lohi = q & 1;
+        const u32 s = 8 * n + 4 * lohi + 2 * slot + a;
+        const float4 sv = *reinterpret_cast<const float4*>(tb + t * 256 + s * 16 + 4 * rg);
+        const float f = lohi ? fsc20 : fsc24;
+        acc[t][0] = fmaf(sv.x, fmaf(f, dq[0], m32sx[q]), acc[t][0]);   // d sc (2^-e sum(code x) - 32 sum(x))
+        acc[t][1] = fmaf(sv.y, fmaf(f, dq[1], m32sx[q]), acc[t][1]);
+        acc[t][2] = fmaf(sv.z, fmaf(f, dq[2], m32sx[q]), acc[t][2]);
+        acc[t][3] = fmaf(sv.w, fmaf(f, dq[3], m32sx[q]), acc[t][3]);
+      };
+      mf_float4 dp0 = (mf_float4){0.f, 0.f, 0.f, 0.f}, dp1 = dp0;
 #pragma unroll
       for (int na = 0; na < 4; na++) {
         // The two qh bits of a code go to bits 4, 5 of its 16-bit half (beside a low nibble) or 8, 9 (above a high
@@ -243,10 +260,16 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
         hi.z = (q.y & 0x00F000F0u) | (hbx & 0x03000300u);
         hi.w = (qb8 & 0x00F000F0u) | (hby & 0x03000300u);
         const mf_float4 zero = (mf_float4){0.f, 0.f, 0.f, 0.f};
-        dacc[2 * na] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mf_half8, lo),
-                                                              __builtin_bit_cast(mf_half8, breg[2 * na]), zero, 0, 0, 0);
-        dacc[2 * na + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mf_half8, hi),
-                                                                  __builtin_bit_cast(mf_half8, breg[2 * na + 1]), zero, 0, 0, 0);
+        const mf_float4 d0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mf_half8, lo),
+                                                                    __builtin_bit_cast(mf_half8, breg[2 * na]), zero, 0, 0, 0);
+        const mf_float4 d1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mf_half8, hi),
+                                                                    __builtin_bit_cast(mf_half8, breg[2 * na + 1]), zero, 0, 0, 0);
+        if (na > 0) {
+          fold(2 * na - 2, dp0);
+          fold(2 * na - 1, dp1);
+        }
+        dp0 = d0;
+        dp1 = d1;
       }
       if constexpr (decltype(refill)::value) {
         // this tile's stage is free: request its next super-block
@@ -260,22 +283,15 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
         st[t].sc = ld4(rowp[t] + (off + 192 + 4 * kg));
         st[t].d = ld2(rowp[t] + (off + 208));
       }
-      // (c) fold: rows 4 rg .. 4 rg + 3 of the column's sub-block s = 8 n + 4 lohi + 2 slot + a
-#pragma unroll
-      for (int q = 0; q < 8; q++) {
-        const u32 n = q >> 2, a = (q >> 1) & 1, lohi = q & 1;
-        const u32 s = 8 * n + 4 * lohi + 2 * slot + a;
-        const float4 sv = *reinterpret_cast<const float4*>(tb + t * 256 + s * 16 + 4 * rg);
-        const float f = lohi ? fsc20 : fsc24;
-        acc[t][0] = fmaf(sv.x, fmaf(f, dacc[q][0], m32sx[q]), acc[t][0]);   // d sc (2^-e sum(code x) - 32 sum(x))
-        acc[t][1] = fmaf(sv.y, fmaf(f, dacc[q][1], m32sx[q]), acc[t][1]);
-        acc[t][2] = fmaf(sv.z, fmaf(f, dacc[q][2], m32sx[q]), acc[t][2]);
-        acc[t][3] = fmaf(sv.w, fmaf(f, dacc[q][3], m32sx[q]), acc[t][3]);
-      }
+      fold(6, dp0);
+      fold(7, dp1);
     }
     wave_lds_fence();
   };
 
+  for (;;) {
+#pragma unroll
+  for (int t = 0; t < T; t++) acc[t] = (mf_float4){0.f, 0.f, 0.f, 0.f};
   if constexpr (!CHUNK) {
     u32 sb = kslice;
     for (; sb + NWK < nsb; sb += NWK) process(stA, sb, sb + NWK, mf_true{});
@@ -298,6 +314,8 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
     }
   }
 
+  const u32 next = grp + gridDim.x;
+  const bool walk = !CHUNK && next < ngroups;   // (rows staged in chunks: one group per workgroup)
   // ---- add up the columns of a token inside the wavefront, then the k-slices through LDS ------------
 #pragma unroll
   for (int t = 0; t < T; t++) {
@@ -321,12 +339,18 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
     const u32 r = o & 15, m = (o >> 4) % M, tt = (o / (16 * M)) % T, rgp = o / (16 * M * T);
     float v = 0.f;
     for (u32 k = 0; k < NWK; k++) v += part[(((rgp << lg_nwk) + k) * GEMV_MFMA_TMAX + tt) * MP * 16 + m * 16 + r];
-    const u32 row = ((blockIdx.x * NWR + rgp) * T + tt) * 16 + r;
+    const u32 row = ((grp * NWR + rgp) * T + tt) * 16 + r;
     if (row < out_dim) {
       const size_t oi = (size_t)m * out_dim + row;
       if (ADD) v += residual[oi];
       out[oi] = v;
     }
+  }
+  if (!walk) break;
+  grp = next;
+  set_rows(grp);
+  load_sb(stA, kslice);
+  __syncthreads();   // every partial sum has been read
   }
 }
 

@@ -103,6 +103,8 @@ def test_gemv_plan_picks_the_kernel_for_the_shape():
     assert lds == 64 + 8 * 3 * 1024 + 8 * 3 * 4 * 64 + 4 * 16 * (4 + 32 + 1024)
     assert quant.gemv_plan(12, 2, 4096, 12288, add=True)[0] == "q4_k_gemv_mfma_add_f32_tbatch2"
     assert quant.gemv_plan(12, 2, 4096, 4096)[1] == 256 and quant.gemv_plan(12, 2, 1024, 3584)[1] == 112
+    # more groups of 48 rows than compute units: 256 workgroups walk them (9496 tiles of the 151936-row head)
+    assert quant.gemv_plan(14, 4, 4096, 151936)[1] == 256 and quant.gemv_plan(12, 4, 4096, 12288 + 48)[1] == 256
     # rows of a multiple of 2048 values whose activations do not fit the staging buffer: staged a chunk at a time,
     # 8 wavefronts x 2 super-blocks x 4 tokens of LDS image
     name, grid, block, lds = quant.gemv_plan(12, 4, 12288, 4096)

@@ -188,7 +188,7 @@ def test_linearity_and_determinism_at_full_size(gpu):
 
 
 MFMA_SHAPES = [(256, 17), (512, 100), (768, 33), (1024, 3584), (2048, 48), (2304, 250), (4096, 1024), (8192, 300),
-               (6144, 40), (12288, 530), (16384, 64), (26624, 33), (8448, 20)]
+               (6144, 40), (12288, 530), (16384, 64), (26624, 33), (8448, 20), (2048, 20011), (512, 70003)]
 
 
 @pytest.mark.parametrize("in_dim,out_dim", MFMA_SHAPES)
@@ -196,7 +196,8 @@ MFMA_SHAPES = [(256, 17), (512, 100), (768, 33), (1024, 3584), (2048, 48), (2304
 def test_q4_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
     """2..4 tokens of a Q4_K matrix run on the matrix cores where the activations fit the staging buffer or the row is
     a multiple of 2048 values (staged a chunk at a time: whole chunks, a half-filled last chunk at 6144 and 26624, several
-    row tiles per wavefront): odd row counts, every k-slice split (1, 2, 3, 4, 8, 9, 16, 32 super-blocks), with and
+    row tiles per wavefront; 20011 x 2048 and 70003 x 512 have more row groups than the 256 workgroups launched, which
+    walk them with the activations staged once): odd row counts, every k-slice split (1, 2, 3, 4, 8, 9, 16, 32 super-blocks), with and
     without residual. 8448 values (33 super-blocks) are neither: three and four tokens stay on the vector ALU."""
     rng = np.random.default_rng(in_dim * 131 + out_dim * 7 + tokens)
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
