@@ -1,7 +1,7 @@
 // Decode GEMV on the matrix cores for M = 1..4 tokens, Q4_K: out[m][o] = (residual[m][o] +) sum_j x[m][j] * deq(W[o][j]).
 //
 // Same kernel ABI as the vector-ALU GEMV (gemv.cuh): (w_raw, x, [residual,] out, in_dim, out_dim), x rows at
-// stride in_dim, out/residual rows at stride out_dim. Launch: block = 1024 threads (16 wavefronts), grid and
+// stride in_dim, out/residual rows at stride out_dim. Launch: block = 512 threads (8 wavefronts), grid and
 // dynamic shared memory from gemv_config.h (gemv_mfma_grid, gemv_mfma_lds_bytes).
 //
 // Why the matrix cores for a matrix-vector product: the vector ALU needs one fused multiply-add per weight
@@ -26,8 +26,9 @@
 // belongs to one sub-block, so the fp32 scale d * sc and the min term dmin * m * sum(x) are applied here:
 // the lanes that decoded the 6-bit fields (A layout) hand them over through a wave-private LDS buffer.
 //
-// Work split: a workgroup owns 16 * T * NWR rows; its 16 wavefronts are NWK k-slices (super-blocks kslice,
-// kslice + NWK, ...) times NWR row groups, NWK = min(16, largest power of two <= in_dim / 256). Partial sums meet in LDS
+// Work split: a workgroup owns 16 * T * NWR rows at a time (and walks such row groups blockIdx.x, blockIdx.x + gridDim.x,
+// ... with the activations staged once where the host launches fewer workgroups than groups); its 8 wavefronts are NWK k-slices (super-blocks kslice,
+// kslice + NWK, ...) times NWR row groups, NWK = min(8, largest power of two <= in_dim / 256). Partial sums meet in LDS
 // and are added in a fixed order, so results are reproducible.
 #pragma once
 #include "common.cuh"
