@@ -403,13 +403,28 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
   const uint32_t cap = top1_token_cap(w_type), stride = cogni_gemv_top1_partials(w_type, out_dim);
-  for (uint32_t t0 = 0; t0 < tokens; t0 += cap) {
-    const uint32_t m = tokens - t0 < cap ? tokens - t0 : cap;
+  uint32_t m = 0;
+  for (uint32_t t0 = 0; t0 < tokens; t0 += m) {
+    const uint32_t left = tokens - t0;
+    m = left < cap ? left : cap;
     uint32_t grid = 0, block = 0, shmem = 0;
-    int rc = cogni_gemv_launch_dims(w_type, m, in_dim, out_dim, &grid, &block, &shmem);
-    if (rc != 0) return rc;
-    std::string name = std::string(type_prefix(w_type)) + "_gemv_top1_partial_f32";
-    if (m > 1) name += "_tbatch" + std::to_string(m);
+    std::string name;
+    // three or four tokens of a Q4_K or Q6_K matrix: the matrix-core kernel with the arg-max inside, where its
+    // workgroups fit the caller's partial buffers (sized for the vector-ALU kernels)
+    const uint32_t mm = left < (uint32_t)GEMV_MFMA_MAX_TOKENS ? left : (uint32_t)GEMV_MFMA_MAX_TOKENS;
+    if (mm >= 3 && gemv_mfma_supported(w_type, (int)mm, in_dim) && gemv_mfma_grid((int)mm, in_dim, out_dim) <= stride) {
+      m = mm;
+      grid = gemv_mfma_grid((int)m, in_dim, out_dim);
+      block = GEMV_MFMA_WAVES * 64;
+      shmem = gemv_mfma_lds_bytes(w_type, (int)m, in_dim);
+      name = std::string(type_prefix(w_type)) + "_gemv_mfma_top1_partial_f32_tbatch" + std::to_string(m);
+    } else {
+      int rc = cogni_gemv_launch_dims(w_type, m, in_dim, out_dim, &grid, &block, &shmem);
+      if (rc != 0) return rc;
+      name = std::string(type_prefix(w_type)) + "_gemv_top1_partial_f32";
+      if (m > 1) name += "_tbatch" + std::to_string(m);
+    }
+    int rc = 0;
     // the group's partial results: [token in group][workgroup], inside the group's share of the caller's buffers
     uint64_t xm = x + (uint64_t)t0 * in_dim * 4, pi = partial_ids + (uint64_t)t0 * stride * 4, pv = partial_values + (uint64_t)t0 * stride * 4;
     uint64_t oi = top1_ids + (uint64_t)t0 * 4, ov = top1_values + (uint64_t)t0 * 4;

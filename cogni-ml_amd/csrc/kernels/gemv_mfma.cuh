@@ -62,9 +62,13 @@ __device__ __forceinline__ void wave_lds_fence() {
 // wavefronts are eight k-slices and each stages and reads the activations of its own super-blocks only, so a wavefront
 // stages them C super-blocks at a time into a region of its own (no workgroup barrier), with the next chunk's
 // activations requested while the current one is consumed.
-template <int M, bool ADD, int T, bool CHUNK = false>
+// TOP1: instead of the row values a workgroup stores, per token, the largest of all its rows and that row's index
+// (out[token * gridDim.x + blockIdx.x], top_ids[...]: the layout of the vector-ALU top-1 kernels, finished by
+// top1_reduce_f32); of equal values the lowest row wins.
+template <int M, bool ADD, int T, bool CHUNK = false, bool TOP1 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float* x, const float* residual,
-                                                   float* out, u32 in_dim, u32 out_dim) {
+                                                   float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr) {
+  static_assert(!TOP1 || !ADD, "TOP1 is a mode of the plain GEMV");
   constexpr int MP = M <= 1 ? 1 : (M <= 2 ? 2 : 4);   // token slots in the column index
   constexpr int ND = MP;                              // accumulator tiles per 16 rows and super-block
   constexpr int BB = 144;
@@ -167,6 +171,8 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   load_sb(stA, kslice);
 
   mf_float4 acc[T];
+  float run_best = -__builtin_inff();   // TOP1: wavefront m keeps token m's best over the row groups it has seen
+  u32 run_id = 0xFFFFFFFFu;
 
   // ---- stage the activations: one wavefront per (token, super-block) -----------------------------------
   auto stage_xv = [&](u32 i0) {
@@ -383,43 +389,70 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   }
   __syncthreads();
   const u32 nout = NWR * T * 16 * M;
+  const u32 group_rows = NWR * T * 16;
+  float* tv = reinterpret_cast<float*>(lds + 64);   // TOP1: the group's row values [token][row in group], in the handover space
   for (u32 o = tid; o < nout; o += GEMV_MFMA_WAVES * 64) {
     const u32 r = o & 15, m = (o >> 4) % M, tt = (o / (16 * M)) % T, rgp = o / (16 * M * T);
     float v = 0.f;
     for (u32 k = 0; k < NWK; k++) v += part[(((rgp << lg_nwk) + k) * GEMV_MFMA_TMAX + tt) * MP * 16 + m * 16 + r];
     const u32 row = ((grp * NWR + rgp) * T + tt) * 16 + r;
-    if (row < out_dim) {
+    if constexpr (TOP1) {
+      tv[m * group_rows + (rgp * T + tt) * 16 + r] = v;
+    } else if (row < out_dim) {
       const size_t oi = (size_t)m * out_dim + row;
       if (ADD) v += residual[oi];
       out[oi] = v;
+    }
+  }
+  if constexpr (TOP1) {
+    __syncthreads();
+    if (wave < M) {
+      const u32 row_base = grp * group_rows;
+      float best = -__builtin_inff();
+      u32 best_id = 0xFFFFFFFFu;
+      for (u32 i = lane; i < group_rows; i += 64)
+        if (row_base + i < out_dim) top1_take(best, best_id, tv[(u32)wave * group_rows + i], row_base + i);
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const float ov = __shfl_xor(best, d, 64);
+        const u32 oi = (u32)__shfl_xor((int)best_id, d, 64);
+        top1_take(best, best_id, ov, oi);
+      }
+      top1_take(run_best, run_id, best, best_id);
     }
   }
   if (!walk) break;
   grp = next;
   __syncthreads();   // every partial sum has been read
   }
+  if constexpr (TOP1) {
+    if (wave < M && lane == 0) {
+      out[(size_t)wave * gridDim.x + blockIdx.x] = run_best;
+      top_ids[(size_t)wave * gridDim.x + blockIdx.x] = run_id == 0xFFFFFFFFu ? 0u : run_id;
+    }
+  }
 }
 
 // The tile count per wavefront follows from the grid the host chose (gemv_mfma_grid); tile count and
 // round structure are template parameters so that register use and loads in flight are compile-time constants.
 // Shapes outside gemv_mfma_supported() must not be launched.
-template <int M, bool ADD>
+template <int M, bool ADD, bool TOP1 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const float* x, const float* residual,
-                                                       float* out, u32 in_dim, u32 out_dim) {
+                                                       float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr) {
   const u32 nsb = in_dim >> 8;
   const u32 lg = gemv_mfma_log2_kslices(nsb);
   const u32 nwr = GEMV_MFMA_WAVES >> lg;
   const u32 ntiles = (out_dim + 15) >> 4;
   const u32 t = (ntiles + gridDim.x * nwr - 1) / (gridDim.x * nwr);
   if (gemv_mfma_chunked(M, in_dim)) {
-    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true>(w, x, residual, out, in_dim, out_dim);
-    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true>(w, x, residual, out, in_dim, out_dim);
-    else q4k_gemv_mfma_core<M, ADD, 3, true>(w, x, residual, out, in_dim, out_dim);
+    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
+    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
+    else q4k_gemv_mfma_core<M, ADD, 3, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
     return;
   }
-  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1>(w, x, residual, out, in_dim, out_dim);
-  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2>(w, x, residual, out, in_dim, out_dim);
-  else q4k_gemv_mfma_core<M, ADD, 3>(w, x, residual, out, in_dim, out_dim);
+  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
+  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
+  else q4k_gemv_mfma_core<M, ADD, 3, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
 }
 
 #define GEMV_MFMA_ENTRY(NAME, M)                                                                              \
@@ -432,4 +465,11 @@ __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const f
                                                                          const float* residual, float* out,   \
                                                                          u32 in_dim, u32 out_dim) {           \
     q4k_gemv_mfma_dispatch<M, true>(w, x, residual, out, in_dim, out_dim);                                    \
+  }
+// (w_raw, x, partial_ids, partial_values, in_dim, out_dim): the parameter list of the vector-ALU top-1 kernels
+#define GEMV_MFMA_TOP1_ENTRY(NAME, M)                                                                          \
+  extern "C" __global__ __launch_bounds__(GEMV_MFMA_WAVES * 64) void NAME(const uint8_t* w, const float* x,    \
+                                                                         u32* partial_ids, float* partial_values, \
+                                                                         u32 in_dim, u32 out_dim) {            \
+    q4k_gemv_mfma_dispatch<M, false, true>(w, x, nullptr, partial_values, in_dim, out_dim, partial_ids);       \
   }

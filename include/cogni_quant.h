@@ -164,8 +164,11 @@ int cogni_embed_dev(uint64_t w_raw, uint32_t w_type, uint64_t token_ids, uint64_
 
 /* Output head without the logits: for each token the index of the largest element of W x and that value
  * (top1_ids: u32[tokens], top1_values: f32[tokens]); of equal values the lowest index wins, as in the reference's CPU scan
- * (bin/cuda_mixed_stack_probe.cr:1485-1497). Two launches per group of up to 2 tokens (Q4_K, Q6_K; one token for the other
- * types; kernels for 3 tokens exist but a pair and a single token are faster): kernel "<prefix>_gemv_top1_partial_f32[_tbatchM]" (w_raw, x, partial_ids, partial_values, in_dim, out_dim) -
+ * (bin/cuda_mixed_stack_probe.cr:1485-1497). Two launches per group of tokens. Groups of 3 or 4 tokens of a Q4_K or Q6_K
+ * matrix take the matrix-core kernel "<prefix>_gemv_mfma_top1_partial_f32_tbatchM" (same parameters, the geometry of
+ * cogni_gemv_plan) where that kernel takes the shape and its grid fits the partial buffers; otherwise groups of up to
+ * 2 tokens (Q4_K, Q6_K; one token for the other types):
+ * kernel "<prefix>_gemv_top1_partial_f32[_tbatchM]" (w_raw, x, partial_ids, partial_values, in_dim, out_dim) -
  * the reference's q6_k_gemv_top1_partial_f32 (src/ml/cuda/kernels/q6k_gemv_probe.ptx:1331), with the grid, block and
  * shared memory of the GEMV of that type and token count and one (id, value) per workgroup and token - then
  * "top1_reduce_f32" (partial_ids, partial_values, out_ids, out_values, count:u32), block 1024, grid = tokens of the group -
