@@ -333,7 +333,34 @@ int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uin
     void* params[] = {&w_raw_a, &w_raw_b, &x, &out_a, &out_b, &in_dim, &out_dim};
     return launch("q4_k_dual_gemv_f32", grid, block, shmem, params, stream);
   }
-  // other types, several tokens: the pair as two launches of the kernels cogni_gemv_dev picks
+  // several tokens of a Q4_K pair whose shape the matrix-core kernel takes: groups of up to four tokens, the two
+  // matrices as one of 2 * out_dim rows (the activations are staged once for both); a last single token goes to the
+  // one-token pair kernel
+  if (w_type == COGNI_TYPE_Q4_K && tokens >= 2 && (in_dim % 256) == 0 && (out_dim % 16) == 0 && out_dim <= 0x7FFFFFFFu) {
+    uint32_t cap = 0;
+    for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2 && cap == 0; mt--)
+      if (gemv_mfma_supported(w_type, mt, in_dim)) cap = (uint32_t)mt;
+    if (cap != 0) {
+      uint32_t m = 0;
+      for (uint32_t t0 = 0; t0 < tokens; t0 += m) {
+        const uint32_t left = tokens - t0;
+        m = left < cap ? left : cap;
+        uint64_t xm = x + (uint64_t)t0 * in_dim * 4, oa = out_a + (uint64_t)t0 * out_dim * 4, ob = out_b + (uint64_t)t0 * out_dim * 4;
+        int rc = 0;
+        if (m == 1) {
+          rc = cogni_gemv_dual_dev(w_raw_a, w_raw_b, w_type, xm, oa, ob, in_dim, out_dim, 1, stream);
+        } else {
+          const uint32_t grid = gemv_mfma_grid((int)m, in_dim, 2 * out_dim);
+          const std::string name = "q4_k_dual_gemv_mfma_f32_tbatch" + std::to_string(m);
+          void* params[] = {&w_raw_a, &w_raw_b, &xm, &oa, &ob, &in_dim, &out_dim};
+          rc = launch(name.c_str(), grid, GEMV_MFMA_WAVES * 64, gemv_mfma_lds_bytes(w_type, (int)m, in_dim), params, stream);
+        }
+        if (rc != 0) return rc;
+      }
+      return 0;
+    }
+  }
+  // other types and shapes: the pair as two launches of the kernels cogni_gemv_dev picks
   int rc = cogni_gemv_dev(w_raw_a, w_type, x, 0, out_a, in_dim, out_dim, tokens, stream);
   if (rc != 0) return rc;
   return cogni_gemv_dev(w_raw_b, w_type, x, 0, out_b, in_dim, out_dim, tokens, stream);

@@ -67,8 +67,12 @@ __device__ __forceinline__ void wave_lds_fence() {
 // top1_reduce_f32); of equal values the lowest row wins.
 template <int M, bool ADD, int T, bool CHUNK = false, bool TOP1 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float* x, const float* residual,
-                                                   float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr) {
+                                                   float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr,
+                                                   const uint8_t* w_b = nullptr, float* out_b = nullptr) {
   static_assert(!TOP1 || !ADD, "TOP1 is a mode of the plain GEMV");
+  // matrix pair (w_b set): two matrices of one shape against the same activations (k | v, gate | up) as one matrix of
+  // rows [0, out_dim) of the first and then of the second; out_dim must be a multiple of 16 (a tile is of one matrix)
+  const u32 total_rows = w_b ? 2 * out_dim : out_dim;
   constexpr int MP = M <= 1 ? 1 : (M <= 2 ? 2 : 4);   // token slots in the column index
   constexpr int ND = MP;                              // accumulator tiles per 16 rows and super-block
   constexpr int BB = 144;
@@ -83,7 +87,7 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   const u32 lg_nwk = gemv_mfma_log2_kslices(nsb);
   const u32 NWK = 1u << lg_nwk, NWR = GEMV_MFMA_WAVES >> lg_nwk;
   const u32 kslice = wave & (NWK - 1), rgrp = wave >> lg_nwk;
-  const u32 ntiles = (out_dim + 15) >> 4;
+  const u32 ntiles = (total_rows + 15) >> 4;
   // A workgroup takes the row groups (NWR * T tiles each) blockIdx.x, blockIdx.x + gridDim.x, ... with the activations
   // staged once: a matrix with more groups than compute units (an output head) is launched as one workgroup per unit.
   const u32 ngroups = (ntiles + NWR * T - 1) / (NWR * T);
@@ -121,7 +125,8 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
 #pragma unroll
     for (int t = 0; t < T; t++) {
       const u32 tile = min(tile0 + (u32)t, ntiles - 1);
-      rowp[t] = w + (size_t)min(tile * 16 + ar, out_dim - 1) * row_bytes;
+      const u32 vr = min(tile * 16 + ar, total_rows - 1);
+      rowp[t] = vr < out_dim ? w + (size_t)vr * row_bytes : w_b + (size_t)(vr - out_dim) * row_bytes;
     }
   };
   set_rows(grp);
@@ -398,7 +403,9 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     const u32 row = ((grp * NWR + rgp) * T + tt) * 16 + r;
     if constexpr (TOP1) {
       tv[m * group_rows + (rgp * T + tt) * 16 + r] = v;
-    } else if (row < out_dim) {
+    } else if (row >= out_dim) {
+      if (row < total_rows) out_b[(size_t)m * out_dim + (row - out_dim)] = v;
+    } else {
       const size_t oi = (size_t)m * out_dim + row;
       if (ADD) v += residual[oi];
       out[oi] = v;
@@ -438,21 +445,22 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
 // Shapes outside gemv_mfma_supported() must not be launched.
 template <int M, bool ADD, bool TOP1 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const float* x, const float* residual,
-                                                       float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr) {
+                                                       float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr,
+                                                       const uint8_t* w_b = nullptr, float* out_b = nullptr) {
   const u32 nsb = in_dim >> 8;
   const u32 lg = gemv_mfma_log2_kslices(nsb);
   const u32 nwr = GEMV_MFMA_WAVES >> lg;
-  const u32 ntiles = (out_dim + 15) >> 4;
+  const u32 ntiles = ((w_b ? 2 * out_dim : out_dim) + 15) >> 4;
   const u32 t = (ntiles + gridDim.x * nwr - 1) / (gridDim.x * nwr);
   if (gemv_mfma_chunked(M, in_dim)) {
-    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
-    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
-    else q4k_gemv_mfma_core<M, ADD, 3, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
+    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
+    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
+    else q4k_gemv_mfma_core<M, ADD, 3, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
     return;
   }
-  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
-  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
-  else q4k_gemv_mfma_core<M, ADD, 3, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids);
+  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
+  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
+  else q4k_gemv_mfma_core<M, ADD, 3, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
 }
 
 #define GEMV_MFMA_ENTRY(NAME, M)                                                                              \
@@ -472,4 +480,12 @@ __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const f
                                                                          u32* partial_ids, float* partial_values, \
                                                                          u32 in_dim, u32 out_dim) {            \
     q4k_gemv_mfma_dispatch<M, false, true>(w, x, nullptr, partial_values, in_dim, out_dim, partial_ids);       \
+  }
+// (w_raw_a, w_raw_b, x, out_a, out_b, in_dim, out_dim): the matrix pair, parameters of q4_k_dual_gemv_f32; M tokens at
+// strides in_dim / out_dim; out_dim a multiple of 16; grid and shared memory of the single matrix with 2 * out_dim rows
+#define GEMV_MFMA_DUAL_ENTRY(NAME, M)                                                                          \
+  extern "C" __global__ __launch_bounds__(GEMV_MFMA_WAVES * 64) void NAME(const uint8_t* w_a, const uint8_t* w_b, \
+                                                                         const float* x, float* out_a, float* out_b, \
+                                                                         u32 in_dim, u32 out_dim) {            \
+    q4k_gemv_mfma_dispatch<M, false>(w_a, x, nullptr, out_a, in_dim, out_dim, nullptr, w_b, out_b);            \
   }

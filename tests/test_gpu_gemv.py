@@ -280,10 +280,14 @@ def test_q4_k_matrix_core_kernel_activation_ranges(gpu, oracle):
 
 
 @pytest.mark.parametrize("type_id,in_dim,out_dim,tokens", [(Q4_K, 4096, 12288, 1), (Q4_K, 512, 37, 1), (Q4_K, 1024, 1024, 3),
-                                                            (Q6_K, 512, 40, 1), (Q4_K, 4096, 1024, 1)])
+                                                            (Q6_K, 512, 40, 1), (Q4_K, 4096, 1024, 1), (Q4_K, 4096, 12288, 4),
+                                                            (Q4_K, 4096, 1024, 8), (Q4_K, 12288, 48, 4), (Q4_K, 512, 40, 2),
+                                                            (Q4_K, 2048, 8000, 5), (Q4_K, 768, 12304, 3)])
 def test_dual_gemv_shares_activations(gpu, oracle, type_id, in_dim, out_dim, tokens):
     """Two matrices of one shape against the same x (gate | up, k | v): one launch for one token of a Q4_K pair,
-    including a row count that puts the a | b boundary inside a wavefront's rows."""
+    including a row count that puts the a | b boundary inside a wavefront's rows; several tokens of a Q4_K pair with a
+    multiple of 16 rows go to the matrix-core kernel as one matrix of twice the rows (groups of four tokens and a last
+    single one, activations staged in chunks, more row groups than workgroups), other shapes as two launches."""
     rng = np.random.default_rng(in_dim + 3 * out_dim + tokens)
     raw_a = synth.make_weights(rng, type_id, out_dim, in_dim)
     raw_b = synth.make_weights(rng, type_id, out_dim, in_dim)
