@@ -89,6 +89,18 @@ class QwenProjectionStackRunner:
         while i < len(ents):
             name, src, t, out_dim, in_dim, raw = ents[i]
             nxt = ents[i + 1] if i + 1 < len(ents) else None
+            # several tokens: up to three consecutive projections of one input, type and row length (q | k | v,
+            # gate | up) go to the library as one list (the qmatvec_many seam), which stages the input once for them
+            j = i + 1
+            while count > 1 and j < len(ents) and j - i < 3 and (ents[j][1], ents[j][2], ents[j][4]) == (src, t, in_dim):
+                j += 1
+            if j - i >= 2:
+                grp = ents[i:j]
+                quant.gemv_many_dev([self._w[e[0]].ptr for e in grp], t, self._act[src].ptr + 4 * tok0 * in_dim,
+                                    [self._act[e[0]].ptr + 4 * tok0 * e[3] for e in grp], [e[3] for e in grp], in_dim,
+                                    count, stream)
+                i = j
+                continue
             if nxt is not None and nxt[1:5] == (src, t, out_dim, in_dim):
                 # two projections of one shape on the same input (k | v, gate | up) share one launch
                 quant.gemv_dual_dev(self._w[name].ptr, self._w[nxt[0]].ptr, t, self._act[src].ptr + 4 * tok0 * in_dim,

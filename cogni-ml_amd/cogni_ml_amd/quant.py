@@ -73,6 +73,18 @@ def gemv_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens=1, residual_
                                     ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+def gemv_many_dev(w_ptrs, w_type, x_ptr, out_ptrs, out_dims, in_dim, tokens=1, stream=None):
+    """Several matrices of one type and in_dim against the same activations (q | k | v): the qmatvec_many seam on
+    device pointers."""
+    n = len(w_ptrs)
+    if len(out_ptrs) != n or len(out_dims) != n:
+        raise ValueError("w_ptrs, out_ptrs and out_dims must have the same length")
+    U64, U32 = ctypes.c_uint64 * n, ctypes.c_uint32 * n
+    _check(hip.lib().cogni_gemv_many_dev(U64(*w_ptrs), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(x_ptr), U64(*out_ptrs),
+                                         U32(*out_dims), ctypes.c_uint32(n), ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens),
+                                         stream))
+
+
 def gemv_dual_dev(w_a_ptr, w_b_ptr, w_type, x_ptr, out_a_ptr, out_b_ptr, in_dim, out_dim, tokens=1, stream=None):
     """Two matrices of one shape against the same activations (gate | up, k | v)."""
     _check(hip.lib().cogni_gemv_dual_dev(ctypes.c_uint64(w_a_ptr), ctypes.c_uint64(w_b_ptr), ctypes.c_uint32(int(w_type)),

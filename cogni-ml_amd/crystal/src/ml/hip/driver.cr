@@ -58,6 +58,8 @@ lib LibCogniHIP
                       grid_x : UInt32*, block_x : UInt32*, shared_mem_bytes : UInt32*) : Int32
   fun cogni_gemv_dual_dev(w_raw_a : UInt64, w_raw_b : UInt64, w_type : UInt32, x : UInt64, out_a : UInt64, out_b : UInt64,
                           in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemv_many_dev(w_raw : UInt64*, w_type : UInt32, x : UInt64, out : UInt64*, out_dims : UInt32*, count : UInt32,
+                          in_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_swiglu_dev(gate : UInt64, up : UInt64, out : UInt64, n : UInt32, stream : Void*) : Int32
   fun cogni_gemv_dual_swiglu_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, x : UInt64, out : UInt64,
                                  in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32

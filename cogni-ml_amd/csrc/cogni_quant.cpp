@@ -366,6 +366,58 @@ int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uin
   return cogni_gemv_dev(w_raw_b, w_type, x, 0, out_b, in_dim, out_dim, tokens, stream);
 }
 
+int cogni_gemv_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t x, const uint64_t* out, const uint32_t* out_dims,
+                        uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream) {
+  if (!gemv_type(w_type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for fused matmul: ") + type_name(w_type));
+  if (!w_raw || !out || !out_dims || !x) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_many_dev: null argument");
+  if (count == 0 || count > 8) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_many_dev: count must be 1..8");
+  if (in_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_many_dev: zero dimension");
+  uint64_t total = 0;
+  bool aligned = true;
+  for (uint32_t i = 0; i < count; i++) {
+    if (!w_raw[i] || !out[i] || out_dims[i] == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_many_dev: null pointer or zero rows");
+    total += out_dims[i];
+    aligned = aligned && (out_dims[i] % 16) == 0;
+  }
+  if (count == 2 && out_dims[0] == out_dims[1])
+    return cogni_gemv_dual_dev(w_raw[0], w_raw[1], w_type, x, out[0], out[1], in_dim, out_dims[0], tokens, stream);
+  uint32_t cap = 0;
+  if (w_type == COGNI_TYPE_Q4_K && (count == 2 || count == 3) && tokens >= 2 && aligned && (in_dim % 256) == 0 && total <= 0x7FFFFFFFull)
+    for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2 && cap == 0; mt--)
+      if (gemv_mfma_supported(w_type, mt, in_dim)) cap = (uint32_t)mt;
+  if (cap == 0) {
+    for (uint32_t i = 0; i < count; i++) {
+      const int rc = cogni_gemv_dev(w_raw[i], w_type, x, 0, out[i], in_dim, out_dims[i], tokens, stream);
+      if (rc != 0) return rc;
+    }
+    return 0;
+  }
+  uint32_t m = 0;
+  for (uint32_t t0 = 0; t0 < tokens; t0 += m) {
+    const uint32_t left = tokens - t0;
+    m = left < cap ? left : cap;
+    uint64_t xm = x + (uint64_t)t0 * in_dim * 4;
+    if (m == 1) {   // a last single token: one launch per matrix
+      for (uint32_t i = 0; i < count; i++) {
+        const int rc = cogni_gemv_dev(w_raw[i], w_type, xm, 0, out[i] + (uint64_t)t0 * out_dims[i] * 4, in_dim, out_dims[i], 1, stream);
+        if (rc != 0) return rc;
+      }
+      continue;
+    }
+    uint64_t w[3] = {w_raw[0], w_raw[1], count > 2 ? w_raw[2] : 0};
+    uint64_t o[3] = {out[0] + (uint64_t)t0 * out_dims[0] * 4, out[1] + (uint64_t)t0 * out_dims[1] * 4,
+                     count > 2 ? out[2] + (uint64_t)t0 * out_dims[2] * 4 : 0};
+    uint32_t rows[3] = {out_dims[0], out_dims[1], count > 2 ? out_dims[2] : 0};
+    const uint32_t grid = gemv_mfma_grid((int)m, in_dim, (uint32_t)total);
+    const std::string name = "q4_k_many_gemv_mfma_f32_tbatch" + std::to_string(m);
+    void* params[] = {&w[0], &w[1], &w[2], &xm, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2]};
+    const int rc = launch(name.c_str(), grid, GEMV_MFMA_WAVES * 64, gemv_mfma_lds_bytes(w_type, (int)m, in_dim), params, stream);
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+
 int cogni_swiglu_dev(uint64_t gate, uint64_t up, uint64_t out, uint32_t n, void* stream) {
   if (!gate || !up || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_swiglu_dev: null device pointer");
   if (n == 0) return 0;

@@ -27,3 +27,6 @@ GEMV_MFMA_Q6K_TOP1_ENTRY(q6_k_gemv_mfma_top1_partial_f32_tbatch4, 4)
 GEMV_MFMA_DUAL_ENTRY(q4_k_dual_gemv_mfma_f32_tbatch2, 2)
 GEMV_MFMA_DUAL_ENTRY(q4_k_dual_gemv_mfma_f32_tbatch3, 3)
 GEMV_MFMA_DUAL_ENTRY(q4_k_dual_gemv_mfma_f32_tbatch4, 4)
+GEMV_MFMA_MANY_ENTRY(q4_k_many_gemv_mfma_f32_tbatch2, 2)
+GEMV_MFMA_MANY_ENTRY(q4_k_many_gemv_mfma_f32_tbatch3, 3)
+GEMV_MFMA_MANY_ENTRY(q4_k_many_gemv_mfma_f32_tbatch4, 4)

@@ -65,14 +65,23 @@ __device__ __forceinline__ void wave_lds_fence() {
 // TOP1: instead of the row values a workgroup stores, per token, the largest of all its rows and that row's index
 // (out[token * gridDim.x + blockIdx.x], top_ids[...]: the layout of the vector-ALU top-1 kernels, finished by
 // top1_reduce_f32); of equal values the lowest row wins.
+// Further matrices of the same in_dim behind the first (w, out, out_dim = rows0): rows [0, rows0) are the first's,
+// [rows0, rows0 + rows1) the second's, then the third's. Every row count a multiple of 16 (a tile is of one matrix).
+struct MfMany {
+  const uint8_t* w1;
+  const uint8_t* w2;
+  float* out1;
+  float* out2;
+  u32 rows1, rows2;
+};
 template <int M, bool ADD, int T, bool CHUNK = false, bool TOP1 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float* x, const float* residual,
                                                    float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr,
-                                                   const uint8_t* w_b = nullptr, float* out_b = nullptr) {
+                                                   const MfMany* many = nullptr) {
   static_assert(!TOP1 || !ADD, "TOP1 is a mode of the plain GEMV");
-  // matrix pair (w_b set): two matrices of one shape against the same activations (k | v, gate | up) as one matrix of
-  // rows [0, out_dim) of the first and then of the second; out_dim must be a multiple of 16 (a tile is of one matrix)
-  const u32 total_rows = w_b ? 2 * out_dim : out_dim;
+  // several matrices against the same activations (q | k | v, gate | up) as one matrix of all their rows
+  const u32 rows1 = many ? many->rows1 : 0u, rows2 = many ? many->rows2 : 0u;
+  const u32 total_rows = out_dim + rows1 + rows2;
   constexpr int MP = M <= 1 ? 1 : (M <= 2 ? 2 : 4);   // token slots in the column index
   constexpr int ND = MP;                              // accumulator tiles per 16 rows and super-block
   constexpr int BB = 144;
@@ -126,7 +135,9 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     for (int t = 0; t < T; t++) {
       const u32 tile = min(tile0 + (u32)t, ntiles - 1);
       const u32 vr = min(tile * 16 + ar, total_rows - 1);
-      rowp[t] = vr < out_dim ? w + (size_t)vr * row_bytes : w_b + (size_t)(vr - out_dim) * row_bytes;
+      if (!many || vr < out_dim) rowp[t] = w + (size_t)vr * row_bytes;
+      else if (vr < out_dim + rows1) rowp[t] = many->w1 + (size_t)(vr - out_dim) * row_bytes;
+      else rowp[t] = many->w2 + (size_t)(vr - out_dim - rows1) * row_bytes;
     }
   };
   set_rows(grp);
@@ -404,7 +415,8 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     if constexpr (TOP1) {
       tv[m * group_rows + (rgp * T + tt) * 16 + r] = v;
     } else if (row >= out_dim) {
-      if (row < total_rows) out_b[(size_t)m * out_dim + (row - out_dim)] = v;
+      if (row < out_dim + rows1) many->out1[(size_t)m * rows1 + (row - out_dim)] = v;
+      else if (row < total_rows) many->out2[(size_t)m * rows2 + (row - out_dim - rows1)] = v;
     } else {
       const size_t oi = (size_t)m * out_dim + row;
       if (ADD) v += residual[oi];
@@ -446,21 +458,21 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
 template <int M, bool ADD, bool TOP1 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const float* x, const float* residual,
                                                        float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr,
-                                                       const uint8_t* w_b = nullptr, float* out_b = nullptr) {
+                                                       const MfMany* many = nullptr) {
   const u32 nsb = in_dim >> 8;
   const u32 lg = gemv_mfma_log2_kslices(nsb);
   const u32 nwr = GEMV_MFMA_WAVES >> lg;
-  const u32 ntiles = ((w_b ? 2 * out_dim : out_dim) + 15) >> 4;
+  const u32 ntiles = (out_dim + (many ? many->rows1 + many->rows2 : 0u) + 15) >> 4;
   const u32 t = (ntiles + gridDim.x * nwr - 1) / (gridDim.x * nwr);
   if (gemv_mfma_chunked(M, in_dim)) {
-    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
-    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
-    else q4k_gemv_mfma_core<M, ADD, 3, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
+    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+    else q4k_gemv_mfma_core<M, ADD, 3, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
     return;
   }
-  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
-  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
-  else q4k_gemv_mfma_core<M, ADD, 3, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, w_b, out_b);
+  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+  else q4k_gemv_mfma_core<M, ADD, 3, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
 }
 
 #define GEMV_MFMA_ENTRY(NAME, M)                                                                              \
@@ -487,5 +499,16 @@ __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const f
   extern "C" __global__ __launch_bounds__(GEMV_MFMA_WAVES * 64) void NAME(const uint8_t* w_a, const uint8_t* w_b, \
                                                                          const float* x, float* out_a, float* out_b, \
                                                                          u32 in_dim, u32 out_dim) {            \
-    q4k_gemv_mfma_dispatch<M, false>(w_a, x, nullptr, out_a, in_dim, out_dim, nullptr, w_b, out_b);            \
+    const MfMany many = {w_b, nullptr, out_b, nullptr, out_dim, 0u};                                           \
+    q4k_gemv_mfma_dispatch<M, false>(w_a, x, nullptr, out_a, in_dim, out_dim, nullptr, &many);                 \
+  }
+// (w0, w1, w2, x, out0, out1, out2, in_dim, rows0, rows1, rows2): up to three matrices of one in_dim against the same
+// activations (q | k | v); rows2 may be 0; every row count a multiple of 16; out_i rows at stride rows_i; grid and shared
+// memory of a single matrix with rows0 + rows1 + rows2 rows
+#define GEMV_MFMA_MANY_ENTRY(NAME, M)                                                                          \
+  extern "C" __global__ __launch_bounds__(GEMV_MFMA_WAVES * 64) void NAME(                                     \
+      const uint8_t* w0, const uint8_t* w1, const uint8_t* w2, const float* x, float* out0, float* out1, float* out2, \
+      u32 in_dim, u32 rows0, u32 rows1, u32 rows2) {                                                           \
+    const MfMany many = {w1, w2, out1, out2, rows1, rows2};                                                    \
+    q4k_gemv_mfma_dispatch<M, false>(w0, x, nullptr, out0, in_dim, rows0, nullptr, &many);                     \
   }

@@ -122,9 +122,23 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
  * used by src/ml/cuda/qwen_recurrent_layer_runner.cr:519-520): output row r of the launch is row r of W_a for
  * r < out_dim and row r - out_dim of W_b above; block and dynamic shared memory as cogni_gemv_launch_dims gives for
  * one token, grid_x = ceil(2*out_dim / rows per workgroup), grid_y = tokens (one token per slice, x + y*in_dim,
- * out_* + y*out_dim, the reference's ..._batched entry). Every other case is issued as two cogni_gemv_dev calls. */
+ * out_* + y*out_dim, the reference's ..._batched entry). Several tokens of a Q4_K pair with out_dim a multiple of 16
+ * and a row length the matrix-core kernel takes: "q4_k_dual_gemv_mfma_f32_tbatchM", same parameters, block 512, grid and
+ * shared memory of one matrix with 2*out_dim rows (cogni_gemv_plan), per group of up to four tokens. Every other case is
+ * issued as two cogni_gemv_dev calls. */
 int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uint64_t x, uint64_t out_a, uint64_t out_b,
                         uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
+
+/* Several matrices of one type and in_dim against the same activations (q | k | v, gate | up) on device pointers: the
+ * reference's qmatvec_many seam (src/ml/gguf/qwen35_cpu.cr:1419-1445), which hands a list of weights and one x to the
+ * GPU arm.  out[i][m*out_dims[i] + o] = sum_j x[m*in_dim + j] * deq(W_i[o][j]).
+ * Two or three Q4_K matrices, two or more tokens, every out_dims[i] a multiple of 16 and a row length the matrix-core
+ * kernel takes: one launch per group of up to four tokens of "q4_k_many_gemv_mfma_f32_tbatchM"
+ * (w0, w1, w2, x, out0, out1, out2, in_dim, rows0, rows1, rows2), block 512, grid and shared memory of one matrix with
+ * the sum of the rows (cogni_gemv_plan), the activations staged once for all of them. Two matrices of one shape: as
+ * cogni_gemv_dual_dev. Everything else: one cogni_gemv_dev per matrix. count in 1..8. */
+int cogni_gemv_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t x, const uint64_t* out, const uint32_t* out_dims,
+                        uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream);
 
 /* out[i] = silu(gate[i]) * up[i], silu(g) = g / (1 + exp(-g)) in fp32: kernel "swiglu_f32" (gate, up, out, n:u32),
  * block 256, grid ceil(n/256) - the reference's swiglu_f32 (bin/cuda_ffn_sequence_probe.cr:46-84, CPU form :189-191). */

@@ -309,6 +309,37 @@ def test_dual_gemv_shares_activations(gpu, oracle, type_id, in_dim, out_dim, tok
         d.close()
 
 
+@pytest.mark.parametrize("type_id,in_dim,dims,tokens", [(Q4_K, 4096, (4096, 1024, 1024), 4), (Q4_K, 1024, (48, 16, 160), 7),
+                                                        (Q4_K, 12288, (64, 32), 3), (Q4_K, 2048, (12288, 4096, 32), 2),
+                                                        (Q4_K, 512, (40, 16, 16), 4), (Q6_K, 512, (32, 48, 16), 4),
+                                                        (Q4_K, 1024, (64, 32, 16), 1), (Q4_K, 256, (16, 16, 16, 16), 3)])
+def test_many_gemv_shares_activations(gpu, oracle, type_id, in_dim, dims, tokens):
+    """Several matrices against one x in one call (q | k | v): two or three Q4_K matrices with multiples of 16 rows and
+    two or more tokens run as one matrix-core launch per group of four tokens, everything else matrix by matrix. Either
+    way the values are those of cogni_gemv_dev on each matrix, bit for bit where both take the matrix cores."""
+    rng = np.random.default_rng(in_dim + sum(dims) + tokens)
+    raws = [synth.make_weights(rng, type_id, d, in_dim) for d in dims]
+    x = synth.make_activations(rng, tokens, in_dim)
+    ws, xd = [DevArray(r) for r in raws], DevArray(x)
+    outs = [DevArray(nbytes=4 * tokens * d) for d in dims]
+    quant.gemv_many_dev([w.ptr for w in ws], type_id, xd.ptr, [o.ptr for o in outs], list(dims), in_dim, tokens)
+    zero = {d: np.zeros(d, dtype=np.float32) for d in dims}
+    for raw, o, d in zip(raws, outs, dims):
+        got = o.read(np.float32, tokens * d)
+        want = oracle.matmul_add(x, tokens, in_dim, raw, type_id, d, zero[d], threads=8).astype(np.float64)
+        dense = np.abs(oracle.dequantize(raw, type_id, d * in_dim)).reshape(d, in_dim)
+        assert np.all(np.abs(got.astype(np.float64) - want) <= gemv_tolerance(x, dense, tokens, in_dim).reshape(-1))
+        single = run_gemv(raw, type_id, x, in_dim, d, tokens)
+        if all("mfma" in quant.gemv_plan(type_id, m, in_dim, d)[0] for m in {min(tokens, 4), tokens % 4 or 4} if m >= 2) and tokens % 4 != 1:
+            assert np.array_equal(got, single)
+        else:
+            assert np.max(np.abs(got - single)) <= 2e-5 * max(1e-30, float(np.abs(single).max()))
+    for a in ws + outs + [xd]:
+        a.close()
+    with pytest.raises(quant.QuantError):
+        quant.gemv_many_dev([], type_id, 0, [], [], in_dim, tokens)
+
+
 def test_swiglu_kernel_and_fused_gate_up(gpu, oracle):
     """swiglu_f32 against the oracle's float32 form, and the fused gate/up + SwiGLU launch against the
     two-step composition (same bits: same GEMV arithmetic, same device function) and the oracle."""
