@@ -3,8 +3,8 @@
 The HIP counterpart of the reference's FFN sequence probe (bin/cuda_ffn_sequence_probe.cr:3, 254-266 for the
 CPU form, 314-440 for the launches): weights and activations stay on the device, the lifecycle goes through
 ResidentSequenceRunner. Where the reference launches gate, up, the activation and down as four kernels per token,
-one token here is two launches (gate | up | SwiGLU fused, then down with the residual add); several tokens go
-through the weight-stationary kernels (gate | up pair, swiglu_f32, down).
+a group of up to four tokens here is two launches (gate | up | SwiGLU fused, then down with the residual add); an FFN width
+that is not a multiple of 16 goes through the weight-stationary kernels for several tokens (gate | up pair, swiglu_f32, down).
 
 With `norm` and `add` the sequence is the whole FFN half of a decoder layer (src/ml/gguf/qwen35_cpu.cr:1705-1725):
 r = x + add (the attention output joining the residual stream), h = rmsnorm(r, norm), out = r + down(silu(gate h) * up h).
@@ -77,8 +77,9 @@ class FFNSequenceRunner:
             quant.add_rmsnorm_dev(x, self._add.ptr + 4 * tok0 * h, self._norm.ptr, self._res.ptr + 4 * tok0 * h, normed, h,
                                   count, self._eps, st)
             x = normed
-        if count == 1:
-            quant.gemv_dual_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, x, act, h, f, 1, st)
+        if count == 1 or f % 16 == 0:
+            # gate | up | SwiGLU in one launch (several tokens: per group of four on the matrix cores)
+            quant.gemv_dual_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, x, act, h, f, count, st)
         else:
             g, u = self._gate.ptr + 4 * tok0 * f, self._up.ptr + 4 * tok0 * f
             quant.gemv_dual_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, x, g, u, h, f, count, st)

@@ -434,6 +434,34 @@ int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, 
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dual_swiglu_dev: zero dimension");
   if ((in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "Q4_K GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  // several tokens, out_dim a multiple of 16 and a row length the matrix-core kernel takes: groups of up to four tokens
+  // on the matrix cores (gate tile and up tile side by side in a wavefront, two tiles per wavefront, 256 workgroups at
+  // most, which walk the row groups with the activations staged once); a last single token as below
+  uint32_t cap = 0;
+  if (tokens >= 2 && (out_dim % 16) == 0 && out_dim <= 0x7FFFFFFFu)
+    for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2 && cap == 0; mt--)
+      if (gemv_mfma_supported(w_type, mt, in_dim)) cap = (uint32_t)mt;
+  if (cap != 0) {
+    uint32_t m = 0;
+    for (uint32_t t0 = 0; t0 < tokens; t0 += m) {
+      const uint32_t left = tokens - t0;
+      m = left < cap ? left : cap;
+      uint64_t xm = x + (uint64_t)t0 * in_dim * 4, om = out + (uint64_t)t0 * out_dim * 4;
+      int rc = 0;
+      if (m == 1) {
+        rc = cogni_gemv_dual_swiglu_dev(w_gate, w_up, w_type, xm, om, in_dim, out_dim, 1, stream);
+      } else {
+        const uint32_t nwr = GEMV_MFMA_WAVES >> gemv_mfma_log2_kslices(in_dim >> 8);
+        const uint32_t groups = (out_dim / 16 + nwr - 1) / nwr;   // pairs of tiles, one pair per wavefront
+        const uint32_t g = gemv_mfma_chunked((int)m, in_dim) || groups <= 256u ? groups : 256u;
+        const std::string name = "q4_k_dual_gemv_swiglu_mfma_f32_tbatch" + std::to_string(m);
+        void* params[] = {&w_gate, &w_up, &xm, &om, &in_dim, &out_dim};
+        rc = launch(name.c_str(), g, GEMV_MFMA_WAVES * 64, gemv_mfma_lds_bytes(w_type, (int)m, in_dim), params, stream);
+      }
+      if (rc != 0) return rc;
+    }
+    return 0;
+  }
   uint32_t grid = 0, block = 0, shmem = 0;
   int rc = cogni_gemv_launch_dims(w_type, 1, in_dim, out_dim, &grid, &block, &shmem);
   if (rc != 0) return rc;

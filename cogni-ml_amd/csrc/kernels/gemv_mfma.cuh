@@ -74,11 +74,15 @@ struct MfMany {
   float* out2;
   u32 rows1, rows2;
 };
-template <int M, bool ADD, int T, bool CHUNK = false, bool TOP1 = false>
+// SWIGLU (gate = w, up = many->w1, many->rows1 = out_dim, a multiple of 16): the tiles alternate gate tile p, up tile p,
+// so a wavefront with an even tile count holds both and the workgroup stores out[m][o] = silu(gate . x) * (up . x)
+// (swiglu_one, the function of swiglu_f32) - no gate or up vectors in memory.
+template <int M, bool ADD, int T, bool CHUNK = false, bool TOP1 = false, bool SWIGLU = false>
 __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float* x, const float* residual,
                                                    float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr,
                                                    const MfMany* many = nullptr) {
   static_assert(!TOP1 || !ADD, "TOP1 is a mode of the plain GEMV");
+  static_assert(!SWIGLU || (T % 2 == 0 && !ADD && !TOP1), "SWIGLU pairs a gate tile with an up tile");
   // several matrices against the same activations (q | k | v, gate | up) as one matrix of all their rows
   const u32 rows1 = many ? many->rows1 : 0u, rows2 = many ? many->rows2 : 0u;
   const u32 total_rows = out_dim + rows1 + rows2;
@@ -135,7 +139,8 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
     for (int t = 0; t < T; t++) {
       const u32 tile = min(tile0 + (u32)t, ntiles - 1);
       const u32 vr = min(tile * 16 + ar, total_rows - 1);
-      if (!many || vr < out_dim) rowp[t] = w + (size_t)vr * row_bytes;
+      if constexpr (SWIGLU) rowp[t] = ((tile & 1) ? many->w1 : w) + (size_t)min((tile >> 1) * 16 + ar, out_dim - 1) * row_bytes;
+      else if (!many || vr < out_dim) rowp[t] = w + (size_t)vr * row_bytes;
       else if (vr < out_dim + rows1) rowp[t] = many->w1 + (size_t)(vr - out_dim) * row_bytes;
       else rowp[t] = many->w2 + (size_t)(vr - out_dim - rows1) * row_bytes;
     }
@@ -407,6 +412,19 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   const u32 nout = NWR * T * 16 * M;
   const u32 group_rows = NWR * T * 16;
   float* tv = reinterpret_cast<float*>(lds + 64);   // TOP1: the group's row values [token][row in group], in the handover space
+  if constexpr (SWIGLU) {
+    for (u32 o = tid; o < nout / 2; o += GEMV_MFMA_WAVES * 64) {
+      const u32 r = o & 15, m = (o >> 4) % M, pp = (o / (16 * M)) % (T / 2), rgp = o / (16 * M * (T / 2));
+      float g = 0.f, u = 0.f;
+      for (u32 k = 0; k < NWK; k++) {
+        const u32 base = (((rgp << lg_nwk) + k) * GEMV_MFMA_TMAX + 2 * pp) * MP * 16 + m * 16 + r;
+        g += part[base];
+        u += part[base + MP * 16];
+      }
+      const u32 row = ((((grp * NWR + rgp) * T) >> 1) + pp) * 16 + r;
+      if (row < out_dim) out[(size_t)m * out_dim + row] = swiglu_one(g, u);
+    }
+  } else
   for (u32 o = tid; o < nout; o += GEMV_MFMA_WAVES * 64) {
     const u32 r = o & 15, m = (o >> 4) % M, tt = (o / (16 * M)) % T, rgp = o / (16 * M * T);
     float v = 0.f;
@@ -511,4 +529,16 @@ __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const f
       u32 in_dim, u32 rows0, u32 rows1, u32 rows2) {                                                           \
     const MfMany many = {w1, w2, out1, out2, rows1, rows2};                                                    \
     q4k_gemv_mfma_dispatch<M, false>(w0, x, nullptr, out0, in_dim, rows0, nullptr, &many);                     \
+  }
+// (w_gate, w_up, x, out, in_dim, out_dim): the parameters of q4_k_dual_gemv_swiglu_f32; M tokens at strides in_dim /
+// out_dim; out_dim a multiple of 16; two tiles per wavefront: grid = min(256, ceil(out_dim / 16 / row groups per workgroup))
+#define GEMV_MFMA_SWIGLU_ENTRY(NAME, M)                                                                        \
+  extern "C" __global__ __launch_bounds__(GEMV_MFMA_WAVES * 64) void NAME(const uint8_t* w_gate, const uint8_t* w_up, \
+                                                                         const float* x, float* out, u32 in_dim, \
+                                                                         u32 out_dim) {                        \
+    const MfMany many = {w_up, nullptr, nullptr, nullptr, out_dim, 0u};                                        \
+    if (gemv_mfma_chunked(M, in_dim))                                                                          \
+      q4k_gemv_mfma_core<M, false, 2, true, false, true>(w_gate, x, nullptr, out, in_dim, out_dim, nullptr, &many); \
+    else                                                                                                       \
+      q4k_gemv_mfma_core<M, false, 2, false, false, true>(w_gate, x, nullptr, out, in_dim, out_dim, nullptr, &many); \
   }

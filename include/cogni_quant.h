@@ -149,7 +149,10 @@ int cogni_swiglu_dev(uint64_t gate, uint64_t up, uint64_t out, uint32_t n, void*
  * i.e. the reference's gate/up GEMVs followed by swiglu_f32 (bin/cuda_ffn_sequence_probe.cr: FFN sequence) without
  * the intermediate vectors. Kernel "q4_k_dual_gemv_swiglu_f32" (w_gate, w_up, x, out, in_dim, out_dim): block and
  * dynamic shared memory as for one token of cogni_gemv_launch_dims, grid_x = ceil(out_dim / (rows per workgroup / 2)),
- * grid_y = tokens (one token per slice). Other types return COGNI_ERR_UNSUPPORTED_TYPE: compose
+ * grid_y = tokens (one token per slice). Several tokens with out_dim a multiple of 16 and a row length the matrix-core
+ * kernel takes: "q4_k_dual_gemv_swiglu_mfma_f32_tbatchM", same parameters, per group of up to four tokens, block 512,
+ * shared memory as cogni_gemv_plan gives for the token count, grid = min(256, out_dim / 16 / row groups per workgroup).
+ * Other types return COGNI_ERR_UNSUPPORTED_TYPE: compose
  * cogni_gemv_dual_dev and cogni_swiglu_dev. */
 int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t x, uint64_t out, uint32_t in_dim,
                                uint32_t out_dim, uint32_t tokens, void* stream);

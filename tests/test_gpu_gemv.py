@@ -373,6 +373,28 @@ def test_swiglu_kernel_and_fused_gate_up(gpu, oracle):
         assert np.max(np.abs(fused - ref)) <= 1e-4 * np.max(np.abs(ref))
         for d in (wg, wu, xd, og, ou, o2, of):
             d.close()
+    # several tokens, a multiple of 16 rows: the matrix-core kernel with gate and up tiles side by side; the same bits as
+    # the matrix-core pair kernel followed by swiglu_f32 on the same token groups (walking row groups, chunked activations,
+    # a last single token)
+    for in_dim, out_dim, tokens in ((4096, 12288, 4), (1024, 160, 7), (12288, 48, 3), (512, 48, 2), (2048, 8208, 5)):
+        raw_g = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+        raw_u = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+        x = synth.make_activations(rng, tokens, in_dim)
+        wg, wu, xd = DevArray(raw_g), DevArray(raw_u), DevArray(x)
+        n = tokens * out_dim
+        og, ou, o2, of = (DevArray(nbytes=4 * n) for _ in range(4))
+        quant.gemv_dual_dev(wg.ptr, wu.ptr, Q4_K, xd.ptr, og.ptr, ou.ptr, in_dim, out_dim, tokens)
+        quant.swiglu_dev(og.ptr, ou.ptr, o2.ptr, n)
+        quant.gemv_dual_swiglu_dev(wg.ptr, wu.ptr, Q4_K, xd.ptr, of.ptr, in_dim, out_dim, tokens)
+        fused, two_step = of.read(np.float32, n), o2.read(np.float32, n)
+        assert np.array_equal(fused, two_step), (in_dim, out_dim, tokens)
+        zero = np.zeros(out_dim, dtype=np.float32)
+        ref = oracle.swiglu(oracle.matmul_add(x, tokens, in_dim, raw_g, Q4_K, out_dim, zero, threads=8),
+                            oracle.matmul_add(x, tokens, in_dim, raw_u, Q4_K, out_dim, zero, threads=8))
+        assert cosine(fused, ref) >= 0.999999
+        assert np.max(np.abs(fused - ref)) <= 1e-4 * np.max(np.abs(ref))
+        for d in (wg, wu, xd, og, ou, o2, of):
+            d.close()
     with pytest.raises(quant.QuantError, match="Unsupported quant type for the fused gate/up SwiGLU: Q6_K"):
         quant.gemv_dual_swiglu_dev(1, 1, Q6_K, 1, 1, 256, 16, 1)
     for d in (gd, ud, od):
