@@ -253,10 +253,10 @@ int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, ui
   if (!kernel || !grid_x || !block_x || !shared_mem_bytes || !gemv_type(type) || tokens < 1 ||
       tokens > COGNI_MAX_GEMV_TOKENS || in_dim == 0 || out_dim == 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_plan: bad argument");
-  // two to four tokens of a Q4_K matrix and three or four of a Q6_K matrix go to the matrix-core kernels; one token
+  // two to four tokens of a Q4_K matrix and three or four of a Q5_K or Q6_K matrix go to the matrix-core kernels; one token
   // is faster on the vector ALU
   if (tokens >= 2 && gemv_mfma_supported(type, (int)tokens, in_dim)) {
-    std::snprintf(buf, sizeof buf, "q%c_k_gemv_mfma_%sf32_tbatch%u", type == COGNI_TYPE_Q6_K ? '6' : '4', add ? "add_" : "",
+    std::snprintf(buf, sizeof buf, "q%c_k_gemv_mfma_%sf32_tbatch%u", type == COGNI_TYPE_Q6_K ? '6' : (type == COGNI_TYPE_Q5_K ? '5' : '4'), add ? "add_" : "",
                   tokens);
     *kernel = buf;
     *grid_x = gemv_mfma_grid((int)tokens, in_dim, out_dim);
@@ -519,7 +519,8 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
     // three or four tokens of a Q4_K or Q6_K matrix: the matrix-core kernel with the arg-max inside, where its
     // workgroups fit the caller's partial buffers (sized for the vector-ALU kernels)
     const uint32_t mm = left < (uint32_t)GEMV_MFMA_MAX_TOKENS ? left : (uint32_t)GEMV_MFMA_MAX_TOKENS;
-    if (mm >= 3 && gemv_mfma_supported(w_type, (int)mm, in_dim) && gemv_mfma_grid((int)mm, in_dim, out_dim) <= stride) {
+    if (mm >= 3 && (w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q6_K) && gemv_mfma_supported(w_type, (int)mm, in_dim) &&
+        gemv_mfma_grid((int)mm, in_dim, out_dim) <= stride) {
       m = mm;
       grid = gemv_mfma_grid((int)m, in_dim, out_dim);
       block = GEMV_MFMA_WAVES * 64;

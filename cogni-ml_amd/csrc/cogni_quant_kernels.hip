@@ -33,3 +33,7 @@ GEMV_MFMA_MANY_ENTRY(q4_k_many_gemv_mfma_f32_tbatch4, 4)
 GEMV_MFMA_SWIGLU_ENTRY(q4_k_dual_gemv_swiglu_mfma_f32_tbatch2, 2)
 GEMV_MFMA_SWIGLU_ENTRY(q4_k_dual_gemv_swiglu_mfma_f32_tbatch3, 3)
 GEMV_MFMA_SWIGLU_ENTRY(q4_k_dual_gemv_swiglu_mfma_f32_tbatch4, 4)
+GEMV_MFMA_Q5K_ENTRY(q5_k_gemv_mfma_f32_tbatch3, 3)
+GEMV_MFMA_Q5K_ENTRY(q5_k_gemv_mfma_f32_tbatch4, 4)
+GEMV_MFMA_Q5K_ADD_ENTRY(q5_k_gemv_mfma_add_f32_tbatch3, 3)
+GEMV_MFMA_Q5K_ADD_ENTRY(q5_k_gemv_mfma_add_f32_tbatch4, 4)

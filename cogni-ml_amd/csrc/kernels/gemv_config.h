@@ -115,11 +115,11 @@ static inline GEMV_HD unsigned gemv_mfma_log2_kslices(unsigned nsb) {
 static inline GEMV_HD int gemv_mfma_chunked(int tokens, unsigned in_dim) {
   return (unsigned)tokens * (in_dim >> 8) > (unsigned)GEMV_MFMA_MAX_UNITS(tokens) && (in_dim & 2047u) == 0;
 }
-// Shapes the matrix-core kernels take: Q4_K with 1..4 tokens, Q6_K with 3 or 4 (its columns are laid out for four
+// Shapes the matrix-core kernels take: Q4_K with 1..4 tokens, Q5_K and Q6_K with 3 or 4 (its columns are laid out for four
 // tokens, and two are as fast on the vector ALU); in_dim a multiple of 256, all activations staged at once or in_dim a
 // multiple of 2048.
 static inline int gemv_mfma_supported(unsigned type, int tokens, unsigned in_dim) {
-  if ((type != 12 && type != 14) || tokens < (type == 14 ? 3 : 1) || tokens > GEMV_MFMA_MAX_TOKENS || in_dim == 0 ||
+  if ((type != 12 && type != 13 && type != 14) || tokens < (type == 12 ? 1 : 3) || tokens > GEMV_MFMA_MAX_TOKENS || in_dim == 0 ||
       (in_dim & 255u))
     return 0;
   return (unsigned)tokens * (in_dim >> 8) <= (unsigned)GEMV_MFMA_MAX_UNITS(tokens) || (in_dim & 2047u) == 0;

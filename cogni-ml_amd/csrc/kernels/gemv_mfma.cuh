@@ -77,7 +77,10 @@ struct MfMany {
 // SWIGLU (gate = w, up = many->w1, many->rows1 = out_dim, a multiple of 16): the tiles alternate gate tile p, up tile p,
 // so a wavefront with an even tile count holds both and the workgroup stores out[m][o] = silu(gate . x) * (up . x)
 // (swiglu_one, the function of swiglu_f32) - no gate or up vectors in memory.
-template <int M, bool ADD, int T, bool CHUNK = false, bool TOP1 = false, bool SWIGLU = false>
+// Q5: Q5_K blocks (176 B: the Q4_K header, qh[32], qs[128]): bit 2g / 2g + 1 of qh[l] is the fifth bit of the low /
+// high nibble of qs[32 g + l]; it is or-ed in beside the nibble (bit 4, or bit 8 next to a high nibble left in place),
+// so the codes 0..31 stay exact binary16 subnormals. One more 16-byte load per lane and super-block.
+template <int M, bool ADD, int T, bool CHUNK = false, bool TOP1 = false, bool SWIGLU = false, bool Q5 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float* x, const float* residual,
                                                    float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr,
                                                    const MfMany* many = nullptr) {
@@ -88,7 +91,7 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   const u32 total_rows = out_dim + rows1 + rows2;
   constexpr int MP = M <= 1 ? 1 : (M <= 2 ? 2 : 4);   // token slots in the column index
   constexpr int ND = MP;                              // accumulator tiles per 16 rows and super-block
-  constexpr int BB = 144;
+  constexpr int BB = Q5 ? 176 : 144, QOFF = Q5 ? 48 : 16;
   constexpr int NPRE = GEMV_MFMA_MAX_UNITS(M) / GEMV_MFMA_WAVES;   // staging units (token, super-block) per wavefront
   constexpr int C = NPRE / M;                                      // CHUNK: super-blocks of a k-slice staged at a time
   extern __shared__ uint4 mf_lds4[];
@@ -147,15 +150,16 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
   };
   set_rows(grp);
 
-  struct Stage { uint4 hdr, q0, q1; };
+  struct Stage { uint4 hdr, q0, q1, hq; };
   Stage stA[T];
   auto load_sb = [&](Stage* st, u32 sb) {
     const u32 off = sb * BB;
 #pragma unroll
     for (int t = 0; t < T; t++) {
       st[t].hdr = ld16(rowp[t] + off);
-      st[t].q0 = ld16(rowp[t] + (off + 16 + 16 * kg));
-      st[t].q1 = ld16(rowp[t] + (off + 80 + 16 * kg));
+      st[t].q0 = ld16(rowp[t] + (off + QOFF + 16 * kg));
+      st[t].q1 = ld16(rowp[t] + (off + QOFF + 64 + 16 * kg));
+      if constexpr (Q5) st[t].hq = ld16(rowp[t] + (off + 16 + 16 * (kg & 1)));
     }
   };
   // The activations are requested ahead of the weights, by every wavefront of the workgroup (hence the
@@ -325,6 +329,16 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
             a4.y = (wa >> 8) & mask;
             a4.z = wb & mask;
             a4.w = (wb >> 8) & mask;
+            if constexpr (Q5) {
+              const uint4 hq = st[tb0 + t].hq;
+              const u32 sh = 2 * (kg >> 1) + 4 * j + (t4 & 1);   // bit 2 g + (high nibble) of every qh byte, g = kg / 2 + 2 j
+              const u32 ba = (((t4 & 2) ? hq.z : hq.x) >> sh) & 0x01010101u, bb = (((t4 & 2) ? hq.w : hq.y) >> sh) & 0x01010101u;
+              const int up = (t4 & 1) ? 8 : 4;
+              a4.x |= (ba & 0x00010001u) << up;
+              a4.y |= ((ba >> 8) & 0x00010001u) << up;
+              a4.z |= (bb & 0x00010001u) << up;
+              a4.w |= ((bb >> 8) & 0x00010001u) << up;
+            }
             const int d = MP == 1 ? 0 : (MP == 2 ? (t4 & 1) : 2 * j + (t4 & 1));
             dacc[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mf_half8, a4),
                                                                 __builtin_bit_cast(mf_half8, breg[j * 4 + t4]),
@@ -473,7 +487,7 @@ __device__ __forceinline__ void q4k_gemv_mfma_core(const uint8_t* w, const float
 // The tile count per wavefront follows from the grid the host chose (gemv_mfma_grid); tile count and
 // round structure are template parameters so that register use and loads in flight are compile-time constants.
 // Shapes outside gemv_mfma_supported() must not be launched.
-template <int M, bool ADD, bool TOP1 = false>
+template <int M, bool ADD, bool TOP1 = false, bool Q5 = false>
 __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const float* x, const float* residual,
                                                        float* out, u32 in_dim, u32 out_dim, u32* top_ids = nullptr,
                                                        const MfMany* many = nullptr) {
@@ -483,14 +497,14 @@ __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const f
   const u32 ntiles = (out_dim + (many ? many->rows1 + many->rows2 : 0u) + 15) >> 4;
   const u32 t = (ntiles + gridDim.x * nwr - 1) / (gridDim.x * nwr);
   if (gemv_mfma_chunked(M, in_dim)) {
-    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
-    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
-    else q4k_gemv_mfma_core<M, ADD, 3, true, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+    if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, true, TOP1, false, Q5>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+    else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, true, TOP1, false, Q5>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+    else q4k_gemv_mfma_core<M, ADD, 3, true, TOP1, false, Q5>(w, x, residual, out, in_dim, out_dim, top_ids, many);
     return;
   }
-  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
-  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
-  else q4k_gemv_mfma_core<M, ADD, 3, false, TOP1>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+  if (t <= 1) q4k_gemv_mfma_core<M, ADD, 1, false, TOP1, false, Q5>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+  else if (t == 2) q4k_gemv_mfma_core<M, ADD, 2, false, TOP1, false, Q5>(w, x, residual, out, in_dim, out_dim, top_ids, many);
+  else q4k_gemv_mfma_core<M, ADD, 3, false, TOP1, false, Q5>(w, x, residual, out, in_dim, out_dim, top_ids, many);
 }
 
 #define GEMV_MFMA_ENTRY(NAME, M)                                                                              \
@@ -541,4 +555,16 @@ __device__ __forceinline__ void q4k_gemv_mfma_dispatch(const uint8_t* w, const f
       q4k_gemv_mfma_core<M, false, 2, true, false, true>(w_gate, x, nullptr, out, in_dim, out_dim, nullptr, &many); \
     else                                                                                                       \
       q4k_gemv_mfma_core<M, false, 2, false, false, true>(w_gate, x, nullptr, out, in_dim, out_dim, nullptr, &many); \
+  }
+// Q5_K: the same parameter lists as GEMV_MFMA_ENTRY / GEMV_MFMA_ADD_ENTRY
+#define GEMV_MFMA_Q5K_ENTRY(NAME, M)                                                                          \
+  extern "C" __global__ __launch_bounds__(GEMV_MFMA_WAVES * 64) void NAME(const uint8_t* w, const float* x,   \
+                                                                         float* out, u32 in_dim, u32 out_dim) { \
+    q4k_gemv_mfma_dispatch<M, false, false, true>(w, x, nullptr, out, in_dim, out_dim);                       \
+  }
+#define GEMV_MFMA_Q5K_ADD_ENTRY(NAME, M)                                                                      \
+  extern "C" __global__ __launch_bounds__(GEMV_MFMA_WAVES * 64) void NAME(const uint8_t* w, const float* x,   \
+                                                                         const float* residual, float* out,   \
+                                                                         u32 in_dim, u32 out_dim) {           \
+    q4k_gemv_mfma_dispatch<M, true, false, true>(w, x, residual, out, in_dim, out_dim);                       \
   }

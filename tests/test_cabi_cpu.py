@@ -121,7 +121,10 @@ def test_gemv_plan_picks_the_kernel_for_the_shape():
     assert quant.gemv_plan(14, 3, 12288, 4096, add=True)[0] == "q6_k_gemv_mfma_add_f32_tbatch3"
     assert quant.gemv_plan(14, 2, 4096, 4096)[0] == "q6_k_gemv_f32_tbatch2"
     assert quant.gemv_plan(14, 4, 8448, 4096)[0] == "q6_k_gemv_f32_tbatch4"
-    assert quant.gemv_plan(13, 4, 4096, 4096)[0] == "q5_k_gemv_f32_tbatch4"
+    assert quant.gemv_plan(13, 4, 4096, 4096)[0] == "q5_k_gemv_mfma_f32_tbatch4"     # Q5_K: as Q6_K, from three tokens
+    assert quant.gemv_plan(13, 3, 12288, 4096, add=True)[0] == "q5_k_gemv_mfma_add_f32_tbatch3"
+    assert quant.gemv_plan(13, 2, 4096, 4096)[0] == "q5_k_gemv_f32_tbatch2"          # two tokens: the vector-ALU pair is as fast
+    assert quant.gemv_plan(13, 4, 8448, 4096)[0] == "q5_k_gemv_f32_tbatch4"
     assert quant.gemv_plan(12, 8, 4096, 4096)[0] == "q4_k_gemv_f32_tbatch8"
     with pytest.raises(quant.QuantError):
         quant.gemv_plan(12, 9, 4096, 4096)

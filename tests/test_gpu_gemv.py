@@ -212,6 +212,39 @@ def test_q4_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
 
 
 @pytest.mark.parametrize("in_dim,out_dim", MFMA_SHAPES)
+@pytest.mark.parametrize("tokens", [2, 3, 4, 7])
+def test_q5_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
+    """Three and four tokens of a Q5_K matrix run through the Q4_K matrix-core kernel with the fifth bit or-ed in beside
+    the nibble (two tokens stay on the vector ALU): the same shape rule, with and without residual."""
+    rng = np.random.default_rng(in_dim * 139 + out_dim * 13 + tokens)
+    raw = synth.make_weights(rng, Q5_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = rng.standard_normal(tokens * out_dim).astype(np.float32)
+    m = min(tokens, 4)
+    name = quant.gemv_plan(Q5_K, m, in_dim, out_dim)[0]
+    expect_mfma = m >= 3 and (m * (in_dim // 256) <= 64 or in_dim % 2048 == 0)
+    assert name == ("q5_k_gemv_mfma_f32_tbatch%d" % m if expect_mfma else "q5_k_gemv_f32_tbatch%d" % m), name
+    check(oracle, raw, Q5_K, x, in_dim, out_dim, tokens, None, "%dx%d M=%d" % (in_dim, out_dim, tokens))
+    check(oracle, raw, Q5_K, x, in_dim, out_dim, tokens, res, "%dx%d M=%d add" % (in_dim, out_dim, tokens))
+
+
+def test_q5_k_matrix_core_kernel_element_order(gpu, oracle):
+    """One-hot activations pick single weights out of every position of a super-block: a fifth bit taken from the wrong
+    byte or bit position shows as a wrong value."""
+    rng = np.random.default_rng(79)
+    in_dim, out_dim, tokens = 512, 48, 4
+    raw = synth.make_weights(rng, Q5_K, out_dim, in_dim)
+    dense = oracle.dequantize(raw, Q5_K, out_dim * in_dim).reshape(out_dim, in_dim)
+    for base in range(0, in_dim, tokens):
+        x = np.zeros((tokens, in_dim), dtype=np.float32)
+        for m in range(tokens):
+            x[m, base + m] = 1.0
+        got = run_gemv(raw, Q5_K, np.ascontiguousarray(x.reshape(-1)), in_dim, out_dim, tokens).reshape(tokens, out_dim)
+        for m in range(tokens):
+            assert np.allclose(got[m], dense[:, base + m], rtol=0, atol=1e-5 * np.max(np.abs(dense))), (base, m)
+
+
+@pytest.mark.parametrize("in_dim,out_dim", MFMA_SHAPES)
 @pytest.mark.parametrize("tokens", [3, 4, 7])
 def test_q6_k_matrix_core_kernel_shapes(gpu, oracle, in_dim, out_dim, tokens):
     """Three and four tokens of a Q6_K matrix run on the matrix cores under the same shape rule as Q4_K (7 tokens:
