@@ -159,8 +159,9 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
         const float inv = __builtin_bit_cast(float, (u32)(127 - sh) << 23);
         const float s0 = v.x * scale, s1 = v.y * scale, s2 = v.z * scale, s3 = v.w * scale;
         const _Float16 h0 = (_Float16)s0, h1 = (_Float16)s1, h2 = (_Float16)s2, h3 = (_Float16)s3;
-        const _Float16 l0 = (_Float16)(s0 - (float)h0), l1 = (_Float16)(s1 - (float)h1),
-                       l2 = (_Float16)(s2 - (float)h2), l3 = (_Float16)(s3 - (float)h3);
+        // (x * scale is exact, so fma(x, scale, -hi) is the same value as (x * scale) - hi, in one mixed-precision instruction)
+        const _Float16 l0 = (_Float16)fmaf(v.x, scale, -(float)h0), l1 = (_Float16)fmaf(v.y, scale, -(float)h1),
+                       l2 = (_Float16)fmaf(v.z, scale, -(float)h2), l3 = (_Float16)fmaf(v.w, scale, -(float)h3);
         // k-slot order inside a run of 8 weights is 0,2,1,3,4,6,5,7 (how the nibble masks deliver them)
         typedef _Float16 h4 __attribute__((ext_vector_type(4)));
         const h4 hv = {h0, h2, h1, h3}, lv = {l0, l2, l1, l3};
