@@ -5,6 +5,7 @@ import os
 import re
 import struct
 
+import numpy as np
 import pytest
 
 from cogni_ml_amd import hip, quant
@@ -196,3 +197,38 @@ def test_runner_rejects_invalid_active_counts():
         r.run_repeated(0)
     r.reset_active_tokens()
     assert r.active_tokens == 4
+
+
+def test_matrix_core_gemv_grid_covers_every_row():
+    """The matrix-core kernels derive the tiles per wavefront from the grid they are launched with and cover rows
+    beyond one group per workgroup only by walking (not where the activations are staged in chunks): for a sweep of
+    shapes the planned grid must reach every 16-row tile under exactly those rules, and its LDS must fit a compute unit."""
+    def log2_kslices(nsb):
+        lg = 0
+        while lg < 3 and (2 << lg) <= nsb:
+            lg += 1
+        return lg
+    rng = np.random.default_rng(5)
+    shapes = [(4096, 12288), (12288, 4096), (4096, 151936), (256, 1), (256, 17), (512, 70003), (2048, 20011), (26624, 33),
+              (4096, 12288 + 48), (4096, 24576), (6144, 40), (8192, 300000)]
+    shapes += [(256 * int(rng.integers(1, 120)), int(rng.integers(1, 200000))) for _ in range(300)]
+    checked = 0
+    for t in (12, 13, 14):
+        for tokens in (2, 3, 4):
+            for in_dim, out_dim in shapes:
+                name, grid, block, lds = quant.gemv_plan(t, tokens, in_dim, out_dim)
+                if "mfma" not in name:
+                    continue
+                checked += 1
+                nsb = in_dim // 256
+                units = tokens * nsb
+                chunked = units > (64 if tokens >= 3 else 96)
+                assert not chunked or in_dim % 2048 == 0
+                nwr = 8 >> log2_kslices(nsb)
+                ntiles = (out_dim + 15) // 16
+                tk = -(-ntiles // (grid * nwr))                      # what the kernel computes from gridDim.x
+                T = 1 if tk <= 1 else (2 if tk == 2 else 3)
+                groups = -(-ntiles // (nwr * T))
+                assert block == 512 and 0 < grid <= groups and lds <= 160 * 1024, (name, in_dim, out_dim, grid)
+                assert grid == groups or (grid == 256 and not chunked), (name, in_dim, out_dim, grid, groups)
+    assert checked > 500
