@@ -4,17 +4,33 @@
 Headline (the JSON line on stdout): Q4_K decode GEMV, W = 12288 x 4096 (in_dim 4096 -> out_dim 12288,
 the ffn_gate/ffn_up shape), M = 1, fp32 activations and accumulation. One "step" is one GEMV launch.
 Weights are seeded synthetic super-blocks, already resident in HBM; consecutive steps read different
-copies of the matrix (more bytes in total than the 256 MB last-level cache) so every step streams
-its 28 MB from HBM. The K timed steps are captured into one HIP graph and bracketed by HIP events
-on the launch stream.
+copies of the matrix, and a copy comes round again only after more bytes than the 256 MB last-level
+cache holds, so every step streams its 28 MB from HBM.
+
+How a workload is timed (`measure`): the K = --steps launches are captured into HIP graphs; after the
+--warmup launches the graphs are replayed untimed for a fixed wall time (the clocks of an idle GPU take
+tens of milliseconds to come up, however few warm-up steps the caller asks for); then R samples are
+taken back to back, each one exactly K steps (or a whole number of replays of them when K steps are
+shorter than a couple of milliseconds), bracketed by HIP events on the launch stream. The figure
+reported is the median sample; min, max, R and the length of the timed region go into the line as well.
+The CPU baseline runs after the GPU work, so the GPU never waits idle in front of a timed region.
+
+The same line carries, under "cases", every other configuration (Q8_0 and the other K-quant GEMVs, the
+510 MB output head, the prefill GEMM at M = 64 / 512 / 2048, the projection stack at M = 1 / 4 / 8), each
+with its fraction of the roofline that bounds it and, for matrices under 16 MB, the time a kernel that
+only reads the same bytes takes.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
-  python bench.py --mode cases      per-shape table (key=value blocks, stderr) + the JSON line
+  python bench.py --mode cases      more shapes and fused sequences in the same line
   python bench.py --mode pmc        plain launches of the dominant kernel and of a copy kernel of
                                     known size, for rocprofv3 --pmc / --kernel-trace runs
+  python bench.py --mode pmc-gemm   plain launches of the M = 512 prefill GEMM for the same purpose
+  python bench.py --mode ceiling    empty launch, read-only stream, matrix-core-only loop
 """
 import argparse
+import ctypes
 import json
+import math
 import os
 import sys
 import time
@@ -28,12 +44,16 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E, published
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 matrix peak, published
-# HBM bytes one q4_k_gemv_f32 launch moves at 12288x4096, M=1: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# (13974.0 and 48.0 per dispatch), scaled by what a 512 MiB copy kernel reads on the same counters (2.0, 1.0)
-MEASURED_TRAFFIC_BYTES = int((13967.0 * 2.0 + 48.0 * 1.0) * 1024)
 LLC_BYTES = 256 << 20           # last-level (Infinity) cache
 Q4_K, Q5_K, Q6_K, Q8_0 = 12, 13, 14, 8
 TYPE_NAME = {Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", Q8_0: "Q8_0"}
+MEASURE_HSACO = os.path.join(ROOT, "cogni-ml_amd", "lib", "measure_kernels_gfx950.hsaco")
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+
+RAMP_MS = 150.0        # untimed replays right before the timed samples
+MIN_SAMPLE_MS = 2.0    # a sample is at least this long (whole replays of the K steps)
+MIN_TIMED_MS = 20.0    # all samples together
+MIN_SAMPLES, MAX_SAMPLES = 5, 60
 
 
 def log(*a):
@@ -45,16 +65,111 @@ def gemv_bytes(w_bytes, in_dim, out_dim, tokens):
     return w_bytes + 4 * tokens * in_dim + 4 * tokens * out_dim
 
 
+def rotation(steps, copies, needed):
+    """How `copies` buffers are walked by consecutive steps so that a buffer is read again only after `needed` others:
+    returns (C, G): step number n (counted across replays) reads buffer n % C, and G = C / gcd(steps, C) graphs of
+    `steps` launches each, replayed in turn, continue that sequence without a seam."""
+    best = None
+    for c in range(min(copies, max(1, needed)), copies + 1):
+        g = c // math.gcd(steps, c)
+        if best is None or g < best[1] or (g == best[1] and c > best[0]):
+            best = (c, g)
+    return best
+
+
+class Rotating:
+    """Launches that walk a set of equivalent buffers (weight copies, runner instances)."""
+
+    def __init__(self, launch, copies, bytes_per_copy):
+        self.launch, self.copies = launch, copies
+        # buffers that must be read in between before one comes round again: more than the last-level cache holds
+        self.needed = min(copies, max(2, int(math.ceil(1.1 * LLC_BYTES / max(1, bytes_per_copy)))))
+
+
+def measure(hip, stream, rot, steps, warmup, graph=True):
+    """Time `steps` launches of rot.launch(copy_index, stream) per sample; see the module docstring.
+    Returns a dict: us (median per step), us_min, us_max, samples, replays_per_sample, timed_region_ms, graphed."""
+    C, G = rotation(steps, rot.copies, rot.needed)
+    graphs, execs = [], []
+    if graph:
+        try:
+            for g in range(G):
+                stream.begin_capture(1)
+                for i in range(steps):
+                    rot.launch((g * steps + i) % C, stream)
+                gr = stream.end_capture()
+                graphs.append(gr)
+                ex = gr.instantiate()
+                ex.upload(stream)
+                execs.append(ex)
+            stream.synchronize()
+        except Exception as e:   # stream capture unavailable: direct launches
+            log("graph capture failed (%s); timing direct launches" % e)
+            for o in execs + graphs:
+                o.close()
+            graphs, execs = [], []
+    counter = [0]
+
+    def replay():
+        if execs:
+            execs[counter[0] % G].launch(stream)
+        else:
+            for i in range(steps):
+                rot.launch((counter[0] * steps + i) % C, stream)
+        counter[0] += 1
+
+    for i in range(warmup):
+        rot.launch(i % C, stream)
+    # a first estimate of one replay, then untimed replays for RAMP_MS
+    e0, e1 = hip.Event(), hip.Event()
+    stream.synchronize()
+    e0.record(stream)
+    replay()
+    e1.record(stream)
+    e1.synchronize()
+    est_ms = max(e0.elapsed_ms(e1), 1e-3)
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < RAMP_MS:
+        for _ in range(max(1, min(64, int(5.0 / est_ms)))):
+            replay()
+        stream.synchronize()
+    e0.record(stream)
+    replay()
+    e1.record(stream)
+    e1.synchronize()
+    est_ms = max(e0.elapsed_ms(e1), 1e-3)
+    inner = max(1, int(math.ceil(MIN_SAMPLE_MS / est_ms)))
+    samples = int(min(MAX_SAMPLES, max(MIN_SAMPLES, math.ceil(MIN_TIMED_MS / (inner * est_ms)))))
+    # keep the GPU busy between the estimate and the samples, then enqueue every sample without a host wait in between
+    events = [hip.Event() for _ in range(samples + 1)]
+    for _ in range(inner):
+        replay()
+    events[0].record(stream)
+    for s in range(samples):
+        for _ in range(inner):
+            replay()
+        events[s + 1].record(stream)
+    events[-1].synchronize()
+    hip.synchronize()
+    per_step_us = sorted(events[s].elapsed_ms(events[s + 1]) * 1e3 / (inner * steps) for s in range(samples))
+    region_ms = events[0].elapsed_ms(events[-1])
+    for o in execs + graphs + events + [e0, e1]:
+        o.close()
+    return {"us": per_step_us[len(per_step_us) // 2], "us_min": per_step_us[0], "us_max": per_step_us[-1],
+            "samples": samples, "replays_per_sample": inner, "timed_region_ms": region_ms, "graphed": bool(execs),
+            "buffers_rotated": C}
+
+
 class GemvCase:
     """Rotating weight copies + activations + output for one (type, shape, tokens)."""
 
-    def __init__(self, hip, quant, synth, rng, w_type, out_dim, in_dim, tokens, min_total_bytes=2 * LLC_BYTES,
-                 max_copies=24):
+    def __init__(self, hip, quant, synth, rng, w_type, out_dim, in_dim, tokens, min_total_bytes=2 * LLC_BYTES + (32 << 20),
+                 max_copies=96):
         from cogni_ml_amd.types import TensorType
         self.hip, self.quant = hip, quant
         self.w_type, self.out_dim, self.in_dim, self.tokens = w_type, out_dim, in_dim, tokens
         self.w_bytes = TensorType(w_type).data_bytes(in_dim) * out_dim
-        self.copies = int(max(1, min(max_copies, -(-min_total_bytes // self.w_bytes))))
+        self.copies = int(max(2, min(max_copies, -(-min_total_bytes // self.w_bytes))))
         self.host_w = synth.make_weights(rng, w_type, out_dim, in_dim)
         self.host_x = synth.make_activations(rng, tokens, in_dim)
         self.w = []
@@ -70,9 +185,12 @@ class GemvCase:
         self.out = hip.DeviceBuffer(4 * tokens * out_dim)
         self.bytes_per_step = gemv_bytes(self.w_bytes, in_dim, out_dim, tokens)
 
-    def launch(self, step, stream):
-        self.quant.gemv_dev(self.w[step % self.copies].ptr, self.w_type, self.x.ptr, self.out.ptr, self.in_dim,
+    def launch(self, copy, stream):
+        self.quant.gemv_dev(self.w[copy].ptr, self.w_type, self.x.ptr, self.out.ptr, self.in_dim,
                             self.out_dim, self.tokens, 0, stream.handle)
+
+    def rotating(self):
+        return Rotating(self.launch, self.copies, self.w_bytes)
 
     def read_out(self):
         out = np.empty(self.tokens * self.out_dim, dtype=np.float32)
@@ -85,66 +203,66 @@ class GemvCase:
             b.close()
 
 
-def time_steps(hip, stream, launch, steps, warmup, graph=True):
-    """Run `warmup` untimed and exactly `steps` timed launches on `stream`; returns ms for the timed region.
-    The timed launches are captured into one HIP graph so host launch latency does not gate the GPU."""
-    graph_wanted = bool(graph)
-    graph, exe = None, None
-    try:
-        if not graph_wanted:
-            raise RuntimeError("direct launches requested")
-        stream.begin_capture(1)
-        for i in range(steps):
-            launch(warmup + i, stream)
-        graph = stream.end_capture()
-        exe = graph.instantiate()
-        exe.upload(stream)
-        stream.synchronize()
-    except Exception as e:  # stream capture unavailable or not wanted: direct launches
-        if graph_wanted:
-            log("graph capture failed (%s); timing direct launches" % e)
-        graph, exe = None, None
-    # the warm-up runs once the graph is built, directly ahead of the timed region: capture and instantiation are
-    # host work during which the GPU would otherwise sit idle and drop its clocks
-    for i in range(warmup):
-        launch(i, stream)
-    e0, e1 = hip.Event(), hip.Event()
-    hip.synchronize()
-    e0.record(stream)
-    if exe is not None:
-        exe.launch(stream)
-    else:
-        for i in range(steps):
-            launch(warmup + i, stream)
-    e1.record(stream)
-    e1.synchronize()
-    hip.synchronize()
-    ms = e0.elapsed_ms(e1)
-    for o in (exe, graph):
-        if o is not None:
-            o.close()
-    e0.close()
-    e1.close()
-    return ms, exe is not None
+class MeasureKernels:
+    """The bench-only code object: copy, read-only stream, matrix-core loop."""
+
+    def __init__(self, hip):
+        if not os.path.exists(MEASURE_HSACO):
+            raise RuntimeError("%s is missing: run __graft_entry__.build() first" % MEASURE_HSACO)
+        self.hip = hip
+        self.mod = hip.HIPModule.load(open(MEASURE_HSACO, "rb").read(), "measure_kernels_gfx950")
+        self.sink = hip.DeviceBuffer(4 * 65536)
+
+    def fn(self, name):
+        return self.mod.function(name)
+
+    def read_floor(self, stream, case, steps, warmup):
+        """Best time of a kernel that only reads the weight bytes of `case` (same rotating buffers): (us, grid)."""
+        read_fn = self.fn("read_bytes_16")
+        best = None
+        for grid in (256, 512, 1024, 2048, 4096):
+            if grid * 256 * 16 > 2 * case.w_bytes and grid > 256:
+                break
+            boxes = [self.hip.KernelParams(ctypes.c_uint64(b.ptr), ctypes.c_uint64(self.sink.ptr),
+                                           ctypes.c_uint64(case.w_bytes & ~15)) for b in case.w]
+
+            def rd(copy, st, grid=grid, boxes=boxes):
+                with self.hip.with_stream(st):
+                    self.hip.launch(read_fn, grid, 1, 1, 256, 1, 1, boxes[copy], "read")
+            r = measure(self.hip, stream, Rotating(rd, case.copies, case.w_bytes), steps, warmup)
+            if best is None or r["us"] < best[0]:
+                best = (r["us"], grid)
+        return best
 
 
-def bench_gemm(hip, quant, synth, rng, stream, tokens, out_dim, in_dim, steps, warmup, graph=True, Q4_K=Q4_K):
-    """Prefill GEMM (x repack + MFMA kernel) at `tokens`, Q4_K unless another type is given; returns (ms per call, TFLOP/s)."""
-    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+def gemv_record(r, bytes_per_step):
+    gbps = bytes_per_step / r["us"] / 1e3
+    return {"us": round(r["us"], 3), "us_min": round(r["us_min"], 3), "us_max": round(r["us_max"], 3),
+            "gbps": round(gbps, 1), "frac_hbm": round(gbps / HBM_PEAK_GBPS, 4), "bytes": bytes_per_step,
+            "samples": r["samples"], "timed_region_ms": round(r["timed_region_ms"], 2)}
+
+
+def bench_gemm(hip, quant, synth, rng, stream, w_type, tokens, out_dim, in_dim, steps, warmup, graph=True):
+    """Prefill GEMM (x repack + MFMA kernel, every launch of the call) at `tokens`; returns the case record."""
+    raw = synth.make_weights(rng, w_type, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
-    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens, out_dim)
+    wsb = quant.gemm_workspace_bytes(w_type, in_dim, tokens, out_dim)
     bufs = [hip.DeviceBuffer(n) for n in (raw.nbytes, x.nbytes, 4 * tokens * out_dim, wsb)]
     hip.copy_htod(bufs[0].ptr, raw, raw.nbytes, "w")
     hip.copy_htod(bufs[1].ptr, x, x.nbytes, "x")
 
-    def launch(i, st):
-        quant.gemm_dev(bufs[0].ptr, Q4_K, bufs[1].ptr, bufs[2].ptr, in_dim, out_dim, tokens, bufs[3].ptr, wsb, 0,
+    def launch(copy, st):
+        quant.gemm_dev(bufs[0].ptr, w_type, bufs[1].ptr, bufs[2].ptr, in_dim, out_dim, tokens, bufs[3].ptr, wsb, 0,
                        st.handle)
-    ms, _ = time_steps(hip, stream, launch, steps, warmup, graph)
+    r = measure(hip, stream, Rotating(launch, 1, raw.nbytes), steps, warmup, graph)
     for b in bufs:
         b.close()
-    per = ms / steps
-    return per, 2.0 * tokens * out_dim * in_dim / (per * 1e-3) / 1e12
+    flops = 2.0 * tokens * out_dim * in_dim
+    tf = flops / r["us"] / 1e6
+    return {"us": round(r["us"], 2), "us_min": round(r["us_min"], 2), "us_max": round(r["us_max"], 2),
+            "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
+            "samples": r["samples"], "timed_region_ms": round(r["timed_region_ms"], 2),
+            "includes": "activation repack + GEMM (+ plane sum where the k range is split)"}
 
 
 def cpu_baseline(oracle, case, budget_s=10.0, threads=1):
@@ -162,11 +280,26 @@ def cpu_baseline(oracle, case, budget_s=10.0, threads=1):
     return ref, reps, el
 
 
+def recorded_traffic():
+    """HBM bytes per launch of the headline kernel as the profiler counted them, from profiles/traffic.json (written
+    from two rocprofv3 --pmc runs; the file names the commit and the command). None if there is no record."""
+    try:
+        rec = json.load(open(TRAFFIC_JSON))
+        return int(rec["bytes_per_launch"]), rec
+    except Exception as e:
+        log("no recorded traffic (%s)" % e)
+        return None, None
+
+
+def steps_for(args, bytes_per_step, cap_bytes=6e9):
+    return int(max(4, min(args.steps, cap_bytes // max(1, bytes_per_step))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--mode", choices=["headline", "cases", "pmc", "pmc-gemm", "ceiling"], default="headline")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--seed", type=int, default=1234)
@@ -179,6 +312,7 @@ def main():
     from cogni_ml_amd import hip, quant, synth
     from oracle import oracle
 
+    t_start = time.perf_counter()
     ctx = hip.Context.create(0)
     quant.init(0)
     log("device=%s arch=%s compute_units=%d clock_mhz=%d host_cores=%d" % (
@@ -188,8 +322,8 @@ def main():
 
     if args.mode == "pmc-gemm":
         # plain launches of the prefill GEMM (M = 512) for profiler runs
-        per, tf = bench_gemm(hip, quant, synth, rng, stream, 512, 12288, 4096, args.steps, args.warmup, graph=False)
-        log("pmc-gemm mode: M=512 ms=%.5f tflops=%.1f" % (per, tf))
+        rec = bench_gemm(hip, quant, synth, rng, stream, Q4_K, 512, 12288, 4096, args.steps, args.warmup, graph=False)
+        log("pmc-gemm mode: M=512 us=%.2f tflops=%.1f" % (rec["us"], rec["tflops"]))
         return
 
     head = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1)
@@ -197,15 +331,14 @@ def main():
     if args.mode == "pmc":
         # plain (uncaptured) launches so a profiler attributes counters per dispatch; the copy kernel moves a
         # known number of bytes and calibrates the counters' units
-        mod = hip.HIPModule.load_builtin()
-        copy_fn = mod.function("copy_bytes_16")
-        import ctypes
+        mk = MeasureKernels(hip)
+        copy_fn = mk.fn("copy_bytes_16")
         nbytes = 512 << 20
         src, dst = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(nbytes)
         params = hip.KernelParams(ctypes.c_uint64(src.ptr), ctypes.c_uint64(dst.ptr), ctypes.c_uint64(nbytes))
         with hip.with_stream(stream):
             for i in range(args.warmup + args.steps):
-                head.launch(i, stream)
+                head.launch(i % head.copies, stream)
             for i in range(8):
                 hip.launch(copy_fn, 8192, 1, 1, 256, 1, 1, params, "copy_bytes_16")
         stream.synchronize()
@@ -216,27 +349,24 @@ def main():
     if args.mode == "ceiling":
         # what the machine gives a trivial kernel under the same timing method: an empty launch, and a
         # read-only stream over the same rotating weight buffers
-        import ctypes
-        mod = hip.HIPModule.load_builtin()
-        copy_fn, read_fn = mod.function("copy_bytes_16"), mod.function("read_bytes_16")
-        sink = hip.DeviceBuffer(4 * 65536)
-        nul = hip.KernelParams(ctypes.c_uint64(head.w[0].ptr), ctypes.c_uint64(sink.ptr), ctypes.c_uint64(0))
+        mk = MeasureKernels(hip)
+        copy_fn, read_fn = mk.fn("copy_bytes_16"), mk.fn("read_bytes_16")
+        nul = hip.KernelParams(ctypes.c_uint64(head.w[0].ptr), ctypes.c_uint64(mk.sink.ptr), ctypes.c_uint64(0))
 
-        def empty(i, st):
+        def empty(copy, st):
             with hip.with_stream(st):
                 hip.launch(copy_fn, 768, 1, 1, 256, 1, 1, nul, "empty")
-        ms, _ = time_steps(hip, stream, empty, args.steps, args.warmup)
-        log("empty_kernel_us=%.3f" % (ms / args.steps * 1e3))
+        r = measure(hip, stream, Rotating(empty, 1, 1 << 30), args.steps, args.warmup)
+        log("empty_kernel_us=%.3f" % r["us"])
         for grid in (256, 512, 1024, 2048, 4096, 8192):
-            boxes = [hip.KernelParams(ctypes.c_uint64(b.ptr), ctypes.c_uint64(sink.ptr), ctypes.c_uint64(head.w_bytes))
+            boxes = [hip.KernelParams(ctypes.c_uint64(b.ptr), ctypes.c_uint64(mk.sink.ptr), ctypes.c_uint64(head.w_bytes))
                      for b in head.w]
 
-            def rd(i, st, grid=grid, boxes=boxes):
+            def rd(copy, st, grid=grid, boxes=boxes):
                 with hip.with_stream(st):
-                    hip.launch(read_fn, grid, 1, 1, 256, 1, 1, boxes[i % len(boxes)], "read")
-            ms, _ = time_steps(hip, stream, rd, args.steps, args.warmup)
-            us = ms / args.steps * 1e3
-            log("read_only grid=%d us=%.3f gbps=%.1f" % (grid, us, head.w_bytes / us / 1e3))
+                    hip.launch(read_fn, grid, 1, 1, 256, 1, 1, boxes[copy], "read")
+            r = measure(hip, stream, Rotating(rd, head.copies, head.w_bytes), args.steps, args.warmup)
+            log("read_only grid=%d us=%.3f gbps=%.1f" % (grid, r["us"], head.w_bytes / r["us"] / 1e3))
         # a loop of nothing but fp16 MFMAs on every SIMD of the chip, one and two wavefronts per SIMD, short and long
         # (the clock the chip sustains under that load is part of the answer)
         ops = hip.DeviceBuffer(7 * 64 * 16)
@@ -244,90 +374,117 @@ def main():
         hip.copy_htod(ops.ptr, vals, vals.nbytes, "mfma operands")
         res = hip.DeviceBuffer(4 * 512 * 1024)
         for name, block in (("mfma_f16_ceiling_w4", 256), ("mfma_f16_ceiling_w8", 512)):
-            fn = mod.function(name)
+            fn = mk.fn(name)
             for wgs in (256, 1024):
                 for iters in (128, 1024):
                     box = hip.KernelParams(ctypes.c_uint64(ops.ptr), ctypes.c_uint64(res.ptr), ctypes.c_uint32(iters))
 
-                    def mm(i, st, fn=fn, wgs=wgs, block=block, box=box):
+                    def mm(copy, st, fn=fn, wgs=wgs, block=block, box=box):
                         with hip.with_stream(st):
                             hip.launch(fn, wgs, 1, 1, block, 1, 1, box, "mfma")
-                    reps = 20
-                    ms, _ = time_steps(hip, stream, mm, reps, 3)
-                    us = ms / reps * 1e3
+                    r = measure(hip, stream, Rotating(mm, 1, 1 << 30), 20, 3)
                     flops = 2.0 * 32 * 32 * 16 * 12 * iters * (block // 64) * wgs
                     log("%s workgroups=%d iters=%d us=%.2f tflops=%.1f frac_of_published_peak=%.3f" % (
-                        name, wgs, iters, us, flops / us / 1e6, flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS))
+                        name, wgs, iters, r["us"], flops / r["us"] / 1e6, flops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS))
         return
 
-    # ---- parity spot check of the measured kernel against the oracle, and the CPU baseline ------------
+    mk = MeasureKernels(hip)
+    cases = {}
+
+    # ---- the headline: timed first, checked against the oracle afterwards -------------------------------------
     head.launch(0, stream)
     stream.synchronize()
     got = head.read_out()
-    ref, cpu_reps, cpu_s = cpu_baseline(oracle, head, args.cpu_seconds)
-    dense_max = float(np.max(np.abs(oracle.dequantize(head.host_w[:16 * 144 * 256], Q4_K, 256 * 4096))))
-    max_diff = float(np.max(np.abs(got - ref)))
-    cos = float(got.astype(np.float64) @ ref.astype(np.float64) /
-                np.sqrt((got.astype(np.float64) @ got.astype(np.float64)) * (ref.astype(np.float64) @ ref.astype(np.float64))))
-    ok = cos >= 0.99999 and max_diff <= 1e-3
-    cpu_gbps = head.bytes_per_step * cpu_reps / cpu_s / 1e9
-    # the same restatement with the rows divided among the host cores this job may use (16 on a one-GPU box)
-    mt_cores = max(1, min(16, os.cpu_count() or 1))
-    _, mt_reps, mt_s = cpu_baseline(oracle, head, min(3.0, args.cpu_seconds), threads=mt_cores)
-    mt_gbps = head.bytes_per_step * mt_reps / mt_s / 1e9
-    log("cpu_baseline: 1 thread %.4f GB/s (%d reps, %.1f s); %d threads %.4f GB/s (%d reps, %.1f s); gcc -O2 -ffp-contract=off, "
-        "stands in for the reference's Crystal QuantMatmul" % (cpu_gbps, cpu_reps, cpu_s, mt_cores, mt_gbps, mt_reps, mt_s))
-
-    # ---- timed region ------------------------------------------------------------------------------------
-    ms, graphed = time_steps(hip, stream, head.launch, args.steps, args.warmup)
-    ms_per_step = ms / args.steps
-    gbps = head.bytes_per_step / (ms_per_step * 1e-3) / 1e9
-
+    hr = measure(hip, stream, head.rotating(), args.steps, args.warmup)
+    ms_per_step = hr["us"] * 1e-3
+    gbps = head.bytes_per_step / hr["us"] / 1e3
     # cache-resident figure (one copy only), reported beside the HBM one
-    hot_ms, _ = time_steps(hip, stream, lambda i, s: head.launch(0, s), args.steps, args.warmup)
-    hot_gbps = head.bytes_per_step / (hot_ms / args.steps * 1e-3) / 1e9
-
+    hot = measure(hip, stream, Rotating(lambda c, s: head.launch(0, s), 1, head.w_bytes), args.steps, args.warmup)
+    hot_gbps = head.bytes_per_step / hot["us"] / 1e3
+    floor_us, floor_grid = mk.read_floor(stream, head, args.steps, args.warmup)
     log("case=q4_k_gemv ffn_up\ntype=Q4_K\nshape=%dx%d\ntokens=1\nraw_bytes=%d\ncopies=%d\nreps=%d\nwarmup=%d\n"
-        "hip_ms=%.5f\ncpu_ms=%.3f\ncos=%.8f\nmax_diff=%g\nok=%s\ngbps_hbm=%.1f\ngbps_cache_hot=%.1f\ngraph=%s" % (
-            head.in_dim, head.out_dim, head.w_bytes, head.copies, args.steps, args.warmup, ms_per_step,
-            cpu_s / cpu_reps * 1e3, cos, max_diff, str(ok).lower(), gbps, hot_gbps, graphed))
+        "hip_us=%.3f\nhip_us_min=%.3f\nhip_us_max=%.3f\nsamples=%d\ngbps_hbm=%.1f\ngbps_cache_hot=%.1f\nread_only_us=%.3f\ngraph=%s" % (
+            head.in_dim, head.out_dim, head.w_bytes, hr["buffers_rotated"], args.steps, args.warmup, hr["us"], hr["us_min"],
+            hr["us_max"], hr["samples"], gbps, hot_gbps, floor_us, hr["graphed"]))
 
+    def gemv_case(name, w_type, out_dim, in_dim, tokens, floor=None):
+        c = GemvCase(hip, quant, synth, rng, w_type, out_dim, in_dim, tokens)
+        steps = steps_for(args, c.bytes_per_step)
+        r = measure(hip, stream, c.rotating(), steps, min(args.warmup, steps))
+        rec = gemv_record(r, c.bytes_per_step)
+        rec["steps"] = steps
+        if floor if floor is not None else c.w_bytes < (16 << 20):
+            fu, fg = mk.read_floor(stream, c, steps, min(args.warmup, steps))
+            rec["read_only_us"] = round(fu, 3)
+            rec["x_read_only"] = round(r["us"] / fu, 3)
+        cases[name] = rec
+        log("case=%s\ntype=%s\nshape=%dx%d\ntokens=%d\nraw_bytes=%d\ncopies=%d\nreps=%d\nhip_us=%.3f\ngbps_hbm=%.1f\nfrac_hbm=%.4f\n%s" % (
+            name, TYPE_NAME[w_type], in_dim, out_dim, tokens, c.w_bytes, r["buffers_rotated"], steps, r["us"], rec["gbps"],
+            rec["frac_hbm"], "read_only_us=%.3f\n" % rec["read_only_us"] if "read_only_us" in rec else ""))
+        c.close()
+
+    # config 1, the rest of config 2, config 3
+    gemv_case("cfg1 q8_0 gemv 3584x1024 M=1", Q8_0, 3584, 1024, 1)
+    gemv_case("cfg2 q4_k gemv down 4096x12288 M=1", Q4_K, 4096, 12288, 1)
+    gemv_case("cfg3 q6_k gemv output head 151936x4096 M=1", Q6_K, 151936, 4096, 1)
+    gemv_case("cfg3 q6_k gemv down 4096x12288 M=1", Q6_K, 4096, 12288, 1)
+    gemv_case("cfg3 q5_k gemv 4096x4096 M=1", Q5_K, 4096, 4096, 1)
+    # several tokens against one pass over the weights (what config 5's row batches are made of)
+    gemv_case("q4_k gemv 12288x4096 M=4", Q4_K, 12288, 4096, 4)
+    gemv_case("q4_k gemv 12288x4096 M=8", Q4_K, 12288, 4096, 8)
+    if args.mode == "cases":
+        gemv_case("q4_k gemv 4096x12288 M=4", Q4_K, 4096, 12288, 4)
+        gemv_case("q4_k gemv 4096x12288 M=8", Q4_K, 4096, 12288, 8)
+        gemv_case("q6_k gemv 4096x12288 M=4", Q6_K, 4096, 12288, 4)
+        gemv_case("q6_k gemv 4096x12288 M=8", Q6_K, 4096, 12288, 8)
+        gemv_case("q5_k gemv 4096x4096 M=4", Q5_K, 4096, 4096, 4)
+
+    # config 4: prefill GEMM
     gemm = {}
-    for tokens in ((64, 512, 2048) if args.mode == "cases" else (512,)):
-        gsteps = max(10, min(200, args.steps // 10))
-        per, tf = bench_gemm(hip, quant, synth, rng, stream, tokens, 12288, 4096, gsteps, 5)
-        gemm["M=%d" % tokens] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
-        log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
-            tokens, gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
-
+    for tokens in (64, 512, 2048):
+        gsteps = max(5, min(100, args.steps, int(4e12 // (2.0 * tokens * 12288 * 4096))))
+        rec = bench_gemm(hip, quant, synth, rng, stream, Q4_K, tokens, 12288, 4096, gsteps, min(5, args.warmup))
+        rec["steps"] = gsteps
+        gemm["M=%d" % tokens] = rec
+        cases["cfg4 q4_k gemm 12288x4096 M=%d" % tokens] = rec
+        log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
+            tokens, gsteps, rec["us"], rec["tflops"], rec["frac_mfma_f16"]))
     if args.mode == "cases":
-        gsteps = max(10, min(200, args.steps // 10))
-        per, tf = bench_gemm(hip, quant, synth, rng, stream, 512, 4096, 12288, gsteps, 5, Q4_K=Q6_K)
-        gemm["q6_k down 4096x12288 M=512"] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
-        log("case=q6_k_gemm prefill\ntype=Q6_K\nshape=12288x4096\ntokens=512\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
-            gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
-        per, tf = bench_gemm(hip, quant, synth, rng, stream, 512, 12288, 4096, gsteps, 5, Q4_K=Q5_K)
-        gemm["q5_k 12288x4096 M=512"] = {"ms": round(per, 5), "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4)}
-        log("case=q5_k_gemm prefill\ntype=Q5_K\nshape=4096x12288\ntokens=512\nreps=%d\nhip_ms=%.5f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
-            gsteps, per, tf, tf / MFMA_F16_PEAK_TFLOPS))
+        for name, t, o, i in (("q6_k gemm down 4096x12288 M=512", Q6_K, 4096, 12288), ("q5_k gemm 12288x4096 M=512", Q5_K, 12288, 4096)):
+            rec = bench_gemm(hip, quant, synth, rng, stream, t, 512, o, i, 50, 5)
+            cases[name] = rec
+            log("case=%s\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (name, rec["us"], rec["tflops"], rec["frac_mfma_f16"]))
 
-    extra = {}
-    if args.mode == "cases":
-        table = [
-            ("q8_0 ffn_up 0.8B", Q8_0, 3584, 1024, 1), ("q4_k ffn_down", Q4_K, 4096, 12288, 1),
-            ("q6_k ffn_down", Q6_K, 4096, 12288, 1), ("q5_k attn_qkv-like", Q5_K, 4096, 4096, 1),
-            ("q6_k output head", Q6_K, 151936, 4096, 1),
-            ("q4_k ffn_up M=4", Q4_K, 12288, 4096, 4), ("q4_k ffn_up M=8", Q4_K, 12288, 4096, 8),
-        ]
-        for name, t, out_dim, in_dim, tokens in table:
-            c = GemvCase(hip, quant, synth, rng, t, out_dim, in_dim, tokens)
-            steps = max(20, min(args.steps, int(2e9 // c.bytes_per_step)))
-            cms, _ = time_steps(hip, stream, c.launch, steps, min(args.warmup, steps))
-            cg = c.bytes_per_step / (cms / steps * 1e-3) / 1e9
-            extra[name] = {"gbps": round(cg, 1), "ms": round(cms / steps, 5), "frac_hbm": round(cg / HBM_PEAK_GBPS, 4)}
-            log("case=%s\ntype=%s\nshape=%dx%d\ntokens=%d\nraw_bytes=%d\ncopies=%d\nreps=%d\nhip_ms=%.5f\ngbps_hbm=%.1f\n" % (
-                name, TYPE_NAME[t], in_dim, out_dim, tokens, c.w_bytes, c.copies, steps, cms / steps, cg))
-            c.close()
+    # config 5: the mixed-quant projection stack, back to back in one stream. Three resident layers are walked in turn
+    # (364 MB of weights), so that a layer's weights come from HBM as they do in a model of many layers; the figure
+    # with one layer alone (121.5 MB, which the last-level cache keeps between repetitions) is reported beside it.
+    from cogni_ml_amd.projection_stack import QwenProjectionStackRunner, Weights
+    layers = [Weights.synthetic(rng) for _ in range(3)]
+    for tokens in (1, 4, 8):
+        xs = synth.make_activations(rng, tokens, layers[0].hidden)
+        runners = [QwenProjectionStackRunner.from_weights(w, tokens, xs) for w in layers]
+        for r_ in runners:
+            r_.upload_weights()
+            r_.reset_sequence()
+
+        def seq(copy, st, runners=runners):
+            with hip.with_stream(st):
+                runners[copy].run_sequence()
+        nbytes = runners[0].bytes_per_sequence()
+        steps = max(6, min(args.steps, 300))
+        r = measure(hip, stream, Rotating(seq, 3, layers[0].raw_bytes), steps, min(args.warmup, 10))
+        rec = gemv_record(r, nbytes)
+        rec["steps"] = steps
+        r1 = measure(hip, stream, Rotating(seq, 1, layers[0].raw_bytes), steps, min(args.warmup, 10))
+        rec["us_cache_resident"] = round(r1["us"], 3)
+        rec["gbps_cache_resident"] = round(nbytes / r1["us"] / 1e3, 1)
+        rec["launches_per_sequence"] = "q|k|v, o, gate|up, down per group of tokens"
+        cases["cfg5 projection stack M=%d" % tokens] = rec
+        log("case=projection stack (q,k,v,o,gate,up Q4_K + down Q6_K)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_us=%.3f\n"
+            "gbps_hbm=%.1f\nfrac_hbm=%.4f\nhip_us_cache_resident=%.3f\n" % (
+                tokens, layers[0].raw_bytes, steps, r["us"], rec["gbps"], rec["frac_hbm"], r1["us"]))
+        for r_ in runners:
+            r_.close()
 
     if args.mode == "cases":
         # output head without the logits: RMSNorm -> Q6_K vocabulary projection with arg-max -> top-1 reduce (510 MB)
@@ -338,38 +495,28 @@ def main():
             ohead.upload_weights()
             ohead.reset_sequence()
 
-            def hseq(i, st, ohead=ohead):
+            def hseq(copy, st, ohead=ohead):
                 with hip.with_stream(st):
                     ohead.run_sequence()
-            reps = 20
-            hms, _ = time_steps(hip, stream, hseq, reps, 3)
-            hg = ohead.bytes_per_sequence() / (hms / reps * 1e-3) / 1e9
-            extra["q6_k output head top-1 M=%d" % tokens] = {"gbps": round(hg, 1), "ms": round(hms / reps, 5), "frac_hbm": round(hg / HBM_PEAK_GBPS, 4)}
-            log("case=output head top-1 (rmsnorm -> q6_k gemv top1 partial -> reduce)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\ngbps_hbm=%.1f\n" % (
-                tokens, hw.output_raw.size, reps, hms / reps, hg))
+            r = measure(hip, stream, Rotating(hseq, 1, hw.output_raw.size), 10, 3)
+            cases["q6_k output head top-1 M=%d" % tokens] = gemv_record(r, ohead.bytes_per_sequence())
+            log("case=output head top-1 (rmsnorm -> q6_k gemv top1 partial -> reduce)\ntokens=%d\nhip_us=%.3f\n" % (tokens, r["us"]))
             ohead.close()
 
-    if args.mode == "cases":
         # the gate | up pair of one layer against the same x in one launch (q4_k_dual_gemv_f32)
-        a = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES)
-        b = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES)
+        a = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES + (32 << 20))
+        b = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1, min_total_bytes=LLC_BYTES + (32 << 20))
         out_b = hip.DeviceBuffer(4 * 12288)
 
-        def dual(i, st):
-            quant.gemv_dual_dev(a.w[i % a.copies].ptr, b.w[i % b.copies].ptr, Q4_K, a.x.ptr, a.out.ptr, out_b.ptr, 4096, 12288,
-                                1, st.handle)
+        def dual(copy, st):
+            quant.gemv_dual_dev(a.w[copy].ptr, b.w[copy].ptr, Q4_K, a.x.ptr, a.out.ptr, out_b.ptr, 4096, 12288, 1, st.handle)
         dsteps = max(20, min(args.steps, 1000))
-        dms, _ = time_steps(hip, stream, dual, dsteps, min(args.warmup, dsteps))
-        dbytes = 2 * a.w_bytes + 4 * 4096 + 2 * 4 * 12288
-        dg = dbytes / (dms / dsteps * 1e-3) / 1e9
-        extra["q4_k gate|up pair, one launch"] = {"gbps": round(dg, 1), "ms": round(dms / dsteps, 5), "frac_hbm": round(dg / HBM_PEAK_GBPS, 4)}
-        log("case=q4_k gate|up pair in one launch\ntype=Q4_K\nshape=2 x 4096x12288\ntokens=1\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\ngbps_hbm=%.1f\n" % (
-            2 * a.w_bytes, dsteps, dms / dsteps, dg))
-        a.close()
-        b.close()
-        out_b.close()
+        r = measure(hip, stream, Rotating(dual, min(a.copies, b.copies), 2 * a.w_bytes), dsteps, min(args.warmup, dsteps))
+        cases["q4_k gate|up pair, one launch"] = gemv_record(r, 2 * a.w_bytes + 4 * 4096 + 2 * 4 * 12288)
+        log("case=q4_k gate|up pair in one launch\nhip_us=%.3f\n" % r["us"])
+        for o in (a, b, out_b):
+            o.close()
 
-    if args.mode == "cases":
         # FFN sequence of one layer: gate | up | SwiGLU in one launch, then Q6_K down with the residual add
         from cogni_ml_amd.ffn_sequence import FFNSequenceRunner
         graw = [synth.make_weights(rng, Q4_K, 12288, 4096) for _ in range(2)] + [synth.make_weights(rng, Q6_K, 4096, 12288)]
@@ -382,40 +529,37 @@ def main():
             ffn.upload_weights()
             ffn.reset_sequence()
 
-            def fseq(i, st, ffn=ffn):
+            def fseq(copy, st, ffn=ffn):
                 with hip.with_stream(st):
                     ffn.run_sequence()
-            reps = max(20, min(args.steps // 4, 300))
-            fms, _ = time_steps(hip, stream, fseq, reps, 10)
-            fg = ffn.bytes_per_sequence() / (fms / reps * 1e-3) / 1e9
-            extra["%s M=%d" % ("add+rmsnorm+ffn" if block else "ffn sequence", tokens)] = {"gbps": round(fg, 1), "ms": round(fms / reps, 5), "frac_hbm": round(fg / HBM_PEAK_GBPS, 4)}
-            log("case=ffn sequence (gate|up Q4_K -> SwiGLU -> down Q6_K + residual)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\n"
-                "gbps=%.1f\nnote=weights %.0f MB stay in the 256 MB last-level cache between repetitions\n" % (
-                    tokens, sum(r.size for r in graw), reps, fms / reps, fg, sum(r.size for r in graw) / 1e6))
+            r = measure(hip, stream, Rotating(fseq, 1, sum(x_.size for x_ in graw)), max(20, min(args.steps // 4, 300)), 10)
+            rec = gemv_record(r, ffn.bytes_per_sequence())
+            rec["note"] = "weights (%.0f MB) stay in the last-level cache between repetitions" % (sum(x_.size for x_ in graw) / 1e6)
+            cases["%s M=%d" % ("add+rmsnorm+ffn" if block else "ffn sequence", tokens)] = rec
+            log("case=ffn sequence (gate|up Q4_K -> SwiGLU -> down Q6_K + residual)%s\ntokens=%d\nhip_us=%.3f\n" % (
+                " with add+rmsnorm" if block else "", tokens, r["us"]))
             ffn.close()
 
-    if args.mode == "cases":
-        # config 5: the mixed-quant projection stack, resident, back to back in one stream
-        from cogni_ml_amd.projection_stack import QwenProjectionStackRunner, Weights
-        wts = Weights.synthetic(rng)
-        for tokens in (1, 4, 8):
-            runner = QwenProjectionStackRunner.from_weights(wts, tokens, synth.make_activations(rng, tokens, wts.hidden))
-            runner.upload_weights()
-            runner.reset_sequence()
+    gpu_seconds = time.perf_counter() - t_start
 
-            def seq(i, st, runner=runner):
-                with hip.with_stream(st):
-                    runner.run_sequence()
-            reps = max(20, min(args.steps // 4, 300))
-            sms, _ = time_steps(hip, stream, seq, reps, 10)
-            sg = runner.bytes_per_sequence() / (sms / reps * 1e-3) / 1e9
-            extra["projection stack M=%d" % tokens] = {"gbps": round(sg, 1), "ms": round(sms / reps, 5),
-                                                        "frac_hbm": round(sg / HBM_PEAK_GBPS, 4)}
-            log("case=projection stack (q,k,v,o,gate,up Q4_K + down Q6_K)\ntokens=%d\nraw_bytes=%d\nreps=%d\nhip_ms=%.5f\n"
-                "gbps=%.1f\nnote=weights %.0f MB stay in the 256 MB last-level cache between repetitions\n" % (
-                    tokens, wts.raw_bytes, reps, sms / reps, sg, wts.raw_bytes / 1e6))
-            runner.close()
+    # ---- the oracle: parity of the measured kernel's output, and the CPU baseline (after the GPU work) ---------
+    ref, cpu_reps, cpu_s = cpu_baseline(oracle, head, args.cpu_seconds)
+    dense_max = float(np.max(np.abs(oracle.dequantize(head.host_w[:16 * 144 * 256], Q4_K, 256 * 4096))))
+    max_diff = float(np.max(np.abs(got - ref)))
+    cos = float(got.astype(np.float64) @ ref.astype(np.float64) /
+                np.sqrt((got.astype(np.float64) @ got.astype(np.float64)) * (ref.astype(np.float64) @ ref.astype(np.float64))))
+    tol = 1e-4 * float(np.linalg.norm(head.host_x)) * dense_max
+    ok = cos >= 0.99999 and max_diff <= 1e-3 and max_diff <= tol
+    cpu_gbps = head.bytes_per_step * cpu_reps / cpu_s / 1e9
+    # the same restatement with the rows divided among the host cores this job may use (16 on a one-GPU box)
+    mt_cores = max(1, min(16, os.cpu_count() or 1))
+    _, mt_reps, mt_s = cpu_baseline(oracle, head, min(3.0, args.cpu_seconds), threads=mt_cores)
+    mt_gbps = head.bytes_per_step * mt_reps / mt_s / 1e9
+    log("cpu_baseline: 1 thread %.4f GB/s (%d reps, %.1f s); %d threads %.4f GB/s (%d reps, %.1f s); gcc -O2 -ffp-contract=off, "
+        "stands in for the reference's Crystal QuantMatmul\ncpu_ms=%.3f\ncos=%.8f\nmax_diff=%g\nok=%s" % (
+            cpu_gbps, cpu_reps, cpu_s, mt_cores, mt_gbps, mt_reps, mt_s, cpu_s / cpu_reps * 1e3, cos, max_diff, str(ok).lower()))
 
+    traffic, traffic_rec = recorded_traffic()
     result = {
         "metric": "Q4_K GEMV GB/s 4096x12288 M=1",
         "value": round(gbps, 1),
@@ -432,15 +576,22 @@ def main():
         "config": {
             "workload": "Q4_K decode GEMV, W 12288x4096 (in 4096 -> out 12288), M=1, fp32 x, fp32 accumulate",
             "weight_bytes": head.w_bytes, "bytes_per_step": head.bytes_per_step,
-            "weight_copies_rotated": head.copies, "timed_region": "hip graph of K launches" if graphed else "K direct launches",
+            "weight_copies_rotated": hr["buffers_rotated"],
+            "timed_region": ("median of %d samples, each %d replay(s) of a hip graph of K launches" if hr["graphed"] else
+                             "median of %d samples, each %d x K direct launches") % (hr["samples"], hr["replays_per_sample"]),
         },
+        "us_per_step": {"median": round(hr["us"], 3), "min": round(hr["us_min"], 3), "max": round(hr["us_max"], 3)},
+        "timed_region_ms": round(hr["timed_region_ms"], 2),
         "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "cache_hot_gbps": round(hot_gbps, 1),
+        "read_only_kernel_same_bytes": {"us": round(floor_us, 3), "grid": floor_grid, "gbps": round(head.w_bytes / floor_us / 1e3, 1)},
         "prefill_gemm_q4k_12288x4096": gemm,
-        "parity": {"cos": round(cos, 8), "max_diff": max_diff, "ok": ok, "tol_1e-4_x_wmax": 1e-4 * float(np.linalg.norm(head.host_x)) * dense_max},
+        "parity": {"cos": round(cos, 8), "max_diff": max_diff, "ok": ok, "tol_1e-4_x_wmax": tol},
         "roofline": {
             "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+            "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
+            "traffic_source": None if traffic_rec is None else "profiles/traffic.json: rocprofv3 --pmc record for %s at commit %s, not counted in this run" % (
+                traffic_rec.get("kernel"), traffic_rec.get("commit")),
         },
         "cpu_baseline": {
             "value": round(cpu_gbps, 4), "unit": "GB/s", "cores": 1, "kind": "port",
@@ -449,9 +600,9 @@ def main():
         },
         "cpu_baseline_all_cores": {"value": round(mt_gbps, 4), "unit": "GB/s", "cores": mt_cores, "kind": "port",
                                    "sample": "%d x the same GEMV, rows divided among %d threads, %.1f s" % (mt_reps, mt_cores, mt_s)},
+        "cases": cases,
+        "gpu_phase_seconds": round(gpu_seconds, 1),
     }
-    if extra:
-        result["cases"] = extra
     head.close()
     stream.close()
     ctx.close()

@@ -223,6 +223,12 @@ class QuantWeight:
     def matmul(self, x, rows=1, bias=None):
         xa = np.ascontiguousarray(x, dtype=np.float32)
         ba = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        if rows <= 0:
+            raise ValueError("rows must be positive, got %d" % rows)
+        if xa.size < rows * self.in_dim:   # the library copies rows*in_dim floats from this buffer
+            raise ValueError("x has %d elements, rows*in_dim is %d" % (xa.size, rows * self.in_dim))
+        if ba is not None and ba.size < self.out_dim:
+            raise ValueError("bias has %d elements, out_dim is %d" % (ba.size, self.out_dim))
         res = np.empty(rows * self.out_dim, dtype=np.float32)
         _check(hip.lib().cogni_weight_matmul(self._handle, ctypes.c_void_p(xa.ctypes.data), ctypes.c_int32(rows),
                                              ctypes.c_void_p(ba.ctypes.data if ba is not None else None),

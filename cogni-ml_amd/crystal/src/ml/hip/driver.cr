@@ -92,6 +92,8 @@ lib LibCogniHIP
   fun cogni_last_error : UInt8*
 end
 
+require "../cuda/driver"   # for the backend-neutral ML::CUDA::ResidentSequenceRunner only
+
 module ML::HIP
   alias DevicePtr = LibCogniHIP::Deviceptr
   @@current_stream = Pointer(Void).null
@@ -321,60 +323,10 @@ module ML::HIP
       params, Pointer(Void*).null), "hipModuleLaunchKernel(#{label})"
   end
 
-  # Unchanged from ML::CUDA::ResidentSequenceRunner (src/ml/cuda/driver.cr:288-342): pure host logic.
-  class ResidentSequenceRunner
-    getter tokens : Int32
-
-    def initialize(@tokens : Int32,
-                   @upload_weights : Proc(Nil),
-                   @reset_sequence : Proc(Nil),
-                   @run_token : Proc(Int32, Nil),
-                   @read_outputs : Proc(Nil)? = nil,
-                   @run_sequence_override : Proc(Int32, Nil)? = nil)
-      raise ArgumentError.new("tokens must be positive") unless @tokens > 0
-      @active_tokens = @tokens
-    end
-
-    def active_tokens : Int32
-      @active_tokens
-    end
-
-    def active_tokens=(@active_tokens : Int32) : Int32
-      raise ArgumentError.new("active_tokens must be positive") unless @active_tokens > 0
-      raise ArgumentError.new("active_tokens must be <= tokens") unless @active_tokens <= @tokens
-      @active_tokens
-    end
-
-    def reset_active_tokens : Nil
-      @active_tokens = @tokens
-    end
-
-    def upload_weights : Nil
-      @upload_weights.call
-    end
-
-    def reset_sequence : Nil
-      @reset_sequence.call
-    end
-
-    def run_sequence : Nil
-      if override = @run_sequence_override
-        override.call(@active_tokens)
-      else
-        @active_tokens.times { |tok| @run_token.call(tok) }
-      end
-    end
-
-    def run_repeated(reps : Int32) : Int32
-      raise ArgumentError.new("reps must be positive") unless reps > 0
-      reps.times { run_sequence }
-      reps * @active_tokens
-    end
-
-    def read_outputs : Nil
-      @read_outputs.try(&.call)
-    end
-  end
+  # The resident-sequence facade is backend neutral in the reference (src/ml/cuda/driver.cr:288-342: five procs and a
+  # token count, no driver call), so the HIP runners use that very class rather than a second copy of it. Requiring
+  # the CUDA binding file does not link libcuda: Crystal only links a `lib` whose funs are called.
+  alias ResidentSequenceRunner = ML::CUDA::ResidentSequenceRunner
 
   # The GPU arm of the projection router: same shape as Qwen35Metal.matmul(qw, x, batch) : Array(Float32)?
   # (src/ml/gguf/qwen35_cpu.cr:1398-1412, 1478-1490). nil = not eligible, fall back to QuantMatmul.matmul_add.

@@ -1,14 +1,13 @@
 // The gfx950 code object: every kernel is an unmangled extern "C" __global__ symbol so a host can
 // fetch it by name with hipModuleGetFunction after hipModuleLoadData, the way the reference loads
 // its PTX modules (src/ml/cuda/driver.cr:115-127).
-#include "kernels/dequant.cuh"
-#include "kernels/gemv.cuh"
-#include "kernels/gemv_mfma.cuh"
-#include "kernels/gemv_mfma_q6k.cuh"
-#include "kernels/gemm_q4k.cuh"
-#include "kernels/gemm_q6k.cuh"
-#include "kernels/norm.cuh"
-#include "kernels/util.cuh"
+#include "kernels/dequant.hpp"
+#include "kernels/gemv.hpp"
+#include "kernels/gemv_mfma.hpp"
+#include "kernels/gemv_mfma_q6k.hpp"
+#include "kernels/gemm_q4k.hpp"
+#include "kernels/gemm_q6k.hpp"
+#include "kernels/norm.hpp"
 
 GEMV_MFMA_ENTRY(q4_k_gemv_mfma_f32_tbatch2, 2)
 GEMV_MFMA_ENTRY(q4_k_gemv_mfma_f32_tbatch3, 3)

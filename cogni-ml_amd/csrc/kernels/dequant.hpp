@@ -11,7 +11,7 @@
 // each store instruction writes 1 KiB of contiguous memory. Signature of every kernel:
 //   (const uint8_t* w_raw, float* out, uint64 n_elements), block = 256 threads, any grid size.
 #pragma once
-#include "common.cuh"
+#include "common.hpp"
 
 #define DEQ_BLOCK 256
 #define DEQ_WAVES (DEQ_BLOCK / WAVE)

@@ -37,7 +37,7 @@
 // consumed (two 64 KiB buffers); the raw weight bytes of the next super-block are copied into the one 28 KiB
 // buffer as soon as every wavefront has taken the current ones into registers.
 #pragma once
-#include "common.cuh"
+#include "common.hpp"
 
 #define GEMM_BM 128
 #define GEMM_BN 192
@@ -66,7 +66,7 @@ __device__ __forceinline__ u32 gemm_k_element(u32 ks, u32 kg, u32 e) {
 #ifndef PACK_TOK
 #define PACK_TOK 8
 #endif
-// Q6: the element order of the Q6_K kernel (gemm_q6k.cuh) instead of the Q4_K one.
+// Q6: the element order of the Q6_K kernel (gemm_q6k.hpp) instead of the Q4_K one.
 template <bool Q6>
 __device__ __forceinline__ void pack_x_core(const float* __restrict__ x, uint4* __restrict__ xp, u32 m, u32 in_dim) {
   // [32 (k-step, k-group)][32 tokens] uint4, each (k-step, k-group) row padded by one uint4 so that the

@@ -1,5 +1,5 @@
 // Prefill GEMM over raw Q6_K weights: out[m][n] = (bias[n] +) sum_k x[m][k] * deq(W[n][k]), M >= 9.
-// Same tiling, operand layouts, x workspace format and epilogue as the Q4_K kernel (gemm_q4k.cuh): 128 tokens x 192
+// Same tiling, operand layouts, x workspace format and epilogue as the Q4_K kernel (gemm_q4k.hpp): 128 tokens x 192
 // rows per workgroup, 4 wavefronts = 2 row halves x 2 k-step halves, v_mfma_f32_32x32x16_f16 with fp32 accumulation,
 // x as fp16 in LDS (two 64 KiB buffers filled by global_load_lds_dwordx4). What differs is the weight side:
 //
@@ -23,7 +23,7 @@
 // packed multiply gives fp16((q - 32) * (d * sc)). The 8 values come in byte order 0,2,1,3,4,6,5,7;
 // pack_x_f16_q6k writes x accordingly (gemm_k_element_q6k).
 #pragma once
-#include "gemm_q4k.cuh"
+#include "gemm_q4k.hpp"
 
 // Element (0..255) of a super-block that k-slot (ks, kg, e) of the MFMA stands for: ks = 8 n + 2 qd + h8.
 __device__ __forceinline__ u32 gemm_k_element_q6k(u32 ks, u32 kg, u32 e) {

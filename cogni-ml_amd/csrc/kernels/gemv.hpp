@@ -31,7 +31,7 @@
 // into the block scale.
 #pragma once
 #include <type_traits>
-#include "common.cuh"
+#include "common.hpp"
 #include "gemv_config.h"
 
 

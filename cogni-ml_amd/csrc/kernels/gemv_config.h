@@ -30,7 +30,7 @@ static inline int gemv_rows_per_block(unsigned type, int tokens) {
 // token group it is working on. per_set_f4 = float4 count of one column set for that token group.
 #define GEMV_LDS_BYTES 49152
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
+#if defined(__HIPCC__)
 #define GEMV_HD __host__ __device__
 #else
 #define GEMV_HD
@@ -97,7 +97,7 @@ static inline unsigned gemv_lds_bytes(unsigned type, int tokens, unsigned in_dim
   return (unsigned)(per_set_f4 * ch) * 16u + (unsigned)(mg * nsum * 64 * ch) * 4u;
 }
 
-// ---- matrix-core GEMV (gemv_mfma.cuh): 8 wavefronts per workgroup ------------------------------------
+// ---- matrix-core GEMV (gemv_mfma.hpp): 8 wavefronts per workgroup ------------------------------------
 #define GEMV_MFMA_WAVES 8
 #define GEMV_MFMA_TMAX 3            // 16-row tiles a wavefront carries at most
 #define GEMV_MFMA_MAX_TOKENS 4

@@ -1,6 +1,6 @@
 // Decode GEMV on the matrix cores for M = 1..4 tokens, Q4_K: out[m][o] = (residual[m][o] +) sum_j x[m][j] * deq(W[o][j]).
 //
-// Same kernel ABI as the vector-ALU GEMV (gemv.cuh): (w_raw, x, [residual,] out, in_dim, out_dim), x rows at
+// Same kernel ABI as the vector-ALU GEMV (gemv.hpp): (w_raw, x, [residual,] out, in_dim, out_dim), x rows at
 // stride in_dim, out/residual rows at stride out_dim. Launch: block = 512 threads (8 wavefronts), grid and
 // dynamic shared memory from gemv_config.h (gemv_mfma_grid, gemv_mfma_lds_bytes).
 //
@@ -31,7 +31,7 @@
 // kslice + NWK, ...) times NWR row groups, NWK = min(8, largest power of two <= in_dim / 256). Partial sums meet in LDS
 // and are added in a fixed order, so results are reproducible.
 #pragma once
-#include "common.cuh"
+#include "common.hpp"
 #include "gemv_config.h"
 
 typedef _Float16 mf_half8 __attribute__((ext_vector_type(8)));

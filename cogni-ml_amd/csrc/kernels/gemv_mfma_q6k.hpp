@@ -1,6 +1,6 @@
 // Decode GEMV on the matrix cores for M = 3, 4 tokens, Q6_K: out[m][o] = (residual[m][o] +) sum_j x[m][j] * deq(W[o][j]).
 //
-// Same kernel ABI, launch geometry and work split as the Q4_K kernel in gemv_mfma.cuh (block = 8 wavefronts = k-slices x
+// Same kernel ABI, launch geometry and work split as the Q4_K kernel in gemv_mfma.hpp (block = 8 wavefronts = k-slices x
 // row groups, 16-row tiles, activations as binary16 hi + lo pairs in LDS, partial sums added in a fixed order); dynamic
 // shared memory from gemv_mfma_lds_bytes(14, ...). What differs is the block format (210 B: ql[128], qh[64],
 // scales:i8[16], d:f16 - src/ml/gguf/dequant.cr:195-236):
@@ -19,9 +19,9 @@
 //
 // Rows are only 2-byte aligned (210-byte blocks): all weight loads are 8, 4 or 2 bytes at any alignment.
 #pragma once
-#include "common.cuh"
+#include "common.hpp"
 #include "gemv_config.h"
-#include "gemv_mfma.cuh"
+#include "gemv_mfma.hpp"
 
 // TOP1: instead of the row values a workgroup stores, per token, the largest of all its rows and that row's index
 // (out[token * gridDim.x + blockIdx.x], top_ids[...]: the layout of the vector-ALU top-1 kernels, finished by

@@ -4,7 +4,7 @@
 //   inv = 1 / sqrt(sum(x^2) / dim + eps);  out[i] = (x[i] * inv) * norm[i]
 // The add form first forms r = x + add, stores r (the residual stream) and normalises r.
 #pragma once
-#include "common.cuh"
+#include "common.hpp"
 
 #define NORM_BLOCK 256
 #define NORM_KEEP 4   // float4 a thread keeps across the reduction on the short-row path

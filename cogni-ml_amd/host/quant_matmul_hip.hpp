@@ -77,6 +77,12 @@ class QuantWeight {
   uint64_t device_ptr() const { return cogni_weight_device_ptr(handle_); }
   // ComputeBackend#matmul(x, rows, qw, bias) (compute.cr:50); bias may be null (qmatvec_nobias)
   std::vector<float> matmul(const std::vector<float>& x, int rows, const std::vector<float>* bias = nullptr) const {
+    if (rows <= 0) throw std::invalid_argument("matmul: rows must be positive");
+    if (x.size() < (size_t)rows * (size_t)in_dim_)   // the library copies rows*in_dim floats from this buffer
+      throw std::invalid_argument("matmul: x has " + std::to_string(x.size()) + " elements, rows*in_dim is " +
+                                  std::to_string((size_t)rows * (size_t)in_dim_));
+    if (bias && bias->size() < (size_t)out_dim_)
+      throw std::invalid_argument("matmul: bias has " + std::to_string(bias->size()) + " elements, out_dim is " + std::to_string(out_dim_));
     std::vector<float> result((size_t)rows * out_dim_);
     qcheck(cogni_weight_matmul(handle_, x.data(), rows, bias ? bias->data() : nullptr, result.data()));
     return result;

@@ -147,6 +147,11 @@ static int gpu_probe() {
   EXPECT(qw.device_ptr() != 0);
   std::vector<float> via_qw = qw.matmul(x, 1);
   EXPECT(std::memcmp(via_qw.data(), gpu.data(), 4 * out_dim) == 0);
+  // a buffer shorter than the shape says is refused before the library reads from it
+  std::vector<float> short_x(in_dim - 1), short_bias(out_dim - 1);
+  EXPECT(throws_with<std::invalid_argument>([&] { qw.matmul(short_x, 1); }, "rows*in_dim is 4096"));
+  EXPECT(throws_with<std::invalid_argument>([&] { qw.matmul(x, 2); }, "rows*in_dim is 8192"));
+  EXPECT(throws_with<std::invalid_argument>([&] { qw.matmul(x, 1, &short_bias); }, "out_dim is 1024"));
   // qmatvec_many: the same weight twice against one x, and no weights at all
   std::vector<std::vector<float>> many = QuantWeight::matvec_many({&qw, &qw}, x);
   EXPECT(many.size() == 2 && std::memcmp(many[0].data(), gpu.data(), 4 * out_dim) == 0 &&

@@ -151,6 +151,21 @@ def test_argument_errors_do_not_need_a_gpu():
     assert e.value.code == -2
 
 
+def test_quant_weight_matmul_checks_buffer_sizes_before_the_library_reads_them():
+    # cogni_weight_matmul copies rows*in_dim floats from x and out_dim from bias: a short buffer must never reach it.
+    # (The checks sit in front of the library call, so a weight without a device copy is enough to exercise them.)
+    qw = quant.QuantWeight.__new__(quant.QuantWeight)
+    qw.out_dim, qw.in_dim, qw._handle = 8, 256, None
+    with pytest.raises(ValueError, match="x has 255 elements, rows\\*in_dim is 256"):
+        qw.matmul(np.zeros(255, dtype=np.float32))
+    with pytest.raises(ValueError, match="x has 256 elements, rows\\*in_dim is 512"):
+        qw.matmul(np.zeros(256, dtype=np.float32), rows=2)
+    with pytest.raises(ValueError, match="bias has 7 elements, out_dim is 8"):
+        qw.matmul(np.zeros(256, dtype=np.float32), bias=np.zeros(7, dtype=np.float32))
+    with pytest.raises(ValueError, match="rows must be positive"):
+        qw.matmul(np.zeros(256, dtype=np.float32), rows=0)
+
+
 def gpu_present():
     return os.path.exists("/dev/kfd")
 
