@@ -127,6 +127,18 @@ def gemv_top1_dev(w_ptr, w_type, x_ptr, partial_ids_ptr, partial_values_ptr, top
                                          ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+TOP1_NOALLOC_MAX_PARTIALS = 65536
+
+
+def gemv_top1_noalloc_dev(w_ptr, w_type, x_ptr, top1_ids_ptr, top1_values_ptr, in_dim, out_dim, tokens=1, stream=None):
+    """gemv_top1_dev with the partial results in the library's static device array: allocates nothing. Fails when
+    tokens * gemv_top1_partials() exceeds TOP1_NOALLOC_MAX_PARTIALS; calls that overlap on one GPU race."""
+    _check(hip.lib().cogni_gemv_top1_noalloc_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(x_ptr),
+                                                 ctypes.c_uint64(top1_ids_ptr), ctypes.c_uint64(top1_values_ptr),
+                                                 ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens),
+                                                 stream))
+
+
 def rmsnorm_dev(x_ptr, norm_ptr, out_ptr, dim, tokens=1, eps=1.0e-6, stream=None):
     _check(hip.lib().cogni_rmsnorm_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(out_ptr),
                                        ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))

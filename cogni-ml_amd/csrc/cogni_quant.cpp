@@ -4,6 +4,7 @@
 // (hsaco_blob.S) and loaded with hipModuleLoadData; every launch goes through
 // hipModuleLaunchKernel with the kernel ABI the header documents. There is no host fallback.
 #include "cogni_quant.h"
+#include "internal.h"
 #include "kernels/gemv_config.h"
 
 #include <hip/hip_runtime_api.h>
@@ -133,6 +134,8 @@ struct cogni_quant_weight {
 extern "C" {
 
 const char* cogni_last_error(void) { return g_err.c_str(); }
+int cogni_internal_fail(int code, const char* text) { return fail(code, text); }
+int cogni_internal_hip_fail(int hip_error, const char* what) { return hip_fail((hipError_t)hip_error, what); }
 
 // ---- geometry (reader.cr:51-78, 119-127) -----------------------------------------------------
 int32_t cogni_block_bytes(uint32_t type) {
@@ -217,6 +220,26 @@ int cogni_quant_init(int32_t ordinal) {
   if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(COGNI_ERR_NO_DEVICE, std::string("device is ") + prop.gcnArchName + ", the code object is gfx950 only");
   HIP_TRY(hipModuleLoadData(&g_rt.mod, cogni_hsaco_begin), "hipModuleLoadData(cogni_quant gfx950 code object)");
+  // the static scratch of the entry point that allocates nothing: its device address, once per device
+  if (int rc = cogni_internal_noalloc_setup(ordinal)) {
+    (void)hipModuleUnload(g_rt.mod);
+    g_rt.mod = nullptr;
+    return rc;
+  }
+  // its kernels are resolved now, so that a call under stream capture finds them in the table
+  for (const char* t : {"q8_0", "q4_k", "q5_k", "q6_k"}) {
+    for (const char* sfx : {"", "_tbatch2", "_tbatch3"}) {
+      hipFunction_t fn = nullptr;
+      const std::string name = std::string(t) + "_gemv_top1_partial_f32" + sfx;
+      if (hipModuleGetFunction(&fn, g_rt.mod, name.c_str()) == hipSuccess) g_rt.fns.emplace(name, fn);
+    }
+  }
+  for (const char* name : {"q4_k_gemv_mfma_top1_partial_f32_tbatch3", "q4_k_gemv_mfma_top1_partial_f32_tbatch4",
+                           "q6_k_gemv_mfma_top1_partial_f32_tbatch3", "q6_k_gemv_mfma_top1_partial_f32_tbatch4", "top1_reduce_f32"}) {
+    hipFunction_t fn = nullptr;
+    HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
+    g_rt.fns.emplace(name, fn);
+  }
   g_rt.compute_units = prop.multiProcessorCount;
   g_rt.ordinal = ordinal;
   g_rt.ready = true;

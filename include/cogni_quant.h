@@ -196,6 +196,19 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
                         uint64_t top1_ids, uint64_t top1_values, uint32_t in_dim, uint32_t out_dim, uint32_t tokens,
                         void* stream);
 
+/* cogni_gemv_top1_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same launches and the same results, with the per-workgroup partial
+ * results in a static device array inside the library instead of caller-owned buffers. No counterpart in the
+ * reference. Allocates nothing and frees nothing. Limit: tokens * cogni_gemv_top1_partials(w_type, out_dim) must not
+ * exceed COGNI_TOP1_NOALLOC_MAX_PARTIALS (512 KiB of device memory per GPU, held until the process ends); beyond it the
+ * call fails with COGNI_ERR_INVALID_ARGUMENT and launches nothing. Every call on a GPU uses that GPU's one array: calls
+ * that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered and safe. Nothing in the
+ * array needs clearing between calls (every slot read was written by the same call). Needs cogni_quant_init on the
+ * current device. */
+enum { COGNI_TOP1_NOALLOC_MAX_PARTIALS = 65536 };
+int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t top1_ids, uint64_t top1_values,
+                                uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
+
 /* Prefill GEMM for `tokens` > 8 (Q4_K, Q5_K, Q6_K): out[m*out_dim + o] = (bias ? bias[o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j]).
  * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
  * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:

@@ -1,0 +1,68 @@
+"""cogni_gemv_top1_noalloc_dev (the output-head arg-max with its partial results in the library's static device array)
+against cogni_gemv_top1_dev (the same launches with caller-owned partial buffers): ids and values must agree bit for bit,
+on two calls in a row, the second with a smaller input, so that what the first call left in the array is shown not to
+matter. Collected last: a failure here must not hide the other GPU tests."""
+import numpy as np
+import pytest
+
+from cogni_ml_amd import quant, synth
+from gpu_common import DevArray, gpu  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+
+
+def top1_both(raw, t, x, in_dim, out_dim, tokens):
+    """(ids, values) from the existing entry point and from the one that allocates nothing, on the same device inputs."""
+    stride = quant.gemv_top1_partials(t, out_dim)
+    wd, xd = DevArray(raw), DevArray(x)
+    pi, pv = DevArray(nbytes=4 * tokens * stride), DevArray(nbytes=4 * tokens * stride)
+    oi, ov = DevArray(nbytes=4 * tokens), DevArray(nbytes=4 * tokens)
+    ni, nv = DevArray(np.full(tokens, 0xFFFFFFFF, dtype=np.uint32)), DevArray(np.full(tokens, np.nan, dtype=np.float32))
+    try:
+        quant.gemv_top1_dev(wd.ptr, t, xd.ptr, pi.ptr, pv.ptr, oi.ptr, ov.ptr, in_dim, out_dim, tokens)
+        quant.gemv_top1_noalloc_dev(wd.ptr, t, xd.ptr, ni.ptr, nv.ptr, in_dim, out_dim, tokens)
+        return (oi.read(np.uint32, tokens), ov.read(np.float32, tokens)), (ni.read(np.uint32, tokens), nv.read(np.float32, tokens))
+    finally:
+        for d in (wd, xd, pi, pv, oi, ov, ni, nv):
+            d.close()
+
+
+# (first call, second call): the second is smaller in rows, row length or tokens, and of another type in two of the pairs
+PAIRS = [
+    ((Q6_K, 1024, 40003, 4), (Q6_K, 512, 3001, 1)),     # matrix-core kernel walking row groups, then one token
+    ((Q4_K, 2048, 20011, 7), (Q4_K, 256, 530, 2)),      # 4 + 3 tokens, then a pair on the vector ALU
+    ((Q8_0, 1024, 3584, 3), (Q5_K, 512, 1001, 2)),      # one launch pair per token
+]
+
+
+@pytest.mark.parametrize("first,second", PAIRS)
+def test_noalloc_top1_equals_top1_with_caller_buffers_twice_in_a_row(gpu, oracle, first, second):
+    for call, (t, in_dim, out_dim, tokens) in enumerate((first, second)):
+        print("case type=%d in_dim=%d out_dim=%d tokens=%d call=%d" % (t, in_dim, out_dim, tokens, call), flush=True)
+        rng = np.random.default_rng(out_dim * 7 + tokens)
+        raw = synth.make_weights(rng, t, out_dim, in_dim)
+        x = synth.make_activations(rng, tokens, in_dim)
+        (ids, vals), (nids, nvals) = top1_both(raw, t, x, in_dim, out_dim, tokens)
+        assert np.array_equal(ids, nids), (call, ids, nids)
+        assert np.array_equal(vals.view(np.uint32), nvals.view(np.uint32)), (call, vals, nvals)
+        # and both are the oracle's winner within the GEMV tolerance (bit equality alone would also hold for two wrong answers)
+        want = oracle.matmul_add(x, tokens, in_dim, raw, t, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).reshape(tokens, out_dim)
+        for tok in range(tokens):
+            top = float(want[tok].max())
+            scale = float(np.abs(want[tok]).max())
+            assert abs(float(nvals[tok]) - top) <= 1e-4 * scale
+            assert want[tok][nids[tok]] >= top - 1e-4 * scale
+
+
+def test_noalloc_top1_rejects_what_does_not_fit_the_static_array(gpu):
+    """Q8_0 has one workgroup per 16 rows: 8 tokens x 9496 partial results exceed the 65536 the array holds. The call must
+    fail before it launches anything (the pointers are never dereferenced)."""
+    out_dim = 151936
+    assert 8 * quant.gemv_top1_partials(Q8_0, out_dim) > quant.TOP1_NOALLOC_MAX_PARTIALS
+    with pytest.raises(quant.QuantError, match="exceed the static scratch of 65536") as e:
+        quant.gemv_top1_noalloc_dev(0x1000, Q8_0, 0x1000, 0x1000, 0x1000, 1024, out_dim, 8)
+    assert e.value.code == -1
+    # the operator's own argument checks still apply
+    with pytest.raises(quant.QuantError, match="Unsupported quant type"):
+        quant.gemv_top1_noalloc_dev(0x1000, 20, 0x1000, 0x1000, 0x1000, 1024, 64, 1)
