@@ -85,6 +85,45 @@ def gemv_many_dev(w_ptrs, w_type, x_ptr, out_ptrs, out_dims, in_dim, tokens=1, s
                                          stream))
 
 
+def gemv_image_bytes(w_type, in_dim, tokens):
+    """Bytes of the activation image of the one-pass multi-token GEMV; 0 = no such kernel for the combination."""
+    f = hip.lib().cogni_gemv_image_bytes
+    f.restype = ctypes.c_size_t
+    return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens))
+
+
+def gemv_packed_launch_dims(total_rows):
+    """(grid_x, block_x, shared_mem_bytes) of the one-pass kernel for a launch of total_rows rows."""
+    g, b, sh = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+    _check(hip.lib().cogni_gemv_packed_launch_dims(ctypes.c_uint32(total_rows), ctypes.byref(g), ctypes.byref(b), ctypes.byref(sh)))
+    return g.value, b.value, sh.value
+
+
+def gemv_pack_dev(x_ptr, w_type, in_dim, tokens, image_ptr, stream=None):
+    """x[tokens][in_dim] (fp32) -> the image gemv_packed_dev reads."""
+    _check(hip.lib().cogni_gemv_pack_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim),
+                                         ctypes.c_uint32(tokens), ctypes.c_uint64(image_ptr), stream))
+
+
+def gemv_packed_dev(w_ptrs, w_type, image_ptr, out_ptrs, out_dims, in_dim, tokens, residual_ptr=0, stream=None):
+    """Up to 8 matrices against one packed activation block of 2..8 tokens, the weights read once for all tokens."""
+    n = len(w_ptrs)
+    if len(out_ptrs) != n or len(out_dims) != n:
+        raise ValueError("w_ptrs, out_ptrs and out_dims must have the same length")
+    U64, U32 = ctypes.c_uint64 * n, ctypes.c_uint32 * n
+    _check(hip.lib().cogni_gemv_packed_dev(U64(*w_ptrs), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr),
+                                           ctypes.c_uint64(residual_ptr), U64(*out_ptrs), U32(*out_dims), ctypes.c_uint32(n),
+                                           ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens), stream))
+
+
+def gemv_packed_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, image_ptr, out_ptr, in_dim, out_dim, tokens, stream=None):
+    """out = silu(x W_gate^T) * (x W_up^T) against a packed activation block of 2..8 tokens, one launch."""
+    _check(hip.lib().cogni_gemv_packed_swiglu_dev(ctypes.c_uint64(w_gate_ptr), ctypes.c_uint64(w_up_ptr),
+                                                  ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr),
+                                                  ctypes.c_uint64(out_ptr), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim),
+                                                  ctypes.c_uint32(tokens), stream))
+
+
 def gemv_dual_dev(w_a_ptr, w_b_ptr, w_type, x_ptr, out_a_ptr, out_b_ptr, in_dim, out_dim, tokens=1, stream=None):
     """Two matrices of one shape against the same activations (gate | up, k | v)."""
     _check(hip.lib().cogni_gemv_dual_dev(ctypes.c_uint64(w_a_ptr), ctypes.c_uint64(w_b_ptr), ctypes.c_uint32(int(w_type)),

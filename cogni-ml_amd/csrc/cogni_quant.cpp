@@ -48,6 +48,12 @@ struct Runtime {
   int compute_units = 0;
   hipModule_t mod = nullptr;
   std::unordered_map<std::string, hipFunction_t> fns;
+  // activation images of the one-pass multi-token GEMV for the calls that bring none: one slot per stream
+  static constexpr int kImageSlots = 8;
+  void* image_pool = nullptr;
+  size_t image_slot_bytes = 0;
+  void* image_stream[kImageSlots] = {};
+  bool image_used[kImageSlots] = {};
 };
 Runtime g_rt;
 std::mutex g_mu;
@@ -74,6 +80,23 @@ int launch(const char* name, uint32_t grid, uint32_t block, uint32_t shmem, void
   if (rc != 0) return rc;
   HIP_TRY(hipModuleLaunchKernel(fn, grid, grid_y, 1, block, 1, 1, shmem, (hipStream_t)stream, params, nullptr),
           std::string("hipModuleLaunchKernel(") + name + ")");
+  return 0;
+}
+
+// The library-owned activation image of `stream` (0 if every slot belongs to another stream). Work on one stream is
+// ordered, so a stream's slot is free again by the time its next call writes it; different streams never share one.
+uint64_t image_for_stream(void* stream) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (!g_rt.ready || !g_rt.image_pool) return 0;
+  for (int i = 0; i < Runtime::kImageSlots; i++)
+    if (g_rt.image_used[i] && g_rt.image_stream[i] == stream)
+      return (uint64_t)(uintptr_t)g_rt.image_pool + (uint64_t)i * g_rt.image_slot_bytes;
+  for (int i = 0; i < Runtime::kImageSlots; i++)
+    if (!g_rt.image_used[i]) {
+      g_rt.image_used[i] = true;
+      g_rt.image_stream[i] = stream;
+      return (uint64_t)(uintptr_t)g_rt.image_pool + (uint64_t)i * g_rt.image_slot_bytes;
+    }
   return 0;
 }
 
@@ -240,6 +263,13 @@ int cogni_quant_init(int32_t ordinal) {
     HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
     g_rt.fns.emplace(name, fn);
   }
+  g_rt.image_slot_bytes = ((size_t)gemv_mt_image_bytes(GEMV_MT_MAX_IN_DIM) + 255) & ~(size_t)255;
+  HIP_TRY(hipMalloc(&g_rt.image_pool, g_rt.image_slot_bytes * Runtime::kImageSlots), "hipMalloc(activation images)");
+  for (const char* name : {"pack_x_mt_f16", "q4_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32"}) {
+    hipFunction_t fn = nullptr;
+    HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
+    g_rt.fns.emplace(name, fn);
+  }
   g_rt.compute_units = prop.multiProcessorCount;
   g_rt.ordinal = ordinal;
   g_rt.ready = true;
@@ -250,6 +280,7 @@ int cogni_quant_shutdown(void) {
   std::lock_guard<std::mutex> lk(g_mu);
   if (!g_rt.ready) return 0;
   (void)hipModuleUnload(g_rt.mod);
+  if (g_rt.image_pool) (void)hipFree(g_rt.image_pool);
   g_rt = Runtime();
   return 0;
 }
@@ -268,6 +299,98 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
   unsigned long long n = n_elements;
   void* params[] = {&w_raw, &out, &n};
   return launch(name, grid, 256, 0, params, stream);
+}
+
+// ---- several tokens in one pass over the weights: pack the activations once, then one launch per matrix list ------
+size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {
+  return gemv_mt_supported(w_type, (int)tokens, in_dim) ? (size_t)gemv_mt_image_bytes(in_dim) : 0;
+}
+
+int cogni_gemv_packed_launch_dims(uint32_t total_rows, uint32_t* grid_x, uint32_t* block_x, uint32_t* shared_mem_bytes) {
+  if (!grid_x || !block_x || !shared_mem_bytes || total_rows == 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_launch_dims: bad argument");
+  *grid_x = gemv_mt_grid(total_rows);
+  *block_x = GEMV_MT_WAVES * 64;
+  *shared_mem_bytes = gemv_mt_lds_bytes();
+  return 0;
+}
+
+int cogni_gemv_pack_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t image, void* stream) {
+  if (!gemv_mt_supported(w_type, (int)tokens, in_dim))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack_dev: no one-pass kernel for this type, token count and in_dim "
+                                            "(cogni_gemv_image_bytes is 0)");
+  if (!x || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack_dev: null device pointer");
+  void* params[] = {&x, &image, &tokens, &in_dim};
+  return launch("pack_x_mt_f16", 2 * (in_dim >> 8), 256, 0, params, stream);
+}
+
+int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,
+                          const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream) {
+  if (!w_raw || !out || !out_dims || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: null argument");
+  if (count == 0 || count > 8) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: count must be 1..8");
+  if (!gemv_mt_supported(w_type, (int)tokens, in_dim))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: no one-pass kernel for this type, token count and in_dim");
+  if (residual && count != 1) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: a residual goes with a single matrix");
+  for (uint32_t i = 0; i < count; i++)
+    if (!w_raw[i] || !out[i] || out_dims[i] == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: null pointer or zero rows");
+  // up to three matrices per launch, as one matrix of all their rows; a matrix whose row count is not a multiple of 16
+  // ends its launch (a tile of 16 rows is of one matrix)
+  for (uint32_t i0 = 0; i0 < count;) {
+    uint64_t w[3] = {0, 0, 0}, o[3] = {0, 0, 0};
+    uint32_t rows[3] = {0, 0, 0}, n = 0;
+    uint64_t total = 0;
+    while (n < 3 && i0 + n < count) {
+      w[n] = w_raw[i0 + n], o[n] = out[i0 + n], rows[n] = out_dims[i0 + n];
+      total += rows[n];
+      n++;
+      if (rows[n - 1] % 16 != 0) break;
+    }
+    if (total > 0x7FFFFFFFull) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: too many rows");
+    uint64_t res = i0 == 0 ? residual : 0;
+    void* params[] = {&w[0], &w[1], &w[2], &image, &res, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2], &tokens};
+    const int rc = launch("q4_k_gemv_mt_f32", gemv_mt_grid((uint32_t)total), GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(), params, stream);
+    if (rc != 0) return rc;
+    i0 += n;
+  }
+  return 0;
+}
+
+int cogni_gemv_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t image, uint64_t out, uint32_t in_dim,
+                                 uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (!w_gate || !w_up || !image || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: null device pointer");
+  if (out_dim == 0 || out_dim > 0x7FFFFFFFu) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: bad out_dim");
+  if (!gemv_mt_supported(w_type, (int)tokens, in_dim))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: no one-pass kernel for this type, token count and in_dim");
+  const uint32_t groups = (out_dim + 15) / 16;
+  void* params[] = {&w_gate, &w_up, &image, &out, &in_dim, &out_dim, &tokens};
+  return launch("q4_k_gemv_mt_swiglu_f32", groups < 256u ? groups : 256u, GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(), params, stream);
+}
+
+// Token groups of up to 8 through the library's own image of `stream`: pack, then the matrices. false = not taken (no
+// kernel for the shape, or every image slot belongs to another stream): the caller goes the older way.
+static bool try_one_pass(const uint64_t* w_raw, uint32_t w_type, uint64_t x, uint64_t residual, const uint64_t* out,
+                         const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, uint32_t min_tokens,
+                         void* stream, int* rc_out) {
+  if (tokens < min_tokens || !gemv_mt_supported(w_type, 2, in_dim)) return false;
+  const uint64_t image = image_for_stream(stream);
+  if (!image) return false;
+  *rc_out = 0;
+  for (uint32_t t0 = 0; t0 < tokens;) {
+    const uint32_t m = tokens - t0 < (uint32_t)GEMV_MT_MAX_TOKENS ? tokens - t0 : (uint32_t)GEMV_MT_MAX_TOKENS;
+    uint64_t o[8];
+    for (uint32_t i = 0; i < count; i++) o[i] = out[i] + (uint64_t)t0 * out_dims[i] * 4;
+    const uint64_t xm = x + (uint64_t)t0 * in_dim * 4, rm = residual ? residual + (uint64_t)t0 * out_dims[0] * 4 : 0;
+    if (m == 1) {   // a last single token: the one-token kernels
+      for (uint32_t i = 0; i < count && *rc_out == 0; i++)
+        *rc_out = cogni_gemv_dev(w_raw[i], w_type, xm, i == 0 ? rm : 0, o[i], in_dim, out_dims[i], 1, stream);
+    } else {
+      *rc_out = cogni_gemv_pack_dev(xm, w_type, in_dim, m, image, stream);
+      if (*rc_out == 0) *rc_out = cogni_gemv_packed_dev(w_raw, w_type, image, rm, o, out_dims, count, in_dim, m, stream);
+    }
+    if (*rc_out != 0) return true;
+    t0 += m;
+  }
+  return true;
 }
 
 int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, uint32_t out_dim, const char** kernel,
@@ -299,6 +422,11 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: zero dimension");
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  // five tokens and more of a matrix the one-pass kernel takes: groups of up to eight, the weights read once per group
+  {
+    int rc = 0;
+    if (try_one_pass(&w_raw, w_type, x, residual, &out, &out_dim, 1, in_dim, tokens, 5, stream, &rc)) return rc;
+  }
   // tokens per launch: groups of up to 4 where the matrix-core kernel takes the shape (several passes over
   // the weights are still cheaper than one pass on the vector ALU, measured up to 8 tokens); Q8_0 up to 8; the
   // vector-ALU kernels of the K-quants hold two tokens in registers (a third costs a second pass over the staged
@@ -356,6 +484,13 @@ int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uin
     void* params[] = {&w_raw_a, &w_raw_b, &x, &out_a, &out_b, &in_dim, &out_dim};
     return launch("q4_k_dual_gemv_f32", grid, block, shmem, params, stream);
   }
+  // several tokens of a pair the one-pass kernel takes: the activations packed once, both matrices in one launch
+  if (tokens >= 2) {
+    const uint64_t ws[2] = {w_raw_a, w_raw_b}, os[2] = {out_a, out_b};
+    const uint32_t dims[2] = {out_dim, out_dim};
+    int rc = 0;
+    if (try_one_pass(ws, w_type, x, 0, os, dims, 2, in_dim, tokens, 2, stream, &rc)) return rc;
+  }
   // several tokens of a Q4_K pair whose shape the matrix-core kernel takes: groups of up to four tokens, the two
   // matrices as one of 2 * out_dim rows (the activations are staged once for both); a last single token goes to the
   // one-token pair kernel
@@ -402,6 +537,10 @@ int cogni_gemv_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t x, cons
     if (!w_raw[i] || !out[i] || out_dims[i] == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_many_dev: null pointer or zero rows");
     total += out_dims[i];
     aligned = aligned && (out_dims[i] % 16) == 0;
+  }
+  if (count >= 2 && tokens >= 2) {   // the one-pass kernel: one image for all of them, up to three matrices per launch
+    int rc = 0;
+    if (try_one_pass(w_raw, w_type, x, 0, out, out_dims, count, in_dim, tokens, 2, stream, &rc)) return rc;
   }
   if (count == 2 && out_dims[0] == out_dims[1])
     return cogni_gemv_dual_dev(w_raw[0], w_raw[1], w_type, x, out[0], out[1], in_dim, out_dims[0], tokens, stream);
@@ -457,6 +596,27 @@ int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, 
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dual_swiglu_dev: zero dimension");
   if ((in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "Q4_K GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
+  // several tokens of a pair the one-pass kernel takes: the activations packed once per group of up to eight tokens, gate
+  // tile and up tile side by side in a workgroup, which stores silu(gate) * up
+  if (tokens >= 2 && gemv_mt_supported(w_type, 2, in_dim) && out_dim <= 0x7FFFFFFFu) {
+    const uint64_t image = image_for_stream(stream);
+    if (image) {
+      for (uint32_t t0 = 0; t0 < tokens;) {
+        const uint32_t m = tokens - t0 < (uint32_t)GEMV_MT_MAX_TOKENS ? tokens - t0 : (uint32_t)GEMV_MT_MAX_TOKENS;
+        const uint64_t xm = x + (uint64_t)t0 * in_dim * 4, om = out + (uint64_t)t0 * out_dim * 4;
+        int rc;
+        if (m == 1) {
+          rc = cogni_gemv_dual_swiglu_dev(w_gate, w_up, w_type, xm, om, in_dim, out_dim, 1, stream);
+        } else {
+          rc = cogni_gemv_pack_dev(xm, w_type, in_dim, m, image, stream);
+          if (rc == 0) rc = cogni_gemv_packed_swiglu_dev(w_gate, w_up, w_type, image, om, in_dim, out_dim, m, stream);
+        }
+        if (rc != 0) return rc;
+        t0 += m;
+      }
+      return 0;
+    }
+  }
   // several tokens, out_dim a multiple of 16 and a row length the matrix-core kernel takes: groups of up to four tokens
   // on the matrix cores (gate tile and up tile side by side in a wavefront, two tiles per wavefront, 256 workgroups at
   // most, which walk the row groups with the activations staged once); a last single token as below

@@ -88,3 +88,9 @@ __device__ __forceinline__ void k4_pair(u32 s0, u32 s1, u32 s2, u32 sh, bool upp
   sc_pair = upper ? sc_up : sc_lo;
   m_pair = upper ? m_up : m_lo;
 }
+
+// silu(g) * u in fp32: g / (1 + exp(-g)), then times u (bin/cuda_ffn_sequence_probe.cr:189-191)
+__device__ __forceinline__ float swiglu_one(float g, float u) {
+  const float s = g / (1.0f + expf(-g));
+  return s * u;
+}

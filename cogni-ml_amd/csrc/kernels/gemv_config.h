@@ -152,3 +152,34 @@ static inline unsigned gemv_mfma_lds_bytes(unsigned type, int tokens, unsigned i
   return 64u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * 1024u + GEMV_MFMA_WAVES * GEMV_MFMA_TMAX * (unsigned)mp * 64u +
          units * (4u + 4u * nsums + 1024u);
 }
+
+// ---- several tokens in one pass over a Q4_K matrix (gemv_mt.hpp): 8 wavefronts = 8 k-slices, activations packed once ----
+#define GEMV_MT_WAVES 8
+#define GEMV_MT_TMAX 3              // 16-row tiles a wavefront carries at most
+#define GEMV_MT_MAX_TOKENS 8
+#define GEMV_MT_MAX_IN_DIM 4096u
+// tiles per wavefront: as many as keep 256 workgroups busy, at most GEMV_MT_TMAX (host and kernel use the same rule)
+static inline GEMV_HD unsigned gemv_mt_tiles(unsigned ntiles, unsigned grid) {
+  (void)grid;
+  unsigned t = ntiles / 256u;
+  if (t < 1) t = 1;
+  if (t > (unsigned)GEMV_MT_TMAX) t = GEMV_MT_TMAX;
+  return t;
+}
+// Shapes the kernel takes: Q4_K, 2..8 tokens, in_dim 2048 or 4096 (one or two super-blocks per k-slice).
+static inline int gemv_mt_supported(unsigned type, int tokens, unsigned in_dim) {
+  return type == 12 && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && (in_dim == 2048u || in_dim == 4096u);
+}
+static inline unsigned gemv_mt_grid(unsigned total_rows) {
+  const unsigned ntiles = (total_rows + 15) / 16, t = gemv_mt_tiles(ntiles, 0);
+  const unsigned groups = (ntiles + t - 1) / t;
+  return groups < 256u ? groups : 256u;   // more groups than compute units: the workgroups walk them
+}
+static inline unsigned gemv_mt_lds_bytes(void) {
+  // the k-slices' partial sums, then per wavefront a slot of 16 rows x 144 bytes for each of its 2 x GEMV_MT_TMAX units
+  return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u + GEMV_MT_WAVES * 2u * GEMV_MT_TMAX * 2304u;
+}
+// bytes of the activation image pack_x_mt_f16 writes: the operands, then 20 floats per (super-block, token pair)
+static inline unsigned long long gemv_mt_image_bytes(unsigned in_dim) {
+  return (unsigned long long)(in_dim >> 8) * (8192u + 4u * 80u);
+}

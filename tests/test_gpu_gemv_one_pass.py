@@ -1,0 +1,161 @@
+"""Decode GEMV for 2..8 tokens in one pass over a Q4_K matrix (activations packed once, q4_k_gemv_mt_f32) vs the CPU oracle.
+
+Bars, both asserted: the north-star bound max|err| <= 1e-4 * ||x||_2 * max|w_row| per token and row, and the reference's own
+probe gate (cos >= 0.99999, max_diff <= 1e-3 * max(1, max|ref| / 64): the probe's absolute 1e-3 is meant for outputs of order
+10..100). The kernel feeds the activations as two binary16 terms (22 bits), so it is also held to 2e-5 of each token's
+output scale."""
+import numpy as np
+import pytest
+
+from cogni_ml_amd import quant, synth
+from gpu_common import DevArray, gpu  # noqa: F401
+from helpers import Q4_K, Q6_K, cosine, gemv_tolerance
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_rows(oracle, raw, x, in_dim, out_dim, tokens):
+    want = oracle.matmul_add(x, tokens, in_dim, raw, Q4_K, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).astype(np.float64)
+    dense = np.abs(oracle.dequantize(raw, Q4_K, out_dim * in_dim)).reshape(out_dim, in_dim)
+    return want, gemv_tolerance(x, dense, tokens, in_dim).reshape(-1)
+
+
+def assert_bars(got, want, tol, tokens, out_dim, what):
+    err = np.abs(got.astype(np.float64) - want)
+    worst = int(np.argmax(err / np.maximum(tol, 1e-30)))
+    assert np.all(err <= tol), "%s: err %.3e > tol %.3e at %d" % (what, err[worst], tol[worst], worst)
+    g, w_ = got.reshape(tokens, out_dim).astype(np.float64), want.reshape(tokens, out_dim)
+    for m in range(tokens):
+        scale = float(np.max(np.abs(w_[m])))
+        if scale == 0.0:
+            assert not g[m].any()
+            continue
+        assert cosine(g[m], w_[m]) >= 0.99999, (what, m)
+        assert np.max(np.abs(g[m] - w_[m])) <= 1e-3 * max(1.0, scale / 64.0), (what, m)
+        assert np.max(np.abs(g[m] - w_[m])) <= 2e-5 * scale, (what, m)
+
+
+ONE_PASS_SHAPES = [(4096, 12288), (4096, 4096), (2048, 1024), (4096, 37), (2048, 50), (4096, 1040), (2048, 16 * 3 * 256 * 2 + 40),
+                   (4096, 16 * 300 + 7), (2048, 16 * 600)]
+
+
+@pytest.mark.parametrize("in_dim,out_dim", ONE_PASS_SHAPES)
+@pytest.mark.parametrize("tokens", [5, 6, 7, 8])
+def test_five_to_eight_tokens_in_one_pass(gpu, oracle, in_dim, out_dim, tokens):
+    """cogni_gemv_dev with 5..8 tokens: one pack and one launch. Shapes: one, two and three tiles per wavefront, a single
+    partial tile, row counts that are not multiples of 16, more row groups than workgroups (24616 rows: the workgroups walk
+    two groups each, refilling their slots), both super-block counts per k-slice; with and without residual."""
+    print("case in_dim=%d out_dim=%d tokens=%d" % (in_dim, out_dim, tokens), flush=True)
+    assert quant.gemv_image_bytes(Q4_K, in_dim, tokens) == (in_dim // 256) * (8192 + 320)
+    rng = np.random.default_rng(in_dim * 13 + out_dim * 7 + tokens)
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = rng.standard_normal(tokens * out_dim).astype(np.float32)
+    want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens)
+    w, xd, od, rd = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim), DevArray(res)
+    quant.gemv_dev(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+    plain = od.read(np.float32, tokens * out_dim)
+    assert_bars(plain, want, tol, tokens, out_dim, "%dx%d M=%d" % (in_dim, out_dim, tokens))
+    quant.gemv_dev(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens, rd.ptr)
+    added = od.read(np.float32, tokens * out_dim)
+    assert np.array_equal(added, plain + res)          # the residual is one fp32 add on the finished sum
+    for a in (w, xd, od, rd):
+        a.close()
+
+
+@pytest.mark.parametrize("tokens", [2, 3, 4, 8])
+def test_explicit_image_and_matrix_lists(gpu, oracle, tokens):
+    """The caller-owned image: pack once, then a list of matrices (q | k | v | odd one) against it in one call. A matrix
+    whose row count is not a multiple of 16 ends its launch; the values are those of the same kernel on each matrix alone,
+    bit for bit (a row's arithmetic does not depend on its neighbours)."""
+    in_dim, dims = 4096, (4096, 1024, 1040, 24, 16, 160)
+    rng = np.random.default_rng(tokens)
+    raws = [synth.make_weights(rng, Q4_K, d, in_dim) for d in dims]
+    x = synth.make_activations(rng, tokens, in_dim)
+    ws, xd = [DevArray(r) for r in raws], DevArray(x)
+    image = DevArray(nbytes=quant.gemv_image_bytes(Q4_K, in_dim, tokens))
+    outs = [DevArray(nbytes=4 * tokens * d) for d in dims]
+    quant.gemv_pack_dev(xd.ptr, Q4_K, in_dim, tokens, image.ptr)
+    quant.gemv_packed_dev([w.ptr for w in ws], Q4_K, image.ptr, [o.ptr for o in outs], list(dims), in_dim, tokens)
+    single = DevArray(nbytes=4 * tokens * max(dims))
+    for raw, w, o, d in zip(raws, ws, outs, dims):
+        got = o.read(np.float32, tokens * d)
+        want, tol = oracle_rows(oracle, raw, x, in_dim, d, tokens)
+        assert_bars(got, want, tol, tokens, d, "list member %d rows M=%d" % (d, tokens))
+        quant.gemv_packed_dev([w.ptr], Q4_K, image.ptr, [single.ptr], [d], in_dim, tokens)
+        assert np.array_equal(got, single.read(np.float32, tokens * d))
+    for a in ws + outs + [xd, image, single]:
+        a.close()
+
+
+def test_one_pass_activation_ranges(gpu, oracle):
+    """Activations far outside the binary16 range, zeros and mixed magnitudes must come out as from fp32 arithmetic: the
+    image scales every (token, super-block) by its own power of two."""
+    rng = np.random.default_rng(78)
+    in_dim, out_dim, tokens = 4096, 528, 8
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim).reshape(tokens, in_dim)
+    x[0] *= np.float32(1e-30)                       # far below the smallest binary16 subnormal
+    x[1] *= np.float32(1e30)                        # far above the largest binary16 number
+    x[2, :256] = 0.0                                # an all-zero super-block
+    x[2, 256:512] *= np.float32(1e-12)
+    x[2, 700] = np.float32(3e7)                     # one huge value among small ones
+    x[3] = np.where(rng.random(in_dim) < 0.5, x[3] * np.float32(1e-6), x[3] * np.float32(1e4)).astype(np.float32)
+    x[4] = 0.0                                      # a whole token of zeros
+    x[5] = np.float32(1.0)                          # constants: the min term alone decides the sign of many rows
+    x[6] = -x[7]                                    # a token and its negative
+    x = np.ascontiguousarray(x.reshape(-1))
+    want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens)
+    w, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim)
+    quant.gemv_dev(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+    got = od.read(np.float32, tokens * out_dim)
+    assert_bars(got, want, tol, tokens, out_dim, "activation ranges")
+    g = got.reshape(tokens, out_dim)
+    assert not g[4].any()
+    # (not bit for bit: the matrix cores' internal sums are not symmetric under a change of sign)
+    assert np.max(np.abs(g[6] + g[7])) <= 2e-5 * float(np.abs(g[7]).max())
+    for a in (w, xd, od):
+        a.close()
+
+
+def test_one_pass_element_order_and_scale_positions(gpu, oracle):
+    """A matrix whose codes, scales and mins each appear in exactly one place at a time: a swapped sub-block, nibble half,
+    k-group or scale byte puts the unit activation's weight in the wrong output."""
+    in_dim, out_dim, tokens = 2048, 16, 8
+    rng = np.random.default_rng(5)
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    w = DevArray(raw)
+    od = DevArray(nbytes=4 * tokens * out_dim)
+    dense = oracle.dequantize(raw, Q4_K, out_dim * in_dim).reshape(out_dim, in_dim)
+    for base in (0, 31, 32, 255, 256 + 64 + 9, 1024 + 200, 2047):
+        x = np.zeros((tokens, in_dim), dtype=np.float32)
+        for m in range(tokens):                     # token m picks out column base + 37 m (mod in_dim)
+            x[m, (base + 37 * m) % in_dim] = 1.0
+        xd = DevArray(np.ascontiguousarray(x.reshape(-1)))
+        quant.gemv_dev(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+        got = od.read(np.float32, tokens * out_dim).reshape(tokens, out_dim)
+        for m in range(tokens):
+            col = dense[:, (base + 37 * m) % in_dim]
+            assert np.allclose(got[m], col, rtol=0, atol=2e-6 * float(np.abs(dense).max())), (base, m)
+        xd.close()
+    for a in (w, od):
+        a.close()
+
+
+def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
+    """9 and 13 tokens: a group of eight in one pass, the rest as the token count decides (one token on the vector ALU,
+    five in one pass); in_dim 1024 and Q6_K have no one-pass kernel and keep their older paths."""
+    rng = np.random.default_rng(11)
+    for in_dim, out_dim, tokens in ((4096, 272, 9), (2048, 100, 13), (1024, 64, 8)):
+        raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+        x = synth.make_activations(rng, tokens, in_dim)
+        want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens)
+        w, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim)
+        quant.gemv_dev(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+        assert_bars(od.read(np.float32, tokens * out_dim), want, tol, tokens, out_dim, "%dx%d M=%d" % (in_dim, out_dim, tokens))
+        for a in (w, xd, od):
+            a.close()
+    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(Q6_K, 4096, 8) == 0
+    assert quant.gemv_image_bytes(Q4_K, 4096, 1) == 0 and quant.gemv_image_bytes(Q4_K, 4096, 9) == 0
+    with pytest.raises(quant.QuantError, match="no one-pass kernel"):
+        quant.gemv_pack_dev(0x1000, Q4_K, 1024, 8, 0x1000)
