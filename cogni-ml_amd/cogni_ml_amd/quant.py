@@ -85,6 +85,13 @@ def gemv_many_dev(w_ptrs, w_type, x_ptr, out_ptrs, out_dims, in_dim, tokens=1, s
                                          stream))
 
 
+def gemv_one_pass_from(w_type, in_dim):
+    """Token count from which gemv_dev packs the activations and reads the weights once (0: never for this shape)."""
+    f = hip.lib().cogni_gemv_one_pass_from
+    f.restype = ctypes.c_uint32
+    return int(f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim)))
+
+
 def gemv_image_bytes(w_type, in_dim, tokens):
     """Bytes of the activation image of the one-pass multi-token GEMV; 0 = no such kernel for the combination."""
     f = hip.lib().cogni_gemv_image_bytes
@@ -92,10 +99,11 @@ def gemv_image_bytes(w_type, in_dim, tokens):
     return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens))
 
 
-def gemv_packed_launch_dims(total_rows):
+def gemv_packed_launch_dims(w_type, in_dim, total_rows):
     """(grid_x, block_x, shared_mem_bytes) of the one-pass kernel for a launch of total_rows rows."""
     g, b, sh = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
-    _check(hip.lib().cogni_gemv_packed_launch_dims(ctypes.c_uint32(total_rows), ctypes.byref(g), ctypes.byref(b), ctypes.byref(sh)))
+    _check(hip.lib().cogni_gemv_packed_launch_dims(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(total_rows),
+                                                   ctypes.byref(g), ctypes.byref(b), ctypes.byref(sh)))
     return g.value, b.value, sh.value
 
 

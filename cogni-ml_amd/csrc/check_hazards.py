@@ -1,0 +1,118 @@
+#!/usr/bin/env python3
+"""Build-time check of the gfx950 code object for two instruction-spacing rules that the compiler keeps for the code it
+emits itself but cannot keep for instructions written inside asm statements:
+
+  * a vector instruction that writes a scalar register (v_readfirstlane_b32, v_readlane_b32, a compare with a scalar
+    destination, a carry-out) must be five wait states ahead of a memory instruction that reads that register as its
+    scalar base;
+  * a write of M0 must be one wait state ahead of a global load that writes to LDS.
+
+An instruction is one wait state, "s_nop N" is N + 1. The scan is linear over each kernel of the disassembly (this
+library's own code object, made by llvm-objdump); labels do not reset it, so a sequence that is only adjacent in the
+file, not in execution, can be reported too: better that than the reverse.
+
+usage: check_hazards.py <llvm-objdump> <code object>       exit status 1 and a report when a rule is broken
+"""
+import re
+import subprocess
+import sys
+
+VALU_SGPR_TO_VMEM = 5
+M0_TO_LDS_DMA = 1
+# vector instructions whose second operand is a scalar destination (carry or scale flag)
+SDST_SECOND = ("v_mad_u64_u32", "v_mad_i64_i32", "v_add_co_u32", "v_sub_co_u32", "v_subrev_co_u32", "v_addc_co_u32",
+               "v_subb_co_u32", "v_subbrev_co_u32", "v_div_scale_f32", "v_div_scale_f64")
+SREG = re.compile(r"^s(\d+)$|^s\[(\d+):(\d+)\]$")
+
+
+def sregs(operand):
+    """The scalar registers an operand names, as a set of numbers."""
+    m = SREG.match(operand.strip())
+    if not m:
+        return set()
+    if m.group(1) is not None:
+        return {int(m.group(1))}
+    return set(range(int(m.group(2)), int(m.group(3)) + 1))
+
+
+def written_sgprs(mnemonic, operands):
+    if not mnemonic.startswith("v_") or not operands:
+        return set()
+    out = set(sregs(operands[0]))
+    if mnemonic.startswith(SDST_SECOND) and len(operands) > 1:
+        out |= sregs(operands[1])
+    return out
+
+
+def is_vmem(mnemonic):
+    return mnemonic.startswith(("global_", "buffer_", "flat_", "scratch_"))
+
+
+def vmem_scalar_base(mnemonic, operands):
+    """Scalar registers a memory instruction reads: every scalar operand it has (base pair, resource, offset)."""
+    out = set()
+    for op in operands:
+        out |= sregs(op.split(" ")[0])
+    return out
+
+
+def check(lines):
+    problems = []
+    kernel = "?"
+    recent = []      # (wait states since, written sgprs, text) of recent vector-writes-scalar instructions
+    m0_age = None    # wait states since the last write of m0
+    for raw in lines:
+        line = raw.split("//")[0].strip()
+        if not line:
+            continue
+        lab = re.match(r"^[0-9a-f]+ <([^>]+)>:$", line)
+        if lab:
+            if not lab.group(1).startswith("L"):
+                kernel = lab.group(1)
+                recent, m0_age = [], None
+            continue
+        if line.endswith(":") or line.startswith((".", "Disassembly", "/")) or "file format" in line:
+            continue
+        parts = line.split(None, 1)
+        mnemonic = parts[0]
+        operands = [o.strip() for o in parts[1].split(",")] if len(parts) > 1 else []
+        if is_vmem(mnemonic):
+            used = vmem_scalar_base(mnemonic, operands)
+            for age, regs, text in recent:
+                if age < VALU_SGPR_TO_VMEM and used & regs:
+                    problems.append("%s: '%s' reads s%s %d wait state(s) after '%s' (needs %d)" % (
+                        kernel, line, sorted(used & regs), age, text, VALU_SGPR_TO_VMEM))
+            if "_lds_" in mnemonic and m0_age is not None and m0_age < M0_TO_LDS_DMA:
+                problems.append("%s: '%s' %d wait state(s) after a write of m0 (needs %d)" % (kernel, line, m0_age, M0_TO_LDS_DMA))
+        states = 1
+        if mnemonic == "s_nop" and operands:
+            states = int(operands[0], 0) + 1
+        recent = [(age + states, regs, text) for age, regs, text in recent if age + states < 8]
+        if m0_age is not None:
+            m0_age += states
+        w = written_sgprs(mnemonic, operands)
+        if w:
+            recent.append((0, w, line))
+        if mnemonic.startswith("s_") and operands and operands[0] == "m0":
+            m0_age = 0
+    return problems
+
+
+def main(argv):
+    if len(argv) != 3:
+        print(__doc__)
+        return 2
+    dis = subprocess.run([argv[1], "-d", "--no-show-raw-insn", argv[2]], check=True, capture_output=True, text=True).stdout
+    problems = check(dis.splitlines())
+    n = dis.count("\n")
+    if problems:
+        print("check_hazards: %d problem(s) in %s" % (len(problems), argv[2]))
+        for p in problems[:40]:
+            print("  " + p)
+        return 1
+    print("check_hazards: %s clean (%d lines of disassembly)" % (argv[2], n))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv))

@@ -263,9 +263,9 @@ int cogni_quant_init(int32_t ordinal) {
     HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
     g_rt.fns.emplace(name, fn);
   }
-  g_rt.image_slot_bytes = ((size_t)gemv_mt_image_bytes(GEMV_MT_MAX_IN_DIM) + 255) & ~(size_t)255;
+  g_rt.image_slot_bytes = ((size_t)gemv_mt_image_bytes(COGNI_TYPE_Q6_K, GEMV_MT_MAX_IN_DIM) + 255) & ~(size_t)255;
   HIP_TRY(hipMalloc(&g_rt.image_pool, g_rt.image_slot_bytes * Runtime::kImageSlots), "hipMalloc(activation images)");
-  for (const char* name : {"pack_x_mt_f16", "q4_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32"}) {
+  for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32"}) {
     hipFunction_t fn = nullptr;
     HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
     g_rt.fns.emplace(name, fn);
@@ -303,15 +303,18 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 
 // ---- several tokens in one pass over the weights: pack the activations once, then one launch per matrix list ------
 size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {
-  return gemv_mt_supported(w_type, (int)tokens, in_dim) ? (size_t)gemv_mt_image_bytes(in_dim) : 0;
+  return gemv_mt_supported(w_type, (int)tokens, in_dim) ? (size_t)gemv_mt_image_bytes(w_type, in_dim) : 0;
 }
 
-int cogni_gemv_packed_launch_dims(uint32_t total_rows, uint32_t* grid_x, uint32_t* block_x, uint32_t* shared_mem_bytes) {
-  if (!grid_x || !block_x || !shared_mem_bytes || total_rows == 0)
+uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim) { return gemv_mt_from(w_type, in_dim); }
+
+int cogni_gemv_packed_launch_dims(uint32_t w_type, uint32_t in_dim, uint32_t total_rows, uint32_t* grid_x, uint32_t* block_x,
+                                  uint32_t* shared_mem_bytes) {
+  if (!grid_x || !block_x || !shared_mem_bytes || total_rows == 0 || !gemv_mt_supported(w_type, 2, in_dim))
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_launch_dims: bad argument");
-  *grid_x = gemv_mt_grid(total_rows);
+  *grid_x = gemv_mt_grid(w_type, in_dim, total_rows);
   *block_x = GEMV_MT_WAVES * 64;
-  *shared_mem_bytes = gemv_mt_lds_bytes();
+  *shared_mem_bytes = gemv_mt_lds_bytes(w_type);
   return 0;
 }
 
@@ -321,7 +324,7 @@ int cogni_gemv_pack_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t t
                                             "(cogni_gemv_image_bytes is 0)");
   if (!x || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack_dev: null device pointer");
   void* params[] = {&x, &image, &tokens, &in_dim};
-  return launch("pack_x_mt_f16", 2 * (in_dim >> 8), 256, 0, params, stream);
+  return launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_mt_q6k_f16" : "pack_x_mt_q4k_f16", 2 * (in_dim >> 8), 256, 0, params, stream);
 }
 
 int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,
@@ -348,7 +351,8 @@ int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image
     if (total > 0x7FFFFFFFull) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: too many rows");
     uint64_t res = i0 == 0 ? residual : 0;
     void* params[] = {&w[0], &w[1], &w[2], &image, &res, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2], &tokens};
-    const int rc = launch("q4_k_gemv_mt_f32", gemv_mt_grid((uint32_t)total), GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(), params, stream);
+    const int rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt_f32" : "q4_k_gemv_mt_f32", gemv_mt_grid(w_type, in_dim, (uint32_t)total),
+                          GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type), params, stream);
     if (rc != 0) return rc;
     i0 += n;
   }
@@ -359,11 +363,11 @@ int cogni_gemv_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type
                                  uint32_t out_dim, uint32_t tokens, void* stream) {
   if (!w_gate || !w_up || !image || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: null device pointer");
   if (out_dim == 0 || out_dim > 0x7FFFFFFFu) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: bad out_dim");
-  if (!gemv_mt_supported(w_type, (int)tokens, in_dim))
+  if (!gemv_mt_supported(w_type, (int)tokens, in_dim) || w_type != COGNI_TYPE_Q4_K)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: no one-pass kernel for this type, token count and in_dim");
   const uint32_t groups = (out_dim + 15) / 16;
   void* params[] = {&w_gate, &w_up, &image, &out, &in_dim, &out_dim, &tokens};
-  return launch("q4_k_gemv_mt_swiglu_f32", groups < 256u ? groups : 256u, GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(), params, stream);
+  return launch("q4_k_gemv_mt_swiglu_f32", groups < 256u ? groups : 256u, GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type), params, stream);
 }
 
 // Token groups of up to 8 through the library's own image of `stream`: pack, then the matrices. false = not taken (no
@@ -422,10 +426,11 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
   if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: zero dimension");
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
-  // five tokens and more of a matrix the one-pass kernel takes: groups of up to eight, the weights read once per group
-  {
+  // several tokens of a matrix the one-pass kernel takes: groups of up to eight, the weights read once per group, from
+  // the token count at which pack + one pass measures faster than the kernels below
+  if (const uint32_t from = gemv_mt_from(w_type, in_dim)) {
     int rc = 0;
-    if (try_one_pass(&w_raw, w_type, x, residual, &out, &out_dim, 1, in_dim, tokens, 5, stream, &rc)) return rc;
+    if (try_one_pass(&w_raw, w_type, x, residual, &out, &out_dim, 1, in_dim, tokens, from, stream, &rc)) return rc;
   }
   // tokens per launch: groups of up to 4 where the matrix-core kernel takes the shape (several passes over
   // the weights are still cheaper than one pass on the vector ALU, measured up to 8 tokens); Q8_0 up to 8; the

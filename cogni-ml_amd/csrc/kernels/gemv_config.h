@@ -153,33 +153,44 @@ static inline unsigned gemv_mfma_lds_bytes(unsigned type, int tokens, unsigned i
          units * (4u + 4u * nsums + 1024u);
 }
 
-// ---- several tokens in one pass over a Q4_K matrix (gemv_mt.hpp): 8 wavefronts = 8 k-slices, activations packed once ----
+// ---- several tokens in one pass over a Q4_K or Q6_K matrix (gemv_mt.hpp): 8 wavefronts = 8 k-slices, activations packed once
 #define GEMV_MT_WAVES 8
-#define GEMV_MT_TMAX 3              // 16-row tiles a wavefront carries at most
+#define GEMV_MT_TMAX 3              // 16-row tiles a wavefront carries at most (Q4_K; Q6_K two)
 #define GEMV_MT_MAX_TOKENS 8
-#define GEMV_MT_MAX_IN_DIM 4096u
-// tiles per wavefront: as many as keep 256 workgroups busy, at most GEMV_MT_TMAX (host and kernel use the same rule)
-static inline GEMV_HD unsigned gemv_mt_tiles(unsigned ntiles, unsigned grid) {
-  (void)grid;
+#define GEMV_MT_MAX_IN_DIM 12288u
+// Shapes the kernels take: Q4_K or Q6_K, 2..8 tokens, in_dim a multiple of 2048 up to 12288 (1..6 super-blocks per k-slice).
+static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned in_dim) {
+  return (type == 12 || type == 14) && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && in_dim != 0 && (in_dim & 2047u) == 0 &&
+         in_dim <= GEMV_MT_MAX_IN_DIM;
+}
+// Token count from which one matrix goes through pack + one pass rather than the per-token-group kernels (0: never): where
+// the pair measures faster. Q6_K from three tokens; Q4_K from four on rows longer than 4096 values, else from five.
+static inline unsigned gemv_mt_from(unsigned type, unsigned in_dim) {
+  if (!gemv_mt_supported(type, 2, in_dim)) return 0;
+  return type == 14 ? 3u : (in_dim > 4096u ? 4u : 5u);
+}
+// tiles per wavefront: rows of more than 4096 values one (the operands are streamed); else as many as keep 256 workgroups
+// busy, at most three (Q4_K) or two (Q6_K: its units are larger). Host and kernel use the same rule.
+static inline GEMV_HD unsigned gemv_mt_tiles(unsigned type, unsigned in_dim, unsigned ntiles) {
+  if (in_dim > 4096u) return 1;
+  const unsigned tmax = type == 14 ? 2u : (unsigned)GEMV_MT_TMAX;
   unsigned t = ntiles / 256u;
   if (t < 1) t = 1;
-  if (t > (unsigned)GEMV_MT_TMAX) t = GEMV_MT_TMAX;
+  if (t > tmax) t = tmax;
   return t;
 }
-// Shapes the kernel takes: Q4_K, 2..8 tokens, in_dim 2048 or 4096 (one or two super-blocks per k-slice).
-static inline int gemv_mt_supported(unsigned type, int tokens, unsigned in_dim) {
-  return type == 12 && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && (in_dim == 2048u || in_dim == 4096u);
-}
-static inline unsigned gemv_mt_grid(unsigned total_rows) {
-  const unsigned ntiles = (total_rows + 15) / 16, t = gemv_mt_tiles(ntiles, 0);
+static inline unsigned gemv_mt_grid(unsigned type, unsigned in_dim, unsigned total_rows) {
+  const unsigned ntiles = (total_rows + 15) / 16, t = gemv_mt_tiles(type, in_dim, ntiles);
   const unsigned groups = (ntiles + t - 1) / t;
   return groups < 256u ? groups : 256u;   // more groups than compute units: the workgroups walk them
 }
-static inline unsigned gemv_mt_lds_bytes(void) {
-  // the k-slices' partial sums, then per wavefront a slot of 16 rows x 144 bytes for each of its 2 x GEMV_MT_TMAX units
-  return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u + GEMV_MT_WAVES * 2u * GEMV_MT_TMAX * 2304u;
+// the k-slices' partial sums, then per wavefront the slots of its units: 6 x (16 rows x 144 B) for Q4_K, 4 x (16 rows x 240 B)
+// for Q6_K
+static inline unsigned gemv_mt_lds_bytes(unsigned type) {
+  return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u + GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : 6u * 2304u);
 }
-// bytes of the activation image pack_x_mt_f16 writes: the operands, then 20 floats per (super-block, token pair)
-static inline unsigned long long gemv_mt_image_bytes(unsigned in_dim) {
-  return (unsigned long long)(in_dim >> 8) * (8192u + 4u * 80u);
+// bytes of the activation image: 8 KiB of operands per super-block, then per (super-block, token pair) the two scales and
+// the sub-block sums (Q4_K 20 floats, Q6_K 36)
+static inline unsigned long long gemv_mt_image_bytes(unsigned type, unsigned in_dim) {
+  return (unsigned long long)(in_dim >> 8) * (8192u + 4u * (type == 14 ? 144u : 80u));
 }

@@ -80,7 +80,8 @@ const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add);
  * No GPU needed. */
 int cogni_gemv_launch_dims(uint32_t type, uint32_t tokens, uint32_t in_dim, uint32_t out_dim, uint32_t* grid_x,
                            uint32_t* block_x, uint32_t* shared_mem_bytes);
-/* The kernel the library itself launches for this shape, with its geometry: for 2..4 tokens of a Q4_K matrix and
+/* The kernel the library itself launches for this shape where the call does not go through pack + one pass (see
+ * cogni_gemv_one_pass_from), with its geometry: for 2..4 tokens of a Q4_K matrix and
  * 3 or 4 tokens of a Q5_K or Q6_K matrix whose activations fit the staging buffer (tokens * in_dim / 256 <= 96, or 64 from
  * 3 tokens) or whose in_dim is a multiple of 2048 (staged a chunk at a time) that is the matrix-core variant
  * "q4_k_gemv_mfma_[add_]f32_tbatchM" / "q5_k_..." / "q6_k_gemv_mfma_[add_]f32_tbatchM" (same parameter list, block 512), otherwise the kernel
@@ -107,8 +108,9 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 
 /* Decode GEMV, weights read once for all tokens:
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
- * fp32 accumulation. tokens >= 1; five and more tokens of a matrix the one-pass kernel takes (see cogni_gemv_pack_dev
- * below) go in groups of up to 8 with the weights read once per group; otherwise they are issued as consecutive launches
+ * fp32 accumulation. tokens >= 1; several tokens of a matrix the one-pass kernel takes (see cogni_gemv_pack_dev below;
+ * Q6_K from three tokens, Q4_K from four on rows longer than 4096 values, else from five) go in groups of up to 8 with
+ * the weights read once per group; otherwise they are issued as consecutive launches
  * of the token count that measures
  * fastest for the type and shape: up to 4 where cogni_gemv_plan picks the matrix-core kernel, else pairs for the
  * K-quants (one group of three when the count is odd and the matrix is short enough for one workgroup per row group) and up to 8 for Q8_0. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
@@ -117,38 +119,47 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
                    uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 
-/* Several tokens in ONE pass over the weights (Q4_K, in_dim 2048 or 4096, 2..8 tokens): the activations are packed once
- * into an image - per 256-value super-block the matrix-core operands of its eight instructions (x as two binary16 terms,
- * scaled per token and super-block), then the scales and sub-block sums - and every matrix that meets those activations
- * (q | k | v | gate | up of a layer) is one launch that reads its weights once for all the tokens. The reference's
- * multi-token kernels stop at four tokens per pass (tbatch4, src/ml/cuda/kernels/q4k_gemv_probe.ptx:437-768).
+/* Several tokens in ONE pass over the weights (Q4_K and Q6_K, in_dim a multiple of 2048 up to 12288, 2..8 tokens): the
+ * activations are packed once into an image - per 256-value super-block the matrix-core operands of its instructions (x as
+ * two binary16 terms, scaled per token and super-block), then the scales and sub-block sums - and every matrix that meets
+ * those activations (q | k | v | gate | up of a layer) is one launch that reads its weights once for all the tokens. The
+ * reference's multi-token kernels stop at four tokens per pass (tbatch4, src/ml/cuda/kernels/q4k_gemv_probe.ptx:437-768,
+ * q6k_gemv_probe.ptx:977). The image depends on the weight type (Q4_K and Q6_K order their sub-blocks differently).
  *   cogni_gemv_image_bytes  size of the image for (type, in_dim, tokens); 0 = no one-pass kernel for that combination.
- *   cogni_gemv_pack_dev     kernel "pack_x_mt_f16" (x, image, tokens:u32, in_dim:u32), block 256, grid 2 * in_dim / 256.
+ *   cogni_gemv_pack_dev     kernel "pack_x_mt_q4k_f16" | "pack_x_mt_q6k_f16" (x, image, tokens:u32, in_dim:u32), block 256,
+ *                           grid 2 * in_dim / 256.
  *   cogni_gemv_packed_dev   `count` (1..8) matrices of one type and in_dim against the image:
  *                           out[i][m*out_dims[i] + o] = (residual ? residual[m*out_dims[0] + o] : 0) + sum_j x[m][j] deq(W_i[o][j])
- *                           (a residual only with count == 1). Kernel "q4_k_gemv_mt_f32" (w0, w1, w2, image, residual, out0,
- *                           out1, out2, in_dim, rows0, rows1, rows2, tokens), block 512, up to three matrices per launch as
- *                           one matrix of all their rows (a matrix whose row count is not a multiple of 16 ends its launch),
- *                           grid = min(256, row groups), dynamic shared memory 122880 bytes.
+ *                           (a residual only with count == 1). Kernel "q4_k_gemv_mt_f32" | "q6_k_gemv_mt_f32" (w0, w1, w2,
+ *                           image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens), block 512, up to three
+ *                           matrices per launch as one matrix of all their rows (a matrix whose row count is not a multiple
+ *                           of 16 ends its launch), geometry from cogni_gemv_packed_launch_dims.
  * The image is caller-owned device memory; pack and GEMV are ordered by the stream. Accuracy: about 5e-7 of max|out|
  * (22-bit activations, exact weights, fp32 accumulation).
- * cogni_gemv_dev (5 tokens and more), cogni_gemv_dual_dev and cogni_gemv_many_dev (2 tokens and more) take this path by
+ * cogni_gemv_dev (from 3 to 5 tokens on, by type and row length), cogni_gemv_dual_dev and cogni_gemv_many_dev (2 tokens
+ * and more) take this path by
  * themselves with an image the library keeps per stream (8 streams at most; a ninth falls back to the kernels
  * cogni_gemv_plan describes). A graph captured from one stream carries that stream's image: replay it on one stream at a
  * time, and not beside eager calls on the capture stream. */
 size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
-/* Launch geometry of "q4_k_gemv_mt_f32" for a launch of total_rows rows (all its matrices together): a workgroup's eight
- * wavefronts carry t = clamp(tiles / 256, 1, 3) tiles of 16 rows at a time, a row group is t tiles, grid_x = min(256, row
- * groups) and the workgroups walk the groups blockIdx.x, blockIdx.x + grid_x, ... No GPU needed. */
-int cogni_gemv_packed_launch_dims(uint32_t total_rows, uint32_t* grid_x, uint32_t* block_x, uint32_t* shared_mem_bytes);
+/* The token count from which cogni_gemv_dev takes this path for one matrix (Q6_K 3; Q4_K 4 on rows longer than 4096 values,
+ * else 5), 0 where it never does; below it the call runs the kernel cogni_gemv_plan names. No GPU needed. */
+uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim);
+/* Launch geometry of the one-pass kernel for a launch of total_rows rows (all its matrices together): a workgroup's eight
+ * wavefronts carry t tiles of 16 rows at a time (in_dim above 4096: t = 1; else t = clamp(tiles / 256, 1, 3), Q6_K at most 2),
+ * a row group is t tiles, grid_x = min(256, row groups) and the workgroups walk the groups blockIdx.x, blockIdx.x +
+ * grid_x, ...; block_x = 512; shared_mem_bytes 122880 (Q4_K) or 135168 (Q6_K). No GPU needed. */
+int cogni_gemv_packed_launch_dims(uint32_t w_type, uint32_t in_dim, uint32_t total_rows, uint32_t* grid_x, uint32_t* block_x,
+                                  uint32_t* shared_mem_bytes);
 int cogni_gemv_pack_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t image, void* stream);
 int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,
                           const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream);
 /* The gate and up projections and the SwiGLU against an image, one launch:
  *   out[m*out_dim + o] = silu(sum_j x[m][j] deq(W_gate[o][j])) * sum_j x[m][j] deq(W_up[o][j])
  * Kernel "q4_k_gemv_mt_swiglu_f32" (w_gate, w_up, image, out, in_dim, out_dim, tokens), block 512, grid = min(256,
- * ceil(out_dim / 16)), dynamic shared memory as q4_k_gemv_mt_f32. The values of cogni_gemv_packed_dev on the pair
- * followed by cogni_swiglu_dev, bit for bit. cogni_gemv_dual_swiglu_dev takes this path for 2 tokens and more. */
+ * ceil(out_dim / 16)), dynamic shared memory as q4_k_gemv_mt_f32. Q4_K only. The values of
+ * cogni_gemv_packed_dev on the pair followed by cogni_swiglu_dev, bit for bit. cogni_gemv_dual_swiglu_dev takes this path
+ * for 2 tokens and more. */
 int cogni_gemv_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t image, uint64_t out, uint32_t in_dim,
                                  uint32_t out_dim, uint32_t tokens, void* stream);
 

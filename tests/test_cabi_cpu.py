@@ -214,6 +214,52 @@ def test_runner_rejects_invalid_active_counts():
     assert r.active_tokens == 4
 
 
+def test_one_pass_geometry_and_thresholds():
+    """Pack + one pass over the weights: which shapes have a kernel, the size of the activation image (8 KiB of operands
+    per super-block, then two scales and the sub-block sums per super-block and token pair), where gemv_dev switches to it,
+    and that the planned grid reaches every 16-row tile: a workgroup's eight wavefronts split the row, a row group is t
+    tiles and the workgroups walk the groups with stride grid."""
+    assert quant.gemv_image_bytes(12, 4096, 8) == 16 * (8192 + 4 * 80)
+    assert quant.gemv_image_bytes(14, 12288, 2) == 48 * (8192 + 4 * 144)
+    for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1024, 4), (12, 14336, 4), (13, 4096, 4), (8, 4096, 4), (12, 0, 4)):
+        assert quant.gemv_image_bytes(t, in_dim, tokens) == 0, (t, in_dim, tokens)
+    assert [quant.gemv_one_pass_from(12, d) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 5, 4, 4, 0, 0]
+    assert [quant.gemv_one_pass_from(t, 4096) for t in (14, 13, 8)] == [3, 0, 0]
+    rng = np.random.default_rng(11)
+    for t, tmax, lds in ((12, 3, 8 * 3 * 8 * 16 * 4 + 8 * 6 * 16 * 144), (14, 2, 8 * 3 * 8 * 16 * 4 + 8 * 4 * 16 * 240)):
+        for in_dim in (2048, 4096, 6144, 8192, 10240, 12288):
+            for rows in [1, 15, 16, 17, 4096, 4097, 12288, 8 * 4096 - 16, 151936] + [int(r) for r in rng.integers(1, 400000, 40)]:
+                grid, block, shmem = quant.gemv_packed_launch_dims(t, in_dim, rows)
+                ntiles = -(-rows // 16)
+                tiles = 1 if in_dim > 4096 else max(1, min(tmax, ntiles // 256))     # the kernel's own rule
+                groups = -(-ntiles // tiles)
+                assert (block, shmem) == (512, lds) and shmem <= 160 * 1024
+                assert grid == min(256, groups) and grid >= 1
+    for bad in ((12, 1024, 16), (13, 4096, 16), (12, 4096, 0)):
+        with pytest.raises(quant.QuantError):
+            quant.gemv_packed_launch_dims(*bad)
+
+
+def test_one_pass_argument_errors_do_not_need_a_gpu():
+    with pytest.raises(quant.QuantError, match="no one-pass kernel") as e:
+        quant.gemv_pack_dev(0x1000, 12, 1024, 4, 0x2000)
+    assert e.value.code == -1
+    with pytest.raises(quant.QuantError, match="null device pointer"):
+        quant.gemv_pack_dev(0, 12, 4096, 4, 0x2000)
+    with pytest.raises(quant.QuantError, match="count must be 1..8"):
+        quant.gemv_packed_dev([], 12, 0x2000, [], [], 4096, 4)
+    with pytest.raises(quant.QuantError, match="no one-pass kernel"):
+        quant.gemv_packed_dev([0x1000], 13, 0x2000, [0x3000], [16], 4096, 4)
+    with pytest.raises(quant.QuantError, match="a residual goes with a single matrix"):
+        quant.gemv_packed_dev([0x1000, 0x1100], 12, 0x2000, [0x3000, 0x3100], [16, 16], 4096, 4, residual_ptr=0x4000)
+    with pytest.raises(quant.QuantError, match="null pointer or zero rows"):
+        quant.gemv_packed_dev([0x1000, 0x1100], 12, 0x2000, [0x3000, 0x3100], [16, 0], 4096, 4)
+    with pytest.raises(quant.QuantError, match="no one-pass kernel"):
+        quant.gemv_packed_swiglu_dev(0x1000, 0x1100, 14, 0x2000, 0x3000, 4096, 16, 4)
+    with pytest.raises(quant.QuantError, match="bad out_dim"):
+        quant.gemv_packed_swiglu_dev(0x1000, 0x1100, 12, 0x2000, 0x3000, 4096, 0, 4)
+
+
 def test_matrix_core_gemv_grid_covers_every_row():
     """The matrix-core kernels derive the tiles per wavefront from the grid they are launched with and cover rows
     beyond one group per workgroup only by walking (not where the activations are staged in chunks): for a sweep of

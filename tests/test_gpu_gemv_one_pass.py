@@ -1,4 +1,5 @@
-"""Decode GEMV for 2..8 tokens in one pass over a Q4_K matrix (activations packed once, q4_k_gemv_mt_f32) vs the CPU oracle.
+"""Decode GEMV for 2..8 tokens in one pass over a Q4_K or Q6_K matrix (activations packed once, q4_k_gemv_mt_f32 /
+q6_k_gemv_mt_f32) vs the CPU oracle.
 
 Bars, both asserted: the north-star bound max|err| <= 1e-4 * ||x||_2 * max|w_row| per token and row, and the reference's own
 probe gate (cos >= 0.99999, max_diff <= 1e-3 * max(1, max|ref| / 64): the probe's absolute 1e-3 is meant for outputs of order
@@ -14,9 +15,9 @@ from helpers import Q4_K, Q6_K, cosine, gemv_tolerance
 pytestmark = pytest.mark.gpu
 
 
-def oracle_rows(oracle, raw, x, in_dim, out_dim, tokens):
-    want = oracle.matmul_add(x, tokens, in_dim, raw, Q4_K, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).astype(np.float64)
-    dense = np.abs(oracle.dequantize(raw, Q4_K, out_dim * in_dim)).reshape(out_dim, in_dim)
+def oracle_rows(oracle, raw, x, in_dim, out_dim, tokens, type_id=Q4_K):
+    want = oracle.matmul_add(x, tokens, in_dim, raw, type_id, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).astype(np.float64)
+    dense = np.abs(oracle.dequantize(raw, type_id, out_dim * in_dim)).reshape(out_dim, in_dim)
     return want, gemv_tolerance(x, dense, tokens, in_dim).reshape(-1)
 
 
@@ -144,7 +145,7 @@ def test_one_pass_element_order_and_scale_positions(gpu, oracle):
 
 def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
     """9 and 13 tokens: a group of eight in one pass, the rest as the token count decides (one token on the vector ALU,
-    five in one pass); in_dim 1024 and Q6_K have no one-pass kernel and keep their older paths."""
+    five in one pass); in_dim 1024, in_dim above 12288 and Q5_K have no one-pass kernel and keep their older paths."""
     rng = np.random.default_rng(11)
     for in_dim, out_dim, tokens in ((4096, 272, 9), (2048, 100, 13), (1024, 64, 8)):
         raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
@@ -155,7 +156,75 @@ def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
         assert_bars(od.read(np.float32, tokens * out_dim), want, tol, tokens, out_dim, "%dx%d M=%d" % (in_dim, out_dim, tokens))
         for a in (w, xd, od):
             a.close()
-    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(Q6_K, 4096, 8) == 0
+    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(13, 4096, 8) == 0
+    assert quant.gemv_image_bytes(Q4_K, 14336, 8) == 0 and quant.gemv_image_bytes(Q6_K, 4096, 8) == 16 * (8192 + 576)
     assert quant.gemv_image_bytes(Q4_K, 4096, 1) == 0 and quant.gemv_image_bytes(Q4_K, 4096, 9) == 0
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
         quant.gemv_pack_dev(0x1000, Q4_K, 1024, 8, 0x1000)
+
+
+LONG_AND_Q6K = [(Q4_K, 12288, 4096), (Q4_K, 6144, 530), (Q4_K, 8192, 16 * 300 + 5), (Q4_K, 10240, 33),
+                (Q6_K, 12288, 4096), (Q6_K, 4096, 4096), (Q6_K, 2048, 1040), (Q6_K, 4096, 16 * 2 * 256 * 2 + 24), (Q6_K, 6144, 50),
+                (Q6_K, 8192, 16 * 257), (Q6_K, 2048, 37)]
+
+
+@pytest.mark.parametrize("type_id,in_dim,out_dim", LONG_AND_Q6K)
+@pytest.mark.parametrize("tokens", [5, 8])
+def test_long_rows_and_q6_k_in_one_pass(gpu, oracle, type_id, in_dim, out_dim, tokens):
+    """Rows of 6144..12288 values (three to six super-blocks per k-slice: the activation operands are streamed through two
+    register sets, Q6_K with four LDS slots for six units) and Q6_K at every row length: one and two tiles per wavefront,
+    partial tiles, more row groups than workgroups, odd super-blocks (blocks that start 2 bytes off a 4-byte boundary)."""
+    print("case type=%d in_dim=%d out_dim=%d tokens=%d" % (type_id, in_dim, out_dim, tokens), flush=True)
+    assert quant.gemv_image_bytes(type_id, in_dim, tokens) == (in_dim // 256) * (8192 + (576 if type_id == Q6_K else 320))
+    rng = np.random.default_rng(type_id * 1000003 + in_dim * 13 + out_dim * 7 + tokens)
+    raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = rng.standard_normal(tokens * out_dim).astype(np.float32)
+    want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens, type_id)
+    w, xd, od, rd = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim), DevArray(res)
+    quant.gemv_dev(w.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+    plain = od.read(np.float32, tokens * out_dim)
+    assert_bars(plain, want, tol, tokens, out_dim, "type %d %dx%d M=%d" % (type_id, in_dim, out_dim, tokens))
+    quant.gemv_dev(w.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, tokens, rd.ptr)
+    assert np.array_equal(od.read(np.float32, tokens * out_dim), plain + res)
+    for a in (w, xd, od, rd):
+        a.close()
+
+
+def test_q6_k_one_pass_element_order_and_scale_positions(gpu, oracle):
+    """Unit activations pick single weights out of a Q6_K matrix: a swapped quarter, half, nibble, high-bit pair, k-group or
+    scale byte puts another weight there. Every element position of a super-block is visited, in an even and an odd block."""
+    in_dim, out_dim, tokens = 2048, 16, 8
+    rng = np.random.default_rng(6)
+    raw = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    w = DevArray(raw)
+    od = DevArray(nbytes=4 * tokens * out_dim)
+    dense = oracle.dequantize(raw, Q6_K, out_dim * in_dim).reshape(out_dim, in_dim)
+    for base in range(0, 512, 8):
+        x = np.zeros((tokens, in_dim), dtype=np.float32)
+        for m in range(tokens):                     # token m picks out column base + m
+            x[m, base + m] = 1.0
+        xd = DevArray(np.ascontiguousarray(x.reshape(-1)))
+        quant.gemv_dev(w.ptr, Q6_K, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+        got = od.read(np.float32, tokens * out_dim).reshape(tokens, out_dim)
+        for m in range(tokens):
+            assert np.allclose(got[m], dense[:, base + m], rtol=0, atol=2e-6 * float(np.abs(dense).max())), (base, m)
+        xd.close()
+    for a in (w, od):
+        a.close()
+
+
+def test_q6_k_lists_share_one_image(gpu, oracle):
+    """Two Q6_K matrices against one activation block through the list operator (one pack, one launch)."""
+    in_dim, dims, tokens = 4096, (1024, 272), 6
+    rng = np.random.default_rng(66)
+    raws = [synth.make_weights(rng, Q6_K, d, in_dim) for d in dims]
+    x = synth.make_activations(rng, tokens, in_dim)
+    ws, xd = [DevArray(r) for r in raws], DevArray(x)
+    outs = [DevArray(nbytes=4 * tokens * d) for d in dims]
+    quant.gemv_many_dev([w_.ptr for w_ in ws], Q6_K, xd.ptr, [o.ptr for o in outs], list(dims), in_dim, tokens)
+    for raw, o, d in zip(raws, outs, dims):
+        want, tol = oracle_rows(oracle, raw, x, in_dim, d, tokens, Q6_K)
+        assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, "q6_k list member %d" % d)
+    for a in ws + outs + [xd]:
+        a.close()
