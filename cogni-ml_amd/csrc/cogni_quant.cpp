@@ -122,6 +122,13 @@ const char* type_name(uint32_t type) {
     case COGNI_TYPE_IQ4_NL: return "IQ4_NL";
     case COGNI_TYPE_F16: return "F16";
     case COGNI_TYPE_F32: return "F32";
+    case 2: return "Q4_0";
+    case 3: return "Q4_1";
+    case 6: return "Q5_0";
+    case 7: return "Q5_1";
+    case 10: return "Q2_K";
+    case 11: return "Q3_K";
+    case 15: return "Q8_K";
     default: return "unknown";
   }
 }
@@ -129,6 +136,8 @@ const char* type_name(uint32_t type) {
 bool gemv_type(uint32_t t) {
   return t == COGNI_TYPE_Q8_0 || t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q5_K || t == COGNI_TYPE_Q6_K;
 }
+// F32, F16, IQ4_NL: the arms of the reference's dispatch served by the plain kernels (quant_matmul.cr:30-32)
+bool plain_type(uint32_t t) { return t == COGNI_TYPE_F32 || t == COGNI_TYPE_F16 || t == COGNI_TYPE_IQ4_NL; }
 bool k_quant(uint32_t t) { return t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q5_K || t == COGNI_TYPE_Q6_K; }
 
 // Bytes of one weight row, the reference's row_bytes (quant_matmul.cr:46-47, 241-242).
@@ -420,10 +429,16 @@ int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, ui
 
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out, uint32_t in_dim,
                    uint32_t out_dim, uint32_t tokens, void* stream) {
-  if (!gemv_type(w_type))
+  if (!gemv_type(w_type) && !plain_type(w_type))
     return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for fused matmul: ") + type_name(w_type));
   if (!w_raw || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: null device pointer");
   if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_dev: zero dimension");
+  if (plain_type(w_type)) {   // any token count in one launch: a wavefront per row, the workgroups walk the rows
+    const char* name = w_type == COGNI_TYPE_F32 ? "f32_gemv_plain_f32" : (w_type == COGNI_TYPE_F16 ? "f16_gemv_plain_f32" : "iq4_nl_gemv_plain_f32");
+    const uint32_t groups = (out_dim + 3) / 4;
+    void* params[] = {&w_raw, &x, &residual, &out, &in_dim, &out_dim, &tokens};
+    return launch(name, groups < 65536u ? groups : 65536u, 256, 0, params, stream);
+  }
   if (k_quant(w_type) && (in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
   // several tokens of a matrix the one-pass kernel takes: groups of up to eight, the weights read once per group, from
@@ -876,7 +891,7 @@ int cogni_dequantize(const void* data, size_t data_bytes, uint32_t type, int64_t
 int cogni_weight_create(cogni_quant_weight** qw, const void* raw, size_t raw_bytes, uint32_t type, int32_t out_dim,
                         int32_t in_dim) {
   if (!qw || !raw) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_create: null argument");
-  if (!gemv_type(type))
+  if (!gemv_type(type) && !plain_type(type))
     return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for fused matmul: ") + type_name(type));
   if (out_dim <= 0 || in_dim <= 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_weight_create: dimensions must be positive");
   if (k_quant(type) && in_dim % 256 != 0)

@@ -3,6 +3,7 @@
 // its PTX modules (src/ml/cuda/driver.cr:115-127).
 #include "kernels/dequant.hpp"
 #include "kernels/gemv.hpp"
+#include "kernels/gemv_plain.hpp"
 #include "kernels/gemv_mfma.hpp"
 #include "kernels/gemv_mfma_q6k.hpp"
 #include "kernels/gemv_mt.hpp"

@@ -110,12 +110,16 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
  * fp32 accumulation. tokens >= 1; several tokens of a matrix the one-pass kernel takes (see cogni_gemv_pack_dev below;
  * Q6_K from three tokens, Q4_K from four on rows longer than 4096 values, else from five) go in groups of up to 8 with
- * the weights read once per group; otherwise they are issued as consecutive launches
- * of the token count that measures
+ * the weights read once per group; otherwise they are issued as consecutive launches of the token count that measures
  * fastest for the type and shape: up to 4 where cogni_gemv_plan picks the matrix-core kernel, else pairs for the
- * K-quants (one group of three when the count is odd and the matrix is short enough for one workgroup per row group) and up to 8 for Q8_0. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the
- * same, bin/cuda_q4k_gemv_probe.cr:125); Q8_0 accepts any in_dim >= 1 (its last block is clipped,
- * quant_matmul.cr:241,259). Types: Q8_0, Q4_K, Q5_K, Q6_K. */
+ * K-quants (one group of three when the count is odd and the matrix is short enough for one workgroup per row group)
+ * and up to 8 for Q8_0. in_dim must be a multiple of 256 for Q4_K/Q5_K/Q6_K (the reference requires the same,
+ * bin/cuda_q4k_gemv_probe.cr:125); Q8_0 accepts any in_dim >= 1 (its last block is clipped, quant_matmul.cr:241,259).
+ * Types: Q8_0, Q4_K, Q5_K, Q6_K on the kernels above; F32, F16 and IQ4_NL (the remaining arms of
+ * QuantMatmul.matmul_add, quant_matmul.cr:30-32, 272-368) on plain row kernels "f32_gemv_plain_f32" |
+ * "f16_gemv_plain_f32" | "iq4_nl_gemv_plain_f32" (w_raw, x, residual, out, in_dim:u32, out_dim:u32, tokens:u32), block 256
+ * (a wavefront per output row), any in_dim >= 1 and any token count in one launch. Every other ggml type is refused with
+ * COGNI_ERR_UNSUPPORTED_TYPE and the reference's message. */
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
                    uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 

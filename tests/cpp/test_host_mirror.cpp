@@ -62,8 +62,8 @@ static void host_errors() {
   EXPECT(data_bytes(TensorType::Q6_K, 151936LL * 4096) == 510504960LL);
   std::vector<float> x(256), bias(1);
   std::vector<uint8_t> w(144);
-  EXPECT(throws_with<QuantError>([&] { QuantMatmul::matmul_add(x, 1, 256, w.data(), w.size(), TensorType::IQ4_NL, 1, bias); },
-                                 "Unsupported quant type for fused matmul: IQ4_NL"));
+  EXPECT(throws_with<QuantError>([&] { QuantMatmul::matmul_add(x, 1, 256, w.data(), w.size(), TensorType::Q4_0, 1, bias); },
+                                 "Unsupported quant type for fused matmul: Q4_0"));
   EXPECT(throws_with<QuantError>([&] { QuantMatmul::matmul_add(x, 1, 100, w.data(), w.size(), TensorType::Q4_K, 1, bias); },
                                  "in_dim multiple of 256"));
   EXPECT(throws_with<QuantError>([&] { Dequant::dequantize(w.data(), w.size(), TensorType::Q2_K, 256); },

@@ -137,8 +137,8 @@ def test_argument_errors_do_not_need_a_gpu():
     import numpy as np
     x = np.zeros(256, dtype=np.float32)
     w = np.zeros(144, dtype=np.uint8)
-    with pytest.raises(quant.QuantError, match="Unsupported quant type for fused matmul: IQ4_NL") as e:
-        quant.matmul_add(x, 1, 256, w, 20, 1, None)
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for fused matmul: Q4_0") as e:
+        quant.matmul_add(x, 1, 256, w, 2, 1, None)
     assert e.value.code == -2
     with pytest.raises(quant.QuantError, match="requires in_dim multiple of 256") as e:
         quant.matmul_add(x, 1, 100, w, 12, 1, None)
