@@ -26,6 +26,7 @@ only reads the same bytes takes.
                                     known size, for rocprofv3 --pmc / --kernel-trace runs
   python bench.py --mode pmc-gemm   plain launches of the M = 512 prefill GEMM for the same purpose
   python bench.py --mode ceiling    empty launch, read-only stream, matrix-core-only loop
+  python bench.py --launch direct   the same work without HIP graphs (for rocprofv3 --kernel-trace)
 """
 import argparse
 import ctypes
@@ -86,12 +87,15 @@ class Rotating:
         self.needed = min(copies, max(2, int(math.ceil(1.1 * LLC_BYTES / max(1, bytes_per_copy)))))
 
 
+USE_GRAPHS = True   # --launch direct clears it: every launch goes to the stream one by one (profiler runs)
+
+
 def measure(hip, stream, rot, steps, warmup, graph=True):
     """Time `steps` launches of rot.launch(copy_index, stream) per sample; see the module docstring.
     Returns a dict: us (median per step), us_min, us_max, samples, replays_per_sample, timed_region_ms, graphed."""
     C, G = rotation(steps, rot.copies, rot.needed)
     graphs, execs = [], []
-    if graph:
+    if graph and USE_GRAPHS:
         try:
             for g in range(G):
                 stream.begin_capture(1)
@@ -99,16 +103,15 @@ def measure(hip, stream, rot, steps, warmup, graph=True):
                     rot.launch((g * steps + i) % C, stream)
                 gr = stream.end_capture()
                 graphs.append(gr)
-                ex = gr.instantiate()
-                ex.upload(stream)
-                execs.append(ex)
+                ex = gr.instantiate()   # (no hipGraphUpload: the ramp below replays every graph before anything is timed,
+                execs.append(ex)        #  and a profiler that reads kernel arguments cannot follow them into device memory)
             stream.synchronize()
         except Exception as e:   # stream capture unavailable: direct launches
             log("graph capture failed (%s); timing direct launches" % e)
             for o in execs + graphs:
                 o.close()
             graphs, execs = [], []
-    counter = [0]
+    counter = [0]   # replays so far: each is `steps` launches (warm-up launches come on top)
 
     def replay():
         if execs:
@@ -157,7 +160,7 @@ def measure(hip, stream, rot, steps, warmup, graph=True):
         o.close()
     return {"us": per_step_us[len(per_step_us) // 2], "us_min": per_step_us[0], "us_max": per_step_us[-1],
             "samples": samples, "replays_per_sample": inner, "timed_region_ms": region_ms, "graphed": bool(execs),
-            "buffers_rotated": C}
+            "buffers_rotated": C, "launches": warmup + counter[0] * steps}
 
 
 class GemvCase:
@@ -302,8 +305,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--mode", choices=["headline", "cases", "pmc", "pmc-gemm", "ceiling"], default="headline")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--launch", choices=["graph", "direct"], default="graph",
+                    help="direct: no HIP graphs, for runs under rocprofv3 (it crashes in hipGraphLaunch when a graph is "
+                         "replayed back to back); per-step times then include the host's launch cost, kernel durations do not")
     ap.add_argument("--seed", type=int, default=1234)
     args = ap.parse_args()
+    global USE_GRAPHS
+    USE_GRAPHS = args.launch == "graph"
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path has no multi-GPU part (run with --gpus 1)")
     if args.steps <= 0 or args.warmup < 0:
@@ -400,6 +408,8 @@ def main():
     gbps = head.bytes_per_step / hr["us"] / 1e3
     # cache-resident figure (one copy only), reported beside the HBM one
     hot = measure(hip, stream, Rotating(lambda c, s: head.launch(0, s), 1, head.w_bytes), args.steps, args.warmup)
+    # (for reading a kernel trace of this run: the first dispatches of the headline kernel, in order)
+    log("headline_dispatch_order=1 parity launch, %d over rotating copies, %d over one copy" % (hr["launches"], hot["launches"]))
     hot_gbps = head.bytes_per_step / hot["us"] / 1e3
     floor_us, floor_grid = mk.read_floor(stream, head, args.steps, args.warmup)
     log("case=q4_k_gemv ffn_up\ntype=Q4_K\nshape=%dx%d\ntokens=1\nraw_bytes=%d\ncopies=%d\nreps=%d\nwarmup=%d\n"

@@ -421,19 +421,88 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   if constexpr (TOP1) top1_store();
 }
 
+// ---- one token of a small Q8_0 matrix -----------------------------------------------------------
+// A matrix of a few megabytes is over before the memory system is busy: its launch is a chain of latencies (dispatch,
+// activations, barrier, first rows, reduction) and the staging above spends two of them one after the other. Where a row is
+// one column set, every workgroup has one row group, the weights are at most GEMV_SMALL_BYTES and a lane's share of x is
+// small (Q8_0: 16 values; the 64 values of a K-quant lane cost more to fetch per wavefront than the staging they would
+// replace - Q5_K 4096x4096 7.8 us this way against 4.9), a lane takes its share of x straight from global memory into
+// registers (the wavefronts of a compute unit hit the same lines), requests its R rows at once behind it, and nothing waits
+// for another wavefront: no LDS, no barrier. The arithmetic and its order are those of gemv_core (F::compute on the same
+// operands, the same sums, wave_sum), so the values are the same bit for bit.
+#define GEMV_SMALL_BYTES (16u << 20)
+template <class F>
+__device__ __forceinline__ bool gemv_small_shape(u32 in_dim, u32 out_dim) {
+  const u32 nb = F::nblocks(in_dim);
+  const u32 group_rows = GEMV_WAVES * F::rows(1);
+  return F::NF4 <= 4 && nb <= (u32)F::BPS && (size_t)out_dim * F::row_bytes(nb) <= GEMV_SMALL_BYTES &&
+         (size_t)gridDim.x * group_rows >= out_dim;
+}
+template <class F, bool ADD>
+__device__ __forceinline__ void gemv_small_core(const uint8_t* __restrict__ w, const float* __restrict__ x,
+                                                const float* __restrict__ residual, float* __restrict__ out, u32 in_dim,
+                                                u32 out_dim) {
+  constexpr int R = F::rows(1), NF4 = F::NF4, NSUM = F::NSUM;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const typename F::Lane ln(lane);
+  const u32 nb = F::nblocks(in_dim);
+  const size_t row_bytes = F::row_bytes(nb);
+  const u32 row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
+  if (row0 >= out_dim) return;   // (whole wavefronts; nothing below meets another wavefront)
+  float4 xr[1][NF4];
+#pragma unroll
+  for (int i = 0; i < NF4; i++) xr[0][i] = F::load_x(x, F::x_elem(0, lane, i), in_dim);
+  const uint8_t* rowp[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) rowp[r] = w + (size_t)min(row0 + r, out_dim - 1) * row_bytes;
+  typename F::template Stage<R> st;
+  F::template load<R>(st, rowp, ln, 0, nb);
+  float sx[1][NSUM];
+#pragma unroll
+  for (int k = 0; k < NSUM; k++) {
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NF4 / NSUM; i++) a += hsum4(xr[0][k * (NF4 / NSUM) + i]);
+    sx[0][k] = a;
+  }
+  const bool valid = (u32)ln.jb < nb;
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    float c[1];
+    F::template compute<R, 1>(st, r, ln, xr, sx, c);
+    float v = wave_sum(0.0f + (valid ? c[0] : 0.0f));
+    const u32 row = row0 + r;
+    if (lane == 0 && row < out_dim) {
+      if (ADD) v += residual[row];
+      out[row] = v;
+    }
+  }
+}
+template <class F, int M, bool ADD>
+__device__ __forceinline__ void gemv_entry(const uint8_t* w, const float* x, const float* residual, float* out, u32 in_dim, u32 out_dim) {
+  if constexpr (M == 1) {
+    if (gemv_small_shape<F>(in_dim, out_dim)) {
+      gemv_small_core<F, ADD>(w, x, residual, out, in_dim, out_dim);
+      return;
+    }
+  }
+  gemv_core<F, M, ADD>(w, x, residual, out, in_dim, out_dim);
+}
+
 // ---- entry points ---------------------------------------------------------------------------
 // M = 1, 2: ask for at least 3 wavefronts per SIMD so a 12288-row matrix is resident in one round
 #define GEMV_OCC(M) __attribute__((amdgpu_waves_per_eu((M) <= 1 ? 3 : 1)))
 #define GEMV_ENTRY(NAME, FMT, M)                                                                                \
   extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(M) void NAME(const uint8_t* w, const float* x, float* out,   \
                                                                  u32 in_dim, u32 out_dim) {                     \
-    gemv_core<FMT, M, false>(w, x, nullptr, out, in_dim, out_dim);                                              \
+    gemv_entry<FMT, M, false>(w, x, nullptr, out, in_dim, out_dim);                                             \
   }
 #define GEMV_ADD_ENTRY(NAME, FMT, M)                                                                            \
   extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(M) void NAME(const uint8_t* w, const float* x,               \
                                                                  const float* residual, float* out, u32 in_dim, \
                                                                  u32 out_dim) {                                 \
-    gemv_core<FMT, M, true>(w, x, residual, out, in_dim, out_dim);                                              \
+    gemv_entry<FMT, M, true>(w, x, residual, out, in_dim, out_dim);                                             \
   }
 
 #define GEMV_FAMILY(PFX, FMT)                        \

@@ -12,7 +12,9 @@
 #ifndef GEMV_ROWS_Q6K
 #define GEMV_ROWS_Q6K(M) 2
 #endif
+#ifndef GEMV_ROWS_Q80
 #define GEMV_ROWS_Q80(M) 4
+#endif
 
 // rows of the weight matrix one workgroup produces
 static inline int gemv_rows_per_block(unsigned type, int tokens) {
