@@ -56,6 +56,17 @@ lib LibCogniHIP
                      in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemv_plan(type : UInt32, tokens : UInt32, add : Int32, in_dim : UInt32, out_dim : UInt32, kernel : UInt8**,
                       grid_x : UInt32*, block_x : UInt32*, shared_mem_bytes : UInt32*) : Int32
+  fun cogni_gemv_one_pass_from(w_type : UInt32, in_dim : UInt32) : UInt32
+  fun cogni_gemv_image_bytes(w_type : UInt32, in_dim : UInt32, tokens : UInt32) : LibC::SizeT
+  fun cogni_gemv_packed_launch_dims(w_type : UInt32, in_dim : UInt32, total_rows : UInt32,
+                                    grid_x : UInt32*, block_x : UInt32*, shared_mem_bytes : UInt32*) : Int32
+  fun cogni_gemv_pack_dev(x : UInt64, w_type : UInt32, in_dim : UInt32, tokens : UInt32, image : UInt64, stream : Void*) : Int32
+  fun cogni_gemv_packed_dev(w_raw : UInt64*, w_type : UInt32, image : UInt64, residual : UInt64, out : UInt64*,
+                            out_dims : UInt32*, count : UInt32, in_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemv_packed_swiglu_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, image : UInt64, out : UInt64,
+                                   in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemv_top1_noalloc_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, top1_ids : UInt64, top1_values : UInt64,
+                                  in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemv_dual_dev(w_raw_a : UInt64, w_raw_b : UInt64, w_type : UInt32, x : UInt64, out_a : UInt64, out_b : UInt64,
                           in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemv_many_dev(w_raw : UInt64*, w_type : UInt32, x : UInt64, out : UInt64*, out_dims : UInt32*, count : UInt32,
