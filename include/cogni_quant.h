@@ -265,7 +265,12 @@ int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uin
  * x and the dequantized weights are rounded to fp16 and multiplied on the matrix cores with fp32
  * accumulation, the precision of the reference's Metal prefill kernels (src/ml/gguf/kernels/gemm_q4k.metal:
  * 97-105,678-686; Q5_K and Q6_K: gemm_q56k.metal, pipelines mm5 / mm6 src/ml/gguf/qwen35_metal.cr:11035); expect about 5e-4 of
- * max|out| where the GEMV path gives 1e-6. `workspace` is caller-owned device memory of at least
+ * max|out| where the GEMV path gives 1e-6. The conversion of x is the reference's plain `(half)y[i]` (gemm_q4k.metal:678-684):
+ * an activation beyond the binary16 range (|x| > 65504) becomes infinite and its token's outputs Inf or NaN, where the GEMV
+ * kernels (any token count up to 8: they scale every token and super-block by its own power of two) follow fp32. Callers whose
+ * activations can be that large keep to the GEMV path: cogni_set_gemm_threshold(1 << 30). A non-finite activation gives
+ * non-finite outputs for its token on every path (the multi-token GEMV kernels NaN where the reference's sum is +-Inf); the
+ * other tokens of the call are not affected. `workspace` is caller-owned device memory of at least
  * cogni_gemm_workspace_bytes(...) bytes (x repacked as fp16, in the k order of the weight type); nothing is allocated.
  * Kernels: pack_x_f16_q4k (Q4_K and Q5_K) | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
  *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,

@@ -186,3 +186,33 @@ def test_m2048_row_identity(gpu, oracle):
                 sample_tokens=[0, 1, 127, 128, 1000, 1023, 1024, 2046, 2047])
     part = run_gemm(raw, x[1900 * in_dim:], in_dim, out_dim, tokens - 1900, split=False).reshape(-1, out_dim)
     assert np.array_equal(part, got[1900:])
+
+
+def test_activation_magnitude_on_both_sides_of_the_router_threshold(gpu, oracle):
+    """QuantWeight.matmul changes kernels between 8 and 9 rows. Activations up to 3e4 (inside binary16) must pass both bars on
+    both sides; an activation of 1e5 stays exact on the GEMV side (per-super-block scaling) and, as documented for the
+    GEMM (x is converted with a plain float -> half cast, like the reference's Metal kernel), turns that token's outputs
+    non-finite on the GEMM side while every other token stays within the bar."""
+    rng = np.random.default_rng(65504)
+    in_dim, out_dim = 1024, 192
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    zero = np.zeros(out_dim, dtype=np.float32)
+    for rows in (8, 9):
+        x = (synth.make_activations(rng, rows, in_dim) * np.float32(1e4)).astype(np.float32)      # |x| up to about 4e4
+        x = np.clip(x, -3e4, 3e4).astype(np.float32)
+        qw = quant.QuantWeight(raw, Q4_K, out_dim, in_dim, "range")
+        got = qw.matmul(x, rows)
+        want = oracle.matmul_add(x, rows, in_dim, raw, Q4_K, out_dim, zero, threads=8)
+        assert np.max(np.abs(got - want)) <= (2e-3 if rows > 8 else 1e-5) * np.max(np.abs(want)), rows
+        x2 = x.copy().reshape(rows, in_dim)
+        x2[3, 100] = np.float32(1e5)
+        x2 = np.ascontiguousarray(x2.reshape(-1))
+        got2 = qw.matmul(x2, rows).reshape(rows, out_dim)
+        want2 = oracle.matmul_add(x2, rows, in_dim, raw, Q4_K, out_dim, zero, threads=8).reshape(rows, out_dim)
+        others = [r for r in range(rows) if r != 3]
+        assert np.max(np.abs(got2[others] - want2[others])) <= (2e-3 if rows > 8 else 1e-5) * np.max(np.abs(want2)), rows
+        if rows <= 8:
+            assert np.max(np.abs(got2[3] - want2[3])) <= 1e-5 * np.max(np.abs(want2[3]))
+        else:
+            assert not np.isfinite(got2[3]).any()
+        qw.close()

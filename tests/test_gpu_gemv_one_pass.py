@@ -228,3 +228,30 @@ def test_q6_k_lists_share_one_image(gpu, oracle):
         assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, "q6_k list member %d" % d)
     for a in ws + outs + [xd]:
         a.close()
+
+
+@pytest.mark.parametrize("tokens", [1, 2, 4, 8])
+def test_non_finite_activation_stays_in_its_token(gpu, oracle, tokens):
+    """An infinite activation: the reference's sum for that token is +-Inf (or NaN where weights of both signs meet it).
+    Every kernel must give non-finite values for that token's rows that use the element, and must leave the other tokens of
+    the call within the bar (one token: vector ALU; two and four: matrix-core kernels; eight: one pass)."""
+    rng = np.random.default_rng(700 + tokens)
+    in_dim, out_dim = 4096, 64
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim).reshape(tokens, in_dim)
+    bad = tokens - 1
+    x[bad, 777] = np.float32(np.inf)
+    x = np.ascontiguousarray(x.reshape(-1))
+    w, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim)
+    quant.gemv_dev(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+    got = od.read(np.float32, tokens * out_dim).reshape(tokens, out_dim)
+    with np.errstate(all="ignore"):
+        ref = oracle.matmul_add(x, tokens, in_dim, raw, Q4_K, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).reshape(tokens, out_dim)
+    assert not np.isfinite(ref[bad]).any() and not np.isfinite(got[bad]).any()
+    if tokens > 1:
+        good = [m for m in range(tokens) if m != bad]
+        xs = np.ascontiguousarray(x.reshape(tokens, in_dim)[good].reshape(-1))
+        want, tol = oracle_rows(oracle, raw, xs, in_dim, out_dim, len(good))
+        assert np.all(np.abs(got[good].reshape(-1) - want) <= tol)
+    for a in (w, xd, od):
+        a.close()
