@@ -60,6 +60,7 @@ def lib():
         L.mlhip_stream_end_capture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
         L.mlhip_graph_instantiate.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_uint64]
         L.mlhip_graph_upload.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        L.cogni_gemv_release_stream.argtypes = [ctypes.c_void_p]
         L.mlhip_graph_launch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
         L.mlhip_launch_kernel.argtypes = [ctypes.c_void_p] + [ctypes.c_uint32] * 7 + [
             ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p]
@@ -254,6 +255,7 @@ class HIPStream:
     def close(self):
         if self._closed:
             return
+        lib().cogni_gemv_release_stream(self.handle)   # the activation image the library may keep for this stream
         lib().mlhip_stream_destroy(self.handle)
         self._closed = True
 

@@ -317,6 +317,21 @@ size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens)
 
 uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim) { return gemv_mt_from(w_type, in_dim); }
 
+int cogni_gemv_release_stream(void* stream) {
+  int slot = -1;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    for (int i = 0; i < Runtime::kImageSlots; i++)
+      if (g_rt.image_used[i] && g_rt.image_stream[i] == stream) slot = i;
+  }
+  if (slot < 0) return 0;
+  // the slot may only change hands once everything that reads it has run
+  HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize(cogni_gemv_release_stream)");
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_rt.image_used[slot] && g_rt.image_stream[slot] == stream) g_rt.image_used[slot] = false, g_rt.image_stream[slot] = nullptr;
+  return 0;
+}
+
 int cogni_gemv_packed_launch_dims(uint32_t w_type, uint32_t in_dim, uint32_t total_rows, uint32_t* grid_x, uint32_t* block_x,
                                   uint32_t* shared_mem_bytes) {
   if (!grid_x || !block_x || !shared_mem_bytes || total_rows == 0 || !gemv_mt_supported(w_type, 2, in_dim))

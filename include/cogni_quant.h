@@ -149,6 +149,11 @@ size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens)
 /* The token count from which cogni_gemv_dev takes this path for one matrix (Q6_K 3; Q4_K 4 on rows longer than 4096 values,
  * else 5), 0 where it never does; below it the call runs the kernel cogni_gemv_plan names. No GPU needed. */
 uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim);
+/* Gives back the image the library keeps for `stream` (waits for the stream's work first; nothing to do and no error if it
+ * has none). Call it before destroying a stream that ran multi-token GEMVs: the eight slots are otherwise used up by the
+ * first eight streams of the process, and later streams run the per-token-group kernels. A graph captured on the stream
+ * still names the stream's image: release only once such graphs are no longer replayed. */
+int cogni_gemv_release_stream(void* stream);
 /* Launch geometry of the one-pass kernel for a launch of total_rows rows (all its matrices together): a workgroup's eight
  * wavefronts carry t tiles of 16 rows at a time (in_dim above 4096: t = 1; else t = clamp(tiles / 256, 1, 3), Q6_K at most 2),
  * a row group is t tiles, grid_x = min(256, row groups) and the workgroups walk the groups blockIdx.x, blockIdx.x +

@@ -241,6 +241,7 @@ def test_one_pass_geometry_and_thresholds():
 
 
 def test_one_pass_argument_errors_do_not_need_a_gpu():
+    assert hip.lib().cogni_gemv_release_stream(None) == 0          # a stream without an image: nothing to do
     with pytest.raises(quant.QuantError, match="no one-pass kernel") as e:
         quant.gemv_pack_dev(0x1000, 12, 1024, 4, 0x2000)
     assert e.value.code == -1

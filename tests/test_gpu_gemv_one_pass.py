@@ -8,7 +8,7 @@ output scale."""
 import numpy as np
 import pytest
 
-from cogni_ml_amd import quant, synth
+from cogni_ml_amd import hip, quant, synth
 from gpu_common import DevArray, gpu  # noqa: F401
 from helpers import Q4_K, Q6_K, cosine, gemv_tolerance
 
@@ -254,4 +254,27 @@ def test_non_finite_activation_stays_in_its_token(gpu, oracle, tokens):
         want, tol = oracle_rows(oracle, raw, xs, in_dim, out_dim, len(good))
         assert np.all(np.abs(got[good].reshape(-1) - want) <= tol)
     for a in (w, xd, od):
+        a.close()
+
+
+def test_image_slots_return_when_streams_close(gpu, oracle):
+    """The library keeps one activation image per stream, eight at most. A stream that is closed gives its image back, so
+    the twelfth stream of a process still runs the one-pass kernel: its result is bit for bit that of the explicit
+    pack + packed GEMV, which the per-token-group kernels' is not."""
+    rng = np.random.default_rng(12)
+    in_dim, out_dim, tokens = 4096, 256, 8
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    w, xd, od, o2 = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim), DevArray(nbytes=4 * tokens * out_dim)
+    image = DevArray(nbytes=quant.gemv_image_bytes(Q4_K, in_dim, tokens))
+    quant.gemv_pack_dev(xd.ptr, Q4_K, in_dim, tokens, image.ptr)
+    quant.gemv_packed_dev([w.ptr], Q4_K, image.ptr, [o2.ptr], [out_dim], in_dim, tokens)
+    explicit = o2.read(np.float32, tokens * out_dim)
+    for i in range(12):
+        st = hip.HIPStream()
+        quant.gemv_dev(w.ptr, Q4_K, xd.ptr, od.ptr, in_dim, out_dim, tokens, 0, st.handle)
+        st.synchronize()
+        assert np.array_equal(od.read(np.float32, tokens * out_dim), explicit), i
+        st.close()
+    for a in (w, xd, od, o2, image):
         a.close()
