@@ -514,7 +514,7 @@ int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uin
     uint32_t grid = 0, block = 0, shmem = 0;
     int rc = cogni_gemv_launch_dims(w_type, 1, in_dim, out_dim, &grid, &block, &shmem);
     if (rc != 0) return rc;
-    const uint32_t rows = (uint32_t)gemv_rows_per_block(w_type, 1);
+    const uint32_t rows = GEMV_WAVES * GEMV_ROWS_Q4K_PAIR;
     grid = (2 * out_dim + rows - 1) / rows;
     void* params[] = {&w_raw_a, &w_raw_b, &x, &out_a, &out_b, &in_dim, &out_dim};
     return launch("q4_k_dual_gemv_f32", grid, block, shmem, params, stream);
@@ -683,7 +683,7 @@ int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, 
   uint32_t grid = 0, block = 0, shmem = 0;
   int rc = cogni_gemv_launch_dims(w_type, 1, in_dim, out_dim, &grid, &block, &shmem);
   if (rc != 0) return rc;
-  const uint32_t rows = (uint32_t)gemv_rows_per_block(w_type, 1) / 2;   // gate rows per workgroup (as many of up)
+  const uint32_t rows = GEMV_WAVES * GEMV_ROWS_Q4K_PAIR / 2;   // gate rows per workgroup (as many of up)
   grid = (out_dim + rows - 1) / rows;
   void* params[] = {&w_gate, &w_up, &x, &out, &in_dim, &out_dim};
   return launch("q4_k_dual_gemv_swiglu_f32", grid, block, shmem, params, stream, tokens);

@@ -492,7 +492,10 @@ __device__ __forceinline__ void gemv_entry(const uint8_t* w, const float* x, con
 
 // ---- entry points ---------------------------------------------------------------------------
 // M = 1, 2: ask for at least 3 wavefronts per SIMD so a 12288-row matrix is resident in one round
-#define GEMV_OCC(M) __attribute__((amdgpu_waves_per_eu((M) <= 1 ? 3 : 1)))
+#ifndef GEMV_OCC_M1
+#define GEMV_OCC_M1 3
+#endif
+#define GEMV_OCC(M) __attribute__((amdgpu_waves_per_eu((M) <= 1 ? GEMV_OCC_M1 : 1)))
 #define GEMV_ENTRY(NAME, FMT, M)                                                                                \
   extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(M) void NAME(const uint8_t* w, const float* x, float* out,   \
                                                                  u32 in_dim, u32 out_dim) {                     \
@@ -582,22 +585,26 @@ extern "C" __global__ __launch_bounds__(TOP1_REDUCE_BLOCK) void top1_reduce_f32(
 }
 
 // (w_raw_a, w_raw_b, x, out_a, out_b, in_dim, out_dim): one token per grid.y slice (x + y * in_dim, out_* + y * out_dim),
-// grid.x = ceil(2 * out_dim / rows per workgroup), same block and dynamic shared memory as q4_k_gemv_f32.
+// grid.x = ceil(2 * out_dim / (GEMV_WAVES * GEMV_ROWS_Q4K_PAIR)), same block and dynamic shared memory as q4_k_gemv_f32.
 // The reference has this pair as q4_k_dual_gemv_warp4_f32 and ..._batched (q4k_dual_gemv_probe.ptx:5, 233).
+// (the pair kernels keep four rows per wavefront: GEMV_ROWS_Q4K_PAIR)
+struct FmtQ4KPair : FmtQ4K {
+  static constexpr int rows(int) { return GEMV_ROWS_Q4K_PAIR; }
+};
 extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(1) void q4_k_dual_gemv_f32(
     const uint8_t* w_a, const uint8_t* w_b, const float* x, float* out_a, float* out_b, u32 in_dim, u32 out_dim) {
   const size_t tok = blockIdx.y;
-  gemv_core<FmtQ4K, 1, false, true>(w_a, x + tok * in_dim, nullptr, out_a + tok * out_dim, in_dim, out_dim, w_b,
-                                    out_b + tok * out_dim);
+  gemv_core<FmtQ4KPair, 1, false, true>(w_a, x + tok * in_dim, nullptr, out_a + tok * out_dim, in_dim, out_dim, w_b,
+                                        out_b + tok * out_dim);
 }
 
 // (w_gate, w_up, x, out, in_dim, out_dim): out[o] = silu(gate[o]) * up[o] for one token per grid.y slice; block and
-// dynamic shared memory as q4_k_gemv_f32, grid.x = ceil(out_dim / (rows per workgroup / 2)).
+// dynamic shared memory as q4_k_gemv_f32, grid.x = ceil(out_dim / (GEMV_WAVES * GEMV_ROWS_Q4K_PAIR / 2)).
 extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(1) void q4_k_dual_gemv_swiglu_f32(
     const uint8_t* w_gate, const uint8_t* w_up, const float* x, float* out, u32 in_dim, u32 out_dim) {
   const size_t tok = blockIdx.y;
-  gemv_core<FmtQ4K, 1, false, true, true>(w_gate, x + tok * in_dim, nullptr, out + tok * out_dim, in_dim, out_dim, w_up,
-                                          nullptr);
+  gemv_core<FmtQ4KPair, 1, false, true, true>(w_gate, x + tok * in_dim, nullptr, out + tok * out_dim, in_dim, out_dim,
+                                              w_up, nullptr);
 }
 
 // (gate, up, out, n): out[i] = silu(gate[i]) * up[i], the reference's swiglu_f32 (bin/cuda_ffn_sequence_probe.cr:46-84).

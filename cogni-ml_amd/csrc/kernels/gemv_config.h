@@ -7,7 +7,13 @@
 #endif
 #define GEMV_BLOCK (64 * GEMV_WAVES)
 
-#define GEMV_ROWS_Q4K(M) ((M) <= 2 ? 4 : 2)
+// rows per wavefront. One token of a Q4_K matrix: two rows and four workgroups per compute unit (1024 resident workgroups
+// that walk the row groups) measured 7.55 us against 7.9-8.0 for four rows and three workgroups at 12288 x 4096, interleaved
+// runs; 896, 960 or 1088 workgroups lose that again. The one-token matrix-pair kernels keep four rows (no gain there).
+#ifndef GEMV_ROWS_Q4K
+#define GEMV_ROWS_Q4K(M) ((M) == 1 ? 2 : ((M) == 2 ? 4 : 2))
+#endif
+#define GEMV_ROWS_Q4K_PAIR 4
 #define GEMV_ROWS_Q5K(M) 2
 #ifndef GEMV_ROWS_Q6K
 #define GEMV_ROWS_Q6K(M) 2
@@ -66,9 +72,13 @@ static constexpr inline GEMV_HD bool gemv_direct_x(unsigned type, int token_grou
 // number of groups up to one.
 #define GEMV_RESIDENT_WGS 768u
 #define GEMV_RESIDENT_WGS_2 512u
+// (one token of Q4_K: every resident slot is launched, 4 per compute unit, and the workgroups' group counts differ by at
+// most one)
+#define GEMV_RESIDENT_WGS_Q4K 1024u
 static inline unsigned gemv_grid(unsigned type, int tokens, unsigned out_dim) {
   const unsigned rows = (unsigned)gemv_rows_per_block(type, tokens);
   const unsigned groups = (out_dim + rows - 1) / rows;
+  if (type == 12 && tokens == 1) return groups < GEMV_RESIDENT_WGS_Q4K ? groups : GEMV_RESIDENT_WGS_Q4K;
   const unsigned resident = tokens == 1 ? GEMV_RESIDENT_WGS : GEMV_RESIDENT_WGS_2;
   if (tokens > 2 || !gemv_direct_x(type, 1) || groups <= resident) return groups;
   const unsigned per_wg = (groups + resident - 1) / resident;

@@ -72,8 +72,9 @@ int cogni_quant_code_object(const void** image, size_t* size);
 const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add);
 /* Launch geometry of the GEMV kernel for (type, tokens) at this shape: block_x = 256 threads, grid_x =
  * ceil(out_dim / rows_per_block) where rows_per_block depends on the type and token count - except that one token
- * of a K-quant matrix with more than 768 such row groups is launched as at most 768 workgroups, each walking
- * several groups (the kernels accept any grid_x up to the number of row groups) - all other
+ * of a K-quant matrix with more such row groups than workgroups are resident together (Q4_K: 1024 of 8 rows, Q5_K and
+ * Q6_K: 768) is launched as that many workgroups at most, each walking several groups (the kernels accept any grid_x
+ * up to the number of row groups) - all other
  * grid/block extents 1, and shared_mem_bytes of dynamic shared memory (the staged activations), which
  * goes into the shared_mem_bytes argument of the launch (driver.cr:278-286). (The reference's kernels
  * use grid ceil(out_dim/4) x block 128 and no dynamic shared memory, bin/cuda_q4k_gemv_probe.cr:225-230.)
@@ -178,7 +179,7 @@ int cogni_gemv_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type
  * the parameter list of the reference's q4_k_dual_gemv_warp4_f32 (src/ml/cuda/kernels/q4k_dual_gemv_probe.ptx:5-13,
  * used by src/ml/cuda/qwen_recurrent_layer_runner.cr:519-520): output row r of the launch is row r of W_a for
  * r < out_dim and row r - out_dim of W_b above; block and dynamic shared memory as cogni_gemv_launch_dims gives for
- * one token, grid_x = ceil(2*out_dim / rows per workgroup), grid_y = tokens (one token per slice, x + y*in_dim,
+ * one token, grid_x = ceil(2*out_dim / 16), grid_y = tokens (one token per slice, x + y*in_dim,
  * out_* + y*out_dim, the reference's ..._batched entry). Several tokens of a Q4_K pair with out_dim a multiple of 16
  * and a row length the matrix-core kernel takes: "q4_k_dual_gemv_mfma_f32_tbatchM", same parameters, block 512, grid and
  * shared memory of one matrix with 2*out_dim rows (cogni_gemv_plan), per group of up to four tokens. Every other case is
@@ -205,7 +206,7 @@ int cogni_swiglu_dev(uint64_t gate, uint64_t up, uint64_t out, uint32_t n, void*
  *   out[m*out_dim + o] = silu(sum_j x[m][j] deq(W_gate[o][j])) * sum_j x[m][j] deq(W_up[o][j])
  * i.e. the reference's gate/up GEMVs followed by swiglu_f32 (bin/cuda_ffn_sequence_probe.cr: FFN sequence) without
  * the intermediate vectors. Kernel "q4_k_dual_gemv_swiglu_f32" (w_gate, w_up, x, out, in_dim, out_dim): block and
- * dynamic shared memory as for one token of cogni_gemv_launch_dims, grid_x = ceil(out_dim / (rows per workgroup / 2)),
+ * dynamic shared memory as for one token of cogni_gemv_launch_dims, grid_x = ceil(out_dim / 8),
  * grid_y = tokens (one token per slice). Several tokens with out_dim a multiple of 16 and a row length the matrix-core
  * kernel takes: "q4_k_dual_gemv_swiglu_mfma_f32_tbatchM", same parameters, per group of up to four tokens, block 512,
  * shared memory as cogni_gemv_plan gives for the token count, grid = min(256, out_dim / 16 / row groups per workgroup).

@@ -87,8 +87,10 @@ def test_gemv_launch_dims():
     assert quant.gemv_launch_dims(14, 3, 4096, 151936)[0] == groups and quant.gemv_launch_dims(8, 1, 4096, 151936)[0] == 151936 // 16
     # the top-1 scratch holds one entry per workgroup of the widest launch it is used with (one or two tokens)
     assert quant.gemv_top1_partials(14, 151936) == max(g_head, g2)
-    g1 = quant.gemv_launch_dims(12, 1, 256, 17)[0]
-    assert g1 == -(-17 // (12288 // quant.gemv_launch_dims(12, 1, 4096, 12288)[0]))
+    # one token of Q4_K: 8 rows per workgroup, at most 1024 workgroups (four per compute unit), which walk the rest
+    assert quant.gemv_launch_dims(12, 1, 256, 17)[0] == 3 and quant.gemv_launch_dims(12, 1, 4096, 4096)[0] == 512
+    assert quant.gemv_launch_dims(12, 1, 4096, 12288)[0] == 1024 and quant.gemv_launch_dims(12, 1, 4096, 151936)[0] == 1024
+    assert quant.gemv_launch_dims(12, 2, 4096, 12288)[0] == 384                    # two tokens: 768 groups of 16 rows, two per workgroup
     with pytest.raises(quant.QuantError):
         quant.gemv_launch_dims(20, 1, 256, 16)
     with pytest.raises(quant.QuantError):
