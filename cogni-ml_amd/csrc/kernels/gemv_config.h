@@ -75,10 +75,17 @@ static constexpr inline GEMV_HD bool gemv_direct_x(unsigned type, int token_grou
 // (one token of Q4_K: every resident slot is launched, 4 per compute unit, and the workgroups' group counts differ by at
 // most one)
 #define GEMV_RESIDENT_WGS_Q4K 1024u
+// (one token of a Q6_K matrix of many groups: 5 per compute unit. The 151936 x 4096 head, interleaved runs: 93.6 us on 760,
+// 768 or 1024 workgroups, 90.2 on 1280, 91.1 on 1536, 90.8 on 2048; 92.4 - 97.2 on counts that are not multiples of the 256
+// compute units. With only a few groups per workgroup the even split over 768 stays: 12288 rows 10.35 us against 11.1 on
+// 1280, 24576 rows 17.4 against 18.65)
+#define GEMV_RESIDENT_WGS_Q6K 1280u
+#define GEMV_RESIDENT_Q6K_MIN_GROUPS (8u * GEMV_RESIDENT_WGS_Q6K)
 static inline unsigned gemv_grid(unsigned type, int tokens, unsigned out_dim) {
   const unsigned rows = (unsigned)gemv_rows_per_block(type, tokens);
   const unsigned groups = (out_dim + rows - 1) / rows;
   if (type == 12 && tokens == 1) return groups < GEMV_RESIDENT_WGS_Q4K ? groups : GEMV_RESIDENT_WGS_Q4K;
+  if (type == 14 && tokens == 1 && groups >= GEMV_RESIDENT_Q6K_MIN_GROUPS) return GEMV_RESIDENT_WGS_Q6K;
   const unsigned resident = tokens == 1 ? GEMV_RESIDENT_WGS : GEMV_RESIDENT_WGS_2;
   if (tokens > 2 || !gemv_direct_x(type, 1) || groups <= resident) return groups;
   const unsigned per_wg = (groups + resident - 1) / resident;

@@ -72,8 +72,8 @@ int cogni_quant_code_object(const void** image, size_t* size);
 const char* cogni_gemv_kernel_name(uint32_t type, uint32_t tokens, int add);
 /* Launch geometry of the GEMV kernel for (type, tokens) at this shape: block_x = 256 threads, grid_x =
  * ceil(out_dim / rows_per_block) where rows_per_block depends on the type and token count - except that one token
- * of a K-quant matrix with more such row groups than workgroups are resident together (Q4_K: 1024 of 8 rows, Q5_K and
- * Q6_K: 768) is launched as that many workgroups at most, each walking several groups (the kernels accept any grid_x
+ * of a K-quant matrix with more such row groups than workgroups are resident together (Q4_K: 1024 of 8 rows; Q5_K and Q6_K:
+ * 768, Q6_K 1280 from 10240 row groups) is launched as that many workgroups at most, each walking several groups (the kernels accept any grid_x
  * up to the number of row groups) - all other
  * grid/block extents 1, and shared_mem_bytes of dynamic shared memory (the staged activations), which
  * goes into the shared_mem_bytes argument of the launch (driver.cr:278-286). (The reference's kernels

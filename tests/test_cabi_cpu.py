@@ -77,10 +77,10 @@ def test_gemv_launch_dims():
     assert quant.gemv_launch_dims(12, 1, 65536, 4096)[2] <= 49152
     # Q8_0 keeps per-lane sums beside the staged activations: one per 1024-value column set and lane
     assert quant.gemv_launch_dims(8, 1, 1024, 3584)[2] == 1024 * 4 + 256
-    # one token of a long K-quant matrix: at most 768 workgroups that share the row groups evenly
+    # one token of a long K-quant matrix: the workgroups resident together share the row groups (Q6_K 1280, Q5_K 768 evenly)
     g_head = quant.gemv_launch_dims(14, 1, 4096, 151936)[0]
     groups = -(-151936 // 8)
-    assert g_head <= 768 and -(-groups // g_head) * (g_head - 1) < groups
+    assert g_head == 1280 and groups > g_head          # five workgroups per compute unit walk 14 or 15 groups each
     # two tokens (one token group) walk the row groups too, 512 workgroups at most; three tokens and Q8_0 do not
     g2 = quant.gemv_launch_dims(14, 2, 4096, 151936)[0]
     assert g2 <= 512 and -(-groups // g2) * (g2 - 1) < groups

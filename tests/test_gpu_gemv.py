@@ -481,7 +481,7 @@ def test_long_matrices_walk_row_groups(gpu, oracle, type_id, in_dim, out_dim, ad
     rd = DevArray(res) if add else None
     try:
         grid = quant.gemv_launch_dims(type_id, 1, in_dim, out_dim)[0]
-        assert grid <= (1024 if type_id == Q4_K else 768) and grid * 8 < out_dim      # 8 rows per workgroup: they walk
+        assert grid <= {Q4_K: 1024, Q6_K: 768, Q5_K: 768}[type_id] and grid * 8 < out_dim      # 8 rows per workgroup: they walk
         quant.gemv_dev(wd.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, 1, rd.ptr if add else 0)
         full = od.read(np.float32, out_dim)
         piece = 4096                                   # at most 512 row groups: one per workgroup
