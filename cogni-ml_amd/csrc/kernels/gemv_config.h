@@ -14,7 +14,9 @@
 #define GEMV_ROWS_Q4K(M) ((M) == 1 ? 2 : ((M) == 2 ? 4 : 2))
 #endif
 #define GEMV_ROWS_Q4K_PAIR 4
+#ifndef GEMV_ROWS_Q5K
 #define GEMV_ROWS_Q5K(M) 2
+#endif
 #ifndef GEMV_ROWS_Q6K
 #define GEMV_ROWS_Q6K(M) 2
 #endif
