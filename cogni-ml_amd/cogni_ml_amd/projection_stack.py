@@ -89,10 +89,10 @@ class QwenProjectionStackRunner:
         while i < len(ents):
             name, src, t, out_dim, in_dim, raw = ents[i]
             nxt = ents[i + 1] if i + 1 < len(ents) else None
-            # several tokens: up to three consecutive projections of one input, type and row length (q | k | v,
-            # gate | up) go to the library as one list (the qmatvec_many seam), which stages the input once for them
+            # up to three consecutive projections of one input, type and row length (q | k | v, gate | up) go to the
+            # library as one list (the qmatvec_many seam), which stages the input once for them
             j = i + 1
-            while count > 1 and j < len(ents) and j - i < 3 and (ents[j][1], ents[j][2], ents[j][4]) == (src, t, in_dim):
+            while j < len(ents) and j - i < 3 and (ents[j][1], ents[j][2], ents[j][4]) == (src, t, in_dim):
                 j += 1
             if j - i >= 2:
                 grp = ents[i:j]

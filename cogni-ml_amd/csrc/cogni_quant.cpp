@@ -579,6 +579,28 @@ int cogni_gemv_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t x, cons
   }
   if (count == 2 && out_dims[0] == out_dims[1])
     return cogni_gemv_dual_dev(w_raw[0], w_raw[1], w_type, x, out[0], out[1], in_dim, out_dims[0], tokens, stream);
+  // one token of several Q4_K matrices: up to three per launch as one matrix of all their rows (q | k | v: one launch and
+  // one staging of x instead of three)
+  if (tokens == 1 && w_type == COGNI_TYPE_Q4_K && (in_dim % 256) == 0 && total <= 0x7FFFFFFFull) {
+    for (uint32_t i0 = 0; i0 < count; i0 += 3) {
+      const uint32_t n = count - i0 < 3 ? count - i0 : 3;
+      int rc;
+      if (n == 1) {
+        rc = cogni_gemv_dev(w_raw[i0], w_type, x, 0, out[i0], in_dim, out_dims[i0], 1, stream);
+      } else {
+        uint64_t w[3] = {w_raw[i0], w_raw[i0 + 1], n > 2 ? w_raw[i0 + 2] : 0};
+        uint64_t o[3] = {out[i0], out[i0 + 1], n > 2 ? out[i0 + 2] : 0};
+        uint32_t rows[3] = {out_dims[i0], out_dims[i0 + 1], n > 2 ? out_dims[i0 + 2] : 0};
+        uint32_t grid = 0, block = 0, shmem = 0;
+        rc = cogni_gemv_launch_dims(w_type, 1, in_dim, rows[0] + rows[1] + rows[2], &grid, &block, &shmem);
+        if (rc != 0) return rc;
+        void* params[] = {&w[0], &w[1], &w[2], &x, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2]};
+        rc = launch("q4_k_many_gemv_f32", grid, block, shmem, params, stream);
+      }
+      if (rc != 0) return rc;
+    }
+    return 0;
+  }
   uint32_t cap = 0;
   if (w_type == COGNI_TYPE_Q4_K && (count == 2 || count == 3) && tokens >= 2 && aligned && (in_dim % 256) == 0 && total <= 0x7FFFFFFFull)
     for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2 && cap == 0; mt--)

@@ -43,11 +43,20 @@
 // TOP1: instead of the row values the workgroup stores, per token, the largest of its rows and that row's index
 // (out[m * gridDim.x + blockIdx.x], top_ids[same]); of equal values the lowest row wins. The reference's
 // q6_k_gemv_top1_partial_f32 (src/ml/cuda/kernels/q6k_gemv_probe.ptx:1331-1580) for the output head.
-template <class F, int M, bool ADD, bool DUAL = false, bool SWIGLU = false, bool TOP1 = false>
+// LIST (with DUAL, M = 1): up to three matrices of one row length and any row counts as one matrix of all their rows
+// (q | k | v of a decoder layer: the reference's qmatvec_many seam, src/ml/gguf/qwen35_cpu.cr:1419-1445); `list` names
+// them, w / w_b / out / out_b / out_dim are not used.
+struct GemvList {
+  const uint8_t* w[3];
+  float* out[3];
+  u32 rows[3];
+};
+template <class F, int M, bool ADD, bool DUAL = false, bool SWIGLU = false, bool TOP1 = false, bool LIST = false>
 __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const float* __restrict__ x,
                                           const float* __restrict__ residual, float* __restrict__ out,
                                           u32 in_dim, u32 out_dim, const uint8_t* __restrict__ w_b = nullptr,
-                                          float* __restrict__ out_b = nullptr, u32* __restrict__ top_ids = nullptr) {
+                                          float* __restrict__ out_b = nullptr, u32* __restrict__ top_ids = nullptr,
+                                          const GemvList* list = nullptr) {
   constexpr int R = F::rows(M);
   constexpr int MG = M < F::MG_MAX ? M : F::MG_MAX;   // tokens held in registers at a time
   constexpr int NG = (M + MG - 1) / MG;
@@ -68,7 +77,8 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
   const size_t row_bytes = F::row_bytes(nb);
   static_assert(!SWIGLU || (DUAL && M == 1 && !ADD && R % 2 == 0), "SWIGLU is a one-token mode of the matrix pair");
   static_assert(!TOP1 || (!DUAL && !ADD), "TOP1 is a mode of the plain GEMV");
-  const u32 total_rows = DUAL ? 2 * out_dim : out_dim;
+  static_assert(!LIST || (DUAL && M == 1 && !ADD && !SWIGLU), "LIST is a one-token mode of several matrices");
+  const u32 total_rows = LIST ? list->rows[0] + list->rows[1] + list->rows[2] : (DUAL ? 2 * out_dim : out_dim);
   // A workgroup takes the row groups blockIdx.x, blockIdx.x + gridDim.x, ... (GEMV_WAVES * R rows each; with SWIGLU
   // half as many rows of each matrix); a grid of one workgroup per group is the plain case.
   const u32 group_rows = SWIGLU ? GEMV_WAVES * R / 2 : GEMV_WAVES * R;
@@ -84,7 +94,13 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
         rowp[r] = (r < R / 2 ? w : w_b) + (size_t)row * row_bytes;
       } else {
         const u32 row = min(row0 + r, total_rows - 1);
-        rowp[r] = (DUAL && row >= out_dim) ? w_b + (size_t)(row - out_dim) * row_bytes : w + (size_t)row * row_bytes;
+        if constexpr (LIST) {
+          const u32 r0 = list->rows[0], r01 = r0 + list->rows[1];
+          rowp[r] = row < r0 ? list->w[0] + (size_t)row * row_bytes
+                             : (row < r01 ? list->w[1] + (size_t)(row - r0) * row_bytes : list->w[2] + (size_t)(row - r01) * row_bytes);
+        } else {
+          rowp[r] = (DUAL && row >= out_dim) ? w_b + (size_t)(row - out_dim) * row_bytes : w + (size_t)row * row_bytes;
+        }
       }
     }
   };
@@ -278,7 +294,12 @@ __device__ __forceinline__ void gemv_core(const uint8_t* __restrict__ w, const f
           float v = wave_sum(acc[r][m]);
           const u32 row = row0 + r;
           if (lane == 0 && row < total_rows) {
-            if (DUAL && row >= out_dim) {
+            if constexpr (LIST) {   // (one token: m = 0)
+              const u32 r0 = list->rows[0], r01 = r0 + list->rows[1];
+              if (row < r0) list->out[0][row] = v;
+              else if (row < r01) list->out[1][row - r0] = v;
+              else list->out[2][row - r01] = v;
+            } else if (DUAL && row >= out_dim) {
               out_b[(size_t)m * out_dim + (row - out_dim)] = v;
             } else {
               const size_t o = (size_t)m * out_dim + row;
@@ -605,6 +626,16 @@ extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(1) void q4_k_dual_g
   const size_t tok = blockIdx.y;
   gemv_core<FmtQ4KPair, 1, false, true, true>(w_gate, x + tok * in_dim, nullptr, out + tok * out_dim, in_dim, out_dim,
                                               w_up, nullptr);
+}
+
+// (w0, w1, w2, x, out0, out1, out2, in_dim, rows0, rows1, rows2): one token against up to three Q4_K matrices of one row
+// length (rows1 / rows2 may be 0), the parameter list of q4_k_many_gemv_mfma_f32_tbatchM. Block, dynamic shared memory and
+// grid as q4_k_gemv_f32 for a matrix of rows0 + rows1 + rows2 rows. Every row is computed exactly as q4_k_gemv_f32 does it.
+extern "C" __global__ __launch_bounds__(GEMV_BLOCK) GEMV_OCC(1) void q4_k_many_gemv_f32(
+    const uint8_t* w0, const uint8_t* w1, const uint8_t* w2, const float* x, float* out0, float* out1, float* out2, u32 in_dim,
+    u32 rows0, u32 rows1, u32 rows2) {
+  const GemvList list = {{w0, w1, w2}, {out0, out1, out2}, {rows0, rows1, rows2}};
+  gemv_core<FmtQ4K, 1, false, true, false, false, true>(nullptr, x, nullptr, nullptr, in_dim, 0, nullptr, nullptr, nullptr, &list);
 }
 
 // (gate, up, out, n): out[i] = silu(gate[i]) * up[i], the reference's swiglu_f32 (bin/cuda_ffn_sequence_probe.cr:46-84).

@@ -194,7 +194,9 @@ int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uin
  * kernel takes: one launch per group of up to four tokens of "q4_k_many_gemv_mfma_f32_tbatchM"
  * (w0, w1, w2, x, out0, out1, out2, in_dim, rows0, rows1, rows2), block 512, grid and shared memory of one matrix with
  * the sum of the rows (cogni_gemv_plan), the activations staged once for all of them. Two matrices of one shape: as
- * cogni_gemv_dual_dev. Everything else: one cogni_gemv_dev per matrix. count in 1..8. */
+ * cogni_gemv_dual_dev. One token of Q4_K matrices: up to three per launch of "q4_k_many_gemv_f32" (the same parameter
+ * list), block, shared memory and grid as cogni_gemv_launch_dims gives one token of a matrix with the sum of the rows; each
+ * row comes out bit for bit as from cogni_gemv_dev. Everything else: one cogni_gemv_dev per matrix. count in 1..8. */
 int cogni_gemv_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t x, const uint64_t* out, const uint32_t* out_dims,
                         uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream);
 

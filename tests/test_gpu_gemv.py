@@ -378,6 +378,29 @@ def test_many_gemv_shares_activations(gpu, oracle, type_id, in_dim, dims, tokens
         quant.gemv_many_dev([], type_id, 0, [], [], in_dim, tokens)
 
 
+@pytest.mark.parametrize("in_dim,dims", [(4096, (4096, 1024, 1024)), (1024, (37, 5, 130)), (256, (3, 1)), (12288, (48, 77, 9)),
+                                         (512, (8, 8, 8, 20, 7)), (256, (9000, 300, 2)), (2048, (16, 16, 16, 16, 16, 16, 16))])
+def test_one_token_lists_in_one_launch(gpu, oracle, in_dim, dims):
+    """One token against several Q4_K matrices (q | k | v): up to three per launch as one matrix of all their rows. Row counts
+    that put a matrix boundary inside a wavefront's rows and inside a workgroup's, more rows than resident workgroups (the
+    workgroups walk), rows of three column sets, five and seven matrices (launches of three, three and one). Every row must
+    come out bit for bit as from the single-matrix call, and within the bar of the oracle."""
+    rng = np.random.default_rng(in_dim + sum(dims))
+    raws = [synth.make_weights(rng, Q4_K, d, in_dim) for d in dims]
+    x = synth.make_activations(rng, 1, in_dim)
+    ws, xd = [DevArray(r) for r in raws], DevArray(x)
+    outs = [DevArray(nbytes=4 * d) for d in dims]
+    quant.gemv_many_dev([w.ptr for w in ws], Q4_K, xd.ptr, [o.ptr for o in outs], list(dims), in_dim, 1)
+    for raw, o, d in zip(raws, outs, dims):
+        got = o.read(np.float32, d)
+        assert np.array_equal(got, run_gemv(raw, Q4_K, x, in_dim, d, 1))
+        want = oracle.matmul_add(x, 1, in_dim, raw, Q4_K, d, np.zeros(d, dtype=np.float32), threads=8).astype(np.float64)
+        dense = np.abs(oracle.dequantize(raw, Q4_K, d * in_dim)).reshape(d, in_dim)
+        assert np.all(np.abs(got.astype(np.float64) - want) <= gemv_tolerance(x, dense, 1, in_dim).reshape(-1))
+    for a in ws + outs + [xd]:
+        a.close()
+
+
 def test_swiglu_kernel_and_fused_gate_up(gpu, oracle):
     """swiglu_f32 against the oracle's float32 form, and the fused gate/up + SwiGLU launch against the
     two-step composition (same bits: same GEMV arithmetic, same device function) and the oracle."""
