@@ -56,10 +56,15 @@ class QwenProjectionStackRunner:
         self._xs = np.ascontiguousarray(xs, dtype=np.float32)
         self._buffers = []
         self._w = {}
+        self._images = {}   # (input name, weight type) -> packed activation image shared by every list that reads that input
         self._act = {"x": self._alloc(4 * tokens * self.hidden)}
         for name, src, t, out_dim, in_dim, raw in weights.entries:
             self._w[name] = self._alloc(raw.size)
             self._act[name] = self._alloc(4 * tokens * out_dim)
+            # (allocated here, not at first use: the sequence may be issued under stream capture)
+            nbytes = quant.gemv_image_bytes(t, in_dim, quant.MAX_GEMV_TOKENS)
+            if nbytes and (src, int(t)) not in self._images:
+                self._images[(src, int(t))] = self._alloc(nbytes)
         self.outputs = {}
         self._runner = hip.ResidentSequenceRunner(
             tokens, self._upload_weights, self._reset_sequence, self._run_token, self._read_outputs,
@@ -85,6 +90,7 @@ class QwenProjectionStackRunner:
     def _launch(self, tok0, count):
         stream = hip.current_stream_handle()
         ents = self.weights.entries
+        packed = set()
         i = 0
         while i < len(ents):
             name, src, t, out_dim, in_dim, raw = ents[i]
@@ -94,6 +100,19 @@ class QwenProjectionStackRunner:
             j = i + 1
             while j < len(ents) and j - i < 3 and (ents[j][1], ents[j][2], ents[j][4]) == (src, t, in_dim):
                 j += 1
+            if j - i >= 2 and count > 1 and quant.gemv_image_bytes(t, in_dim, min(count, quant.MAX_GEMV_TOKENS)) > 0:
+                # several tokens of a shape the one-pass kernel takes: the input is packed once per sequence step and
+                # every list that reads it (q | k | v, then gate | up) goes against that one image
+                grp = ents[i:j]
+                key = (src, int(t))
+                if key not in packed:
+                    quant.gemv_pack_dev(self._act[src].ptr + 4 * tok0 * in_dim, t, in_dim, count, self._images[key].ptr, stream)
+                    packed.add(key)
+                quant.gemv_packed_dev([self._w[e[0]].ptr for e in grp], t, self._images[key].ptr,
+                                      [self._act[e[0]].ptr + 4 * tok0 * e[3] for e in grp], [e[3] for e in grp], in_dim,
+                                      count, 0, stream)
+                i = j
+                continue
             if j - i >= 2:
                 grp = ents[i:j]
                 quant.gemv_many_dev([self._w[e[0]].ptr for e in grp], t, self._act[src].ptr + 4 * tok0 * in_dim,
