@@ -274,7 +274,7 @@ int cogni_quant_init(int32_t ordinal) {
   }
   g_rt.image_slot_bytes = ((size_t)gemv_mt_image_bytes(COGNI_TYPE_Q6_K, GEMV_MT_MAX_IN_DIM) + 255) & ~(size_t)255;
   HIP_TRY(hipMalloc(&g_rt.image_pool, g_rt.image_slot_bytes * Runtime::kImageSlots), "hipMalloc(activation images)");
-  for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32"}) {
+  for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q5_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32"}) {
     hipFunction_t fn = nullptr;
     HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
     g_rt.fns.emplace(name, fn);
@@ -375,7 +375,7 @@ int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image
     if (total > 0x7FFFFFFFull) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: too many rows");
     uint64_t res = i0 == 0 ? residual : 0;
     void* params[] = {&w[0], &w[1], &w[2], &image, &res, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2], &tokens};
-    const int rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt_f32" : "q4_k_gemv_mt_f32", gemv_mt_grid(w_type, in_dim, (uint32_t)total),
+    const int rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt_f32" : (w_type == COGNI_TYPE_Q5_K ? "q5_k_gemv_mt_f32" : "q4_k_gemv_mt_f32"), gemv_mt_grid(w_type, in_dim, (uint32_t)total),
                           GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type), params, stream);
     if (rc != 0) return rc;
     i0 += n;

@@ -174,14 +174,14 @@ static inline unsigned gemv_mfma_lds_bytes(unsigned type, int tokens, unsigned i
          units * (4u + 4u * nsums + 1024u);
 }
 
-// ---- several tokens in one pass over a Q4_K or Q6_K matrix (gemv_mt.hpp): 8 wavefronts = 8 k-slices, activations packed once
+// ---- several tokens in one pass over a Q4_K, Q5_K or Q6_K matrix (gemv_mt.hpp): 8 wavefronts = 8 k-slices, activations packed once
 #define GEMV_MT_WAVES 8
-#define GEMV_MT_TMAX 3              // 16-row tiles a wavefront carries at most (Q4_K; Q6_K two)
+#define GEMV_MT_TMAX 3              // 16-row tiles a wavefront carries at most (Q4_K, Q5_K; Q6_K two)
 #define GEMV_MT_MAX_TOKENS 8
 #define GEMV_MT_MAX_IN_DIM 12288u
-// Shapes the kernels take: Q4_K or Q6_K, 2..8 tokens, in_dim a multiple of 2048 up to 12288 (1..6 super-blocks per k-slice).
+// Shapes the kernels take: Q4_K, Q5_K or Q6_K, 2..8 tokens, in_dim a multiple of 2048 up to 12288 (1..6 super-blocks per k-slice).
 static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned in_dim) {
-  return (type == 12 || type == 14) && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && in_dim != 0 && (in_dim & 2047u) == 0 &&
+  return (type == 12 || type == 13 || type == 14) && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && in_dim != 0 && (in_dim & 2047u) == 0 &&
          in_dim <= GEMV_MT_MAX_IN_DIM;
 }
 // Token count from which one matrix goes through pack + one pass rather than the per-token-group kernels (0: never): where
@@ -205,13 +205,14 @@ static inline unsigned gemv_mt_grid(unsigned type, unsigned in_dim, unsigned tot
   const unsigned groups = (ntiles + t - 1) / t;
   return groups < 256u ? groups : 256u;   // more groups than compute units: the workgroups walk them
 }
-// the k-slices' partial sums, then per wavefront the slots of its units: 6 x (16 rows x 144 B) for Q4_K, 4 x (16 rows x 240 B)
-// for Q6_K
+// the k-slices' partial sums, then per wavefront the slots of its units: 6 x (16 rows x 144 B) for Q4_K, 6 x (16 rows x
+// 176 B) for Q5_K, 4 x (16 rows x 240 B) for Q6_K
 static inline unsigned gemv_mt_lds_bytes(unsigned type) {
-  return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u + GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : 6u * 2304u);
+  return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u +
+         GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : (type == 13 ? 6u * 2816u : 6u * 2304u));
 }
 // bytes of the activation image: 8 KiB of operands per super-block, then per (super-block, token pair) the two scales and
-// the sub-block sums (Q4_K 20 floats, Q6_K 36)
+// the sub-block sums (Q4_K and Q5_K, which share one image, 20 floats; Q6_K 36)
 static inline unsigned long long gemv_mt_image_bytes(unsigned type, unsigned in_dim) {
   return (unsigned long long)(in_dim >> 8) * (8192u + 4u * (type == 14 ? 144u : 80u));
 }

@@ -1,4 +1,4 @@
-// Decode GEMV for 2..8 tokens in ONE pass over the weights, Q4_K and Q6_K, on the matrix cores:
+// Decode GEMV for 2..8 tokens in ONE pass over the weights, Q4_K, Q5_K and Q6_K, on the matrix cores:
 //   out_i[m][o] = (residual[m][o] +) sum_j x[m][j] * deq(W_i[o][j])      for up to three matrices W_i of one in_dim.
 //
 // Kernels.
@@ -7,12 +7,13 @@
 //     super-block of 256 values the matrix-core operands of its instructions, laid out lane by lane, followed by the
 //     scale and the sub-block sums of every (token, super-block). Written once per activation block, whatever the number
 //     of matrices that block then meets (q | k | v | gate | up of a decoder layer share one).
-//   q4_k_gemv_mt_f32 | q6_k_gemv_mt_f32 (w0, w1, w2, image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens)
+//   q4_k_gemv_mt_f32 | q5_k_gemv_mt_f32 | q6_k_gemv_mt_f32 (w0, w1, w2, image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens)
+//     (Q5_K reads the image pack_x_mt_q4k_f16 writes)
 //     block 512 (8 wavefronts), grid and dynamic shared memory from gemv_config.h (gemv_mt_grid, gemv_mt_lds_bytes).
 //     rows1 / rows2 may be 0 (then w1 / w2 / out1 / out2 are not read); residual (may be null) belongs to the first
 //     matrix. Row counts of all but the last matrix present must be multiples of 16. in_dim must be a multiple of 2048
 //     up to 12288 (8 k-slices of 1..6 super-blocks). out_i rows at stride rows_i (the reference's multi-token kernel
-//     contract, src/ml/cuda/kernels/q4k_gemv_probe.ptx:437-768 and q6k_gemv_probe.ptx:977: x rows at stride in_dim, outs
+//     contract, src/ml/cuda/kernels/q4k_gemv_probe.ptx:437-768, q5k_gemv_probe.ptx:237 and q6k_gemv_probe.ptx:977: x rows at stride in_dim, outs
 //     at stride out_dim; these kernels handle eight tokens where those handle four).
 //   q4_k_gemv_mt_swiglu_f32 (w_gate, w_up, image, out, in_dim, out_dim, tokens)
 //
@@ -20,9 +21,9 @@
 // masked pair of codes read as two binary16 numbers is code * 2^-24 (code * 2^-20 for codes left four bits up), the
 // matrix cores honour subnormals, accumulation is fp32. The activations are fed as two binary16 terms, x * 2^e = hi + lo
 // (22 bits; e per token and super-block, so any fp32 range fits), which makes the 16 rows (token 0..7) x (hi, lo). One
-// instruction covers exactly one sub-block - Q4_K: v_mfma_f32_16x16x32_f16 on a 32-weight sub-block (a lane supplies the
-// low or the high nibbles of 8 bytes), Q6_K: v_mfma_f32_16x16x16_f16 on a 16-weight sub-block (4 bytes) - so the integer
-// scale of that sub-block is applied to the instruction's result, and the terms that do not depend on the codes (Q4_K:
+// instruction covers exactly one sub-block - Q4_K and Q5_K: v_mfma_f32_16x16x32_f16 on a 32-weight sub-block (a lane supplies
+// the low or the high nibbles of 8 bytes, Q5_K with the fifth bit of each from qh), Q6_K: v_mfma_f32_16x16x16_f16 on a 16-weight sub-block (4 bytes) - so the integer
+// scale of that sub-block is applied to the instruction's result, and the terms that do not depend on the codes (Q4_K, Q5_K:
 // dmin * m * sum(x), Q6_K: 32 * d * sc * sum(x)) come from the sub-block sums of the image. A result lane holds two
 // tokens x (hi, lo) of one weight row, the row whose header the same lane reads: the scales never change lanes.
 //
@@ -182,12 +183,20 @@ __device__ __forceinline__ void mt_wait() {
 }
 __device__ __forceinline__ void mt_pin(mt_u32x4& v) { asm volatile("" : "+v"(v)); }
 
-// ---- the two weight formats ----------------------------------------------------------------------------------------------
+// ---- the weight formats --------------------------------------------------------------------------------------------------
 // A format says how a tile's share of a super-block (a unit: 16 rows x one block) is copied to LDS and what a lane does
 // with it. P = 16-byte pieces per row in LDS, NCOPY = copy instructions per unit (the last with LAST lanes), NAUX = 16-byte
-// loads of scales and sums per (super-block, token pair), NSLOT = units a wavefront has room for in LDS.
-struct MtQ4K {
-  static constexpr int BB = 144, P = 9, NCOPY = 3, LAST = 16, NAUX = 5, NSLOT = 6, TMAX = 3;
+// loads of scales and sums per (super-block, token pair), NSLOT = units a wavefront has room for in LDS, TYPE = the GGUF
+// type number (what gemv_config.h's rules are asked with).
+//
+// Q4_K (144 B: d, dmin, scales[12], qs[128]) and Q5_K (176 B: d, dmin, scales[12], qh[32], qs[128]): byte l of qs[32 g ..
+// 32 g + 32) holds element 64 g + l (low nibble, sub-block 2 g) and element 64 g + 32 + l (high nibble, sub-block 2 g + 1);
+// Q5_K adds bit 2 g / 2 g + 1 of qh[l] as the fifth bit of the two. Both read the same activation image (the Q4_K one).
+template <bool Q5>
+struct MtK45 {
+  static constexpr unsigned TYPE = Q5 ? 13 : 12;
+  static constexpr int BB = Q5 ? 176 : 144, P = BB / 16, NCOPY = 3, LAST = 16 * P - 128, NAUX = 5, NSLOT = 6, TMAX = 3;
+  static constexpr int QOFF = Q5 ? 48 : 16;   // where qs starts in the block
   static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_PAIR_BYTES = NAUX * 16;
   // byte offset, inside the row's block, of the piece that goes to place `piece` of the row in LDS
   static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece * 16; }
@@ -206,12 +215,13 @@ struct MtQ4K {
     return a;
   }
   // what a lane takes out of its row's block in LDS
-  struct Raw { uint4 hdr; uint2 q[4]; };
+  struct Raw { uint4 hdr; uint2 q[4], h; };   // (h: the lane's eight qh bytes, Q5_K only)
   static __device__ __forceinline__ Raw read(const char* row, u32 kg) {
     Raw w;
     w.hdr = *reinterpret_cast<const uint4*>(row);
 #pragma unroll
-    for (int g = 0; g < 4; g++) w.q[g] = *reinterpret_cast<const uint2*>(row + 16 + 32 * g + 8 * kg);
+    for (int g = 0; g < 4; g++) w.q[g] = *reinterpret_cast<const uint2*>(row + QOFF + 32 * g + 8 * kg);
+    w.h = Q5 ? *reinterpret_cast<const uint2*>(row + 16 + 8 * kg) : make_uint2(0u, 0u);
     return w;
   }
   // acc[0..3] += this unit's share for tokens (2 rg, 2 rg + 1) x (hi, lo)
@@ -220,6 +230,8 @@ struct MtQ4K {
     mt_float4 dacc[8];
 #pragma unroll
     for (int g = 0; g < 4; g++) {
+      // Q5_K: per byte of t, bit 0 is the fifth bit of the low-nibble element and bit 1 that of the high-nibble element
+      const u32 tx = w.h.x >> (2 * g), ty = w.h.y >> (2 * g);
 #pragma unroll
       for (int par = 0; par < 2; par++) {
         const u32 mask = par ? 0x00F000F0u : 0x000F000Fu;
@@ -228,6 +240,20 @@ struct MtQ4K {
         a4.y = (w.q[g].x >> 8) & mask;
         a4.z = w.q[g].y & mask;
         a4.w = (w.q[g].y >> 8) & mask;
+        if constexpr (Q5) {
+          // a code is nibble | fifth bit << 4: bit 4 of a half for the low nibbles (x 2^-24), bit 8 for the high ones (x 2^-20)
+          if (par == 0) {
+            a4.x |= (tx << 4) & 0x00100010u;   // bytes 0, 2
+            a4.y |= (tx >> 4) & 0x00100010u;   // bytes 1, 3
+            a4.z |= (ty << 4) & 0x00100010u;
+            a4.w |= (ty >> 4) & 0x00100010u;
+          } else {
+            a4.x |= (tx << 7) & 0x01000100u;
+            a4.y |= (tx >> 1) & 0x01000100u;
+            a4.z |= (ty << 7) & 0x01000100u;
+            a4.w |= (ty >> 1) & 0x01000100u;
+          }
+        }
         dacc[2 * g + par] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mt_half8, b[2 * g + par]),
                                                                    __builtin_bit_cast(mt_half8, a4),
                                                                    (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
@@ -267,6 +293,9 @@ struct MtQ4K {
     acc[2] = fmaf(-dmin, mt1, acc[2]);
   }
 };
+typedef MtK45<false> MtQ4K;
+typedef MtK45<true> MtQ5K;
+
 
 // Q6_K (210 B: ql[128], qh[64], scales:i8[16], d). Element 128 n + 32 k + l (half n, quarter k, l < 32) has its low four bits
 // in nibble k / 2 of ql[64 n + 32 (k % 2) + l] and its high two in bits 2 k, 2 k + 1 of qh[32 n + l]; sub-block
@@ -276,6 +305,7 @@ struct MtQ4K {
 // piece 13 is bytes 194..209 (shifted back so that nothing past the end of the matrix is read: d sits at byte 222 of
 // the row) and piece 14 repeats piece 13.
 struct MtQ6K {
+  static constexpr unsigned TYPE = 14;
   static constexpr int BB = 210, P = 15, NCOPY = 4, LAST = 48, NAUX = 9, NSLOT = 4, TMAX = 2;
   static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_PAIR_BYTES = NAUX * 16;
   static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece < 13 ? piece * 16 : 194u; }
@@ -637,7 +667,7 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
 template <class F>
 __device__ __forceinline__ void gemv_mt_dispatch(const MtArgs& a, const uint8_t* image, const float* residual, u32 in_dim, u32 tokens) {
   const u32 ntiles = (a.rows[0] + a.rows[1] + a.rows[2] + 15) >> 4;
-  const u32 t = gemv_mt_tiles(F::BB == 210 ? 14u : 12u, in_dim, ntiles);
+  const u32 t = gemv_mt_tiles(F::TYPE, in_dim, ntiles);
   switch (in_dim >> 11) {
     case 1:
       if (t <= 1) gemv_mt_core<F, 1, 1>(a, image, residual, in_dim, tokens);
@@ -664,6 +694,7 @@ __device__ __forceinline__ void gemv_mt_dispatch(const MtArgs& a, const uint8_t*
     gemv_mt_dispatch<FMT>(a, image, residual, in_dim, tokens);                                                           \
   }
 GEMV_MT_ENTRY(q4_k_gemv_mt_f32, MtQ4K)
+GEMV_MT_ENTRY(q5_k_gemv_mt_f32, MtQ5K)
 GEMV_MT_ENTRY(q6_k_gemv_mt_f32, MtQ6K)
 
 // (w_gate, w_up, image, out, in_dim, out_dim, tokens): out[m][o] = silu(gate . x) * (up . x); block 512, grid = min(256,

@@ -223,12 +223,15 @@ def test_one_pass_geometry_and_thresholds():
     tiles and the workgroups walk the groups with stride grid."""
     assert quant.gemv_image_bytes(12, 4096, 8) == 16 * (8192 + 4 * 80)
     assert quant.gemv_image_bytes(14, 12288, 2) == 48 * (8192 + 4 * 144)
-    for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1024, 4), (12, 14336, 4), (13, 4096, 4), (8, 4096, 4), (12, 0, 4)):
+    assert quant.gemv_image_bytes(13, 4096, 4) == quant.gemv_image_bytes(12, 4096, 4)      # Q5_K reads the Q4_K image
+    for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1024, 4), (12, 14336, 4), (13, 1024, 4), (8, 4096, 4), (12, 0, 4)):
         assert quant.gemv_image_bytes(t, in_dim, tokens) == 0, (t, in_dim, tokens)
     assert [quant.gemv_one_pass_from(12, d) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 5, 4, 4, 0, 0]
-    assert [quant.gemv_one_pass_from(t, 4096) for t in (14, 13, 8)] == [3, 0, 0]
+    assert [quant.gemv_one_pass_from(13, d) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 5, 4, 4, 0, 0]
+    assert [quant.gemv_one_pass_from(t, 4096) for t in (14, 8, 2)] == [3, 0, 0]
     rng = np.random.default_rng(11)
-    for t, tmax, lds in ((12, 3, 8 * 3 * 8 * 16 * 4 + 8 * 6 * 16 * 144), (14, 2, 8 * 3 * 8 * 16 * 4 + 8 * 4 * 16 * 240)):
+    for t, tmax, lds in ((12, 3, 8 * 3 * 8 * 16 * 4 + 8 * 6 * 16 * 144), (13, 3, 8 * 3 * 8 * 16 * 4 + 8 * 6 * 16 * 176),
+                         (14, 2, 8 * 3 * 8 * 16 * 4 + 8 * 4 * 16 * 240)):
         for in_dim in (2048, 4096, 6144, 8192, 10240, 12288):
             for rows in [1, 15, 16, 17, 4096, 4097, 12288, 8 * 4096 - 16, 151936] + [int(r) for r in rng.integers(1, 400000, 40)]:
                 grid, block, shmem = quant.gemv_packed_launch_dims(t, in_dim, rows)
@@ -237,7 +240,7 @@ def test_one_pass_geometry_and_thresholds():
                 groups = -(-ntiles // tiles)
                 assert (block, shmem) == (512, lds) and shmem <= 160 * 1024
                 assert grid == min(256, groups) and grid >= 1
-    for bad in ((12, 1024, 16), (13, 4096, 16), (12, 4096, 0)):
+    for bad in ((12, 1024, 16), (8, 4096, 16), (12, 4096, 0)):
         with pytest.raises(quant.QuantError):
             quant.gemv_packed_launch_dims(*bad)
 
@@ -252,7 +255,7 @@ def test_one_pass_argument_errors_do_not_need_a_gpu():
     with pytest.raises(quant.QuantError, match="count must be 1..8"):
         quant.gemv_packed_dev([], 12, 0x2000, [], [], 4096, 4)
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
-        quant.gemv_packed_dev([0x1000], 13, 0x2000, [0x3000], [16], 4096, 4)
+        quant.gemv_packed_dev([0x1000], 8, 0x2000, [0x3000], [16], 4096, 4)
     with pytest.raises(quant.QuantError, match="a residual goes with a single matrix"):
         quant.gemv_packed_dev([0x1000, 0x1100], 12, 0x2000, [0x3000, 0x3100], [16, 16], 4096, 4, residual_ptr=0x4000)
     with pytest.raises(quant.QuantError, match="null pointer or zero rows"):

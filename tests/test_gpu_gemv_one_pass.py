@@ -1,5 +1,5 @@
-"""Decode GEMV for 2..8 tokens in one pass over a Q4_K or Q6_K matrix (activations packed once, q4_k_gemv_mt_f32 /
-q6_k_gemv_mt_f32) vs the CPU oracle.
+"""Decode GEMV for 2..8 tokens in one pass over a Q4_K, Q5_K or Q6_K matrix (activations packed once, q4_k_gemv_mt_f32 /
+q5_k_gemv_mt_f32 / q6_k_gemv_mt_f32) vs the CPU oracle.
 
 Bars, both asserted: the north-star bound max|err| <= 1e-4 * ||x||_2 * max|w_row| per token and row, and the reference's own
 probe gate (cos >= 0.99999, max_diff <= 1e-3 * max(1, max|ref| / 64): the probe's absolute 1e-3 is meant for outputs of order
@@ -10,7 +10,7 @@ import pytest
 
 from cogni_ml_amd import hip, quant, synth
 from gpu_common import DevArray, gpu  # noqa: F401
-from helpers import Q4_K, Q6_K, cosine, gemv_tolerance
+from helpers import Q4_K, Q5_K, Q6_K, cosine, gemv_tolerance
 
 pytestmark = pytest.mark.gpu
 
@@ -145,7 +145,7 @@ def test_one_pass_element_order_and_scale_positions(gpu, oracle):
 
 def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
     """9 and 13 tokens: a group of eight in one pass, the rest as the token count decides (one token on the vector ALU,
-    five in one pass); in_dim 1024, in_dim above 12288 and Q5_K have no one-pass kernel and keep their older paths."""
+    five in one pass); in_dim 1024 and in_dim above 12288 have no one-pass kernel and keep their older paths."""
     rng = np.random.default_rng(11)
     for in_dim, out_dim, tokens in ((4096, 272, 9), (2048, 100, 13), (1024, 64, 8)):
         raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
@@ -156,7 +156,7 @@ def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
         assert_bars(od.read(np.float32, tokens * out_dim), want, tol, tokens, out_dim, "%dx%d M=%d" % (in_dim, out_dim, tokens))
         for a in (w, xd, od):
             a.close()
-    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(13, 4096, 8) == 0
+    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(Q5_K, 4096, 8) == 16 * (8192 + 320)
     assert quant.gemv_image_bytes(Q4_K, 14336, 8) == 0 and quant.gemv_image_bytes(Q6_K, 4096, 8) == 16 * (8192 + 576)
     assert quant.gemv_image_bytes(Q4_K, 4096, 1) == 0 and quant.gemv_image_bytes(Q4_K, 4096, 9) == 0
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
@@ -164,6 +164,8 @@ def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
 
 
 LONG_AND_Q6K = [(Q4_K, 12288, 4096), (Q4_K, 6144, 530), (Q4_K, 8192, 16 * 300 + 5), (Q4_K, 10240, 33),
+                (Q5_K, 4096, 8192), (Q5_K, 2048, 1040), (Q5_K, 4096, 16 * 3 * 256 * 2 + 24), (Q5_K, 2048, 37), (Q5_K, 4096, 16 * 600),
+                (Q5_K, 12288, 530), (Q5_K, 6144, 16 * 257), (Q5_K, 10240, 50),
                 (Q6_K, 12288, 4096), (Q6_K, 4096, 4096), (Q6_K, 2048, 1040), (Q6_K, 4096, 16 * 2 * 256 * 2 + 24), (Q6_K, 6144, 50),
                 (Q6_K, 8192, 16 * 257), (Q6_K, 2048, 37)]
 
@@ -172,8 +174,9 @@ LONG_AND_Q6K = [(Q4_K, 12288, 4096), (Q4_K, 6144, 530), (Q4_K, 8192, 16 * 300 + 
 @pytest.mark.parametrize("tokens", [5, 8])
 def test_long_rows_and_q6_k_in_one_pass(gpu, oracle, type_id, in_dim, out_dim, tokens):
     """Rows of 6144..12288 values (three to six super-blocks per k-slice: the activation operands are streamed through two
-    register sets, Q6_K with four LDS slots for six units) and Q6_K at every row length: one and two tiles per wavefront,
-    partial tiles, more row groups than workgroups, odd super-blocks (blocks that start 2 bytes off a 4-byte boundary)."""
+    register sets, Q6_K with four LDS slots for six units) and Q5_K and Q6_K at every row length: one, two and three tiles per
+    wavefront, partial tiles, more row groups than workgroups, odd Q6_K super-blocks (blocks that start 2 bytes off a 4-byte
+    boundary)."""
     print("case type=%d in_dim=%d out_dim=%d tokens=%d" % (type_id, in_dim, out_dim, tokens), flush=True)
     assert quant.gemv_image_bytes(type_id, in_dim, tokens) == (in_dim // 256) * (8192 + (576 if type_id == Q6_K else 320))
     rng = np.random.default_rng(type_id * 1000003 + in_dim * 13 + out_dim * 7 + tokens)
@@ -188,6 +191,49 @@ def test_long_rows_and_q6_k_in_one_pass(gpu, oracle, type_id, in_dim, out_dim, t
     quant.gemv_dev(w.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, tokens, rd.ptr)
     assert np.array_equal(od.read(np.float32, tokens * out_dim), plain + res)
     for a in (w, xd, od, rd):
+        a.close()
+
+
+def test_q5_k_one_pass_element_order_and_fifth_bits(gpu, oracle):
+    """Unit activations pick single weights out of a Q5_K matrix: every element position of a super-block, so every bit of
+    every qh byte meets its nibble (a fifth bit taken from the neighbouring sub-block or byte shifts a weight by 16 codes)."""
+    in_dim, out_dim, tokens = 2048, 16, 8
+    rng = np.random.default_rng(55)
+    raw = synth.make_weights(rng, Q5_K, out_dim, in_dim)
+    w = DevArray(raw)
+    od = DevArray(nbytes=4 * tokens * out_dim)
+    dense = oracle.dequantize(raw, Q5_K, out_dim * in_dim).reshape(out_dim, in_dim)
+    for base in list(range(0, 256, 8)) + [256 + 64 + 9, 1024 + 200, 2040]:
+        x = np.zeros((tokens, in_dim), dtype=np.float32)
+        for m in range(tokens):                     # token m picks out column base + m
+            x[m, base + m] = 1.0
+        xd = DevArray(np.ascontiguousarray(x.reshape(-1)))
+        quant.gemv_dev(w.ptr, Q5_K, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+        got = od.read(np.float32, tokens * out_dim).reshape(tokens, out_dim)
+        for m in range(tokens):
+            assert np.allclose(got[m], dense[:, base + m], rtol=0, atol=2e-6 * float(np.abs(dense).max())), (base, m)
+        xd.close()
+    for a in (w, od):
+        a.close()
+
+
+def test_q5_k_and_q4_k_read_one_image(gpu, oracle):
+    """Q5_K takes the Q4_K activation image: one pack serves a Q4_K and a Q5_K matrix of the same input."""
+    in_dim, tokens, d4, d5 = 4096, 7, 272, 1040
+    rng = np.random.default_rng(45)
+    raw4, raw5 = synth.make_weights(rng, Q4_K, d4, in_dim), synth.make_weights(rng, Q5_K, d5, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    w4, w5, xd = DevArray(raw4), DevArray(raw5), DevArray(x)
+    assert quant.gemv_image_bytes(Q5_K, in_dim, tokens) == quant.gemv_image_bytes(Q4_K, in_dim, tokens)
+    image = DevArray(nbytes=quant.gemv_image_bytes(Q4_K, in_dim, tokens))
+    o4, o5 = DevArray(nbytes=4 * tokens * d4), DevArray(nbytes=4 * tokens * d5)
+    quant.gemv_pack_dev(xd.ptr, Q4_K, in_dim, tokens, image.ptr)
+    quant.gemv_packed_dev([w4.ptr], Q4_K, image.ptr, [o4.ptr], [d4], in_dim, tokens)
+    quant.gemv_packed_dev([w5.ptr], Q5_K, image.ptr, [o5.ptr], [d5], in_dim, tokens)
+    for raw, o, d, t in ((raw4, o4, d4, Q4_K), (raw5, o5, d5, Q5_K)):
+        want, tol = oracle_rows(oracle, raw, x, in_dim, d, tokens, t)
+        assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, "type %d against the shared image" % t)
+    for a in (w4, w5, xd, image, o4, o5):
         a.close()
 
 
