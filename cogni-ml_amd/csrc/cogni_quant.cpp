@@ -274,7 +274,8 @@ int cogni_quant_init(int32_t ordinal) {
   }
   g_rt.image_slot_bytes = ((size_t)gemv_mt_image_bytes(COGNI_TYPE_Q6_K, GEMV_MT_MAX_IN_DIM) + 255) & ~(size_t)255;
   HIP_TRY(hipMalloc(&g_rt.image_pool, g_rt.image_slot_bytes * Runtime::kImageSlots), "hipMalloc(activation images)");
-  for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q5_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32"}) {
+  for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q5_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32",
+                           "q4_k_gemv_mt_top1_partial_f32", "q6_k_gemv_mt_top1_partial_f32"}) {
     hipFunction_t fn = nullptr;
     HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
     g_rt.fns.emplace(name, fn);
@@ -756,6 +757,30 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
     m = left < cap ? left : cap;
     uint32_t grid = 0, block = 0, shmem = 0;
     std::string name;
+    int rc = 0;
+    // the group's partial results: [token in group][workgroup], inside the group's share of the caller's buffers
+    uint64_t xm = x + (uint64_t)t0 * in_dim * 4, pi = partial_ids + (uint64_t)t0 * stride * 4, pv = partial_values + (uint64_t)t0 * stride * 4;
+    uint64_t oi = top1_ids + (uint64_t)t0 * 4, ov = top1_values + (uint64_t)t0 * 4;
+    // up to eight tokens of a Q4_K or Q6_K matrix the one-pass kernel takes, from the token count at which pack + one
+    // pass is the faster way to the logits: the weights once for the whole group, the arg-max inside
+    const uint32_t from = (w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q6_K) ? gemv_mt_from(w_type, in_dim) : 0;
+    const uint32_t m8 = left < (uint32_t)GEMV_MT_MAX_TOKENS ? left : (uint32_t)GEMV_MT_MAX_TOKENS;
+    if (from && m8 >= from && gemv_mt_grid(w_type, in_dim, out_dim) <= stride) {
+      if (uint64_t image = image_for_stream(stream)) {
+        m = m8;
+        grid = gemv_mt_grid(w_type, in_dim, out_dim);
+        rc = cogni_gemv_pack_dev(xm, w_type, in_dim, m, image, stream);
+        if (rc != 0) return rc;
+        void* params[] = {&w_raw, &image, &pi, &pv, &in_dim, &out_dim, &m};
+        rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt_top1_partial_f32" : "q4_k_gemv_mt_top1_partial_f32", grid,
+                    GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type), params, stream);
+        if (rc != 0) return rc;
+        void* rparams[] = {&pi, &pv, &oi, &ov, &grid};
+        rc = launch("top1_reduce_f32", m, 1024, 0, rparams, stream);
+        if (rc != 0) return rc;
+        continue;
+      }
+    }
     // three or four tokens of a Q4_K or Q6_K matrix: the matrix-core kernel with the arg-max inside, where its
     // workgroups fit the caller's partial buffers (sized for the vector-ALU kernels)
     const uint32_t mm = left < (uint32_t)GEMV_MFMA_MAX_TOKENS ? left : (uint32_t)GEMV_MFMA_MAX_TOKENS;
@@ -767,15 +792,11 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
       shmem = gemv_mfma_lds_bytes(w_type, (int)m, in_dim);
       name = std::string(type_prefix(w_type)) + "_gemv_mfma_top1_partial_f32_tbatch" + std::to_string(m);
     } else {
-      int rc = cogni_gemv_launch_dims(w_type, m, in_dim, out_dim, &grid, &block, &shmem);
+      rc = cogni_gemv_launch_dims(w_type, m, in_dim, out_dim, &grid, &block, &shmem);
       if (rc != 0) return rc;
       name = std::string(type_prefix(w_type)) + "_gemv_top1_partial_f32";
       if (m > 1) name += "_tbatch" + std::to_string(m);
     }
-    int rc = 0;
-    // the group's partial results: [token in group][workgroup], inside the group's share of the caller's buffers
-    uint64_t xm = x + (uint64_t)t0 * in_dim * 4, pi = partial_ids + (uint64_t)t0 * stride * 4, pv = partial_values + (uint64_t)t0 * stride * 4;
-    uint64_t oi = top1_ids + (uint64_t)t0 * 4, ov = top1_values + (uint64_t)t0 * 4;
     void* params[] = {&w_raw, &xm, &pi, &pv, &in_dim, &out_dim};
     rc = launch(name.c_str(), grid, block, shmem, params, stream);
     if (rc != 0) return rc;

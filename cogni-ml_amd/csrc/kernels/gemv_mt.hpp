@@ -415,10 +415,15 @@ constexpr int mt_stream_wait(int S, int NSLOT, int NA, int NC, int i) {
 // SWIGLU (T = 2, or T = 1 with streamed operands: gate tile, then up tile): the two tiles of a row group are tile grp of
 // w[0] (gate) and tile grp of w[1] (up), rows[0] = rows[1] = out_dim, and the workgroup stores out[0][m][o] = silu(gate . x) * (up . x) (swiglu_one, the function of
 // swiglu_f32): the values of the pair launch followed by swiglu_f32, bit for bit, without the gate and up vectors in memory.
-template <class F, int SBW, int T, bool SWIGLU = false>
+// TOP1 (one matrix): instead of the row values the workgroup stores, per token, the largest of the rows it walked and
+// that row's index (out[0][m * gridDim.x + blockIdx.x], top_ids[same]; of equal values the lowest row wins): the partial
+// results top1_reduce_f32 finishes, as q6_k_gemv_top1_partial_f32 writes them for one token.
+template <class F, int SBW, int T, bool SWIGLU = false, bool TOP1 = false>
 __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __restrict__ image,
-                                             const float* __restrict__ residual, u32 in_dim, u32 tokens) {
+                                             const float* __restrict__ residual, u32 in_dim, u32 tokens,
+                                             u32* __restrict__ top_ids = nullptr) {
   constexpr bool STREAM = SBW > 2;
+  static_assert(!TOP1 || (!SWIGLU && T * 16 * GEMV_MT_MAX_TOKENS <= GEMV_MT_WAVES * 64), "TOP1: a thread owns one (tile, token, row) of a row group");
   static_assert(!SWIGLU || T == (STREAM ? 1 : 2), "SWIGLU pairs a gate tile with an up tile");
   static_assert(!STREAM || T == 1, "streamed operands: one tile per wavefront");
   static_assert(STREAM || SBW * T <= F::NSLOT, "every unit of a row group has a slot");
@@ -445,6 +450,8 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
 
   u32 grp = blockIdx.x;
   if (grp >= ngroups) return;
+  float top_v = -__builtin_inff();   // TOP1: the best row this thread has seen in its place of the row groups
+  u32 top_i = 0xFFFFFFFFu;
 
   // ---- operand sets: the A operands of a super-block and its scales and sub-block sums ----
   mt_u32x4 breg[NSETS][8], auxr[NSETS][F::NAUX];
@@ -539,7 +546,12 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
 #pragma unroll
         for (u32 k = 0; k < GEMV_MT_WAVES; k++) v += part[((k * GEMV_MT_TMAX + t) * 8 + m) * 16 + r];
         const u32 row = (grp * T + t) * 16 + r;
-        if (row < a.rows[0]) {
+        if constexpr (TOP1) {
+          // (the groups a thread walks ascend, so do its rows: among equal values the first one stays; a row past the end
+          // competes as minus infinity under the highest index)
+          const bool real = row < a.rows[0];
+          top1_take(top_v, top_i, real ? v : -__builtin_inff(), real ? row : 0xFFFFFFFFu);
+        } else if (row < a.rows[0]) {
           const size_t oi = (size_t)m * a.rows[0] + row;
           if (residual) v += residual[oi];
           a.out[0][oi] = v;
@@ -659,30 +671,53 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
       between_groups();
     }
   }
+  if constexpr (TOP1) {
+    // the threads' winners meet where the partial sums were: thread o held (tile o / (16 tokens), token (o / 16) % tokens,
+    // row o % 16), so token m's candidates are the T runs of 16 threads from 16 (t tokens + m) on
+    between_groups();
+    u32* const cand_i = reinterpret_cast<u32*>(part + GEMV_MT_WAVES * 64);
+    part[tid] = top_v;
+    cand_i[tid] = top_i;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if ((u32)tid < tokens) {
+      float best = -__builtin_inff();
+      u32 best_id = 0xFFFFFFFFu;
+      for (u32 t = 0; t < (u32)T; t++)
+        for (u32 r = 0; r < 16; r++) {
+          const u32 o = (t * tokens + (u32)tid) * 16 + r;
+          top1_take(best, best_id, part[o], cand_i[o]);
+        }
+      a.out[0][(size_t)tid * gridDim.x + blockIdx.x] = best;
+      top_ids[(size_t)tid * gridDim.x + blockIdx.x] = best_id;
+    }
+  }
 }
 
 // The tile count per wavefront follows from the row count (gemv_mt_tiles, the rule the host sizes the grid with); tile
 // count and super-blocks per k-slice are template parameters so that register use and loads in flight are compile-time
 // constants. Shapes outside gemv_mt_supported() must not be launched.
-template <class F>
-__device__ __forceinline__ void gemv_mt_dispatch(const MtArgs& a, const uint8_t* image, const float* residual, u32 in_dim, u32 tokens) {
+template <class F, bool TOP1 = false>
+__device__ __forceinline__ void gemv_mt_dispatch(const MtArgs& a, const uint8_t* image, const float* residual, u32 in_dim, u32 tokens,
+                                                 u32* top_ids = nullptr) {
   const u32 ntiles = (a.rows[0] + a.rows[1] + a.rows[2] + 15) >> 4;
   const u32 t = gemv_mt_tiles(F::TYPE, in_dim, ntiles);
   switch (in_dim >> 11) {
     case 1:
-      if (t <= 1) gemv_mt_core<F, 1, 1>(a, image, residual, in_dim, tokens);
-      else if (t == 2) gemv_mt_core<F, 1, 2>(a, image, residual, in_dim, tokens);
-      else if constexpr (F::TMAX >= 3) gemv_mt_core<F, 1, 3>(a, image, residual, in_dim, tokens);
+      if (t <= 1) gemv_mt_core<F, 1, 1, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
+      else if (t == 2) gemv_mt_core<F, 1, 2, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
+      else if constexpr (F::TMAX >= 3) gemv_mt_core<F, 1, 3, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
       break;
     case 2:
-      if (t <= 1) gemv_mt_core<F, 2, 1>(a, image, residual, in_dim, tokens);
-      else if (t == 2) gemv_mt_core<F, 2, 2>(a, image, residual, in_dim, tokens);
-      else if constexpr (F::TMAX >= 3) gemv_mt_core<F, 2, 3>(a, image, residual, in_dim, tokens);
+      if (t <= 1) gemv_mt_core<F, 2, 1, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
+      else if (t == 2) gemv_mt_core<F, 2, 2, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
+      else if constexpr (F::TMAX >= 3) gemv_mt_core<F, 2, 3, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
       break;
-    case 3: gemv_mt_core<F, 3, 1>(a, image, residual, in_dim, tokens); break;
-    case 4: gemv_mt_core<F, 4, 1>(a, image, residual, in_dim, tokens); break;
-    case 5: gemv_mt_core<F, 5, 1>(a, image, residual, in_dim, tokens); break;
-    default: gemv_mt_core<F, 6, 1>(a, image, residual, in_dim, tokens); break;
+    case 3: gemv_mt_core<F, 3, 1, false, TOP1>(a, image, residual, in_dim, tokens, top_ids); break;
+    case 4: gemv_mt_core<F, 4, 1, false, TOP1>(a, image, residual, in_dim, tokens, top_ids); break;
+    case 5: gemv_mt_core<F, 5, 1, false, TOP1>(a, image, residual, in_dim, tokens, top_ids); break;
+    default: gemv_mt_core<F, 6, 1, false, TOP1>(a, image, residual, in_dim, tokens, top_ids); break;
   }
 }
 
@@ -696,6 +731,25 @@ __device__ __forceinline__ void gemv_mt_dispatch(const MtArgs& a, const uint8_t*
 GEMV_MT_ENTRY(q4_k_gemv_mt_f32, MtQ4K)
 GEMV_MT_ENTRY(q5_k_gemv_mt_f32, MtQ5K)
 GEMV_MT_ENTRY(q6_k_gemv_mt_f32, MtQ6K)
+
+// (w, image, partial_ids, partial_values, in_dim, out_dim, tokens): the output head's arg-max for 2..8 tokens in one pass
+// over the weights. Grid, block and dynamic shared memory as q4_k_gemv_mt_f32 | q6_k_gemv_mt_f32 for out_dim rows;
+// partial_*[token * gridDim.x + workgroup], finished by top1_reduce_f32 with count = gridDim.x. The one-token kernel's
+// parameter order (src/ml/cuda/kernels/q6k_gemv_probe.ptx:1331-1338) with the image in the place of x and the token count
+// behind.
+#define GEMV_MT_TOP1_ENTRY(NAME, FMT)                                                                                    \
+  extern "C" __global__ __launch_bounds__(GEMV_MT_WAVES * 64) void NAME(const uint8_t* w, const uint8_t* image,          \
+                                                                        u32* partial_ids, float* partial_values,         \
+                                                                        u32 in_dim, u32 out_dim, u32 tokens) {           \
+    /* the absent matrices' row counts: a zero the optimizer cannot see through (with literal zeros it folds the lookup */ \
+    /* of a row's matrix away, and this release of the compiler crashes in its control-flow simplification doing so)    */ \
+    u32 none;                                                                                                            \
+    asm volatile("s_mov_b32 %0, 0" : "=s"(none));                                                                        \
+    const MtArgs a = {{w, w, w}, {partial_values, partial_values, partial_values}, {out_dim, none, none}};               \
+    gemv_mt_dispatch<FMT, true>(a, image, nullptr, in_dim, tokens, partial_ids);                                         \
+  }
+GEMV_MT_TOP1_ENTRY(q4_k_gemv_mt_top1_partial_f32, MtQ4K)
+GEMV_MT_TOP1_ENTRY(q6_k_gemv_mt_top1_partial_f32, MtQ6K)
 
 // (w_gate, w_up, image, out, in_dim, out_dim, tokens): out[m][o] = silu(gate . x) * (up . x); block 512, grid = min(256,
 // ceil(out_dim / 16)), dynamic shared memory as q4_k_gemv_mt_f32. The parameter list of q4_k_dual_gemv_swiglu_f32 with the

@@ -243,7 +243,11 @@ int cogni_embed_dev(uint64_t w_raw, uint32_t w_type, uint64_t token_ids, uint64_
 
 /* Output head without the logits: for each token the index of the largest element of W x and that value
  * (top1_ids: u32[tokens], top1_values: f32[tokens]); of equal values the lowest index wins, as in the reference's CPU scan
- * (bin/cuda_mixed_stack_probe.cr:1485-1497). Two launches per group of tokens. Groups of 3 or 4 tokens of a Q4_K or Q6_K
+ * (bin/cuda_mixed_stack_probe.cr:1485-1497). Groups of up to 8 tokens of a Q4_K or Q6_K matrix the one-pass kernel takes
+ * (from cogni_gemv_one_pass_from(w_type, in_dim) tokens, with the library's image of `stream`) are three launches: the
+ * pack, "q4_k_gemv_mt_top1_partial_f32" | "q6_k_gemv_mt_top1_partial_f32" (w_raw, image, partial_ids, partial_values,
+ * in_dim, out_dim, tokens; the geometry of cogni_gemv_packed_launch_dims) - the weights once for the group, the arg-max
+ * inside - and the reduce below. Otherwise two launches per group of tokens: groups of 3 or 4 tokens of a Q4_K or Q6_K
  * matrix take the matrix-core kernel "<prefix>_gemv_mfma_top1_partial_f32_tbatchM" (same parameters, the geometry of
  * cogni_gemv_plan) where that kernel takes the shape and its grid fits the partial buffers; otherwise groups of up to
  * 2 tokens (Q4_K, Q6_K; one token for the other types):

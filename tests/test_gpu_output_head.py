@@ -101,6 +101,39 @@ def test_top1_on_the_matrix_cores(gpu, oracle, t, in_dim, out_dim, tokens):
     assert list(ids3) == [0] * tokens
 
 
+@pytest.mark.parametrize("t,in_dim,out_dim,tokens", [(Q6_K, 2048, 70001, 8), (Q6_K, 4096, 3000, 3), (Q4_K, 4096, 20011, 5),
+                                                     (Q4_K, 12288, 530, 4), (Q6_K, 6144, 50, 6), (Q4_K, 2048, 17, 8),
+                                                     (Q6_K, 4096, 16 * 2 * 256 * 2 + 24, 7), (Q4_K, 4096, 4099, 13)])
+def test_top1_in_one_pass(gpu, oracle, t, in_dim, out_dim, tokens):
+    """Up to eight tokens of a matrix the one-pass kernel takes: the weights once for the group, the arg-max inside
+    (one, two and three tiles per wavefront, streamed long rows, workgroups that walk several row groups, a partial tile,
+    13 tokens as eight and five). Same bits as that kernel's logits, lowest row among equal values, winner within the GEMV
+    tolerance of the oracle's."""
+    rng = np.random.default_rng(out_dim * 5 + tokens)
+    base = synth.make_weights(rng, t, out_dim, in_dim).reshape(out_dim, -1)
+    x = synth.make_activations(rng, tokens, in_dim)
+    ids, vals, logits = run_top1(np.ascontiguousarray(base).reshape(-1), t, x, in_dim, out_dim, tokens)
+    assert 0 < quant.gemv_one_pass_from(t, in_dim) <= min(tokens, 8)     # gemv_dev (the logits) goes one pass too
+    want = oracle.matmul_add(x, tokens, in_dim, base.reshape(-1), t, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).reshape(tokens, out_dim)
+    for tok in range(tokens):
+        assert ids[tok] == first_max(logits[tok]) and vals[tok] == logits[tok].max(), tok
+        top = float(want[tok].max())
+        assert want[tok][ids[tok]] >= top - 1e-4 * float(np.abs(want[tok]).max())
+    # ties: copies of token 0's winning row at lower and higher indices, in other tiles, row groups and workgroups
+    best = int(ids[0])
+    dup = sorted({out_dim - 1, out_dim // 2, min(best + 17, out_dim - 1), max(best - 1, 0), 3 % out_dim})
+    rows = base.copy()
+    for r in dup:
+        rows[r] = base[best]
+    ids2, vals2, lg2 = run_top1(np.ascontiguousarray(rows).reshape(-1), t, x, in_dim, out_dim, tokens)
+    assert ids2[0] == min(dup + [best]) and vals2[0] == lg2[0].max()
+    for tok in range(1, tokens):
+        assert ids2[tok] == first_max(lg2[tok])
+    rows = np.repeat(base[:1], out_dim, axis=0)
+    ids3, _, _ = run_top1(np.ascontiguousarray(rows).reshape(-1), t, x, in_dim, out_dim, tokens)
+    assert list(ids3) == [0] * tokens
+
+
 def test_output_head_runner(gpu, oracle):
     hidden, vocab, tokens = 1024, 20011, 4
     rng = np.random.default_rng(3)
