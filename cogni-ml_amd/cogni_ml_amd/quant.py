@@ -85,11 +85,11 @@ def gemv_many_dev(w_ptrs, w_type, x_ptr, out_ptrs, out_dims, in_dim, tokens=1, s
                                          stream))
 
 
-def gemv_one_pass_from(w_type, in_dim):
+def gemv_one_pass_from(w_type, in_dim, out_dim):
     """Token count from which gemv_dev packs the activations and reads the weights once (0: never for this shape)."""
     f = hip.lib().cogni_gemv_one_pass_from
     f.restype = ctypes.c_uint32
-    return int(f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim)))
+    return int(f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim)))
 
 
 def gemv_image_bytes(w_type, in_dim, tokens):

@@ -56,7 +56,7 @@ lib LibCogniHIP
                      in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemv_plan(type : UInt32, tokens : UInt32, add : Int32, in_dim : UInt32, out_dim : UInt32, kernel : UInt8**,
                       grid_x : UInt32*, block_x : UInt32*, shared_mem_bytes : UInt32*) : Int32
-  fun cogni_gemv_one_pass_from(w_type : UInt32, in_dim : UInt32) : UInt32
+  fun cogni_gemv_one_pass_from(w_type : UInt32, in_dim : UInt32, out_dim : UInt32) : UInt32
   fun cogni_gemv_release_stream(stream : Void*) : Int32
   fun cogni_gemv_image_bytes(w_type : UInt32, in_dim : UInt32, tokens : UInt32) : LibC::SizeT
   fun cogni_gemv_packed_launch_dims(w_type : UInt32, in_dim : UInt32, total_rows : UInt32,

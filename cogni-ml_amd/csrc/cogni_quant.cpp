@@ -316,7 +316,7 @@ size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens)
   return gemv_mt_supported(w_type, (int)tokens, in_dim) ? (size_t)gemv_mt_image_bytes(w_type, in_dim) : 0;
 }
 
-uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim) { return gemv_mt_from(w_type, in_dim); }
+uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim, uint32_t out_dim) { return gemv_mt_from(w_type, in_dim, out_dim); }
 
 int cogni_gemv_release_stream(void* stream) {
   int slot = -1;
@@ -459,7 +459,7 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
   // several tokens of a matrix the one-pass kernel takes: groups of up to eight, the weights read once per group, from
   // the token count at which pack + one pass measures faster than the kernels below
-  if (const uint32_t from = gemv_mt_from(w_type, in_dim)) {
+  if (const uint32_t from = gemv_mt_from(w_type, in_dim, out_dim)) {
     int rc = 0;
     if (try_one_pass(&w_raw, w_type, x, residual, &out, &out_dim, 1, in_dim, tokens, from, stream, &rc)) return rc;
   }
@@ -763,7 +763,7 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
     uint64_t oi = top1_ids + (uint64_t)t0 * 4, ov = top1_values + (uint64_t)t0 * 4;
     // up to eight tokens of a Q4_K or Q6_K matrix the one-pass kernel takes, from the token count at which pack + one
     // pass is the faster way to the logits: the weights once for the whole group, the arg-max inside
-    const uint32_t from = (w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q6_K) ? gemv_mt_from(w_type, in_dim) : 0;
+    const uint32_t from = (w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q6_K) ? gemv_mt_from(w_type, in_dim, out_dim) : 0;
     const uint32_t m8 = left < (uint32_t)GEMV_MT_MAX_TOKENS ? left : (uint32_t)GEMV_MT_MAX_TOKENS;
     if (from && m8 >= from && gemv_mt_grid(w_type, in_dim, out_dim) <= stride) {
       if (uint64_t image = image_for_stream(stream)) {

@@ -185,9 +185,15 @@ static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned 
          in_dim <= GEMV_MT_MAX_IN_DIM;
 }
 // Token count from which one matrix goes through pack + one pass rather than the per-token-group kernels (0: never): where
-// the pair measures faster. Q6_K from three tokens; Q4_K from four on rows longer than 4096 values, else from five.
-static inline unsigned gemv_mt_from(unsigned type, unsigned in_dim) {
+// the pair measures faster. Q6_K from three tokens; Q4_K and Q5_K from four on rows longer than 4096 values, else from five.
+// Tall matrices of up to 4096 columns (an output head): the workgroups walk many row groups and pay their start once, which
+// puts the kernel ahead earlier - Q6_K from two tokens at GEMV_MT_TALL_ROWS rows, Q4_K and Q5_K from three there and from
+// two at GEMV_MT_VERY_TALL_ROWS.
+#define GEMV_MT_TALL_ROWS 40960u
+#define GEMV_MT_VERY_TALL_ROWS 98304u
+static inline unsigned gemv_mt_from(unsigned type, unsigned in_dim, unsigned out_dim) {
   if (!gemv_mt_supported(type, 2, in_dim)) return 0;
+  if (in_dim <= 4096u && out_dim >= GEMV_MT_TALL_ROWS) return (type == 14 || out_dim >= GEMV_MT_VERY_TALL_ROWS) ? 2u : 3u;
   return type == 14 ? 3u : (in_dim > 4096u ? 4u : 5u);
 }
 // tiles per wavefront: rows of more than 4096 values one (the operands are streamed); else as many as keep 256 workgroups

@@ -110,7 +110,8 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 /* Decode GEMV, weights read once for all tokens:
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
  * fp32 accumulation. tokens >= 1; several tokens of a matrix the one-pass kernel takes (see cogni_gemv_pack_dev below;
- * Q6_K from three tokens, Q4_K and Q5_K from four on rows longer than 4096 values, else from five) go in groups of up to 8 with
+ * cogni_gemv_one_pass_from: Q6_K from three tokens, Q4_K and Q5_K from four on rows longer than 4096 values, else from
+ * five, tall matrices earlier) go in groups of up to 8 with
  * the weights read once per group; otherwise they are issued as consecutive launches of the token count that measures
  * fastest for the type and shape: up to 4 where cogni_gemv_plan picks the matrix-core kernel, else pairs for the
  * K-quants (one group of three when the count is odd and the matrix is short enough for one workgroup per row group)
@@ -149,9 +150,11 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
  * cogni_gemv_plan describes). A graph captured from one stream carries that stream's image: replay it on one stream at a
  * time, and not beside eager calls on the capture stream. */
 size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
-/* The token count from which cogni_gemv_dev takes this path for one matrix (Q6_K 3; Q4_K and Q5_K 4 on rows longer than 4096 values,
- * else 5), 0 where it never does; below it the call runs the kernel cogni_gemv_plan names. No GPU needed. */
-uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim);
+/* The token count from which cogni_gemv_dev and cogni_gemv_top1_dev take this path for one matrix (Q6_K 3; Q4_K and Q5_K 4
+ * on rows longer than 4096 values, else 5; a tall matrix of up to 4096 columns - 40960 rows and more, an output head -
+ * earlier: Q6_K 2, Q4_K and Q5_K 3, and 2 from 98304 rows), 0 where they never do; below it the call runs the kernel
+ * cogni_gemv_plan names. No GPU needed. */
+uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim, uint32_t out_dim);
 /* Gives back the image the library keeps for `stream` (waits for the stream's work first; nothing to do and no error if it
  * has none). Call it before destroying a stream that ran multi-token GEMVs: the eight slots are otherwise used up by the
  * first eight streams of the process, and later streams run the per-token-group kernels. A graph captured on the stream
@@ -244,7 +247,7 @@ int cogni_embed_dev(uint64_t w_raw, uint32_t w_type, uint64_t token_ids, uint64_
 /* Output head without the logits: for each token the index of the largest element of W x and that value
  * (top1_ids: u32[tokens], top1_values: f32[tokens]); of equal values the lowest index wins, as in the reference's CPU scan
  * (bin/cuda_mixed_stack_probe.cr:1485-1497). Groups of up to 8 tokens of a Q4_K or Q6_K matrix the one-pass kernel takes
- * (from cogni_gemv_one_pass_from(w_type, in_dim) tokens, with the library's image of `stream`) are three launches: the
+ * (from cogni_gemv_one_pass_from(w_type, in_dim, out_dim) tokens, with the library's image of `stream`) are three launches: the
  * pack, "q4_k_gemv_mt_top1_partial_f32" | "q6_k_gemv_mt_top1_partial_f32" (w_raw, image, partial_ids, partial_values,
  * in_dim, out_dim, tokens; the geometry of cogni_gemv_packed_launch_dims) - the weights once for the group, the arg-max
  * inside - and the reduce below. Otherwise two launches per group of tokens: groups of 3 or 4 tokens of a Q4_K or Q6_K

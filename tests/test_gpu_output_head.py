@@ -80,7 +80,7 @@ def test_top1_on_the_matrix_cores(gpu, oracle, t, in_dim, out_dim, tokens):
     x = synth.make_activations(rng, tokens, in_dim)
     ids, vals, logits = run_top1(np.ascontiguousarray(base).reshape(-1), t, x, in_dim, out_dim, tokens)
     assert "mfma" in quant.gemv_plan(t, tokens, in_dim, out_dim)[0]
-    assert not 0 < quant.gemv_one_pass_from(t, in_dim) <= tokens      # gemv_dev (the logits) runs that kernel too
+    assert not 0 < quant.gemv_one_pass_from(t, in_dim, out_dim) <= tokens      # gemv_dev (the logits) runs that kernel too
     want = oracle.matmul_add(x, tokens, in_dim, base.reshape(-1), t, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).reshape(tokens, out_dim)
     for tok in range(tokens):
         assert ids[tok] == first_max(logits[tok]) and vals[tok] == logits[tok].max()
@@ -103,17 +103,18 @@ def test_top1_on_the_matrix_cores(gpu, oracle, t, in_dim, out_dim, tokens):
 
 @pytest.mark.parametrize("t,in_dim,out_dim,tokens", [(Q6_K, 2048, 70001, 8), (Q6_K, 4096, 3000, 3), (Q4_K, 4096, 20011, 5),
                                                      (Q4_K, 12288, 530, 4), (Q6_K, 6144, 50, 6), (Q4_K, 2048, 17, 8),
-                                                     (Q6_K, 4096, 16 * 2 * 256 * 2 + 24, 7), (Q4_K, 4096, 4099, 13)])
+                                                     (Q6_K, 4096, 16 * 2 * 256 * 2 + 24, 7), (Q4_K, 4096, 4099, 13),
+                                                     (Q6_K, 2048, 41000, 2), (Q4_K, 2048, 99001, 2), (Q4_K, 2048, 41000, 3)])
 def test_top1_in_one_pass(gpu, oracle, t, in_dim, out_dim, tokens):
     """Up to eight tokens of a matrix the one-pass kernel takes: the weights once for the group, the arg-max inside
     (one, two and three tiles per wavefront, streamed long rows, workgroups that walk several row groups, a partial tile,
-    13 tokens as eight and five). Same bits as that kernel's logits, lowest row among equal values, winner within the GEMV
+    13 tokens as eight and five, tall matrices from two and three tokens). Same bits as that kernel's logits, lowest row among equal values, winner within the GEMV
     tolerance of the oracle's."""
     rng = np.random.default_rng(out_dim * 5 + tokens)
     base = synth.make_weights(rng, t, out_dim, in_dim).reshape(out_dim, -1)
     x = synth.make_activations(rng, tokens, in_dim)
     ids, vals, logits = run_top1(np.ascontiguousarray(base).reshape(-1), t, x, in_dim, out_dim, tokens)
-    assert 0 < quant.gemv_one_pass_from(t, in_dim) <= min(tokens, 8)     # gemv_dev (the logits) goes one pass too
+    assert 0 < quant.gemv_one_pass_from(t, in_dim, out_dim) <= min(tokens, 8)     # gemv_dev (the logits) goes one pass too
     want = oracle.matmul_add(x, tokens, in_dim, base.reshape(-1), t, out_dim, np.zeros(out_dim, dtype=np.float32), threads=8).reshape(tokens, out_dim)
     for tok in range(tokens):
         assert ids[tok] == first_max(logits[tok]) and vals[tok] == logits[tok].max(), tok
