@@ -448,6 +448,9 @@ def main():
         gemv_case("q6_k gemv 4096x12288 M=4", Q6_K, 4096, 12288, 4)
         gemv_case("q6_k gemv 4096x12288 M=8", Q6_K, 4096, 12288, 8)
         gemv_case("q5_k gemv 4096x4096 M=4", Q5_K, 4096, 4096, 4)
+        gemv_case("q5_k gemv attn_qkv 8192x4096 M=8", Q5_K, 8192, 4096, 8)
+        gemv_case("q6_k gemv output head 151936x4096 M=2", Q6_K, 151936, 4096, 2)
+        gemv_case("q6_k gemv output head 151936x4096 M=8", Q6_K, 151936, 4096, 8)
 
     # config 4: prefill GEMM
     gemm = {}
@@ -500,7 +503,7 @@ def main():
         # output head without the logits: RMSNorm -> Q6_K vocabulary projection with arg-max -> top-1 reduce (510 MB)
         from cogni_ml_amd.output_head import QwenOutputHeadRunner, Weights as HeadWeights
         hw = HeadWeights(np.ones(4096, dtype=np.float32), synth.make_weights(rng, Q6_K, 151936, 4096), Q6_K, 4096, 151936)
-        for tokens in (1, 3):
+        for tokens in (1, 3, 8):
             ohead = QwenOutputHeadRunner.from_weights(hw, tokens, synth.make_activations(rng, tokens, 4096).reshape(-1), 1e-6)
             ohead.upload_weights()
             ohead.reset_sequence()

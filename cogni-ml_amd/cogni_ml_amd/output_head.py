@@ -2,7 +2,7 @@
 
 The HIP counterpart of the reference's QwenOutputHeadRunner (src/ml/cuda/qwen_output_head_runner.cr:6-7, 659-760; launches
 :937-940): the default decode-facing path reads back only the top-1 id and value per token; the full logits are read
-only on request (read_logits), through the plain GEMV. Groups of up to three tokens share one pass over the weights.
+only on request (read_logits), through the plain GEMV. Groups of up to eight tokens share one pass over the weights.
 """
 import numpy as np
 
@@ -17,7 +17,7 @@ class Weights:
 
 
 class QwenOutputHeadRunner:
-    GROUP = 3    # tokens per pass over the weights
+    GROUP = quant.MAX_GEMV_TOKENS    # tokens handed to the library at a time: up to eight share one pass over the weights
 
     def __init__(self, weights, tokens, xs, eps, read_logits=False):
         if not tokens > 0:
