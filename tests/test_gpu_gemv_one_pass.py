@@ -260,18 +260,20 @@ def test_q6_k_one_pass_element_order_and_scale_positions(gpu, oracle):
         a.close()
 
 
-def test_q6_k_lists_share_one_image(gpu, oracle):
-    """Two Q6_K matrices against one activation block through the list operator (one pack, one launch)."""
-    in_dim, dims, tokens = 4096, (1024, 272), 6
-    rng = np.random.default_rng(66)
-    raws = [synth.make_weights(rng, Q6_K, d, in_dim) for d in dims]
+@pytest.mark.parametrize("type_id,in_dim,dims,tokens", [(Q6_K, 4096, (1024, 272), 6), (Q5_K, 4096, (8192, 1024, 40), 2),
+                                                        (Q5_K, 6144, (272, 16, 1040, 33), 8)])
+def test_q5_k_and_q6_k_lists_share_one_image(gpu, oracle, type_id, in_dim, dims, tokens):
+    """Q5_K and Q6_K matrices against one activation block through the list operator (one pack, up to three matrices per
+    launch, from two tokens)."""
+    rng = np.random.default_rng(66 + type_id)
+    raws = [synth.make_weights(rng, type_id, d, in_dim) for d in dims]
     x = synth.make_activations(rng, tokens, in_dim)
     ws, xd = [DevArray(r) for r in raws], DevArray(x)
     outs = [DevArray(nbytes=4 * tokens * d) for d in dims]
-    quant.gemv_many_dev([w_.ptr for w_ in ws], Q6_K, xd.ptr, [o.ptr for o in outs], list(dims), in_dim, tokens)
+    quant.gemv_many_dev([w_.ptr for w_ in ws], type_id, xd.ptr, [o.ptr for o in outs], list(dims), in_dim, tokens)
     for raw, o, d in zip(raws, outs, dims):
-        want, tol = oracle_rows(oracle, raw, x, in_dim, d, tokens, Q6_K)
-        assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, "q6_k list member %d" % d)
+        want, tol = oracle_rows(oracle, raw, x, in_dim, d, tokens, type_id)
+        assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, "type %d list member %d" % (type_id, d))
     for a in ws + outs + [xd]:
         a.close()
 
