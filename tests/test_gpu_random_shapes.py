@@ -73,3 +73,47 @@ def test_random_gemm_shapes(gpu, oracle, seed):
         what = "seed %d case %d: type %d M=%d out=%d in=%d bias=%s" % (seed, case, t, tokens, out_dim, in_dim, bias is not None)
         print(what, flush=True)
         check_gemm(oracle, raw, x, in_dim, out_dim, tokens, bias, what, t=t)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_one_pass_shapes(gpu, oracle, seed):
+    """Shapes the one-pass kernels take (in_dim a multiple of 2048 up to 12288; Q4_K, Q5_K, Q6_K), drawn: 2..17 tokens (a
+    group of eight and what is left), single matrices with and without residual, lists of two to five matrices with row
+    counts that are and are not multiples of 16, top-1, activations scaled far out of the binary16 range."""
+    from test_gpu_gemv_one_pass import assert_bars, oracle_rows
+    rng = np.random.default_rng(9100 + seed)
+    for case in range(12):
+        t = [Q4_K, Q5_K, Q6_K][int(rng.integers(0, 3))]
+        in_dim = 2048 * int(rng.integers(1, 7))
+        tokens = int(rng.integers(2, 18))
+        kind = ["single", "residual", "list", "top1"][int(rng.integers(0, 4))]
+        if kind == "top1" and t == Q5_K:
+            kind = "single"
+        count = int(rng.integers(2, 6)) if kind == "list" else 1
+        dims = [int(rng.integers(1, 1500)) if rng.integers(0, 3) else 16 * int(rng.integers(1, 90)) for _ in range(count)]
+        what = "seed %d case %d: type %d in=%d M=%d %s dims=%s" % (seed, case, t, in_dim, tokens, kind, dims)
+        print(what, flush=True)
+        raws = [synth.make_weights(rng, t, d, in_dim) for d in dims]
+        x = synth.make_activations(rng, tokens, in_dim)
+        if rng.integers(0, 4) == 0 and kind != "residual":
+            x *= np.float32(10.0 ** float(rng.integers(-20, 20)))
+        if kind == "residual":
+            res = rng.standard_normal(tokens * dims[0]).astype(np.float32)
+            check_gemv(oracle, raws[0], t, x, in_dim, dims[0], tokens, res, what)
+            continue
+        if kind == "top1":
+            ids, vals, logits = run_top1(raws[0], t, x, in_dim, dims[0], tokens)
+            for tok in range(tokens):
+                assert ids[tok] == int(np.argmax(logits[tok])) or np.isclose(vals[tok], logits[tok].max(), rtol=3e-5, atol=0), what
+            continue
+        ws, xd = [DevArray(r) for r in raws], DevArray(x)
+        outs = [DevArray(nbytes=4 * tokens * d) for d in dims]
+        if kind == "list":
+            quant.gemv_many_dev([w.ptr for w in ws], t, xd.ptr, [o.ptr for o in outs], dims, in_dim, tokens)
+        else:
+            quant.gemv_dev(ws[0].ptr, t, xd.ptr, outs[0].ptr, in_dim, dims[0], tokens)
+        for raw, o, d in zip(raws, outs, dims):
+            want, tol = oracle_rows(oracle, raw, x, in_dim, d, tokens, t)
+            assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, what + " member %d" % d)
+        for a in ws + outs + [xd]:
+            a.close()
