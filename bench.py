@@ -533,7 +533,7 @@ def main():
         # FFN sequence of one layer: gate | up | SwiGLU in one launch, then Q6_K down with the residual add
         from cogni_ml_amd.ffn_sequence import FFNSequenceRunner
         graw = [synth.make_weights(rng, Q4_K, 12288, 4096) for _ in range(2)] + [synth.make_weights(rng, Q6_K, 4096, 12288)]
-        for tokens, block in ((1, False), (4, False), (1, True)):
+        for tokens, block in ((1, False), (4, False), (1, True), (4, True)):
             fx = rng.uniform(-1.0, 1.0, tokens * 4096).astype(np.float32)
             if block:   # the FFN half of a decoder layer: add + RMSNorm ahead of the projections
                 ffn = FFNSequenceRunner(graw[0], graw[1], graw[2], 4096, 12288, tokens, fx, norm=np.ones(4096, dtype=np.float32), add=fx.copy())

@@ -42,6 +42,9 @@ class FFNSequenceRunner:
         self._norm = self._alloc(4 * hidden) if norm is not None else None
         self._add = self._alloc(4 * tokens * hidden) if norm is not None else None
         self._normed = self._alloc(4 * tokens * hidden) if norm is not None else None
+        # several tokens behind the norm: the norm itself writes the activation image gate | up read (no pack launch)
+        image_bytes = quant.gemv_image_bytes(TensorType.Q4_K, hidden, quant.MAX_GEMV_TOKENS) if hidden <= 4096 else 0
+        self._image = self._alloc(image_bytes) if norm is not None and image_bytes and ffn_dim % 16 == 0 else None
         self._gate = self._alloc(4 * tokens * ffn_dim)      # only used when several tokens run together
         self._up = self._alloc(4 * tokens * ffn_dim)
         self._act = self._alloc(4 * tokens * ffn_dim)
@@ -72,13 +75,22 @@ class FFNSequenceRunner:
         st = hip.current_stream_handle()
         h, f = self.hidden, self.ffn_dim
         x, act = self._x.ptr + 4 * tok0 * h, self._act.ptr + 4 * tok0 * f
-        if self._norm is not None:
+        fused_norm = self._image is not None and count >= 2
+        if fused_norm:
+            # r = x + add, and rmsnorm(r) written straight as the activation image gate | up | SwiGLU read
+            quant.add_rmsnorm_pack_dev(x, self._add.ptr + 4 * tok0 * h, self._norm.ptr, self._res.ptr + 4 * tok0 * h, 0,
+                                       TensorType.Q4_K, self._image.ptr, h, count, self._eps, st)
+            quant.gemv_packed_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, self._image.ptr, act, h, f,
+                                         count, st)
+        elif self._norm is not None:
             normed = self._normed.ptr + 4 * tok0 * h
             quant.add_rmsnorm_dev(x, self._add.ptr + 4 * tok0 * h, self._norm.ptr, self._res.ptr + 4 * tok0 * h, normed, h,
                                   count, self._eps, st)
             x = normed
-        if count == 1 or f % 16 == 0:
-            # gate | up | SwiGLU in one launch (several tokens: per group of four on the matrix cores)
+        if fused_norm:
+            pass
+        elif count == 1 or f % 16 == 0:
+            # gate | up | SwiGLU in one launch (several tokens: one pass over both matrices per group of up to eight)
             quant.gemv_dual_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, x, act, h, f, count, st)
         else:
             g, u = self._gate.ptr + 4 * tok0 * f, self._up.ptr + 4 * tok0 * f

@@ -198,6 +198,22 @@ def add_rmsnorm_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_ptr, 
                                            ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
 
 
+def rmsnorm_pack_dev(x_ptr, norm_ptr, out_ptr, w_type, image_ptr, dim, tokens, eps=1.0e-6, stream=None):
+    """rmsnorm_dev that also writes the normalised rows as the one-pass GEMV's activation image (out_ptr may be 0)."""
+    _check(hip.lib().cogni_rmsnorm_pack_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(out_ptr),
+                                            ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr), ctypes.c_uint32(dim),
+                                            ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
+
+def add_rmsnorm_pack_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_ptr, w_type, image_ptr, dim, tokens, eps=1.0e-6,
+                         stream=None):
+    """add_rmsnorm_dev that also writes the normalised rows as the one-pass GEMV's activation image (normed_out_ptr may be 0)."""
+    _check(hip.lib().cogni_add_rmsnorm_pack_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(add_ptr), ctypes.c_uint64(norm_ptr),
+                                                ctypes.c_uint64(residual_out_ptr), ctypes.c_uint64(normed_out_ptr),
+                                                ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr), ctypes.c_uint32(dim),
+                                                ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
+
 def gemm_workspace_bytes(w_type, in_dim, tokens, out_dim=None):
     """Bytes of caller-owned scratch for gemm_dev: the packed activations, and with `out_dim` given also the planes of
     a k-split launch (few tiles), which gemm_dev uses when the workspace has room for them."""

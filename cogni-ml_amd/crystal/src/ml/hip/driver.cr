@@ -79,6 +79,11 @@ lib LibCogniHIP
                         stream : Void*) : Int32
   fun cogni_add_rmsnorm_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,
                             dim : UInt32, tokens : UInt32, eps : Float32, stream : Void*) : Int32
+  fun cogni_rmsnorm_pack_dev(x : UInt64, norm : UInt64, out : UInt64, w_type : UInt32, image : UInt64, dim : UInt32,
+                             tokens : UInt32, eps : Float32, stream : Void*) : Int32
+  fun cogni_add_rmsnorm_pack_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,
+                                 w_type : UInt32, image : UInt64, dim : UInt32, tokens : UInt32, eps : Float32,
+                                 stream : Void*) : Int32
   fun cogni_embed_dev(w_raw : UInt64, w_type : UInt32, token_ids : UInt64, output : UInt64, history : UInt64,
                       token_index : UInt32, hidden_dim : UInt32, vocab_size : UInt32, stream : Void*) : Int32
   fun cogni_gemv_top1_partials(w_type : UInt32, out_dim : UInt32) : UInt32

@@ -275,7 +275,8 @@ int cogni_quant_init(int32_t ordinal) {
   g_rt.image_slot_bytes = ((size_t)gemv_mt_image_bytes(COGNI_TYPE_Q6_K, GEMV_MT_MAX_IN_DIM) + 255) & ~(size_t)255;
   HIP_TRY(hipMalloc(&g_rt.image_pool, g_rt.image_slot_bytes * Runtime::kImageSlots), "hipMalloc(activation images)");
   for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q5_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32",
-                           "q4_k_gemv_mt_top1_partial_f32", "q6_k_gemv_mt_top1_partial_f32"}) {
+                           "q4_k_gemv_mt_top1_partial_f32", "q6_k_gemv_mt_top1_partial_f32", "rmsnorm_pack_q4k_f32",
+                           "rmsnorm_pack_q6k_f32", "add_rmsnorm_pack_q4k_f32", "add_rmsnorm_pack_q6k_f32"}) {
     hipFunction_t fn = nullptr;
     HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
     g_rt.fns.emplace(name, fn);
@@ -823,6 +824,31 @@ int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t resi
   if (tokens == 0) return 0;
   void* params[] = {&x, &add, &norm, &residual_out, &normed_out, &dim, &eps};
   return launch("add_rmsnorm_f32", tokens, 256, 0, params, stream);
+}
+
+// The norms with the activation image of the one-pass GEMV as a second output (norm.hpp): dim must be a shape those
+// kernels take with rows short enough for a thread to keep its values (a multiple of 2048 up to 4096).
+static int norm_pack_check(const char* who, uint32_t w_type, uint32_t dim, uint32_t tokens) {
+  if (!gemv_mt_supported(w_type, tokens < 2 ? 2 : (int)tokens, dim) || dim > 4096u || tokens == 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": needs 1..8 tokens of a row length the one-pass GEMV takes, up to 4096 "
+                                                               "(cogni_gemv_image_bytes) - got type " + type_name(w_type) + ", dim " +
+                                                std::to_string(dim) + ", " + std::to_string(tokens) + " tokens");
+  return 0;
+}
+int cogni_rmsnorm_pack_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t w_type, uint64_t image, uint32_t dim, uint32_t tokens,
+                           float eps, void* stream) {
+  if (!x || !norm || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_pack_dev: null device pointer");
+  if (int rc = norm_pack_check("cogni_rmsnorm_pack_dev", w_type, dim, tokens)) return rc;
+  void* params[] = {&x, &norm, &out, &image, &dim, &tokens, &eps};
+  return launch(w_type == COGNI_TYPE_Q6_K ? "rmsnorm_pack_q6k_f32" : "rmsnorm_pack_q4k_f32", GEMV_MT_MAX_TOKENS, 256, 0, params, stream);
+}
+int cogni_add_rmsnorm_pack_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t w_type,
+                               uint64_t image, uint32_t dim, uint32_t tokens, float eps, void* stream) {
+  if (!x || !add || !norm || !residual_out || !image)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_add_rmsnorm_pack_dev: null device pointer");
+  if (int rc = norm_pack_check("cogni_add_rmsnorm_pack_dev", w_type, dim, tokens)) return rc;
+  void* params[] = {&x, &add, &norm, &residual_out, &normed_out, &image, &dim, &tokens, &eps};
+  return launch(w_type == COGNI_TYPE_Q6_K ? "add_rmsnorm_pack_q6k_f32" : "add_rmsnorm_pack_q4k_f32", GEMV_MT_MAX_TOKENS, 256, 0, params, stream);
 }
 
 int g_gemm_threshold = -1;   // -1: not resolved yet

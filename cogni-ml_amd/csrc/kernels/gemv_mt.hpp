@@ -100,15 +100,9 @@ __device__ __forceinline__ MtPacked mt_pack4(float4 v) {
 // + part) are part (0 = hi, 1 = lo) of x[token][256 sb + 64 g + 32 par + 8 kg + (0,2,1,3,4,6,5,7)] * 2^e. Behind the
 // in_dim / 256 * 8 KiB of operands: [super-block][token pair][20 floats]: 2^-e of the pair's two tokens, two unused, the
 // eight sub-block sums of x (unscaled) of the first token, those of the second. Tokens at and above `tokens` are zero.
-extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
-                                                                    u32 tokens, u32 in_dim) {
-  const u32 lane = threadIdx.x & 63;
-  const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const u32 nsb = in_dim >> 8;
-  const u32 sb = unit >> 3, tok = unit & 7;
-  if (sb >= nsb) return;
-  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (tok < tokens) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+// One wavefront's share of the Q4_K image: (token slot tok, super-block sb) from the lane's four values v (elements
+// 4 lane .. 4 lane + 3 of the super-block; zeros and present = false for a token that is not there).
+__device__ __forceinline__ void mt_pack_store_q4k(uint8_t* __restrict__ image, u32 nsb, u32 sb, u32 tok, u32 lane, float4 v, bool present) {
   const MtPacked pk = mt_pack4(v);
   // element 4 l sits in instruction j = l / 8, k-group (l / 2) % 4, upper half of the lane's eight if l is odd
   const u32 j = lane >> 3, kg = (lane >> 1) & 3;
@@ -122,14 +116,9 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float*
   sm += MT_DPP(sm, MT_ROW_HALF_MIRROR);
   float* aux = reinterpret_cast<float*>(image + (size_t)nsb * 8192) + (size_t)(sb * 4 + (tok >> 1)) * 20;
   if ((lane & 7) == 0) aux[4 + 8 * (tok & 1) + (lane >> 3)] = sm;
-  if (lane == 0) aux[tok & 1] = tok < tokens ? pk.inv : 0.0f;
+  if (lane == 0) aux[tok & 1] = present ? pk.inv : 0.0f;
 }
-
-// Q6_K image: [super-block][sub-block pair p][lane = 16 kg + row][2 x 4 halves]: the halves of lane (kg, row = 2 token +
-// part) for sub-block s = 2 p + (0 | 1) are part of x[token][256 sb + 16 s + 4 kg + (0,2,1,3)] * 2^e. Behind the operands:
-// [super-block][token pair][36 floats]: 2^-e of the two tokens, two unused, the sixteen sub-block sums of x of the first
-// token, those of the second.
-extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q6k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
+extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
                                                                     u32 tokens, u32 in_dim) {
   const u32 lane = threadIdx.x & 63;
   const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -138,6 +127,14 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q6k_f16(const float*
   if (sb >= nsb) return;
   float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
   if (tok < tokens) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  mt_pack_store_q4k(image, nsb, sb, tok, lane, v, tok < tokens);
+}
+
+// Q6_K image: [super-block][sub-block pair p][lane = 16 kg + row][2 x 4 halves]: the halves of lane (kg, row = 2 token +
+// part) for sub-block s = 2 p + (0 | 1) are part of x[token][256 sb + 16 s + 4 kg + (0,2,1,3)] * 2^e. Behind the operands:
+// [super-block][token pair][36 floats]: 2^-e of the two tokens, two unused, the sixteen sub-block sums of x of the first
+// token, those of the second.
+__device__ __forceinline__ void mt_pack_store_q6k(uint8_t* __restrict__ image, u32 nsb, u32 sb, u32 tok, u32 lane, float4 v, bool present) {
   const MtPacked pk = mt_pack4(v);
   // element 4 l sits in sub-block s = l / 4, k-group l % 4
   const u32 s = lane >> 2, kg = lane & 3;
@@ -149,7 +146,18 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q6k_f16(const float*
   sm += MT_DPP(sm, MT_QUAD_2301);
   float* aux = reinterpret_cast<float*>(image + (size_t)nsb * 8192) + (size_t)(sb * 4 + (tok >> 1)) * 36;
   if ((lane & 3) == 0) aux[4 + 16 * (tok & 1) + s] = sm;
-  if (lane == 0) aux[tok & 1] = tok < tokens ? pk.inv : 0.0f;
+  if (lane == 0) aux[tok & 1] = present ? pk.inv : 0.0f;
+}
+extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q6k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
+                                                                    u32 tokens, u32 in_dim) {
+  const u32 lane = threadIdx.x & 63;
+  const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const u32 nsb = in_dim >> 8;
+  const u32 sb = unit >> 3, tok = unit & 7;
+  if (sb >= nsb) return;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tok < tokens) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  mt_pack_store_q6k(image, nsb, sb, tok, lane, v, tok < tokens);
 }
 
 // ---- loads in assembly ---------------------------------------------------------------------------------------------------

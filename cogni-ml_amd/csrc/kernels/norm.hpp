@@ -3,22 +3,41 @@
 // :906 add_rmsnorm_vec_parallel_probe, :1157 and :1324 their batched forms; CPU form src/ml/gguf/qwen35_cpu.cr:484-490).
 //   inv = 1 / sqrt(sum(x^2) / dim + eps);  out[i] = (x[i] * inv) * norm[i]
 // The add form first forms r = x + add, stores r (the residual stream) and normalises r.
+// The pack forms also write the normalised rows as the activation image of the one-pass multi-token GEMV (gemv_mt.hpp), so
+// that the projections behind a norm (q | k | v, gate | up) need no pack launch of their own: a thread of the short-row
+// path holds elements 4 (tid % 64) .. + 3 of super-block 4 k + tid / 64, which is exactly one wavefront per (token,
+// super-block) with the lane order of pack_x_mt_*, and the image comes out bit for bit as from that kernel.
 #pragma once
 #include "common.hpp"
+#include "gemv_mt.hpp"
 
 #define NORM_BLOCK 256
 #define NORM_KEEP 4   // float4 a thread keeps across the reduction on the short-row path
 
-template <bool ADD>
+// IMG: 0 = no image, 12 = the Q4_K (and Q5_K) image, 14 = the Q6_K image. With an image the grid is the image's eight token
+// slots, the workgroups of slots at and above `tokens` write the zeros of an absent token, dim is a multiple of 1024 up to
+// 4096 (the short-row path), and `out` may be null (the normalised rows then exist only as the image).
+template <bool ADD, int IMG = 0>
 __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __restrict__ add,
                                              const float* __restrict__ norm, float* residual_out,
-                                             float* __restrict__ out, u32 dim, float eps) {
+                                             float* __restrict__ out, u32 dim, float eps, uint8_t* __restrict__ image = nullptr,
+                                             u32 tokens = 0) {
   __shared__ float part[NORM_BLOCK / WAVE];
+  if constexpr (IMG != 0) {
+    if (blockIdx.x >= tokens) {
+      const u32 lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+      for (u32 sb = wave; sb < (dim >> 8); sb += NORM_BLOCK / WAVE) {
+        if constexpr (IMG == 14) mt_pack_store_q6k(image, dim >> 8, sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
+        else mt_pack_store_q4k(image, dim >> 8, sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
+      }
+      return;
+    }
+  }
   const u64 base = (u64)blockIdx.x * dim;
   const float* xt = x + base;
   const float* at = ADD ? add + base : nullptr;
   float* rt = ADD ? residual_out + base : nullptr;
-  float* ot = out + base;
+  float* ot = out ? out + base : nullptr;
   const float* st = ADD ? rt : xt;   // second pass: the sum this thread stored (residual_out may be x itself)
   const u32 tid = threadIdx.x;
   const bool vec = (dim & 3u) == 0;   // rows then start 16-byte aligned when the buffers do
@@ -56,11 +75,19 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
       if (i < dim) {
         float4 o;
         o.x = (v[k].x * inv) * w[k].x, o.y = (v[k].y * inv) * w[k].y, o.z = (v[k].z * inv) * w[k].z, o.w = (v[k].w * inv) * w[k].w;
-        *reinterpret_cast<float4*>(ot + i) = o;
+        if (IMG == 0 || out) *reinterpret_cast<float4*>(ot + i) = o;
+        if constexpr (IMG != 0) {
+          // (i < dim holds for whole wavefronts: dim is a multiple of 1024)
+          const u32 sb = 4u * (u32)k + (tid >> 6);
+          if constexpr (IMG == 14) mt_pack_store_q6k(image, dim >> 8, sb, blockIdx.x, tid & 63, o, true);
+          else mt_pack_store_q4k(image, dim >> 8, sb, blockIdx.x, tid & 63, o, true);
+        }
       }
     }
     return;
   }
+  static_assert(IMG == 0 || IMG == 12 || IMG == 14, "image kinds");
+  if constexpr (IMG != 0) return;   // (the host launches the pack forms for the short-row shapes only)
   if (vec) {
     for (u32 i = tid * 4; i < dim; i += NORM_BLOCK * 4) {
       float4 v = *reinterpret_cast<const float4*>(xt + i);
@@ -117,3 +144,21 @@ extern "C" __global__ __launch_bounds__(NORM_BLOCK) void add_rmsnorm_f32(const f
                                                                          float eps) {
   rmsnorm_core<true>(x, add, norm, residual_out, normed_out, dim, eps);
 }
+
+// The same with the normalised rows written as the activation image of the one-pass GEMV as well:
+//   rmsnorm_pack_q4k_f32 | rmsnorm_pack_q6k_f32 (x, norm, out | null, image, dim, tokens, eps)
+//   add_rmsnorm_pack_q4k_f32 | add_rmsnorm_pack_q6k_f32 (x, add, norm, residual_out, normed_out | null, image, dim, tokens, eps)
+// grid.x = 8 (the image's token slots; x, add and the outputs hold `tokens` rows), block 256, dim a multiple of 2048 up
+// to 4096. The image is that of pack_x_mt_q4k_f16 | pack_x_mt_q6k_f16 on the normalised rows, bit for bit.
+#define NORM_PACK_ENTRIES(SFX, IMG)                                                                                          \
+  extern "C" __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_pack_##SFX##_f32(                                         \
+      const float* x, const float* norm, float* out, uint8_t* image, u32 dim, u32 tokens, float eps) {                       \
+    rmsnorm_core<false, IMG>(x, nullptr, norm, nullptr, out, dim, eps, image, tokens);                                       \
+  }                                                                                                                          \
+  extern "C" __global__ __launch_bounds__(NORM_BLOCK) void add_rmsnorm_pack_##SFX##_f32(                                     \
+      const float* x, const float* add, const float* norm, float* residual_out, float* normed_out, uint8_t* image, u32 dim,  \
+      u32 tokens, float eps) {                                                                                               \
+    rmsnorm_core<true, IMG>(x, add, norm, residual_out, normed_out, dim, eps, image, tokens);                                \
+  }
+NORM_PACK_ENTRIES(q4k, 12)
+NORM_PACK_ENTRIES(q6k, 14)

@@ -235,6 +235,21 @@ int cogni_rmsnorm_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t dim, uin
 int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t dim,
                           uint32_t tokens, float eps, void* stream);
 
+/* The two norms with a second output: the normalised rows as the activation image of the one-pass multi-token GEMV
+ * (cogni_gemv_pack_dev below), so that the projections behind a norm (q | k | v, gate | up of a decoder layer) go straight
+ * to cogni_gemv_packed_dev / cogni_gemv_packed_swiglu_dev without a pack launch. `image` holds cogni_gemv_image_bytes(w_type,
+ * dim, tokens) bytes and comes out bit for bit as cogni_gemv_pack_dev writes it from the normalised rows; out / normed_out
+ * may be 0 (the normalised rows then exist only as the image). tokens in 1..8; dim a row length the one-pass kernels take,
+ * up to 4096 (2048 or 4096); w_type names the image (Q4_K and Q5_K share one, Q6_K has its own). Kernels
+ * "rmsnorm_pack_q4k_f32" | "rmsnorm_pack_q6k_f32" (x, norm, out, image, dim:u32, tokens:u32, eps:f32) and
+ * "add_rmsnorm_pack_q4k_f32" | "add_rmsnorm_pack_q6k_f32" (x, add, norm, residual_out, normed_out, image, dim:u32, tokens:u32,
+ * eps:f32), block 256, grid 8 (the image's token slots). No counterpart in the reference, whose multi-token kernels read
+ * fp32 activations (src/ml/cuda/kernels/q4k_gemv_probe.ptx:437-768). */
+int cogni_rmsnorm_pack_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t w_type, uint64_t image, uint32_t dim, uint32_t tokens,
+                           float eps, void* stream);
+int cogni_add_rmsnorm_pack_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t w_type,
+                               uint64_t image, uint32_t dim, uint32_t tokens, float eps, void* stream);
+
 /* One row of a Q4_K or Q6_K embedding matrix chosen by a token id that lives on the device: output[0..hidden_dim) =
  * dequantized row token_ids[0] (zeros if the id is not below vocab_size) and history[token_index] = token_ids[0].
  * Kernel "embed_<prefix>_f32_from_token_id" (w_raw, token_ids:u32*, output, history:u32*, token_index:u32,

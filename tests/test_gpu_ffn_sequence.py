@@ -48,11 +48,12 @@ def test_ffn_sequence_matches_cpu_form(gpu, oracle, hidden, ffn_dim, tokens, res
         stream.close()
 
 
-@pytest.mark.parametrize("tokens", [1, 3])
-def test_ffn_half_of_a_layer(gpu, oracle, tokens):
-    """r = x + attn_out; h = rmsnorm(r); out = r + down(silu(gate h) * up h) - src/ml/gguf/qwen35_cpu.cr:1705-1725."""
-    hidden, ffn_dim = 1024, 1536
-    rng = np.random.default_rng(77 + tokens)
+@pytest.mark.parametrize("hidden,ffn_dim,tokens", [(1024, 1536, 1), (1024, 1536, 3), (2048, 2304, 5), (4096, 1024, 8),
+                                                   (2048, 512, 11)])
+def test_ffn_half_of_a_layer(gpu, oracle, hidden, ffn_dim, tokens):
+    """r = x + attn_out; h = rmsnorm(r); out = r + down(silu(gate h) * up h) - src/ml/gguf/qwen35_cpu.cr:1705-1725.
+    With 2048 or 4096 hidden values and several tokens the norm writes the activation image of gate | up itself."""
+    rng = np.random.default_rng(77 + tokens + hidden)
     gate_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
     up_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
     down_raw = synth.make_weights(rng, Q6_K, hidden, ffn_dim)

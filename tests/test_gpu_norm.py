@@ -45,3 +45,61 @@ def test_rmsnorm_argument_errors(gpu):
     with pytest.raises(quant.QuantError, match="null device pointer"):
         quant.add_rmsnorm_dev(1, 0, 1, 1, 1, 16, 1)
     quant.rmsnorm_dev(1, 1, 1, 16, 0)       # no tokens: nothing is launched
+
+
+@pytest.mark.parametrize("w_type", [12, 13, 14])
+@pytest.mark.parametrize("dim,tokens", [(4096, 8), (4096, 3), (2048, 1), (2048, 6)])
+def test_norms_that_also_write_the_activation_image(gpu, w_type, dim, tokens):
+    """rmsnorm_pack / add_rmsnorm_pack: the normalised rows and residual stream of the plain kernels, bit for bit, and the
+    image cogni_gemv_pack_dev writes from those rows, byte for byte (absent tokens' slots zeroed; the image buffer starts as
+    garbage). With the fp32 output left out the image is the same."""
+    rng = np.random.default_rng(dim + 17 * tokens + w_type)
+    x = (rng.standard_normal(tokens * dim) * 2.5).astype(np.float32)
+    x[:300] *= np.float32(1e-20)                                   # a super-block far below the binary16 range
+    add = rng.standard_normal(tokens * dim).astype(np.float32)
+    w = (1.0 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    eps = 1.0e-6
+    nbytes = quant.gemv_image_bytes(w_type, dim, 8)
+    assert nbytes > 0
+    junk = rng.integers(0, 256, nbytes, dtype=np.uint8)
+    xd, ad, wd = DevArray(x), DevArray(add), DevArray(w)
+    od, rd, nd, od2, rd2 = (DevArray(nbytes=x.nbytes) for _ in range(5))
+    img_ref, img = DevArray(junk), DevArray(junk)
+    try:
+        for with_add in (False, True):
+            if with_add:
+                quant.add_rmsnorm_dev(xd.ptr, ad.ptr, wd.ptr, rd.ptr, nd.ptr, dim, tokens, eps)
+                quant.add_rmsnorm_pack_dev(xd.ptr, ad.ptr, wd.ptr, rd2.ptr, od2.ptr, w_type, img.ptr, dim, tokens, eps)
+                assert np.array_equal(rd2.read(np.float32, x.size), rd.read(np.float32, x.size))
+            else:
+                quant.rmsnorm_dev(xd.ptr, wd.ptr, nd.ptr, dim, tokens, eps)
+                quant.rmsnorm_pack_dev(xd.ptr, wd.ptr, od2.ptr, w_type, img.ptr, dim, tokens, eps)
+            assert np.array_equal(od2.read(np.float32, x.size), nd.read(np.float32, x.size))
+            if tokens >= 2:       # (the pack kernel itself starts at two tokens)
+                quant.gemv_pack_dev(nd.ptr, w_type, dim, tokens, img_ref.ptr)
+                assert np.array_equal(img.read(np.uint8, nbytes), img_ref.read(np.uint8, nbytes))
+            first = img.read(np.uint8, nbytes).copy()
+            # without the fp32 rows
+            hip_junk = DevArray(junk)
+            if with_add:
+                quant.add_rmsnorm_pack_dev(xd.ptr, ad.ptr, wd.ptr, rd2.ptr, 0, w_type, hip_junk.ptr, dim, tokens, eps)
+            else:
+                quant.rmsnorm_pack_dev(xd.ptr, wd.ptr, 0, w_type, hip_junk.ptr, dim, tokens, eps)
+            assert np.array_equal(hip_junk.read(np.uint8, nbytes), first)
+            hip_junk.close()
+    finally:
+        for d in (xd, ad, wd, od, rd, nd, od2, rd2, img_ref, img):
+            d.close()
+
+
+def test_norm_pack_argument_errors(gpu):
+    with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
+        quant.rmsnorm_pack_dev(1, 1, 1, 12, 1, 1024, 4)            # no one-pass kernel for rows of 1024
+    with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
+        quant.rmsnorm_pack_dev(1, 1, 1, 12, 1, 6144, 4)            # longer than a thread keeps
+    with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
+        quant.add_rmsnorm_pack_dev(1, 1, 1, 1, 1, 8, 1, 4096, 4)   # Q8_0 has no image
+    with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
+        quant.rmsnorm_pack_dev(1, 1, 1, 14, 1, 4096, 9)
+    with pytest.raises(quant.QuantError, match="null device pointer"):
+        quant.add_rmsnorm_pack_dev(1, 1, 1, 0, 1, 12, 1, 4096, 4)
