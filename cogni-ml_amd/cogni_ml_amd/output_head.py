@@ -40,6 +40,10 @@ class QwenOutputHeadRunner:
         self._top1_ids = self._alloc(4 * tokens)
         self._top1_values = self._alloc(4 * tokens)
         self._logits = self._alloc(4 * tokens * self.vocab) if read_logits else None
+        # token groups that go through the one-pass kernel: the norm writes that kernel's activation image itself
+        t = weights.output_type
+        self._from = quant.gemv_one_pass_from(t, self.hidden, self.vocab) if int(t) in (12, 14) and self.hidden <= 4096 else 0
+        self._image = self._alloc(quant.gemv_image_bytes(t, self.hidden, quant.MAX_GEMV_TOKENS)) if self._from else None
         self.top1_ids = np.zeros(tokens, dtype=np.int32)
         self.top1_values = np.zeros(tokens, dtype=np.float32)
         self.logits = None
@@ -71,10 +75,17 @@ class QwenOutputHeadRunner:
         st = hip.current_stream_handle()
         h, t = self.hidden, self.weights.output_type
         normed = self._normed.ptr + 4 * tok0 * h
-        quant.rmsnorm_dev(self._x.ptr + 4 * tok0 * h, self._norm.ptr, normed, h, count, self.eps, st)
-        quant.gemv_top1_dev(self._w.ptr, t, normed, self._partial_ids.ptr + 4 * tok0 * self._stride,
-                            self._partial_values.ptr + 4 * tok0 * self._stride, self._top1_ids.ptr + 4 * tok0,
-                            self._top1_values.ptr + 4 * tok0, h, self.vocab, count, st)
+        if self._from and count >= self._from:
+            quant.rmsnorm_pack_dev(self._x.ptr + 4 * tok0 * h, self._norm.ptr, normed if self._logits is not None else 0, t,
+                                   self._image.ptr, h, count, self.eps, st)
+            quant.gemv_packed_top1_dev(self._w.ptr, t, self._image.ptr, self._partial_ids.ptr + 4 * tok0 * self._stride,
+                                       self._partial_values.ptr + 4 * tok0 * self._stride, self._top1_ids.ptr + 4 * tok0,
+                                       self._top1_values.ptr + 4 * tok0, h, self.vocab, count, st)
+        else:
+            quant.rmsnorm_dev(self._x.ptr + 4 * tok0 * h, self._norm.ptr, normed, h, count, self.eps, st)
+            quant.gemv_top1_dev(self._w.ptr, t, normed, self._partial_ids.ptr + 4 * tok0 * self._stride,
+                                self._partial_values.ptr + 4 * tok0 * self._stride, self._top1_ids.ptr + 4 * tok0,
+                                self._top1_values.ptr + 4 * tok0, h, self.vocab, count, st)
         if self._logits is not None:
             quant.gemv_dev(self._w.ptr, t, normed, self._logits.ptr + 4 * tok0 * self.vocab, h, self.vocab, count, 0, st)
 

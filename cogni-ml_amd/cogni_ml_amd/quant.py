@@ -177,6 +177,15 @@ def gemv_top1_dev(w_ptr, w_type, x_ptr, partial_ids_ptr, partial_values_ptr, top
 TOP1_NOALLOC_MAX_PARTIALS = 65536
 
 
+def gemv_packed_top1_dev(w_ptr, w_type, image_ptr, partial_ids_ptr, partial_values_ptr, top1_ids_ptr, top1_values_ptr, in_dim, out_dim,
+                         tokens, stream=None):
+    """Top-1 of up to 8 tokens against a packed activation image (one pass over the weights, arg-max inside, reduce)."""
+    _check(hip.lib().cogni_gemv_packed_top1_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr),
+                                                ctypes.c_uint64(partial_ids_ptr), ctypes.c_uint64(partial_values_ptr),
+                                                ctypes.c_uint64(top1_ids_ptr), ctypes.c_uint64(top1_values_ptr),
+                                                ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
 def gemv_top1_noalloc_dev(w_ptr, w_type, x_ptr, top1_ids_ptr, top1_values_ptr, in_dim, out_dim, tokens=1, stream=None):
     """gemv_top1_dev with the partial results in the library's static device array: allocates nothing. Fails when
     tokens * gemv_top1_partials() exceeds TOP1_NOALLOC_MAX_PARTIALS; calls that overlap on one GPU race."""

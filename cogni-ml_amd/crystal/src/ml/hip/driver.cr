@@ -87,6 +87,9 @@ lib LibCogniHIP
   fun cogni_embed_dev(w_raw : UInt64, w_type : UInt32, token_ids : UInt64, output : UInt64, history : UInt64,
                       token_index : UInt32, hidden_dim : UInt32, vocab_size : UInt32, stream : Void*) : Int32
   fun cogni_gemv_top1_partials(w_type : UInt32, out_dim : UInt32) : UInt32
+  fun cogni_gemv_packed_top1_dev(w_raw : UInt64, w_type : UInt32, image : UInt64, partial_ids : UInt64, partial_values : UInt64,
+                                 top1_ids : UInt64, top1_values : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
+                                 stream : Void*) : Int32
   fun cogni_gemv_top1_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, partial_ids : UInt64, partial_values : UInt64,
                           top1_ids : UInt64, top1_values : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
                           stream : Void*) : Int32

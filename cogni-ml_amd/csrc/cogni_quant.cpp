@@ -808,6 +808,26 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
   return 0;
 }
 
+int cogni_gemv_packed_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t image, uint64_t partial_ids, uint64_t partial_values,
+                               uint64_t top1_ids, uint64_t top1_values, uint32_t in_dim, uint32_t out_dim, uint32_t tokens,
+                               void* stream) {
+  if (!w_raw || !image || !partial_ids || !partial_values || !top1_ids || !top1_values)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_top1_dev: null device pointer");
+  if (out_dim == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_top1_dev: zero dimension");
+  if ((w_type != COGNI_TYPE_Q4_K && w_type != COGNI_TYPE_Q6_K) || tokens == 0 || tokens > (uint32_t)GEMV_MT_MAX_TOKENS ||
+      !gemv_mt_supported(w_type, 2, in_dim))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_top1_dev: no one-pass top-1 kernel for this type, token count and in_dim");
+  uint32_t grid = gemv_mt_grid(w_type, in_dim, out_dim);
+  if (grid > cogni_gemv_top1_partials(w_type, out_dim))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_top1_dev: the partial buffers are sized by cogni_gemv_top1_partials");
+  void* params[] = {&w_raw, &image, &partial_ids, &partial_values, &in_dim, &out_dim, &tokens};
+  int rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt_top1_partial_f32" : "q4_k_gemv_mt_top1_partial_f32", grid,
+                  GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type), params, stream);
+  if (rc != 0) return rc;
+  void* rparams[] = {&partial_ids, &partial_values, &top1_ids, &top1_values, &grid};
+  return launch("top1_reduce_f32", tokens, 1024, 0, rparams, stream);
+}
+
 int cogni_rmsnorm_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t dim, uint32_t tokens, float eps, void* stream) {
   if (!x || !norm || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_dev: null device pointer");
   if (dim == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_dev: zero dimension");

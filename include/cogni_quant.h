@@ -280,6 +280,15 @@ int cogni_gemv_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t pa
                         uint64_t top1_ids, uint64_t top1_values, uint32_t in_dim, uint32_t out_dim, uint32_t tokens,
                         void* stream);
 
+/* The top-1 of up to 8 tokens against a caller-owned activation image (cogni_gemv_pack_dev, or the norms that write it:
+ * cogni_rmsnorm_pack_dev): what cogni_gemv_top1_dev launches behind its own pack - "q4_k_gemv_mt_top1_partial_f32" |
+ * "q6_k_gemv_mt_top1_partial_f32", then "top1_reduce_f32". Q4_K and Q6_K, in_dim a row length the one-pass kernels take,
+ * tokens in 1..8 (an image packed for one token is that token and seven zero slots). partial_ids / partial_values as for
+ * cogni_gemv_top1_dev. */
+int cogni_gemv_packed_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t image, uint64_t partial_ids, uint64_t partial_values,
+                               uint64_t top1_ids, uint64_t top1_values, uint32_t in_dim, uint32_t out_dim, uint32_t tokens,
+                               void* stream);
+
 /* cogni_gemv_top1_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): the same launches and the same results, with the per-workgroup partial
  * results in a static device array inside the library instead of caller-owned buffers. No counterpart in the

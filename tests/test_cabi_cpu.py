@@ -267,6 +267,14 @@ def test_one_pass_argument_errors_do_not_need_a_gpu():
         quant.gemv_packed_dev([0x1000, 0x1100], 12, 0x2000, [0x3000, 0x3100], [16, 0], 4096, 4)
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
         quant.gemv_packed_swiglu_dev(0x1000, 0x1100, 14, 0x2000, 0x3000, 4096, 16, 4)
+    with pytest.raises(quant.QuantError, match="no one-pass top-1 kernel"):
+        quant.gemv_packed_top1_dev(0x1000, 13, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 4096, 1000, 4)    # Q5_K: no top-1 form
+    with pytest.raises(quant.QuantError, match="no one-pass top-1 kernel"):
+        quant.gemv_packed_top1_dev(0x1000, 14, 0x2000, 0x3000, 0x4000, 0x5000, 0x6000, 4096, 1000, 9)
+    with pytest.raises(quant.QuantError, match="null device pointer"):
+        quant.gemv_packed_top1_dev(0x1000, 14, 0, 0x3000, 0x4000, 0x5000, 0x6000, 4096, 1000, 4)
+    with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
+        quant.rmsnorm_pack_dev(0x1000, 0x2000, 0, 12, 0x3000, 1024, 4)
     with pytest.raises(quant.QuantError, match="bad out_dim"):
         quant.gemv_packed_swiglu_dev(0x1000, 0x1100, 12, 0x2000, 0x3000, 4096, 0, 4)
 

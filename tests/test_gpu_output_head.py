@@ -135,9 +135,11 @@ def test_top1_in_one_pass(gpu, oracle, t, in_dim, out_dim, tokens):
     assert list(ids3) == [0] * tokens
 
 
-def test_output_head_runner(gpu, oracle):
-    hidden, vocab, tokens = 1024, 20011, 4
-    rng = np.random.default_rng(3)
+@pytest.mark.parametrize("hidden,vocab,tokens", [(1024, 20011, 4), (2048, 41003, 6), (4096, 3001, 8)])
+def test_output_head_runner(gpu, oracle, hidden, vocab, tokens):
+    """(1024 hidden values: the matrix-core kernel for the group of four; 2048 and 4096: the norm writes the activation image
+    and the group goes through the one-pass kernel with the arg-max inside.)"""
+    rng = np.random.default_rng(3 + hidden)
     w = Weights((1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32), synth.make_weights(rng, Q6_K, vocab, hidden),
                 Q6_K, hidden, vocab)
     xs = (rng.standard_normal(tokens * hidden) * 3).astype(np.float32)
@@ -156,7 +158,7 @@ def test_output_head_runner(gpu, oracle):
             assert runner.top1_ids[tok] == first_max(logits)
             assert abs(runner.top1_values[tok] - logits.max()) <= 1e-4 * np.abs(logits).max()
             dev = runner.logits[tok * vocab:(tok + 1) * vocab]
-            # (a group of four tokens: logits and top-1 both come from the matrix-core kernel, the same sums)
+            # (logits and top-1 of a group come from the same kernel family on the same operands: the same sums)
             assert runner.top1_ids[tok] == first_max(dev) and runner.top1_values[tok] == dev.max()
         # token-local path gives the same ids
         grouped = runner.top1_ids.copy()
