@@ -217,8 +217,9 @@ static inline unsigned gemv_mt_lds_bytes(unsigned type) {
   return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u +
          GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : (type == 13 ? 6u * 2816u : 6u * 2304u));
 }
-// bytes of the activation image: 8 KiB of operands per super-block, then per (super-block, token pair) the two scales and
-// the sub-block sums (Q4_K and Q5_K, which share one image, 20 floats; Q6_K 36)
+// bytes of the activation image: 8 KiB of operands per super-block, then the scales and the sub-block sums: Q4_K and Q5_K
+// (which share one image) 20 floats per (super-block, token pair), Q6_K 16 bytes per (super-block, lane) (its sums are one
+// more matrix-core operand)
 static inline unsigned long long gemv_mt_image_bytes(unsigned type, unsigned in_dim) {
-  return (unsigned long long)(in_dim >> 8) * (8192u + 4u * (type == 14 ? 144u : 80u));
+  return (unsigned long long)(in_dim >> 8) * (8192u + (type == 14 ? 1024u : 320u));
 }

@@ -68,7 +68,7 @@ typedef __attribute__((address_space(3))) void mt_lds_void;
 // weights, and 2^-e.
 struct MtPacked {
   mt_half4 hv, lv;
-  float inv;
+  float inv, scale;   // 2^-e and 2^e
 };
 __device__ __forceinline__ MtPacked mt_pack4(float4 v) {
   // power of two that brings the largest magnitude of the super-block to [2^12, 2^13) (unsigned maximum of the bit
@@ -86,6 +86,7 @@ __device__ __forceinline__ MtPacked mt_pack4(float4 v) {
   sh = sh < -100 ? -100 : sh;  // infinities and NaN: they stay what they are
   const float scale = __builtin_bit_cast(float, (u32)(127 + sh) << 23);
   MtPacked r;
+  r.scale = scale;
   r.inv = __builtin_bit_cast(float, (u32)(127 - sh) << 23);
   const _Float16 h0 = (_Float16)(v.x * scale), h1 = (_Float16)(v.y * scale), h2 = (_Float16)(v.z * scale), h3 = (_Float16)(v.w * scale);
   // (x * scale is exact, so fma(x, scale, -hi) is (x * scale) - hi in one instruction)
@@ -132,8 +133,9 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float*
 
 // Q6_K image: [super-block][sub-block pair p][lane = 16 kg + row][2 x 4 halves]: the halves of lane (kg, row = 2 token +
 // part) for sub-block s = 2 p + (0 | 1) are part of x[token][256 sb + 16 s + 4 kg + (0,2,1,3)] * 2^e. Behind the operands:
-// [super-block][token pair][36 floats]: 2^-e of the two tokens, two unused, the sixteen sub-block sums of x of the first
-// token, those of the second.
+// [super-block][lane = 16 kg + row][16 bytes]: four halves, part of sum(x[token] over sub-block 4 kg + (0,1,2,3)) * 2^(e-4)
+// (the sixteen sub-block sums as one more matrix-core operand: sixteen values of magnitude below 2^e-13 each stay in
+// binary16 range at 2^(e-4)), then 2^-e of tokens 2 kg and 2 kg + 1 (what result lane 16 kg + n needs).
 __device__ __forceinline__ void mt_pack_store_q6k(uint8_t* __restrict__ image, u32 nsb, u32 sb, u32 tok, u32 lane, float4 v, bool present) {
   const MtPacked pk = mt_pack4(v);
   // element 4 l sits in sub-block s = l / 4, k-group l % 4
@@ -141,12 +143,18 @@ __device__ __forceinline__ void mt_pack_store_q6k(uint8_t* __restrict__ image, u
   uint8_t* op = image + ((size_t)(sb * 8 + (s >> 1)) * 64 + kg * 16 + 2 * tok) * 16 + 8 * (s & 1);
   *reinterpret_cast<mt_half4*>(op) = pk.hv;
   *reinterpret_cast<mt_half4*>(op + 16) = pk.lv;
-  float sm = (v.x + v.y) + (v.z + v.w);   // sums of the sixteen sub-blocks (four lanes each), unscaled
+  float sm = (v.x + v.y) + (v.z + v.w);   // sums of the sixteen sub-blocks (four lanes each)
   sm += MT_DPP(sm, MT_QUAD_1032);
   sm += MT_DPP(sm, MT_QUAD_2301);
-  float* aux = reinterpret_cast<float*>(image + (size_t)nsb * 8192) + (size_t)(sb * 4 + (tok >> 1)) * 36;
-  if ((lane & 3) == 0) aux[4 + 16 * (tok & 1) + s] = sm;
-  if (lane == 0) aux[tok & 1] = present ? pk.inv : 0.0f;
+  const float s16 = pk.scale * 0.0625f;   // (powers of two: both products below are exact)
+  const _Float16 sh = (_Float16)(sm * s16), sl = (_Float16)fmaf(sm, s16, -(float)sh);
+  uint8_t* aux = image + (size_t)nsb * 8192 + (size_t)sb * 1024;
+  if ((lane & 3) == 0) {
+    _Float16* ap = reinterpret_cast<_Float16*>(aux + ((s >> 2) * 16 + 2 * tok) * 16) + (s & 3);
+    ap[0] = sh;   // row 2 tok (hi)
+    ap[8] = sl;   // row 2 tok + 1 (lo): the next lane's 16 bytes
+  }
+  if (lane < 16) reinterpret_cast<float*>(aux + ((tok >> 1) * 16 + lane) * 16)[2 + (tok & 1)] = present ? pk.inv : 0.0f;
 }
 extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q6k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
                                                                     u32 tokens, u32 in_dim) {
@@ -205,9 +213,11 @@ struct MtK45 {
   static constexpr unsigned TYPE = Q5 ? 13 : 12;
   static constexpr int BB = Q5 ? 176 : 144, P = BB / 16, NCOPY = 3, LAST = 16 * P - 128, NAUX = 5, NSLOT = 6, TMAX = 3;
   static constexpr int QOFF = Q5 ? 48 : 16;   // where qs starts in the block
-  static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_PAIR_BYTES = NAUX * 16;
+  static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 4 * NAUX * 16;
   // byte offset, inside the row's block, of the piece that goes to place `piece` of the row in LDS
   static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece * 16; }
+  // where a lane's scales and sums start inside a super-block's share of the image: per token pair
+  static __device__ __forceinline__ u32 aux_offset(u32 lane) { return (lane >> 4) * (NAUX * 16); }
 
   struct Aux { float fsc[2], sx[2][8]; };
   static __device__ __forceinline__ Aux aux(const mt_u32x4 (&r)[NAUX]) {
@@ -314,25 +324,22 @@ typedef MtK45<true> MtQ5K;
 // the row) and piece 14 repeats piece 13.
 struct MtQ6K {
   static constexpr unsigned TYPE = 14;
-  static constexpr int BB = 210, P = 15, NCOPY = 4, LAST = 48, NAUX = 9, NSLOT = 4, TMAX = 2;
-  static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_PAIR_BYTES = NAUX * 16;
+  static constexpr int BB = 210, P = 15, NCOPY = 4, LAST = 48, NAUX = 1, NSLOT = 4, TMAX = 2;
+  static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 64 * 16;
   static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece < 13 ? piece * 16 : 194u; }
+  static __device__ __forceinline__ u32 aux_offset(u32 lane) { return lane * 16; }   // 16 bytes of its own per lane
 
-  struct Aux { float fsc[2], sx[2][16]; };
+  // the scales of the lane's two tokens and, as the matrix-core operand of lane (kg, row), the sums of sub-blocks
+  // 4 kg .. 4 kg + 3 of that row's (token, part)
+  struct Aux { float fsc[2]; mt_u32x2 sums; };
   static __device__ __forceinline__ Aux aux(const mt_u32x4 (&r)[NAUX]) {
     Aux a;
-    a.fsc[0] = __uint_as_float(r[0].x), a.fsc[1] = __uint_as_float(r[0].y);
-#pragma unroll
-    for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const mt_u32x4 v = r[1 + 4 * tt + q];
-        a.sx[tt][4 * q] = __uint_as_float(v.x), a.sx[tt][4 * q + 1] = __uint_as_float(v.y);
-        a.sx[tt][4 * q + 2] = __uint_as_float(v.z), a.sx[tt][4 * q + 3] = __uint_as_float(v.w);
-      }
+    a.sums = (mt_u32x2){r[0].x, r[0].y};
+    a.fsc[0] = __uint_as_float(r[0].z), a.fsc[1] = __uint_as_float(r[0].w);
     return a;
   }
-  struct Raw { u32 a[4], b[4], h[4]; uint4 sc; u32 d; };   // [2 n + hh]: ql dword of quarters 0/2, of quarters 1/3, qh dword
+  // [2 n + hh]: ql dword of quarters 0/2, of quarters 1/3, qh dword; sck: the scale bytes of sub-blocks 4 kg .. 4 kg + 3
+  struct Raw { u32 a[4], b[4], h[4]; uint4 sc; u32 d, sck; };
   static __device__ __forceinline__ Raw read(const char* row, u32 kg) {
     Raw w;
 #pragma unroll
@@ -344,13 +351,14 @@ struct MtQ6K {
         w.h[2 * n + hh] = *reinterpret_cast<const u32*>(row + 128 + 32 * n + 16 * hh + 4 * kg);
       }
     w.sc = *reinterpret_cast<const uint4*>(row + 192);
+    w.sck = *reinterpret_cast<const u32*>(row + 192 + 4 * kg);
     w.d = *reinterpret_cast<const unsigned short*>(row + 222);
     return w;
   }
   static __device__ __forceinline__ float sbyte_f(u32 v, int k) { return (float)(int)(signed char)((v >> (8 * k)) & 0xFFu); }
   static __device__ __forceinline__ void unit(const Raw& w, const mt_u32x4 (&b)[8], const Aux& ax, float (&acc)[4]) {
     const u32 scw[4] = {w.sc.x, w.sc.y, w.sc.z, w.sc.w};
-    float lo[4] = {0.f, 0.f, 0.f, 0.f}, hi[4] = {0.f, 0.f, 0.f, 0.f}, mt0 = 0.f, mt1 = 0.f;
+    float lo[4] = {0.f, 0.f, 0.f, 0.f}, hi[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int n = 0; n < 2; n++) {
 #pragma unroll
@@ -376,19 +384,20 @@ struct MtQ6K {
             if (k >= 2) hi[e] = fmaf(sc, r[e], hi[e]);
             else lo[e] = fmaf(sc, r[e], lo[e]);
           }
-          mt0 = fmaf(sc, ax.sx[0][s], mt0);
-          mt1 = fmaf(sc, ax.sx[1][s], mt1);
         }
       }
     }
-    const float dd = h2f(w.d), d24 = dd * MT_TWO_P24, d20 = dd * MT_TWO_P20;
+    // sum (q - 32) x = sum q x - 32 sum x: per sub-block that is sc * sum(x), sixteen of them: one more instruction, the
+    // sums (times 2^(e-4), hi and lo) against the scales as exact binary16 integers
+    const mt_half4 scb = {(_Float16)sbyte_f(w.sck, 0), (_Float16)sbyte_f(w.sck, 1), (_Float16)sbyte_f(w.sck, 2), (_Float16)sbyte_f(w.sck, 3)};
+    const mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), scb,
+                                                                (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    const float dd = h2f(w.d), d24 = dd * MT_TWO_P24, d20 = dd * MT_TWO_P20, d512 = dd * -512.0f;   // 32 * 2^4
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      const float in = fmaf(d24, lo[k], d20 * hi[k]);
+      const float in = fmaf(d24, lo[k], fmaf(d512, off[k], d20 * hi[k]));
       acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
     }
-    acc[0] = fmaf(-32.0f * dd, mt0, acc[0]);   // sum (q - 32) x = sum q x - 32 sum x, on the hi part only
-    acc[2] = fmaf(-32.0f * dd, mt1, acc[2]);
   }
 };
 
@@ -465,11 +474,11 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
   mt_u32x4 breg[NSETS][8], auxr[NSETS][F::NAUX];
   const uint8_t* aux = image + (size_t)nsb * 8192;
   // (uniform bases and two lane offsets: no address registers per load)
-  const u32 lane16 = lane * 16u, rg_off = rg * F::AUX_PAIR_BYTES;
+  const u32 lane16 = lane * 16u, rg_off = F::aux_offset(lane);
   auto issue_set = [&](int i, int set) {
     const u32 sb = wave + 8u * i;
     u64 ob = mt_sbase(image + (size_t)sb * 8192), ob2 = mt_sbase(image + (size_t)sb * 8192 + 4096);
-    u64 ab = mt_sbase(aux + (size_t)sb * (4 * F::AUX_PAIR_BYTES));
+    u64 ab = mt_sbase(aux + (size_t)sb * F::AUX_SB_BYTES);
     mt_settle(ob, ob2, ab);
     mt_load16<0>(breg[set][0], ob, lane16);
     mt_load16<1024>(breg[set][1], ob, lane16);
@@ -480,17 +489,13 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
     mt_load16<2048>(breg[set][6], ob2, lane16);
     mt_load16<3072>(breg[set][7], ob2, lane16);
     mt_load16<0>(auxr[set][0], ab, rg_off);
-    mt_load16<16>(auxr[set][1], ab, rg_off);
-    mt_load16<32>(auxr[set][2], ab, rg_off);
-    mt_load16<48>(auxr[set][3], ab, rg_off);
-    mt_load16<64>(auxr[set][4], ab, rg_off);
-    if constexpr (F::NAUX > 5) {
-      mt_load16<80>(auxr[set][5], ab, rg_off);
-      mt_load16<96>(auxr[set][6], ab, rg_off);
-      mt_load16<112>(auxr[set][7], ab, rg_off);
-      mt_load16<128>(auxr[set][8], ab, rg_off);
+    if constexpr (F::NAUX > 1) {
+      mt_load16<16>(auxr[set][1], ab, rg_off);
+      mt_load16<32>(auxr[set][2], ab, rg_off);
+      mt_load16<48>(auxr[set][3], ab, rg_off);
+      mt_load16<64>(auxr[set][4], ab, rg_off);
     }
-    static_assert(F::NAUX == 5 || F::NAUX == 9, "scale and sum loads per operand set");
+    static_assert(F::NAUX == 1 || F::NAUX == 5, "scale and sum loads per operand set");
   };
   auto pin_set = [&](int set) {
 #pragma unroll

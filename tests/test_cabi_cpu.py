@@ -218,11 +218,11 @@ def test_runner_rejects_invalid_active_counts():
 
 def test_one_pass_geometry_and_thresholds():
     """Pack + one pass over the weights: which shapes have a kernel, the size of the activation image (8 KiB of operands
-    per super-block, then two scales and the sub-block sums per super-block and token pair), where gemv_dev switches to it,
+    per super-block, then the scales and the sub-block sums), where gemv_dev switches to it,
     and that the planned grid reaches every 16-row tile: a workgroup's eight wavefronts split the row, a row group is t
     tiles and the workgroups walk the groups with stride grid."""
     assert quant.gemv_image_bytes(12, 4096, 8) == 16 * (8192 + 4 * 80)
-    assert quant.gemv_image_bytes(14, 12288, 2) == 48 * (8192 + 4 * 144)
+    assert quant.gemv_image_bytes(14, 12288, 2) == 48 * (8192 + 1024)
     assert quant.gemv_image_bytes(13, 4096, 4) == quant.gemv_image_bytes(12, 4096, 4)      # Q5_K reads the Q4_K image
     for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1024, 4), (12, 14336, 4), (13, 1024, 4), (8, 4096, 4), (12, 0, 4)):
         assert quant.gemv_image_bytes(t, in_dim, tokens) == 0, (t, in_dim, tokens)
