@@ -185,7 +185,7 @@ static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned 
          in_dim <= GEMV_MT_MAX_IN_DIM;
 }
 // Token count from which one matrix goes through pack + one pass rather than the per-token-group kernels (0: never): where
-// the pair measures faster. Q6_K from three tokens; Q4_K and Q5_K from four on rows longer than 4096 values, else from five.
+// the pair measures faster. Q6_K from three tokens; Q4_K and Q5_K from four on rows of 4096 values and more, else from five.
 // Tall matrices of up to 4096 columns (an output head): the workgroups walk many row groups and pay their start once, which
 // puts the kernel ahead earlier - Q6_K from two tokens at GEMV_MT_TALL_ROWS rows, Q4_K and Q5_K from three there and from
 // two at GEMV_MT_VERY_TALL_ROWS.
@@ -194,7 +194,7 @@ static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned 
 static inline unsigned gemv_mt_from(unsigned type, unsigned in_dim, unsigned out_dim) {
   if (!gemv_mt_supported(type, 2, in_dim)) return 0;
   if (in_dim <= 4096u && out_dim >= GEMV_MT_TALL_ROWS) return (type == 14 || out_dim >= GEMV_MT_VERY_TALL_ROWS) ? 2u : 3u;
-  return type == 14 ? 3u : (in_dim > 4096u ? 4u : 5u);
+  return type == 14 ? 3u : (in_dim >= 4096u ? 4u : 5u);
 }
 // tiles per wavefront: rows of more than 4096 values one (the operands are streamed); else as many as keep 256 workgroups
 // busy, at most three (Q4_K) or two (Q6_K: its units are larger). Host and kernel use the same rule.
@@ -217,9 +217,9 @@ static inline unsigned gemv_mt_lds_bytes(unsigned type) {
   return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u +
          GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : (type == 13 ? 6u * 2816u : 6u * 2304u));
 }
-// bytes of the activation image: 8 KiB of operands per super-block, then the scales and the sub-block sums: Q4_K and Q5_K
-// (which share one image) 20 floats per (super-block, token pair), Q6_K 16 bytes per (super-block, lane) (its sums are one
-// more matrix-core operand)
+// bytes of the activation image: 8 KiB of operands per super-block, then 16 bytes per (super-block, lane) for the scales and
+// the sub-block sums (one more matrix-core operand). Q4_K and Q5_K share one image, Q6_K has its own.
 static inline unsigned long long gemv_mt_image_bytes(unsigned type, unsigned in_dim) {
-  return (unsigned long long)(in_dim >> 8) * (8192u + (type == 14 ? 1024u : 320u));
+  (void)type;
+  return (unsigned long long)(in_dim >> 8) * (8192u + 1024u);
 }

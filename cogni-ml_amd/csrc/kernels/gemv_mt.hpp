@@ -99,8 +99,10 @@ __device__ __forceinline__ MtPacked mt_pack4(float4 v) {
 
 // Q4_K image: [super-block][instruction j = 2 g + par][lane = 16 kg + row][8 halves]: the halves of lane (kg, row = 2 token
 // + part) are part (0 = hi, 1 = lo) of x[token][256 sb + 64 g + 32 par + 8 kg + (0,2,1,3,4,6,5,7)] * 2^e. Behind the
-// in_dim / 256 * 8 KiB of operands: [super-block][token pair][20 floats]: 2^-e of the pair's two tokens, two unused, the
-// eight sub-block sums of x (unscaled) of the first token, those of the second. Tokens at and above `tokens` are zero.
+// in_dim / 256 * 8 KiB of operands: [super-block][lane = 16 kg + row][16 bytes]: four halves, part of sum(x[token] over
+// sub-block 4 kg + (0,2,1,3)) * 2^(e-5) for kg < 2 and zeros for kg >= 2 (the eight sub-block sums as one more matrix-core
+// operand, in the order in which a masked dword of min bytes delivers them), then 2^-e of tokens 2 kg and 2 kg + 1 (what
+// result lane 16 kg + n needs). Tokens at and above `tokens` are zero.
 // One wavefront's share of the Q4_K image: (token slot tok, super-block sb) from the lane's four values v (elements
 // 4 lane .. 4 lane + 3 of the super-block; zeros and present = false for a token that is not there).
 __device__ __forceinline__ void mt_pack_store_q4k(uint8_t* __restrict__ image, u32 nsb, u32 sb, u32 tok, u32 lane, float4 v, bool present) {
@@ -110,14 +112,23 @@ __device__ __forceinline__ void mt_pack_store_q4k(uint8_t* __restrict__ image, u
   uint8_t* op = image + ((size_t)(sb * 8 + j) * 64 + kg * 16 + 2 * tok) * 16 + 8 * (lane & 1);
   *reinterpret_cast<mt_half4*>(op) = pk.hv;
   *reinterpret_cast<mt_half4*>(op + 16) = pk.lv;
-  // sums of the eight sub-blocks (eight lanes each), unscaled, for the min term
+  // sums of the eight sub-blocks (eight lanes each) for the min term
   float sm = (v.x + v.y) + (v.z + v.w);
   sm += MT_DPP(sm, MT_QUAD_1032);
   sm += MT_DPP(sm, MT_QUAD_2301);
   sm += MT_DPP(sm, MT_ROW_HALF_MIRROR);
-  float* aux = reinterpret_cast<float*>(image + (size_t)nsb * 8192) + (size_t)(sb * 4 + (tok >> 1)) * 20;
-  if ((lane & 7) == 0) aux[4 + 8 * (tok & 1) + (lane >> 3)] = sm;
-  if (lane == 0) aux[tok & 1] = present ? pk.inv : 0.0f;
+  const float s32 = pk.scale * 0.03125f;   // (powers of two: both products below are exact)
+  const _Float16 sh = (_Float16)(sm * s32), sl = (_Float16)fmaf(sm, s32, -(float)sh);
+  uint8_t* aux = image + (size_t)nsb * 8192 + (size_t)sb * 1024;
+  if ((lane & 3) == 0) {
+    // lanes 8 j hold sub-block j: k-group j / 4, slot (0,2,1,3)[j % 4]; lanes 8 j + 4 write the zeros of k-groups 2, 3
+    const u32 sj = lane >> 3, zero = (lane >> 2) & 1;
+    const u32 slot = ((sj & 1) << 1) | ((sj >> 1) & 1);
+    _Float16* ap = reinterpret_cast<_Float16*>(aux + (((sj >> 2) + 2 * zero) * 16 + 2 * tok) * 16) + slot;
+    ap[0] = zero ? (_Float16)0.0f : sh;   // row 2 tok (hi)
+    ap[8] = zero ? (_Float16)0.0f : sl;   // row 2 tok + 1 (lo): the next lane's 16 bytes
+  }
+  if (lane < 16) reinterpret_cast<float*>(aux + ((tok >> 1) * 16 + lane) * 16)[2 + (tok & 1)] = present ? pk.inv : 0.0f;
 }
 extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
                                                                     u32 tokens, u32 in_dim) {
@@ -211,31 +222,28 @@ __device__ __forceinline__ void mt_pin(mt_u32x4& v) { asm volatile("" : "+v"(v))
 template <bool Q5>
 struct MtK45 {
   static constexpr unsigned TYPE = Q5 ? 13 : 12;
-  static constexpr int BB = Q5 ? 176 : 144, P = BB / 16, NCOPY = 3, LAST = 16 * P - 128, NAUX = 5, NSLOT = 6, TMAX = 3;
+  static constexpr int BB = Q5 ? 176 : 144, P = BB / 16, NCOPY = 3, LAST = 16 * P - 128, NAUX = 1, NSLOT = 6, TMAX = 3;
   static constexpr int QOFF = Q5 ? 48 : 16;   // where qs starts in the block
-  static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 4 * NAUX * 16;
+  static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 64 * 16;
   // byte offset, inside the row's block, of the piece that goes to place `piece` of the row in LDS
   static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece * 16; }
-  // where a lane's scales and sums start inside a super-block's share of the image: per token pair
-  static __device__ __forceinline__ u32 aux_offset(u32 lane) { return (lane >> 4) * (NAUX * 16); }
+  // where a lane's scales and sums sit inside a super-block's share of the image: 16 bytes of its own per lane
+  static __device__ __forceinline__ u32 aux_offset(u32 lane) { return lane * 16; }
 
-  struct Aux { float fsc[2], sx[2][8]; };
+  // the scales of the lane's two tokens and, as the matrix-core operand of lane (kg, row), the sums of sub-blocks
+  // 4 kg + (0,2,1,3) of that row's (token, part) (zeros for kg >= 2)
+  struct Aux { float fsc[2]; mt_u32x2 sums; };
   static __device__ __forceinline__ Aux aux(const mt_u32x4 (&r)[NAUX]) {
     Aux a;
-    a.fsc[0] = __uint_as_float(r[0].x), a.fsc[1] = __uint_as_float(r[0].y);
-#pragma unroll
-    for (int tt = 0; tt < 2; tt++) {
-      const mt_u32x4 lo = r[1 + 2 * tt], hi = r[2 + 2 * tt];
-      a.sx[tt][0] = __uint_as_float(lo.x), a.sx[tt][1] = __uint_as_float(lo.y), a.sx[tt][2] = __uint_as_float(lo.z);
-      a.sx[tt][3] = __uint_as_float(lo.w), a.sx[tt][4] = __uint_as_float(hi.x), a.sx[tt][5] = __uint_as_float(hi.y);
-      a.sx[tt][6] = __uint_as_float(hi.z), a.sx[tt][7] = __uint_as_float(hi.w);
-    }
+    a.sums = (mt_u32x2){r[0].x, r[0].y};
+    a.fsc[0] = __uint_as_float(r[0].z), a.fsc[1] = __uint_as_float(r[0].w);
     return a;
   }
   // what a lane takes out of its row's block in LDS
-  struct Raw { uint4 hdr; uint2 q[4], h; };   // (h: the lane's eight qh bytes, Q5_K only)
+  struct Raw { uint4 hdr; uint2 q[4], h; u32 kg; };   // (h: the lane's eight qh bytes, Q5_K only; kg: the lane's k-group)
   static __device__ __forceinline__ Raw read(const char* row, u32 kg) {
     Raw w;
+    w.kg = kg;
     w.hdr = *reinterpret_cast<const uint4*>(row);
 #pragma unroll
     for (int g = 0; g < 4; g++) w.q[g] = *reinterpret_cast<const uint2*>(row + QOFF + 32 * g + 8 * kg);
@@ -285,12 +293,9 @@ struct MtK45 {
     const u32 mB = ((s2 >> 4) & 0x0F0F0F0Fu) | ((s1 >> 2) & 0x30303030u);
     const float sc[8] = {ubyte_f<0>(scA), ubyte_f<1>(scA), ubyte_f<2>(scA), ubyte_f<3>(scA),
                          ubyte_f<0>(scB), ubyte_f<1>(scB), ubyte_f<2>(scB), ubyte_f<3>(scB)};
-    const float mn[8] = {ubyte_f<0>(mA), ubyte_f<1>(mA), ubyte_f<2>(mA), ubyte_f<3>(mA),
-                         ubyte_f<0>(mB), ubyte_f<1>(mB), ubyte_f<2>(mB), ubyte_f<3>(mB)};
     const float dd = h2f(w.hdr.x), dmin = h2f(w.hdr.x >> 16);
-    // (c) sum_j sc_j * result_j, even sub-blocks (low nibbles, 2^-24) and odd ones (high nibbles, 2^-20) apart;
-    //     sum_j m_j * sum(x_j) for the two tokens of this lane
-    float ev[4] = {0.f, 0.f, 0.f, 0.f}, od[4] = {0.f, 0.f, 0.f, 0.f}, mt0 = 0.f, mt1 = 0.f;
+    // (c) sum_j sc_j * result_j, even sub-blocks (low nibbles, 2^-24) and odd ones (high nibbles, 2^-20) apart
+    float ev[4] = {0.f, 0.f, 0.f, 0.f}, od[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 8; j++) {
 #pragma unroll
@@ -298,17 +303,19 @@ struct MtK45 {
         if (j & 1) od[k] = fmaf(sc[j], dacc[j][k], od[k]);
         else ev[k] = fmaf(sc[j], dacc[j][k], ev[k]);
       }
-      mt0 = fmaf(mn[j], ax.sx[0][j], mt0);
-      mt1 = fmaf(mn[j], ax.sx[1][j], mt1);
     }
-    const float d24 = dd * MT_TWO_P24, d20 = dd * MT_TWO_P20;
+    // (d) sum_j m_j * sum(x_j): one more instruction, the eight sub-block sums (times 2^(e-5), hi and lo) against the min
+    //     bytes of k-groups 0 and 1 read as binary16 (m * 2^-24, in the order bytes 0, 2, 1, 3 of the masked dword)
+    const u32 msel = w.kg == 0 ? mA : (w.kg == 1 ? mB : 0u);
+    const mt_u32x2 mb = {msel & 0x00FF00FFu, (msel >> 8) & 0x00FF00FFu};
+    const mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), __builtin_bit_cast(mt_half4, mb),
+                                                                (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    const float d24 = dd * MT_TWO_P24, d20 = dd * MT_TWO_P20, dm29 = dmin * -536870912.0f;   // 2^24 * 2^5
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      const float in = fmaf(d24, ev[k], d20 * od[k]);
+      const float in = fmaf(d24, ev[k], fmaf(dm29, off[k], d20 * od[k]));
       acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
     }
-    acc[0] = fmaf(-dmin, mt0, acc[0]);   // the min term goes to the hi part only
-    acc[2] = fmaf(-dmin, mt1, acc[2]);
   }
 };
 typedef MtK45<false> MtQ4K;

@@ -110,7 +110,7 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 /* Decode GEMV, weights read once for all tokens:
  *   out[m*out_dim + o] = (residual ? residual[m*out_dim + o] : 0) + sum_j x[m*in_dim + j] * deq(W[o][j])
  * fp32 accumulation. tokens >= 1; several tokens of a matrix the one-pass kernel takes (see cogni_gemv_pack_dev below;
- * cogni_gemv_one_pass_from: Q6_K from three tokens, Q4_K and Q5_K from four on rows longer than 4096 values, else from
+ * cogni_gemv_one_pass_from: Q6_K from three tokens, Q4_K and Q5_K from four on rows of 4096 values and more, else from
  * five, tall matrices earlier) go in groups of up to 8 with
  * the weights read once per group; otherwise they are issued as consecutive launches of the token count that measures
  * fastest for the type and shape: up to 4 where cogni_gemv_plan picks the matrix-core kernel, else pairs for the
@@ -151,7 +151,7 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
  * time, and not beside eager calls on the capture stream. */
 size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 /* The token count from which cogni_gemv_dev and cogni_gemv_top1_dev take this path for one matrix (Q6_K 3; Q4_K and Q5_K 4
- * on rows longer than 4096 values, else 5; a tall matrix of up to 4096 columns - 40960 rows and more, an output head -
+ * on rows of 4096 values and more, else 5; a tall matrix of up to 4096 columns - 40960 rows and more, an output head -
  * earlier: Q6_K 2, Q4_K and Q5_K 3, and 2 from 98304 rows), 0 where they never do; below it the call runs the kernel
  * cogni_gemv_plan names. No GPU needed. */
 uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim, uint32_t out_dim);

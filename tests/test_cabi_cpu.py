@@ -221,17 +221,17 @@ def test_one_pass_geometry_and_thresholds():
     per super-block, then the scales and the sub-block sums), where gemv_dev switches to it,
     and that the planned grid reaches every 16-row tile: a workgroup's eight wavefronts split the row, a row group is t
     tiles and the workgroups walk the groups with stride grid."""
-    assert quant.gemv_image_bytes(12, 4096, 8) == 16 * (8192 + 4 * 80)
+    assert quant.gemv_image_bytes(12, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(14, 12288, 2) == 48 * (8192 + 1024)
     assert quant.gemv_image_bytes(13, 4096, 4) == quant.gemv_image_bytes(12, 4096, 4)      # Q5_K reads the Q4_K image
     for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1024, 4), (12, 14336, 4), (13, 1024, 4), (8, 4096, 4), (12, 0, 4)):
         assert quant.gemv_image_bytes(t, in_dim, tokens) == 0, (t, in_dim, tokens)
-    assert [quant.gemv_one_pass_from(12, d, 4096) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 5, 4, 4, 0, 0]
-    assert [quant.gemv_one_pass_from(13, d, 8192) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 5, 4, 4, 0, 0]
+    assert [quant.gemv_one_pass_from(12, d, 4096) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 0]
+    assert [quant.gemv_one_pass_from(13, d, 8192) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 0]
     assert [quant.gemv_one_pass_from(t, 4096, 12288) for t in (14, 8, 2)] == [3, 0, 0]
     # tall matrices of up to 4096 columns (an output head) take the path earlier
     assert [quant.gemv_one_pass_from(14, 4096, r) for r in (40959, 40960, 151936)] == [3, 2, 2]
-    assert [quant.gemv_one_pass_from(12, 4096, r) for r in (40959, 40960, 98303, 98304, 151936)] == [5, 3, 3, 2, 2]
+    assert [quant.gemv_one_pass_from(12, 4096, r) for r in (40959, 40960, 98303, 98304, 151936)] == [4, 3, 3, 2, 2]
     assert [quant.gemv_one_pass_from(13, 2048, r) for r in (40960, 98304)] == [3, 2]
     assert [quant.gemv_one_pass_from(t, 12288, 151936) for t in (12, 14)] == [4, 3] and quant.gemv_one_pass_from(12, 1024, 151936) == 0
     rng = np.random.default_rng(11)

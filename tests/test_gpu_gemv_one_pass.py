@@ -47,7 +47,7 @@ def test_five_to_eight_tokens_in_one_pass(gpu, oracle, in_dim, out_dim, tokens):
     partial tile, row counts that are not multiples of 16, more row groups than workgroups (24616 rows: the workgroups walk
     two groups each, refilling their slots), both super-block counts per k-slice; with and without residual."""
     print("case in_dim=%d out_dim=%d tokens=%d" % (in_dim, out_dim, tokens), flush=True)
-    assert quant.gemv_image_bytes(Q4_K, in_dim, tokens) == (in_dim // 256) * (8192 + 320)
+    assert quant.gemv_image_bytes(Q4_K, in_dim, tokens) == (in_dim // 256) * (8192 + 1024)
     rng = np.random.default_rng(in_dim * 13 + out_dim * 7 + tokens)
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
@@ -156,7 +156,7 @@ def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
         assert_bars(od.read(np.float32, tokens * out_dim), want, tol, tokens, out_dim, "%dx%d M=%d" % (in_dim, out_dim, tokens))
         for a in (w, xd, od):
             a.close()
-    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(Q5_K, 4096, 8) == 16 * (8192 + 320)
+    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(Q5_K, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(Q4_K, 14336, 8) == 0 and quant.gemv_image_bytes(Q6_K, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(Q4_K, 4096, 1) == 0 and quant.gemv_image_bytes(Q4_K, 4096, 9) == 0
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
@@ -178,7 +178,7 @@ def test_long_rows_and_q6_k_in_one_pass(gpu, oracle, type_id, in_dim, out_dim, t
     wavefront, partial tiles, more row groups than workgroups, odd Q6_K super-blocks (blocks that start 2 bytes off a 4-byte
     boundary)."""
     print("case type=%d in_dim=%d out_dim=%d tokens=%d" % (type_id, in_dim, out_dim, tokens), flush=True)
-    assert quant.gemv_image_bytes(type_id, in_dim, tokens) == (in_dim // 256) * (8192 + (1024 if type_id == Q6_K else 320))
+    assert quant.gemv_image_bytes(type_id, in_dim, tokens) == (in_dim // 256) * (8192 + 1024)
     rng = np.random.default_rng(type_id * 1000003 + in_dim * 13 + out_dim * 7 + tokens)
     raw = synth.make_weights(rng, type_id, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
