@@ -243,6 +243,21 @@ def gemm_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_p
                                     ctypes.c_size_t(workspace_bytes), stream))
 
 
+def gemm_pack_dev(x_ptr, w_type, in_dim, tokens, workspace_ptr, workspace_bytes, stream=None):
+    """The first half of gemm_dev: the activations as packed fp16 at the head of the workspace (shared by every projection of
+    one type family that reads them)."""
+    _check(hip.lib().cogni_gemm_pack_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim),
+                                         ctypes.c_uint32(tokens), ctypes.c_uint64(workspace_ptr), ctypes.c_size_t(workspace_bytes),
+                                         stream))
+
+
+def gemm_packed_dev(w_ptr, w_type, workspace_ptr, workspace_bytes, out_ptr, in_dim, out_dim, tokens, bias_ptr=0, stream=None):
+    """The second half of gemm_dev: one matrix against activations gemm_pack_dev has packed."""
+    _check(hip.lib().cogni_gemm_packed_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(workspace_ptr),
+                                           ctypes.c_size_t(workspace_bytes), ctypes.c_uint64(bias_ptr), ctypes.c_uint64(out_ptr),
+                                           ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
 def matmul_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_ptr=0, workspace_bytes=0, bias_ptr=0,
                stream=None):
     """The GEMV/GEMM router (tokens > threshold and Q4_K -> GEMM)."""

@@ -98,6 +98,10 @@ lib LibCogniHIP
   fun cogni_gemm_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, bias : UInt64, out : UInt64,
                      in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
                      workspace : UInt64, workspace_bytes : LibC::SizeT, stream : Void*) : Int32
+  fun cogni_gemm_pack_dev(x : UInt64, w_type : UInt32, in_dim : UInt32, tokens : UInt32,
+                          workspace : UInt64, workspace_bytes : LibC::SizeT, stream : Void*) : Int32
+  fun cogni_gemm_packed_dev(w_raw : UInt64, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT, bias : UInt64,
+                            out : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_matmul_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, bias : UInt64, out : UInt64,
                        in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
                        workspace : UInt64, workspace_bytes : LibC::SizeT, stream : Void*) : Int32

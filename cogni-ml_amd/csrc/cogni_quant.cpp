@@ -899,25 +899,46 @@ size_t cogni_gemm_workspace_bytes_split(uint32_t w_type, uint32_t in_dim, uint32
   return s == 1 ? pack : pack + (size_t)s * tokens * out_dim * sizeof(float);
 }
 
-int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
-                   uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream) {
+// The two halves of cogni_gemm_dev. `who` names the entry point in messages.
+static int gemm_check(const char* who, uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens, uint64_t workspace,
+                      size_t workspace_bytes) {
   if (!gemm_type(w_type))
     return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the prefill GEMM: ") + type_name(w_type));
-  if (!w_raw || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: null device pointer");
-  if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: zero dimension");
+  if (in_dim == 0 || out_dim == 0 || tokens == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": zero dimension");
   if ((in_dim % 256) != 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(type_name(w_type)) + " GEMM requires in_dim multiple of 256, got " + std::to_string(in_dim));
   if ((uint64_t)tokens * out_dim > 0xFFFFFFFFull)
-    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: tokens * out_dim exceeds 2^32 - 1");
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": tokens * out_dim exceeds 2^32 - 1");
   const size_t need = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
   if (!workspace || workspace_bytes < need)
-    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: workspace has " + std::to_string(workspace_bytes) + " bytes, needs " + std::to_string(need));
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": workspace has " + std::to_string(workspace_bytes) + " bytes, needs " + std::to_string(need));
+  return 0;
+}
+
+int cogni_gemm_pack_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes,
+                        void* stream) {
+  if (!x) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_pack_dev: null device pointer");
+  if (int rc = gemm_check("cogni_gemm_pack_dev", w_type, in_dim, 1, tokens, workspace, workspace_bytes)) return rc;
+  const uint32_t mtiles = (tokens + 127) / 128;
+  void* params[] = {&x, &workspace, &tokens, &in_dim};
+  // 8 tokens x one super-block per workgroup
+  return launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_f16_q6k" : "pack_x_f16_q4k", mtiles * 16 * (in_dim / 256), 256, 0, params, stream);
+}
+
+int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
+                   uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream) {
+  if (!w_raw || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_dev: null device pointer");
+  if (int rc = gemm_check("cogni_gemm_dev", w_type, in_dim, out_dim, tokens, workspace, workspace_bytes)) return rc;
+  if (int rc = cogni_gemm_pack_dev(x, w_type, in_dim, tokens, workspace, workspace_bytes, stream)) return rc;
+  return cogni_gemm_packed_dev(w_raw, w_type, workspace, workspace_bytes, bias, out, in_dim, out_dim, tokens, stream);
+}
+
+int cogni_gemm_packed_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t bias, uint64_t out,
+                          uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (!w_raw || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_packed_dev: null device pointer");
+  if (int rc = gemm_check("cogni_gemm_packed_dev", w_type, in_dim, out_dim, tokens, workspace, workspace_bytes)) return rc;
+  const size_t need = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 191) / 192;
-  {
-    void* params[] = {&x, &workspace, &tokens, &in_dim};
-    int rc = launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_f16_q6k" : "pack_x_f16_q4k", mtiles * 16 * (in_dim / 256), 256, 0, params, stream);   // 8 tokens x one super-block per workgroup
-    if (rc != 0) return rc;
-  }
   // a workspace that holds the packed activations only: one workgroup per tile walks the whole row
   uint32_t splits = gemm_splits(in_dim, out_dim, tokens);
   if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) splits = 1;

@@ -327,6 +327,17 @@ size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tok
  * workspace smaller than this, cogni_gemm_dev runs unsplit. No counterpart in the reference (its Metal GEMM does not
  * split k). */
 size_t cogni_gemm_workspace_bytes_split(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens);
+/* The two halves of cogni_gemm_dev for callers whose projections share their activations (q | k | v, gate | up of a layer:
+ * one pack, several GEMMs): cogni_gemm_pack_dev writes the packed fp16 activations to the head of the workspace
+ * (cogni_gemm_workspace_bytes; Q4_K and Q5_K share one layout, Q6_K has its own), cogni_gemm_packed_dev runs the GEMM of one
+ * matrix against them (the k-split planes, when the workspace has room for them, live behind the packed activations and
+ * are reused by every call - calls on one stream are ordered). cogni_gemm_dev is the two in a row. The counterpart of the
+ * packed activation image of the decode kernels (cogni_gemv_pack_dev); no counterpart in the reference, whose Metal GEMM
+ * converts x inside the kernel (gemm_q4k.metal:678-686). */
+int cogni_gemm_pack_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes,
+                        void* stream);
+int cogni_gemm_packed_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t bias, uint64_t out,
+                          uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
                    uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream);
 

@@ -117,6 +117,33 @@ def test_k_split_matches_unsplit(gpu, oracle, tokens, out_dim, in_dim, t):
     assert np.array_equal(run_gemm(raw, x, in_dim, out_dim, tokens, bias, t=t).reshape(tokens, out_dim), got)
 
 
+def test_projections_share_one_packed_activation_block(gpu, oracle):
+    """gemm_pack_dev once, then gemm_packed_dev for several matrices of one type family (Q4_K and Q5_K read the same packed
+    layout; a k-split and an unsplit shape, with and without bias): the bits of gemm_dev on each matrix alone."""
+    tokens, in_dim = 96, 2048
+    rng = np.random.default_rng(321)
+    x = synth.make_activations(rng, tokens, in_dim)
+    members = [(Q4_K, 1000, None), (Q5_K, 384, rng.standard_normal(384).astype(np.float32)), (Q4_K, 4096, None)]
+    raws = [synth.make_weights(rng, t, d, in_dim) for t, d, _ in members]
+    nbytes = max(quant.gemm_workspace_bytes(t, in_dim, tokens, d) for t, d, _ in members)
+    ws, xd = DevArray(nbytes=nbytes), DevArray(x)
+    quant.gemm_pack_dev(xd.ptr, Q4_K, in_dim, tokens, ws.ptr, nbytes)
+    for (t, d, bias), raw in zip(members, raws):
+        wd, od = DevArray(raw), DevArray(nbytes=4 * tokens * d)
+        bd = DevArray(bias) if bias is not None else None
+        quant.gemm_packed_dev(wd.ptr, t, ws.ptr, nbytes, od.ptr, in_dim, d, tokens, bd.ptr if bd else 0)
+        got = od.read(np.float32, tokens * d)
+        assert np.array_equal(got, run_gemm(raw, x, in_dim, d, tokens, bias, t=t)), (t, d)
+        for a_ in (wd, od) + ((bd,) if bd else ()):
+            a_.close()
+    with pytest.raises(quant.QuantError, match="workspace has 16 bytes"):
+        quant.gemm_pack_dev(xd.ptr, Q4_K, in_dim, tokens, ws.ptr, 16)
+    with pytest.raises(quant.QuantError, match="null device pointer"):
+        quant.gemm_packed_dev(0, Q4_K, ws.ptr, nbytes, xd.ptr, in_dim, 16, tokens)
+    for a_ in (ws, xd):
+        a_.close()
+
+
 def test_argument_checks(gpu):
     w, x, o = DevArray(nbytes=4096), DevArray(nbytes=4096), DevArray(nbytes=4096)
     with pytest.raises(quant.QuantError, match="Unsupported quant type for the prefill GEMM") as e:
