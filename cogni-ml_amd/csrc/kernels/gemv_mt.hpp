@@ -45,6 +45,13 @@
 #include "common.hpp"
 #include "gemv_config.h"
 
+// Register sets the streamed activation operands go through (rows above 4096 values). Three measure 2-4 % slower than two
+// at every such shape (Q6_K 4096x12288 15.66 -> 16.00 us, Q4_K 11.84 -> 12.04): the third set's loads stand in front of
+// weight copies.
+#ifndef GEMV_MT_STREAM_SETS
+#define GEMV_MT_STREAM_SETS 2
+#endif
+
 typedef _Float16 mt_half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 mt_half4 __attribute__((ext_vector_type(4)));
 typedef float mt_float4 __attribute__((ext_vector_type(4)));
@@ -419,15 +426,15 @@ struct MtArgs {
 // k-slice, NSLOT units in LDS). Issue order: set 0, unit 0, set 1, unit 1, units 2 .. min(S, NSLOT) - 1 up front; behind unit
 // i's arithmetic: set i + 2, then unit i + NSLOT. NA loads per set, NC copies per unit. The answer is the number of loads
 // issued, by the time of the wait, behind the later of the two.
-constexpr int mt_stream_wait(int S, int NSLOT, int NA, int NC, int i) {
+constexpr int mt_stream_wait(int S, int NSLOT, int NS, int NA, int NC, int i) {
   int pos = 0, end_set[8] = {}, end_unit[8] = {};
   const int up = S < NSLOT ? S : NSLOT;
   for (int u = 0; u < up; u++) {
-    if (u < 2) end_set[u] = (pos += NA);
+    if (u < NS) end_set[u] = (pos += NA);
     end_unit[u] = (pos += NC);
   }
   for (int j = 0; j < i; j++) {   // what was issued behind the units before i
-    if (j + 2 < S) end_set[j + 2] = (pos += NA);
+    if (j + NS < S) end_set[j + NS] = (pos += NA);
     if (j + NSLOT < S) end_unit[j + NSLOT] = (pos += NC);
   }
   const int need = end_set[i] > end_unit[i] ? end_set[i] : end_unit[i];
@@ -451,7 +458,8 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
   static_assert(!SWIGLU || T == (STREAM ? 1 : 2), "SWIGLU pairs a gate tile with an up tile");
   static_assert(!STREAM || T == 1, "streamed operands: one tile per wavefront");
   static_assert(STREAM || SBW * T <= F::NSLOT, "every unit of a row group has a slot");
-  constexpr int NSETS = STREAM ? 2 : SBW, NU = SBW * T, NA = 8 + F::NAUX, NC = F::NCOPY;
+  constexpr int NS = GEMV_MT_STREAM_SETS;   // register sets the streamed operands go through
+  constexpr int NSETS = STREAM ? NS : SBW, NU = SBW * T, NA = 8 + F::NAUX, NC = F::NCOPY;
   extern __shared__ uint4 mt_lds4[];
   char* lds = reinterpret_cast<char*>(mt_lds4);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -655,22 +663,22 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
       set_rows(grp, mat);
 #pragma unroll
       for (int u = 0; u < NSLOT; u++) {
-        if (u < 2) issue_set(u, u);
+        if (u < NS) issue_set(u, u);
         issue_unit(u, 0, u);
       }
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
       auto unit = [&](auto utag) {
         constexpr int i = decltype(utag)::value;
         __builtin_amdgcn_sched_barrier(0);
-        mt_wait<mt_stream_wait(S, NSLOT, NA, NC, i)>();
-        pin_set(i & 1);
-        const typename F::Aux ax = F::aux(auxr[i & 1]);
+        mt_wait<mt_stream_wait(S, NSLOT, NS, NA, NC, i)>();
+        pin_set(i % NS);
+        const typename F::Aux ax = F::aux(auxr[i % NS]);
         const typename F::Raw w = F::read(slots + (i % NSLOT) * F::UNIT_BYTES + ar * (F::P * 16), kg);
-        F::unit(w, breg[i & 1], ax, acc);
+        F::unit(w, breg[i % NS], ax, acc);
         asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
         __builtin_amdgcn_sched_barrier(0);
-        // the set and the slot are free: the operands two super-blocks on, and the unit NSLOT on
-        if constexpr (i + 2 < S) issue_set(i + 2, i & 1);
+        // the set and the slot are free: the operands NS super-blocks on, and the unit NSLOT on
+        if constexpr (i + NS < S) issue_set(i + NS, i % NS);
         if constexpr (i + NSLOT < S) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
           issue_unit(i + NSLOT, 0, i % NSLOT);
