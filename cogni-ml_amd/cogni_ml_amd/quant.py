@@ -243,6 +243,16 @@ def gemm_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_p
                                     ctypes.c_size_t(workspace_bytes), stream))
 
 
+def gemm_plan(w_type, in_dim, out_dim, tokens, workspace_bytes):
+    """(kernel name, grid_x, k splits, block) of the launch gemm_packed_dev makes for this shape and workspace size."""
+    name = ctypes.c_char_p()
+    gx, gy, bx = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+    _check(hip.lib().cogni_gemm_plan(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim),
+                                     ctypes.c_uint32(tokens), ctypes.c_size_t(workspace_bytes), ctypes.byref(name),
+                                     ctypes.byref(gx), ctypes.byref(gy), ctypes.byref(bx)))
+    return name.value.decode(), gx.value, gy.value, bx.value
+
+
 def gemm_pack_dev(x_ptr, w_type, in_dim, tokens, workspace_ptr, workspace_bytes, stream=None):
     """The first half of gemm_dev: the activations as packed fp16 at the head of the workspace (shared by every projection of
     one type family that reads them)."""

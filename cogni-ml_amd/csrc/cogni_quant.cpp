@@ -933,26 +933,56 @@ int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, u
   return cogni_gemm_packed_dev(w_raw, w_type, workspace, workspace_bytes, bias, out, in_dim, out_dim, tokens, stream);
 }
 
+// The launch cogni_gemm_packed_dev makes for a shape and a workspace size: kernel, grid (x = tiles rounded up to a multiple
+// of 8, y = k splits), block.
+struct GemmPlan {
+  const char* kernel;
+  uint32_t grid_x, splits, block;
+};
+static GemmPlan gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens, size_t workspace_bytes) {
+  const uint32_t mtiles = (tokens + 127) / 128;
+  GemmPlan p;
+  // a workspace that holds the packed activations only: one workgroup per tile walks the whole row
+  p.splits = gemm_splits(in_dim, out_dim, tokens);
+  if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) p.splits = 1;
+  const bool wide = w_type == COGNI_TYPE_Q4_K && p.splits == 1 && gemm_q4k_use_wide(out_dim, tokens);
+  p.kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : w_type == COGNI_TYPE_Q5_K ? "q5_k_gemm_f16" : wide ? "q4_k_gemm_wide_f16" : "q4_k_gemm_f16";
+  const uint32_t ntiles = wide ? (out_dim + 255) / 256 : (out_dim + 191) / 192;
+  p.grid_x = 8 * ((mtiles * ntiles + 7) / 8);
+  p.block = wide ? 512 : 256;
+  return p;
+}
+
+int cogni_gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens, size_t workspace_bytes, const char** kernel,
+                    uint32_t* grid_x, uint32_t* grid_y, uint32_t* block_x) {
+  if (!gemm_type(w_type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the prefill GEMM: ") + type_name(w_type));
+  if (in_dim == 0 || out_dim == 0 || tokens == 0 || (in_dim % 256) != 0)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_plan: zero dimension or in_dim not a multiple of 256");
+  const GemmPlan p = gemm_plan(w_type, in_dim, out_dim, tokens, workspace_bytes);
+  if (kernel) *kernel = p.kernel;
+  if (grid_x) *grid_x = p.grid_x;
+  if (grid_y) *grid_y = p.splits;
+  if (block_x) *block_x = p.block;
+  return 0;
+}
+
 int cogni_gemm_packed_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t bias, uint64_t out,
                           uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
   if (!w_raw || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_packed_dev: null device pointer");
   if (int rc = gemm_check("cogni_gemm_packed_dev", w_type, in_dim, out_dim, tokens, workspace, workspace_bytes)) return rc;
   const size_t need = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
-  const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 191) / 192;
-  // a workspace that holds the packed activations only: one workgroup per tile walks the whole row
-  uint32_t splits = gemm_splits(in_dim, out_dim, tokens);
-  if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) splits = 1;
-  const char* kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : w_type == COGNI_TYPE_Q5_K ? "q5_k_gemm_f16" : "q4_k_gemm_f16";
-  const uint32_t grid = 8 * ((mtiles * ntiles + 7) / 8);
+  const GemmPlan p = gemm_plan(w_type, in_dim, out_dim, tokens, workspace_bytes);
+  uint32_t splits = p.splits;
   if (splits == 1) {
     void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};
-    return launch(kernel, grid, 256, 0, params, stream);
+    return launch(p.kernel, p.grid_x, p.block, 0, params, stream);
   }
   uint64_t planes = workspace + need, none = 0;
   uint32_t total = tokens * out_dim;
   {
     void* params[] = {&w_raw, &workspace, &none, &planes, &in_dim, &out_dim, &tokens};
-    int rc = launch(kernel, grid, 256, 0, params, stream, splits);
+    int rc = launch(p.kernel, p.grid_x, p.block, 0, params, stream, splits);
     if (rc != 0) return rc;
   }
   void* params[] = {&planes, &bias, &out, &total, &out_dim, &splits};

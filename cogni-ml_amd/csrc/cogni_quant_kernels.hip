@@ -8,6 +8,7 @@
 #include "kernels/gemv_mfma_q6k.hpp"
 #include "kernels/gemv_mt.hpp"
 #include "kernels/gemm_q4k.hpp"
+#include "kernels/gemm_q4k_wide.hpp"
 #include "kernels/gemm_q6k.hpp"
 #include "kernels/norm.hpp"
 

@@ -257,8 +257,19 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   if (vt >= mtiles * ntiles) return;
   const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
   const size_t row_bytes = (size_t)nkb_all * BS;
-  const u32 sh = 16u * (g & 1);
-  const bool upper = g >= 2;
+  const u32 sh = 16u * kg;
+  // Unpacking the 6-bit (scale, min) pairs takes one of two forms by g >= 2, i.e. by kh, which is the same for a whole
+  // wavefront: written as a select it becomes a scalar branch that cuts the last k-step's scheduling region into
+  // pieces, so the two forms are folded into one through masks the compiler cannot see through.
+  u32 um = kh ? 0xFFFFFFFFu : 0u, mA = kh ? 0x0F0Fu : 0x3F3Fu, mB = kh ? 0x3030u : 0u, shM = kh ? 4u : 0u;
+  um = __builtin_amdgcn_readfirstlane(um);
+  mA = __builtin_amdgcn_readfirstlane(mA);
+  mB = __builtin_amdgcn_readfirstlane(mB);
+  shM = __builtin_amdgcn_readfirstlane(shM);
+  asm volatile("" : "+s"(um), "+s"(mA), "+s"(mB), "+s"(shM));
+  // the fp16 offsets live in registers so that (q & mask) | magic is one v_and_or_b32 (two literals would be two instructions)
+  u32 magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+  asm volatile("" : "+v"(magic_lo), "+v"(magic_hi));
 
   // Weight copies: piece p = 64 i + lane of the tile's super-block, i = wave, wave + 4, ... (27 copies of 64 pieces per
   // workgroup and super-block; every wavefront issues 7, the 28th repeats the last piece into spare LDS so that no
@@ -349,10 +360,11 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
 #pragma unroll
     for (int c = 0; c < 3; c++) {
       const float d = h2f(cur[c].hdr.x), dm = h2f(cur[c].hdr.x >> 16);
-      const u32 s0 = cur[c].hdr.y, s1 = cur[c].hdr.z, s2 = cur[c].hdr.w;
-      const u32 a0 = s0 >> sh, a1 = s1 >> sh, a2 = s2 >> sh;
-      const u32 scp = upper ? ((a2 & 0x0F0Fu) | ((a0 >> 2) & 0x3030u)) : (a0 & 0x3F3Fu);
-      const u32 mp = upper ? (((a2 >> 4) & 0x0F0Fu) | ((a1 >> 2) & 0x3030u)) : (a1 & 0x3F3Fu);
+      const u32 a0 = cur[c].hdr.y >> sh, a1 = cur[c].hdr.z >> sh, a2 = cur[c].hdr.w >> sh;
+      // kh = 0: a0 & 0x3F3F, a1 & 0x3F3F; kh = 1: (a2 & 0x0F0F) | ((a0 >> 2) & 0x3030), ((a2 >> 4) & 0x0F0F) | ((a1 >> 2) & 0x3030)
+      const u32 aS = (um & a2) | (~um & a0), aM = (um & a2) | (~um & a1);
+      const u32 scp = (aS & mA) | ((a0 >> 2) & mB);
+      const u32 mp = ((aM >> shM) & mA) | ((a1 >> 2) & mB);
       S[c][0] = h2_dup(d * ubyte_f<0>(scp));
       S[c][1] = h2_dup(-(dm * ubyte_f<0>(mp)));
       S[c][2] = h2_dup(d * ubyte_f<1>(scp));
@@ -366,7 +378,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       const uint4 Q = h ? cur[c].qb : cur[c].qa;
       const u32 qa = (op & 1) ? Q.z : Q.x, qb = (op & 1) ? Q.w : Q.y;
       const u32 mask = hi ? 0x00F000F0u : 0x000F000Fu;
-      const u32 magic = hi ? 0x54005400u : 0x64006400u;     // 64 + n (n sits 4 bits up) : 1024 + n
+      const u32 magic = hi ? magic_hi : magic_lo;           // 64 + n (n sits 4 bits up) : 1024 + n
       const u32 off = hi ? 0xD400D400u : 0xE400E400u;       // half2(-64) : half2(-1024)
       const u32 sc = S[c][2 * hi], nm = S[c][2 * hi + 1];
       uint4 bw;

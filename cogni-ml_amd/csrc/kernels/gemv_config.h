@@ -223,3 +223,19 @@ static inline unsigned long long gemv_mt_image_bytes(unsigned type, unsigned in_
   (void)type;
   return (unsigned long long)(in_dim >> 8) * (8192u + 1024u);
 }
+
+// ---- prefill GEMM: which Q4_K kernel an unsplit launch takes (gemm_q4k.hpp: 128 x 192 tiles, four wavefronts;
+// gemm_q4k_wide.hpp: 128 x 256 tiles, eight wavefronts). One workgroup per compute unit either way, so a launch runs in
+// rounds of 256 tiles. A round of wide tiles measures 1.24 times a round of the narrower ones (a third more work, done
+// with 25 % fewer activation bytes copied per flop and two wavefronts per SIMD), so the wide kernel is taken where it
+// saves enough whole rounds: 2048 x 12288 is 3 rounds instead of 4, 512 x 12288 (192 wide tiles: a quarter of the
+// compute units idle) and 1024 x 12288 (2 rounds either way) stay with the narrow tiles.
+#define GEMM_ROUND_TILES 256u
+#define GEMM_WIDE_ROUND_COST_X100 124u
+static inline int gemm_q4k_use_wide(unsigned out_dim, unsigned tokens) {
+  const unsigned mtiles = (tokens + 127u) / 128u;
+  const unsigned narrow = mtiles * ((out_dim + 191u) / 192u), wide = mtiles * ((out_dim + 255u) / 256u);
+  if (wide < GEMM_ROUND_TILES) return 0;
+  const unsigned rn = (narrow + GEMM_ROUND_TILES - 1) / GEMM_ROUND_TILES, rw = (wide + GEMM_ROUND_TILES - 1) / GEMM_ROUND_TILES;
+  return rw * GEMM_WIDE_ROUND_COST_X100 < rn * 100u;
+}

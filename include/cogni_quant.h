@@ -315,7 +315,9 @@ int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uin
  * cogni_gemm_workspace_bytes(...) bytes (x repacked as fp16, in the k order of the weight type); nothing is allocated.
  * Kernels: pack_x_f16_q4k (Q4_K and Q5_K) | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
  *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,
- *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/192)/8), no dynamic shared memory.
+ *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/192)/8), no dynamic shared memory; or, for Q4_K launches that fill
+ *          whole rounds of 128 x 256 tiles (cogni_gemm_plan says which), q4_k_gemm_wide_f16 (same arguments), block 512,
+ *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/256)/8).
  * (pack_x_f16_*: block 256, grid ceil(tokens/128)*16*(in_dim/256).) Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 /* The workspace size with which cogni_gemm_dev may also split the k range: a launch with fewer than 128 tiles of
@@ -340,6 +342,12 @@ int cogni_gemm_packed_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, s
                           uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
                    uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream);
+/* The launch cogni_gemm_packed_dev makes for a shape and a workspace of `workspace_bytes`: kernel name, grid (x: tiles,
+ * y: k splits; with y > 1 gemm_sum_splits_f32 follows) and block, for hosts that launch by name (level 1) and for
+ * callers who want to know which of the two Q4_K tilings a shape gets. Any out pointer may be null. The counterpart of
+ * cogni_gemv_plan; the reference picks its Metal prefill pipeline by type only (qwen35_metal.cr:11035). */
+int cogni_gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens, size_t workspace_bytes, const char** kernel,
+                    uint32_t* grid_x, uint32_t* grid_y, uint32_t* block_x);
 
 /* The router of the reference's GPU arm (Qwen35Metal.matmul, src/ml/gguf/qwen35_metal.cr:11404-11449):
  * tokens > threshold and a type with a GEMM kernel -> cogni_gemm_dev, else cogni_gemv_dev. The threshold

@@ -135,6 +135,29 @@ def test_gemv_plan_picks_the_kernel_for_the_shape():
         quant.gemv_plan(20, 1, 4096, 4096)
 
 
+def test_gemm_plan_picks_tile_and_split_for_the_shape():
+    blob = code_object()
+    for k in ("q4_k_gemm_f16", "q4_k_gemm_wide_f16", "q5_k_gemm_f16", "q6_k_gemm_f16", "gemm_sum_splits_f32", "pack_x_f16_q4k", "pack_x_f16_q6k"):
+        assert (k.encode() + b"\x00") in blob, k
+    big = 1 << 40
+    # 512 x 12288: 256 tiles of 128 x 192, one per compute unit; 192 wide tiles would leave a quarter of them idle
+    assert quant.gemm_plan(12, 4096, 12288, 512, big) == ("q4_k_gemm_f16", 256, 1, 256)
+    # 2048 x 12288: 768 wide tiles are three rounds of 256 where the narrow ones need four
+    assert quant.gemm_plan(12, 4096, 12288, 2048, big) == ("q4_k_gemm_wide_f16", 768, 1, 512)
+    assert quant.gemm_plan(12, 4096, 12288, 1024, big) == ("q4_k_gemm_f16", 512, 1, 256)       # two rounds either way
+    assert quant.gemm_plan(12, 4096, 12288, 4096, big) == ("q4_k_gemm_wide_f16", 1536, 1, 512)  # 6 rounds instead of 8
+    # few tiles: the k range is split when the workspace has room for the planes, else not
+    name, gx, gy, block = quant.gemm_plan(12, 4096, 12288, 64, big)
+    assert (name, gx, block) == ("q4_k_gemm_f16", 64, 256) and gy == 4
+    assert quant.gemm_plan(12, 4096, 12288, 64, quant.gemm_workspace_bytes(12, 4096, 64)) == ("q4_k_gemm_f16", 64, 1, 256)
+    # the other types have one tiling
+    assert quant.gemm_plan(13, 4096, 12288, 2048, big)[0] == "q5_k_gemm_f16" and quant.gemm_plan(14, 4096, 12288, 2048, big)[0] == "q6_k_gemm_f16"
+    with pytest.raises(quant.QuantError, match="Unsupported quant type"):
+        quant.gemm_plan(8, 4096, 12288, 512, big)
+    with pytest.raises(quant.QuantError, match="multiple of 256"):
+        quant.gemm_plan(12, 100, 12288, 512, big)
+
+
 def test_argument_errors_do_not_need_a_gpu():
     import numpy as np
     x = np.zeros(256, dtype=np.float32)

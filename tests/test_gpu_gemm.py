@@ -117,6 +117,30 @@ def test_k_split_matches_unsplit(gpu, oracle, tokens, out_dim, in_dim, t):
     assert np.array_equal(run_gemm(raw, x, in_dim, out_dim, tokens, bias, t=t).reshape(tokens, out_dim), got)
 
 
+@pytest.mark.parametrize("tokens,out_dim,in_dim,with_bias", [(128, 65536, 256, False), (130, 65301, 768, True), (100, 65536, 512, False)])
+def test_wide_tiles(gpu, oracle, tokens, out_dim, in_dim, with_bias):
+    """Launches of whole rounds of 128 x 256 tiles go to the eight-wavefront kernel: a clipped last tile with an out_dim that
+    is no multiple of 4, an odd number of super-blocks, a partial token tile and a bias, against the oracle on a sample of
+    tokens; and every output against the four-wavefront kernel's, which adds in the same order (bit for bit)."""
+    rng = np.random.default_rng(out_dim + tokens)
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    bias = rng.standard_normal(out_dim).astype(np.float32) if with_bias else None
+    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens, out_dim)
+    kernel, grid_x, splits, block = quant.gemm_plan(Q4_K, in_dim, out_dim, tokens, wsb)
+    mtiles = (tokens + 127) // 128
+    assert (kernel, splits, block) == ("q4_k_gemm_wide_f16", 1, 512) and grid_x == 8 * ((mtiles * ((out_dim + 255) // 256) + 7) // 8)
+    got = check(oracle, raw, x, in_dim, out_dim, tokens, bias, "wide M=%d N=%d K=%d" % (tokens, out_dim, in_dim),
+                sample_tokens=[0, 1, 31, 32, 63, 64, 97, tokens - 1])
+    # the same rows through the narrow kernel: 8192 rows at a time are fewer than a round of wide tiles
+    for r0 in (0, 8192 * 3, out_dim - 8192):
+        rows = slice(r0, r0 + 8192)
+        assert quant.gemm_plan(Q4_K, in_dim, 8192, tokens, 0)[0] == "q4_k_gemm_f16"
+        part = run_gemm(raw[r0 * (in_dim // 256) * 144:(r0 + 8192) * (in_dim // 256) * 144], x, in_dim, 8192, tokens,
+                        None if bias is None else bias[rows], split=False).reshape(tokens, 8192)
+        assert np.array_equal(part, got[:, rows]), r0
+
+
 def test_projections_share_one_packed_activation_block(gpu, oracle):
     """gemm_pack_dev once, then gemm_packed_dev for several matrices of one type family (Q4_K and Q5_K read the same packed
     layout; a k-split and an unsplit shape, with and without bias): the bits of gemm_dev on each matrix alone."""
