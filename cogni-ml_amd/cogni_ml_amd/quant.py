@@ -92,6 +92,20 @@ def gemv_one_pass_from(w_type, in_dim, out_dim):
     return int(f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim)))
 
 
+def gemv_image_stats():
+    """(slots, in use, pinned by a capture, multi-token calls that found no slot) of the library's activation images."""
+    a, b, c, d = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64()
+    _check(hip.lib().cogni_gemv_image_stats(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c), ctypes.byref(d)))
+    return a.value, b.value, c.value, d.value
+
+
+def gemv_passes(w_type, tokens, in_dim, out_dim):
+    """Passes over the weights gemv_dev makes for such a call (-1: refused)."""
+    f = hip.lib().cogni_gemv_passes
+    f.restype = ctypes.c_int32
+    return f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(tokens), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim))
+
+
 def gemv_image_bytes(w_type, in_dim, tokens):
     """Bytes of the activation image of the one-pass multi-token GEMV; 0 = no such kernel for the combination."""
     f = hip.lib().cogni_gemv_image_bytes

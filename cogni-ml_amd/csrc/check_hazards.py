@@ -5,7 +5,10 @@ emits itself but cannot keep for instructions written inside asm statements:
   * a vector instruction that writes a scalar register (v_readfirstlane_b32, v_readlane_b32, a compare with a scalar
     destination, a carry-out) must be five wait states ahead of a memory instruction that reads that register as its
     scalar base;
-  * a write of M0 must be one wait state ahead of a global load that writes to LDS.
+  * a write of M0 must be one wait state ahead of a global load that writes to LDS;
+  * in the kernels whose copies to LDS set M0 inside asm statements (names with "_mt_"), the compiler does not know
+    that M0 changes, so nothing may read a value of M0 that it assumes to have survived: every instruction that reads
+    M0 must have a write of M0 within the two instructions in front of it, with no label in between.
 
 An instruction is one wait state, "s_nop N" is N + 1. The scan is linear over each kernel of the disassembly (this
 library's own code object, made by llvm-objdump); labels do not reset it, so a sequence that is only adjacent in the
@@ -19,6 +22,21 @@ import sys
 
 VALU_SGPR_TO_VMEM = 5
 M0_TO_LDS_DMA = 1
+M0_WRITE_WITHIN = 2
+# instructions that read M0 without naming it
+M0_IMPLICIT = ("s_movrel", "v_movrel", "s_set_gpr_idx", "s_sendmsg", "ds_gws", "v_interp", "ds_read_addtid", "ds_write_addtid")
+
+
+def reads_m0(mnemonic, operands):
+    if "_lds_" in mnemonic or (is_vmem(mnemonic) and operands and operands[-1].strip().endswith("lds")):
+        return True
+    if mnemonic.startswith(M0_IMPLICIT):
+        return True
+    return any(o.strip() == "m0" for o in operands[1:])
+
+
+def asm_m0_kernel(name):
+    return "_mt_" in name
 # vector instructions whose second operand is a scalar destination (carry or scale flag)
 SDST_SECOND = ("v_mad_u64_u32", "v_mad_i64_i32", "v_add_co_u32", "v_sub_co_u32", "v_subrev_co_u32", "v_addc_co_u32",
                "v_subb_co_u32", "v_subbrev_co_u32", "v_div_scale_f32", "v_div_scale_f64")
@@ -61,6 +79,7 @@ def check(lines):
     kernel = "?"
     recent = []      # (wait states since, written sgprs, text) of recent vector-writes-scalar instructions
     m0_age = None    # wait states since the last write of m0
+    m0_dist = None   # instructions since the last write of m0 in this basic block
     for raw in lines:
         line = raw.split("//")[0].strip()
         if not line:
@@ -70,6 +89,7 @@ def check(lines):
             if not lab.group(1).startswith("L"):
                 kernel = lab.group(1)
                 recent, m0_age = [], None
+            m0_dist = None
             continue
         if line.endswith(":") or line.startswith((".", "Disassembly", "/")) or "file format" in line:
             continue
@@ -84,6 +104,11 @@ def check(lines):
                         kernel, line, sorted(used & regs), age, text, VALU_SGPR_TO_VMEM))
             if "_lds_" in mnemonic and m0_age is not None and m0_age < M0_TO_LDS_DMA:
                 problems.append("%s: '%s' %d wait state(s) after a write of m0 (needs %d)" % (kernel, line, m0_age, M0_TO_LDS_DMA))
+        if asm_m0_kernel(kernel) and reads_m0(mnemonic, operands) and (m0_dist is None or m0_dist > M0_WRITE_WITHIN):
+            problems.append("%s: '%s' reads m0 %s" % (kernel, line, "with no write of m0 in its basic block" if m0_dist is None else
+                                                      "%d instructions after the last write of m0 (at most %d)" % (m0_dist, M0_WRITE_WITHIN)))
+        if m0_dist is not None:
+            m0_dist += 1
         states = 1
         if mnemonic == "s_nop" and operands:
             states = int(operands[0], 0) + 1
@@ -95,6 +120,7 @@ def check(lines):
             recent.append((0, w, line))
         if mnemonic.startswith("s_") and operands and operands[0] == "m0":
             m0_age = 0
+            m0_dist = 0
     return problems
 
 

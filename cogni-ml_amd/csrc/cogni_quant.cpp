@@ -54,6 +54,8 @@ struct Runtime {
   size_t image_slot_bytes = 0;
   void* image_stream[kImageSlots] = {};
   bool image_used[kImageSlots] = {};
+  bool image_pinned[kImageSlots] = {};   // handed out under stream capture: a graph names it, it never changes hands
+  unsigned long long calls_without_image = 0;   // multi-token calls that found every slot taken and made several passes
 };
 Runtime g_rt;
 std::mutex g_mu;
@@ -85,19 +87,29 @@ int launch(const char* name, uint32_t grid, uint32_t block, uint32_t shmem, void
 
 // The library-owned activation image of `stream` (0 if every slot belongs to another stream). Work on one stream is
 // ordered, so a stream's slot is free again by the time its next call writes it; different streams never share one.
+// A slot handed out while `stream` is capturing is baked into the graph, which may be replayed long after the stream is
+// gone: such a slot is pinned, it stays with its stream key until cogni_quant_shutdown and cogni_gemv_release_stream
+// leaves it alone. A call that finds no slot is counted (cogni_gemv_image_stats).
 uint64_t image_for_stream(void* stream) {
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  const bool capturing = stream && hipStreamIsCapturing((hipStream_t)stream, &cs) == hipSuccess && cs == hipStreamCaptureStatusActive;
   std::lock_guard<std::mutex> lk(g_mu);
   if (!g_rt.ready || !g_rt.image_pool) return 0;
-  for (int i = 0; i < Runtime::kImageSlots; i++)
-    if (g_rt.image_used[i] && g_rt.image_stream[i] == stream)
-      return (uint64_t)(uintptr_t)g_rt.image_pool + (uint64_t)i * g_rt.image_slot_bytes;
-  for (int i = 0; i < Runtime::kImageSlots; i++)
+  int slot = -1;
+  for (int i = 0; i < Runtime::kImageSlots && slot < 0; i++)
+    if (g_rt.image_used[i] && g_rt.image_stream[i] == stream) slot = i;
+  for (int i = 0; i < Runtime::kImageSlots && slot < 0; i++)
     if (!g_rt.image_used[i]) {
       g_rt.image_used[i] = true;
       g_rt.image_stream[i] = stream;
-      return (uint64_t)(uintptr_t)g_rt.image_pool + (uint64_t)i * g_rt.image_slot_bytes;
+      slot = i;
     }
-  return 0;
+  if (slot < 0) {
+    g_rt.calls_without_image++;
+    return 0;
+  }
+  if (capturing) g_rt.image_pinned[slot] = true;
+  return (uint64_t)(uintptr_t)g_rt.image_pool + (uint64_t)slot * g_rt.image_slot_bytes;
 }
 
 const char* type_prefix(uint32_t type) {
@@ -252,35 +264,38 @@ int cogni_quant_init(int32_t ordinal) {
   if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(COGNI_ERR_NO_DEVICE, std::string("device is ") + prop.gcnArchName + ", the code object is gfx950 only");
   HIP_TRY(hipModuleLoadData(&g_rt.mod, cogni_hsaco_begin), "hipModuleLoadData(cogni_quant gfx950 code object)");
-  // the static scratch of the entry point that allocates nothing: its device address, once per device
-  if (int rc = cogni_internal_noalloc_setup(ordinal)) {
+  // from here on a failure leaves nothing behind: the module is unloaded, the pool freed, the table emptied, so that a
+  // later call starts from scratch
+  auto undo = [&](int rc) {
     (void)hipModuleUnload(g_rt.mod);
-    g_rt.mod = nullptr;
+    if (g_rt.image_pool) (void)hipFree(g_rt.image_pool);
+    g_rt = Runtime();
     return rc;
-  }
-  // its kernels are resolved now, so that a call under stream capture finds them in the table
-  for (const char* t : {"q8_0", "q4_k", "q5_k", "q6_k"}) {
-    for (const char* sfx : {"", "_tbatch2", "_tbatch3"}) {
-      hipFunction_t fn = nullptr;
-      const std::string name = std::string(t) + "_gemv_top1_partial_f32" + sfx;
-      if (hipModuleGetFunction(&fn, g_rt.mod, name.c_str()) == hipSuccess) g_rt.fns.emplace(name, fn);
-    }
-  }
-  for (const char* name : {"q4_k_gemv_mfma_top1_partial_f32_tbatch3", "q4_k_gemv_mfma_top1_partial_f32_tbatch4",
-                           "q6_k_gemv_mfma_top1_partial_f32_tbatch3", "q6_k_gemv_mfma_top1_partial_f32_tbatch4", "top1_reduce_f32"}) {
+  };
+  auto resolve = [&](const std::string& name, bool required) -> int {
     hipFunction_t fn = nullptr;
-    HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
-    g_rt.fns.emplace(name, fn);
-  }
+    const hipError_t he = hipModuleGetFunction(&fn, g_rt.mod, name.c_str());
+    if (he == hipSuccess) g_rt.fns.emplace(name, fn);
+    else if (required) return hip_fail(he, "hipModuleGetFunction(" + name + ")");
+    return 0;
+  };
+  // the static scratch of the entry point that allocates nothing: its device address, once per device
+  if (int rc = cogni_internal_noalloc_setup(ordinal)) return undo(rc);
+  // its kernels are resolved now, so that a call under stream capture finds them in the table
+  for (const char* t : {"q8_0", "q4_k", "q5_k", "q6_k"})
+    for (const char* sfx : {"", "_tbatch2", "_tbatch3"}) (void)resolve(std::string(t) + "_gemv_top1_partial_f32" + sfx, false);
+  for (const char* name : {"q4_k_gemv_mfma_top1_partial_f32_tbatch3", "q4_k_gemv_mfma_top1_partial_f32_tbatch4",
+                           "q6_k_gemv_mfma_top1_partial_f32_tbatch3", "q6_k_gemv_mfma_top1_partial_f32_tbatch4", "top1_reduce_f32"})
+    if (int rc = resolve(name, true)) return undo(rc);
   g_rt.image_slot_bytes = ((size_t)gemv_mt_image_bytes(COGNI_TYPE_Q6_K, GEMV_MT_MAX_IN_DIM) + 255) & ~(size_t)255;
-  HIP_TRY(hipMalloc(&g_rt.image_pool, g_rt.image_slot_bytes * Runtime::kImageSlots), "hipMalloc(activation images)");
+  if (hipError_t he = hipMalloc(&g_rt.image_pool, g_rt.image_slot_bytes * Runtime::kImageSlots); he != hipSuccess) {
+    g_rt.image_pool = nullptr;
+    return undo(hip_fail(he, "hipMalloc(activation images)"));
+  }
   for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q5_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32",
                            "q4_k_gemv_mt_top1_partial_f32", "q6_k_gemv_mt_top1_partial_f32", "rmsnorm_pack_q4k_f32",
-                           "rmsnorm_pack_q6k_f32", "add_rmsnorm_pack_q4k_f32", "add_rmsnorm_pack_q6k_f32"}) {
-    hipFunction_t fn = nullptr;
-    HIP_TRY(hipModuleGetFunction(&fn, g_rt.mod, name), std::string("hipModuleGetFunction(") + name + ")");
-    g_rt.fns.emplace(name, fn);
-  }
+                           "rmsnorm_pack_q6k_f32", "add_rmsnorm_pack_q4k_f32", "add_rmsnorm_pack_q6k_f32"})
+    if (int rc = resolve(name, true)) return undo(rc);
   g_rt.compute_units = prop.multiProcessorCount;
   g_rt.ordinal = ordinal;
   g_rt.ready = true;
@@ -327,11 +342,51 @@ int cogni_gemv_release_stream(void* stream) {
       if (g_rt.image_used[i] && g_rt.image_stream[i] == stream) slot = i;
   }
   if (slot < 0) return 0;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_rt.image_pinned[slot]) return 0;   // a captured graph names this slot: it stays where it is
+  }
   // the slot may only change hands once everything that reads it has run
   HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize(cogni_gemv_release_stream)");
   std::lock_guard<std::mutex> lk(g_mu);
   if (g_rt.image_used[slot] && g_rt.image_stream[slot] == stream) g_rt.image_used[slot] = false, g_rt.image_stream[slot] = nullptr;
   return 0;
+}
+
+int cogni_gemv_image_stats(uint32_t* slots, uint32_t* in_use, uint32_t* pinned, uint64_t* calls_without_image) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  uint32_t used = 0, pin = 0;
+  for (int i = 0; i < Runtime::kImageSlots; i++) used += g_rt.image_used[i], pin += g_rt.image_pinned[i];
+  if (slots) *slots = Runtime::kImageSlots;
+  if (in_use) *in_use = used;
+  if (pinned) *pinned = pin;
+  if (calls_without_image) *calls_without_image = g_rt.calls_without_image;
+  return 0;
+}
+
+// Passes over the weights cogni_gemv_dev makes for one call (with an image slot at hand): the same rules as the call itself.
+int32_t cogni_gemv_passes(uint32_t w_type, uint32_t tokens, uint32_t in_dim, uint32_t out_dim) {
+  if ((!gemv_type(w_type) && !plain_type(w_type)) || tokens == 0 || in_dim == 0 || out_dim == 0) return -1;
+  if (plain_type(w_type)) return 1;
+  if (k_quant(w_type) && (in_dim % 256) != 0) return -1;
+  const uint32_t from = gemv_mt_from(w_type, in_dim, out_dim);
+  if (from && tokens >= from) return (int32_t)((tokens + GEMV_MT_MAX_TOKENS - 1) / GEMV_MT_MAX_TOKENS);
+  uint32_t cap = k_quant(w_type) ? 2u : (uint32_t)COGNI_MAX_GEMV_TOKENS;
+  bool pairs = k_quant(w_type);
+  for (int mt = GEMV_MFMA_MAX_TOKENS; mt >= 2; mt--)
+    if (gemv_mfma_supported(w_type, mt, in_dim)) {
+      cap = (uint32_t)mt;
+      pairs = false;
+      break;
+    }
+  const bool walks = (uint64_t)gemv_grid(w_type, 2, out_dim) * (uint32_t)gemv_rows_per_block(w_type, 2) < out_dim;
+  int32_t passes = 0;
+  for (uint32_t t0 = 0, m = 0; t0 < tokens; t0 += m, passes++) {
+    const uint32_t left = tokens - t0;
+    m = left < cap ? left : cap;
+    if (pairs && left == 3 && !walks) m = 3;
+  }
+  return passes;
 }
 
 int cogni_gemv_packed_launch_dims(uint32_t w_type, uint32_t in_dim, uint32_t total_rows, uint32_t* grid_x, uint32_t* block_x,

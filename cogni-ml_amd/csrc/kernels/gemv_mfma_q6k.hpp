@@ -154,7 +154,7 @@ __device__ __forceinline__ void q6k_gemv_mfma_core(const uint8_t* w, const float
                             max((u32)__builtin_amdgcn_readlane((int)ab, 32), (u32)__builtin_amdgcn_readlane((int)ab, 48)));
         const int e = (int)((ab4 >> 23) & 0xFFu);
         int sh = 139 - e;                      // scale = 2^sh
-        sh = sh > 100 ? 100 : sh;              // zeros / tiny values: keep 2^-sh a normal number
+        sh = sh > 126 ? 126 : sh;              // zeros / subnormal values: 2^sh and 2^-sh stay normal numbers
         const float scale = __builtin_bit_cast(float, (u32)(127 + sh) << 23);
         const float inv = __builtin_bit_cast(float, (u32)(127 - sh) << 23);
         const float s0 = v.x * scale, s1 = v.y * scale, s2 = v.z * scale, s3 = v.w * scale;

@@ -89,8 +89,9 @@ __device__ __forceinline__ MtPacked mt_pack4(float4 v) {
                       max((u32)__builtin_amdgcn_readlane((int)ab, 32), (u32)__builtin_amdgcn_readlane((int)ab, 48)));
   const int e = (int)((ab4 >> 23) & 0xFFu);
   int sh = 139 - e;            // scale = 2^sh
-  sh = sh > 100 ? 100 : sh;    // zeros and tiny values: keep 2^-sh a normal number
-  sh = sh < -100 ? -100 : sh;  // infinities and NaN: they stay what they are
+  sh = sh > 126 ? 126 : sh;    // zeros and subnormal values: 2^sh and 2^-sh stay normal numbers (every normal input keeps its 22 bits)
+  // (the largest finite magnitudes give sh = -115, infinities and NaN -116: 2^sh and 2^-sh are normal numbers for every
+  // input, so any finite activation lands in the binary16 range and non-finite ones stay what they are)
   const float scale = __builtin_bit_cast(float, (u32)(127 + sh) << 23);
   MtPacked r;
   r.scale = scale;
@@ -120,11 +121,13 @@ __device__ __forceinline__ void mt_pack_store_q4k(uint8_t* __restrict__ image, u
   *reinterpret_cast<mt_half4*>(op) = pk.hv;
   *reinterpret_cast<mt_half4*>(op + 16) = pk.lv;
   // sums of the eight sub-blocks (eight lanes each) for the min term
-  float sm = (v.x + v.y) + (v.z + v.w);
+  // (summed after the scaling, which is exact: the same bits as scaling the sum, and no overflow for activations near
+  // the top of the fp32 range)
+  float sm = (v.x * pk.scale + v.y * pk.scale) + (v.z * pk.scale + v.w * pk.scale);
   sm += MT_DPP(sm, MT_QUAD_1032);
   sm += MT_DPP(sm, MT_QUAD_2301);
   sm += MT_DPP(sm, MT_ROW_HALF_MIRROR);
-  const float s32 = pk.scale * 0.03125f;   // (powers of two: both products below are exact)
+  const float s32 = 0.03125f;
   const _Float16 sh = (_Float16)(sm * s32), sl = (_Float16)fmaf(sm, s32, -(float)sh);
   uint8_t* aux = image + (size_t)nsb * 8192 + (size_t)sb * 1024;
   if ((lane & 3) == 0) {
@@ -161,10 +164,11 @@ __device__ __forceinline__ void mt_pack_store_q6k(uint8_t* __restrict__ image, u
   uint8_t* op = image + ((size_t)(sb * 8 + (s >> 1)) * 64 + kg * 16 + 2 * tok) * 16 + 8 * (s & 1);
   *reinterpret_cast<mt_half4*>(op) = pk.hv;
   *reinterpret_cast<mt_half4*>(op + 16) = pk.lv;
-  float sm = (v.x + v.y) + (v.z + v.w);   // sums of the sixteen sub-blocks (four lanes each)
+  // sums of the sixteen sub-blocks (four lanes each), of the scaled values (exact, and safe near the top of the fp32 range)
+  float sm = (v.x * pk.scale + v.y * pk.scale) + (v.z * pk.scale + v.w * pk.scale);
   sm += MT_DPP(sm, MT_QUAD_1032);
   sm += MT_DPP(sm, MT_QUAD_2301);
-  const float s16 = pk.scale * 0.0625f;   // (powers of two: both products below are exact)
+  const float s16 = 0.0625f;
   const _Float16 sh = (_Float16)(sm * s16), sl = (_Float16)fmaf(sm, s16, -(float)sh);
   uint8_t* aux = image + (size_t)nsb * 8192 + (size_t)sb * 1024;
   if ((lane & 3) == 0) {
@@ -208,6 +212,9 @@ __device__ __forceinline__ void mt_load16(mt_u32x4& dst, u64 sb, u32 voff) {
 // 16 bytes per active lane from addr to LDS byte address lds_base (uniform) + 16 * lane
 __device__ __forceinline__ void mt_copy16(u32 lds_base, const void* addr) {
   const u32 m0 = (u32)__builtin_amdgcn_readfirstlane((int)lds_base);
+  // (M0 cannot be named as clobbered - it is a reserved register and the compiler says it may ignore such a clobber -
+  // so nothing the compiler emits in these kernels may rely on a value of M0: the build checks that every reader of M0
+  // in them sits directly behind a write of M0, check_hazards.py)
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0), "v"(addr) : "memory");
 }
 template <int N>

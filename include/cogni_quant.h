@@ -147,8 +147,10 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
  * cogni_gemv_dev (from 3 to 5 tokens on, by type and row length), cogni_gemv_dual_dev and cogni_gemv_many_dev (2 tokens
  * and more) take this path by
  * themselves with an image the library keeps per stream (8 streams at most; a ninth falls back to the kernels
- * cogni_gemv_plan describes). A graph captured from one stream carries that stream's image: replay it on one stream at a
- * time, and not beside eager calls on the capture stream. */
+ * cogni_gemv_plan describes, which is counted: cogni_gemv_image_stats). A graph captured from one stream carries that
+ * stream's image: replay it on one stream at a time, and not beside eager calls on the capture stream. An image handed
+ * out while its stream is capturing is pinned: it keeps its stream key until cogni_quant_shutdown, so that a graph
+ * replayed after its capture stream was released or destroyed never shares the image with another stream. */
 size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 /* The token count from which cogni_gemv_dev and cogni_gemv_top1_dev take this path for one matrix (Q6_K 3; Q4_K and Q5_K 4
  * on rows of 4096 values and more, else 5; a tall matrix of up to 4096 columns - 40960 rows and more, an output head -
@@ -158,8 +160,17 @@ uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim, uint32_t out
 /* Gives back the image the library keeps for `stream` (waits for the stream's work first; nothing to do and no error if it
  * has none). Call it before destroying a stream that ran multi-token GEMVs: the eight slots are otherwise used up by the
  * first eight streams of the process, and later streams run the per-token-group kernels. A graph captured on the stream
- * still names the stream's image: release only once such graphs are no longer replayed. */
+ * recorded while the stream was capturing keeps the image pinned: the call then changes nothing (see above). */
 int cogni_gemv_release_stream(void* stream);
+/* What became of the library's images: how many slots there are, how many belong to a stream, how many of those are
+ * pinned by a capture, and how many multi-token calls found no slot and ran the per-token-group kernels instead (two or
+ * four passes over the weights where one was possible: slower, same results to the bar). Any pointer may be null. */
+int cogni_gemv_image_stats(uint32_t* slots, uint32_t* in_use, uint32_t* pinned, uint64_t* calls_without_image);
+/* Passes over the weights that cogni_gemv_dev makes for a call of `tokens` tokens when an image slot is at hand: 1 where
+ * the one-pass kernel takes the shape (ceil(tokens / 8) beyond eight tokens), else one per token group of the kernels
+ * cogni_gemv_plan names (groups of up to four on the matrix cores, pairs on the vector ALU, eight for Q8_0). -1 for a
+ * type or shape the call refuses. No GPU needed. */
+int32_t cogni_gemv_passes(uint32_t w_type, uint32_t tokens, uint32_t in_dim, uint32_t out_dim);
 /* Launch geometry of the one-pass kernel for a launch of total_rows rows (all its matrices together): a workgroup's eight
  * wavefronts carry t tiles of 16 rows at a time (in_dim above 4096: t = 1; else t = clamp(tiles / 256, 1, 3), Q6_K at most 2),
  * a row group is t tiles, grid_x = min(256, row groups) and the workgroups walk the groups blockIdx.x, blockIdx.x +
@@ -297,7 +308,9 @@ int cogni_gemv_packed_top1_dev(uint64_t w_raw, uint32_t w_type, uint64_t image, 
  * call fails with COGNI_ERR_INVALID_ARGUMENT and launches nothing. Every call on a GPU uses that GPU's one array: calls
  * that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered and safe. Nothing in the
  * array needs clearing between calls (every slot read was written by the same call). Needs cogni_quant_init on the
- * current device. */
+ * current device. Groups of tokens that go through the one-pass kernel use the library's activation image of `stream`
+ * (allocated by cogni_quant_init, not by the call); recorded under stream capture that image is pinned to the stream
+ * for the life of the library, as described at cogni_gemv_image_bytes. */
 enum { COGNI_TOP1_NOALLOC_MAX_PARTIALS = 65536 };
 int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t top1_ids, uint64_t top1_values,
                                 uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);

@@ -46,6 +46,20 @@ def test_m0_ahead_of_a_load_to_lds():
     assert ch.check(lines("s_mov_b32 m0, s3\nglobal_load_dwordx4 v[4:7], v[2:3], off")) == []      # not a load to LDS
 
 
+def test_m0_readers_in_kernels_with_asm_copies():
+    """Kernels whose copies set M0 inside asm statements: every reader of M0 sits right behind a write of M0."""
+    def mt(text):
+        return ["0000000000001000 <q4_k_gemv_mt_f32>:"] + lines(text)[1:]
+    assert ch.check(mt("s_mov_b32 m0, s3\ns_nop 0\nglobal_load_lds_dwordx4 v[2:3], off")) == []
+    # a reader that relies on an older value of M0: a second copy without its own write, a movrel, a label in between
+    assert len(ch.check(mt("s_mov_b32 m0, s3\ns_nop 0\nglobal_load_lds_dwordx4 v[2:3], off\nv_mov_b32_e32 v1, v2\nglobal_load_lds_dwordx4 v[4:5], off"))) == 1
+    assert len(ch.check(mt("s_mov_b32 m0, s3\ns_nop 0\nv_mov_b32_e32 v1, v2\nv_mov_b32_e32 v1, v2\nv_movrels_b32_e32 v1, v2"))) == 1
+    assert len(ch.check(mt("s_mov_b32 m0, s3\ns_nop 0") + ["0000000000001010 <L1>:", "\tglobal_load_lds_dwordx4 v[2:3], off    // 0: 0"])) == 1
+    assert len(ch.check(mt("v_readlane_b32 s4, v1, m0"))) == 1
+    # the same sequence in a kernel the compiler alone writes M0 for is its own business
+    assert ch.check(lines("s_mov_b32 m0, s3\ns_nop 0\nglobal_load_lds_dwordx4 v[2:3], off\nv_mov_b32_e32 v1, v2\nv_mov_b32_e32 v1, v2\nglobal_load_lds_dwordx4 v[4:5], off")) == []
+
+
 def test_a_new_kernel_starts_clean():
     two = lines("v_readfirstlane_b32 s6, v147") + ["0000000000002000 <k2>:", "\tglobal_load_dword v3, v1, s[6:7]    // 0: 0"]
     assert ch.check(two) == []

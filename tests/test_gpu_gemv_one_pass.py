@@ -119,6 +119,34 @@ def test_one_pass_activation_ranges(gpu, oracle):
         a.close()
 
 
+@pytest.mark.parametrize("type_id", [Q4_K, Q5_K, Q6_K])
+def test_one_pass_activations_near_the_top_of_the_fp32_range(gpu, oracle, type_id):
+    """|x| of 1e35 .. 1e36, beyond 2^116: the image's power of two brings any finite activation into the binary16 range (no
+    clamp on the large side) and the sub-block sums are formed after the scaling, so nothing overflows before the result
+    does. The outputs (up to about 1e38) are finite in the reference's f64 sums and must be here, to the usual bars."""
+    rng = np.random.default_rng(338)
+    in_dim, out_dim, tokens = 2048, 96, 8
+    raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim).reshape(tokens, in_dim)
+    x[0] *= np.float32(1e35)
+    x[1] *= np.float32(2e35)
+    x[2, :256] = np.float32(2.0 ** 117) * np.where(np.arange(256) % 2 == 0, 1.0, -1.0).astype(np.float32)   # one magnitude, alternating signs
+    x[3] *= np.float32(1e-37)                        # and the smallest normal numbers
+    x = np.ascontiguousarray(x.reshape(-1)).astype(np.float32)
+    want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens, type_id)
+    assert np.isfinite(want).all()
+    w, xd, od = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim)
+    quant.gemv_dev(w.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+    got = od.read(np.float32, tokens * out_dim)
+    assert quant.gemv_passes(type_id, tokens, in_dim, out_dim) == 1
+    assert np.isfinite(got).all()
+    g, w_ = got.reshape(tokens, out_dim).astype(np.float64), want.reshape(tokens, out_dim)
+    for m in range(tokens):
+        assert np.max(np.abs(g[m] - w_[m])) <= 2e-5 * float(np.max(np.abs(w_[m]))), m
+    for a in (w, xd, od):
+        a.close()
+
+
 def test_one_pass_element_order_and_scale_positions(gpu, oracle):
     """A matrix whose codes, scales and mins each appear in exactly one place at a time: a swapped sub-block, nibble half,
     k-group or scale byte puts the unit activation's weight in the wrong output."""
@@ -325,4 +353,65 @@ def test_image_slots_return_when_streams_close(gpu, oracle):
         assert np.array_equal(od.read(np.float32, tokens * out_dim), explicit), i
         st.close()
     for a in (w, xd, od, o2, image):
+        a.close()
+
+
+def test_a_ninth_stream_is_counted_and_a_captured_image_stays_pinned(gpu, oracle):
+    """Eight streams hold the eight images; a ninth stream's call runs the per-token-group kernels (within the bar, not
+    the one-pass bits) and is counted. An image handed out under stream capture is pinned: closing the capture stream does
+    not give it back, so a replay of the graph never shares it with another stream."""
+    rng = np.random.default_rng(99)
+    in_dim, out_dim, tokens = 4096, 256, 8
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    w, xd = DevArray(raw), DevArray(x)
+    outs = [DevArray(nbytes=4 * tokens * out_dim) for _ in range(10)]
+    want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens)
+    slots, used0, pinned0, missed0 = quant.gemv_image_stats()
+    assert slots == 8
+    streams = [hip.HIPStream() for _ in range(9)]
+    try:
+        held = []
+        for i, st in enumerate(streams):
+            before = quant.gemv_image_stats()
+            quant.gemv_dev(w.ptr, Q4_K, xd.ptr, outs[i].ptr, in_dim, out_dim, tokens, 0, st.handle)
+            st.synchronize()
+            after = quant.gemv_image_stats()
+            held.append(after[1] > before[1])
+            assert_bars(outs[i].read(np.float32, tokens * out_dim), want, tol, tokens, out_dim, "stream %d" % i)
+        free_at_start = slots - used0
+        assert sum(held) == min(free_at_start, 9)
+        assert quant.gemv_image_stats()[3] - missed0 == 9 - sum(held) >= 1
+    finally:
+        for st in streams:
+            st.close()
+    assert quant.gemv_image_stats()[1] == used0
+    # capture on a fresh stream, close it, then make other streams take every free slot: the replay still gives the
+    # one-pass bits
+    cap = hip.HIPStream()
+    cap.begin_capture(1)
+    quant.gemv_dev(w.ptr, Q4_K, xd.ptr, outs[9].ptr, in_dim, out_dim, tokens, 0, cap.handle)
+    graph = cap.end_capture()
+    ex = graph.instantiate()
+    assert quant.gemv_image_stats()[2] == pinned0 + 1
+    cap.close()
+    assert quant.gemv_image_stats()[2] == pinned0 + 1 and quant.gemv_image_stats()[1] == used0 + 1
+    others = [hip.HIPStream() for _ in range(8)]
+    run = hip.HIPStream()
+    try:
+        for i, st in enumerate(others):
+            quant.gemv_dev(w.ptr, Q4_K, xd.ptr, outs[i].ptr, in_dim, out_dim, tokens, 0, st.handle)
+        for rep in range(3):
+            ex.launch(run)
+            for st in others[:3]:   # eager work on the other streams between the replays
+                quant.gemv_dev(w.ptr, Q4_K, xd.ptr, outs[0].ptr, in_dim, out_dim, tokens, 0, st.handle)
+            run.synchronize()
+            assert_bars(outs[9].read(np.float32, tokens * out_dim), want, tol, tokens, out_dim, "replay %d" % rep)
+    finally:
+        for st in others + [run]:
+            st.synchronize()
+            st.close()
+        ex.close()
+        graph.close()
+    for a in [w, xd] + outs:
         a.close()
