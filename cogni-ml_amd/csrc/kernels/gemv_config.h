@@ -239,3 +239,23 @@ static inline int gemm_q4k_use_wide(unsigned out_dim, unsigned tokens) {
   const unsigned rn = (narrow + GEMM_ROUND_TILES - 1) / GEMM_ROUND_TILES, rw = (wide + GEMM_ROUND_TILES - 1) / GEMM_ROUND_TILES;
   return rw * GEMM_WIDE_ROUND_COST_X100 < rn * 100u;
 }
+
+// ---- one-pass kernel, rows above 4096 values: what a streamed unit waits for (gemv_mt.hpp)
+// vmcnt value that says "operand set i and unit i of a streamed row group have landed" (T = 1, S super-blocks per
+// k-slice, NSLOT units in LDS). Issue order: set 0, unit 0, set 1, unit 1, units 2 .. min(S, NSLOT) - 1 up front; behind unit
+// i's arithmetic: set i + 2, then unit i + NSLOT. NA loads per set, NC copies per unit. The answer is the number of loads
+// issued, by the time of the wait, behind the later of the two.
+static inline GEMV_HD constexpr int mt_stream_wait(int S, int NSLOT, int NS, int NA, int NC, int i) {
+  int pos = 0, end_set[8] = {}, end_unit[8] = {};
+  const int up = S < NSLOT ? S : NSLOT;
+  for (int u = 0; u < up; u++) {
+    if (u < NS) end_set[u] = (pos += NA);
+    end_unit[u] = (pos += NC);
+  }
+  for (int j = 0; j < i; j++) {   // what was issued behind the units before i
+    if (j + NS < S) end_set[j + NS] = (pos += NA);
+    if (j + NSLOT < S) end_unit[j + NSLOT] = (pos += NC);
+  }
+  const int need = end_set[i] > end_unit[i] ? end_set[i] : end_unit[i];
+  return pos - need;
+}

@@ -429,24 +429,7 @@ struct MtArgs {
   u32 rows[3];
 };
 
-// vmcnt value that says "operand set i and unit i of a streamed row group have landed" (T = 1, S super-blocks per
-// k-slice, NSLOT units in LDS). Issue order: set 0, unit 0, set 1, unit 1, units 2 .. min(S, NSLOT) - 1 up front; behind unit
-// i's arithmetic: set i + 2, then unit i + NSLOT. NA loads per set, NC copies per unit. The answer is the number of loads
-// issued, by the time of the wait, behind the later of the two.
-constexpr int mt_stream_wait(int S, int NSLOT, int NS, int NA, int NC, int i) {
-  int pos = 0, end_set[8] = {}, end_unit[8] = {};
-  const int up = S < NSLOT ? S : NSLOT;
-  for (int u = 0; u < up; u++) {
-    if (u < NS) end_set[u] = (pos += NA);
-    end_unit[u] = (pos += NC);
-  }
-  for (int j = 0; j < i; j++) {   // what was issued behind the units before i
-    if (j + NS < S) end_set[j + NS] = (pos += NA);
-    if (j + NSLOT < S) end_unit[j + NSLOT] = (pos += NC);
-  }
-  const int need = end_set[i] > end_unit[i] ? end_set[i] : end_unit[i];
-  return pos - need;
-}
+// (mt_stream_wait, the number a streamed unit waits with, lives in gemv_config.h: host code can test it there)
 
 // SBW: super-blocks per k-slice (in_dim / 2048). SBW <= 2: operands resident in registers, T tiles per wavefront, the next
 // row group requested while this one is worked on. SBW >= 3: T = 1, operands streamed through two register sets.

@@ -14,6 +14,7 @@
 
 #include "ml_hip.hpp"
 #include "quant_matmul_hip.hpp"
+#include "../../cogni-ml_amd/csrc/kernels/gemv_config.h"
 
 extern "C" int oracle_matmul_add(const float* x, int rows, int in_dim, const uint8_t* w_raw, uint32_t w_type,
                                  int out_dim, const float* bias, float* result);
@@ -166,8 +167,47 @@ static int gpu_probe() {
   return 0;
 }
 
+// The vmcnt values of the one-pass kernel's streamed path (mt_stream_wait, gemv_config.h) against a list of what the
+// kernel issues, in its order: up front set u (u < NS) and unit u for u < NSLOT; behind unit i's arithmetic set i + NS and
+// unit i + NSLOT. A unit may start when the youngest load of operand set i and of unit i has landed, i.e. when at most the
+// loads issued after it are outstanding. Every (super-blocks per k-slice, slots, register sets) the kernels are built with,
+// and the neighbouring ones.
+static void stream_wait_spec() {
+  struct Fmt { int slots, nc; };
+  for (int S = 3; S <= 6; S++)
+    for (Fmt f : {Fmt{6, 3}, Fmt{4, 4}})
+      for (int NS = 2; NS <= 3; NS++)
+        for (int NA : {9, 13}) {
+          const int NSLOT = f.slots < S ? f.slots : S, NC = f.nc;
+          std::vector<std::pair<char, int>> issued;
+          auto issue = [&](char kind, int index, int n) { for (int k = 0; k < n; k++) issued.push_back({kind, index}); };
+          for (int u = 0; u < NSLOT; u++) {
+            if (u < NS) issue('s', u, NA);
+            issue('u', u, NC);
+          }
+          for (int i = 0; i < S; i++) {
+            int last = -1, nset = 0, nunit = 0;
+            for (int k = 0; k < (int)issued.size(); k++)
+              if (issued[k].second == i) {
+                last = k;
+                (issued[k].first == 's' ? nset : nunit)++;
+              }
+            EXPECT(nset == NA && nunit == NC);   // both were requested before their wait
+            const int behind = (int)issued.size() - 1 - last;
+            EXPECT(mt_stream_wait(S, NSLOT, NS, NA, NC, i) == behind);
+            EXPECT(behind >= 0 && behind < 64);  // vmcnt has six bits
+            if (i + NS < S) issue('s', i + NS, NA);
+            if (i + NSLOT < S) issue('u', i + NSLOT, NC);
+          }
+        }
+  // a known point: Q4_K at 12288 columns (S = 6, six slots, two sets): unit 0 waits with everything behind unit 0 outstanding
+  EXPECT(mt_stream_wait(6, 6, 2, 9, 3, 0) == 9 + 3 + 4 * 3);
+  EXPECT(mt_stream_wait(6, 6, 2, 9, 3, 5) == 0);
+}
+
 int main(int argc, char** argv) {
   runner_spec();
+  stream_wait_spec();
   host_errors();
   if (argc > 1 && std::string(argv[1]) == "--gpu") gpu_probe();
   std::printf("%s (%d failures)\n", failures == 0 ? "PASSED" : "FAILED", failures);

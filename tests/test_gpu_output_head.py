@@ -135,6 +135,30 @@ def test_top1_in_one_pass(gpu, oracle, t, in_dim, out_dim, tokens):
     assert list(ids3) == [0] * tokens
 
 
+@pytest.mark.parametrize("out_dim", [151936, 248320])
+def test_full_size_heads(gpu, oracle, out_dim):
+    """The vocabulary projections at their real sizes, Q6_K x 4096 columns: 151 936 rows (the configured head) and 248 320
+    (Qwen3.5's, src/ml/gguf/qwen_output_head_runner.cr:895): one token on the vector ALU and eight in one pass, the
+    arg-max inside. The winner is the first maximum of the same kernels' logits, the logits agree with the oracle on every
+    row to the GEMV bars, and the oracle's value at the winner is its maximum up to the tolerance."""
+    rng = np.random.default_rng(out_dim)
+    in_dim = 4096
+    raw = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    dense_max = float(np.abs(oracle.dequantize(raw[:4096 * 16 * 210], Q6_K, 4096 * in_dim)).max())
+    for tokens in (1, 8):
+        x = synth.make_activations(rng, tokens, in_dim)
+        ids, vals, logits = run_top1(raw, Q6_K, x, in_dim, out_dim, tokens)
+        assert quant.gemv_passes(Q6_K, tokens, in_dim, out_dim) == 1
+        want = oracle.matmul_add(x, tokens, in_dim, raw, Q6_K, out_dim, np.zeros(out_dim, dtype=np.float32), threads=16).reshape(tokens, out_dim)
+        for tok in range(tokens):
+            assert ids[tok] == first_max(logits[tok]) and vals[tok] == logits[tok].max(), (tokens, tok)
+            scale = float(np.abs(want[tok]).max())
+            err = float(np.abs(logits[tok].astype(np.float64) - want[tok]).max())
+            assert err <= 1e-4 * float(np.linalg.norm(x[tok * in_dim:(tok + 1) * in_dim])) * dense_max
+            assert err <= 2e-5 * scale, (tokens, tok, err, scale)
+            assert want[tok][ids[tok]] >= float(want[tok].max()) - 2e-5 * scale
+
+
 @pytest.mark.parametrize("hidden,vocab,tokens", [(1024, 20011, 4), (2048, 41003, 6), (4096, 3001, 8)])
 def test_output_head_runner(gpu, oracle, hidden, vocab, tokens):
     """(1024 hidden values: the matrix-core kernel for the group of four; 2048 and 4096: the norm writes the activation image
