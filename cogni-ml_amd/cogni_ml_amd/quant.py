@@ -282,6 +282,20 @@ def gemm_packed_dev(w_ptr, w_type, workspace_ptr, workspace_bytes, out_ptr, in_d
                                            ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+def gemm_packed_add_dev(w_ptr, w_type, workspace_ptr, workspace_bytes, residual_ptr, out_ptr, in_dim, out_dim, tokens, stream=None):
+    """gemm_packed_dev with a [tokens][out_dim] residual added (it may be the output buffer itself)."""
+    _check(hip.lib().cogni_gemm_packed_add_dev(ctypes.c_uint64(w_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(workspace_ptr),
+                                               ctypes.c_size_t(workspace_bytes), ctypes.c_uint64(residual_ptr), ctypes.c_uint64(out_ptr),
+                                               ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
+def gemm_packed_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, workspace_ptr, workspace_bytes, out_ptr, in_dim, out_dim, tokens, stream=None):
+    """silu(x W_gate^T) * (x W_up^T) in one GEMM launch against packed activations (Q4_K)."""
+    _check(hip.lib().cogni_gemm_packed_swiglu_dev(ctypes.c_uint64(w_gate_ptr), ctypes.c_uint64(w_up_ptr), ctypes.c_uint32(int(w_type)),
+                                                  ctypes.c_uint64(workspace_ptr), ctypes.c_size_t(workspace_bytes), ctypes.c_uint64(out_ptr),
+                                                  ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
 def matmul_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_ptr=0, workspace_bytes=0, bias_ptr=0,
                stream=None):
     """The GEMV/GEMM router (tokens > threshold and Q4_K -> GEMM)."""

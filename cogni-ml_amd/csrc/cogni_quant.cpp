@@ -1022,26 +1022,51 @@ int cogni_gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t
   return 0;
 }
 
-int cogni_gemm_packed_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t bias, uint64_t out,
-                          uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
-  if (!w_raw || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_packed_dev: null device pointer");
-  if (int rc = gemm_check("cogni_gemm_packed_dev", w_type, in_dim, out_dim, tokens, workspace, workspace_bytes)) return rc;
+// One matrix against packed activations; `add` is a [out_dim] bias (add_stride 0) or a [tokens][out_dim] residual (add_stride out_dim).
+static int gemm_packed_launch(const char* who, uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t add,
+                              uint32_t add_stride, uint64_t out, uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (!w_raw || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null device pointer");
+  if (int rc = gemm_check(who, w_type, in_dim, out_dim, tokens, workspace, workspace_bytes)) return rc;
   const size_t need = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
   const GemmPlan p = gemm_plan(w_type, in_dim, out_dim, tokens, workspace_bytes);
   uint32_t splits = p.splits;
   if (splits == 1) {
-    void* params[] = {&w_raw, &workspace, &bias, &out, &in_dim, &out_dim, &tokens};
+    void* params[] = {&w_raw, &workspace, &add, &out, &in_dim, &out_dim, &tokens, &add_stride};
     return launch(p.kernel, p.grid_x, p.block, 0, params, stream);
   }
   uint64_t planes = workspace + need, none = 0;
-  uint32_t total = tokens * out_dim;
+  uint32_t total = tokens * out_dim, zero = 0;
   {
-    void* params[] = {&w_raw, &workspace, &none, &planes, &in_dim, &out_dim, &tokens};
+    void* params[] = {&w_raw, &workspace, &none, &planes, &in_dim, &out_dim, &tokens, &zero};
     int rc = launch(p.kernel, p.grid_x, p.block, 0, params, stream, splits);
     if (rc != 0) return rc;
   }
-  void* params[] = {&planes, &bias, &out, &total, &out_dim, &splits};
+  void* params[] = {&planes, &add, &out, &total, &out_dim, &splits, &add_stride};
   return launch("gemm_sum_splits_f32", (total + 1023) / 1024, 256, 0, params, stream);
+}
+
+int cogni_gemm_packed_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t bias, uint64_t out,
+                          uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
+  return gemm_packed_launch("cogni_gemm_packed_dev", w_raw, w_type, workspace, workspace_bytes, bias, 0, out, in_dim, out_dim, tokens, stream);
+}
+
+int cogni_gemm_packed_add_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t residual, uint64_t out,
+                              uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (!residual) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_packed_add_dev: null device pointer");
+  return gemm_packed_launch("cogni_gemm_packed_add_dev", w_raw, w_type, workspace, workspace_bytes, residual, out_dim, out, in_dim, out_dim,
+                            tokens, stream);
+}
+
+int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
+                                 uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream) {
+  if (w_type != COGNI_TYPE_Q4_K)
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the fused gate/up SwiGLU GEMM: ") + type_name(w_type));
+  if (!w_gate || !w_up || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemm_packed_swiglu_dev: null device pointer");
+  if (int rc = gemm_check("cogni_gemm_packed_swiglu_dev", w_type, in_dim, out_dim, tokens, workspace, workspace_bytes)) return rc;
+  // a tile is 128 tokens x 96 rows of each matrix
+  const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 95) / 96;
+  void* params[] = {&w_gate, &w_up, &workspace, &out, &in_dim, &out_dim, &tokens};
+  return launch("q4_k_gemm_swiglu_f16", 8 * ((mtiles * ntiles + 7) / 8), 256, 0, params, stream);
 }
 
 int cogni_set_gemm_threshold(int32_t tokens) {

@@ -7,10 +7,16 @@
 // Kernels:
 //   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 16 * in_dim/256
 //   q4_k_gemm_f16, q5_k_gemm_f16
-//                   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
+//                   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32, bias_stride:u32)
 //                   block 256, grid (8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), k splits), no dynamic LDS
-//                   (156 / 160 KiB static); with k splits > 1 `out` is `splits` planes of [m][out_dim] and bias is null
-//   gemm_sum_splits_f32 (planes, bias|null, out, m*out_dim:u32, out_dim:u32, splits:u32)   block 256, grid ceil(m*out_dim/1024)
+//                   (156 / 160 KiB static); with k splits > 1 `out` is `splits` planes of [m][out_dim] and bias is null.
+//                   bias_stride 0: a [out_dim] bias added to every token; out_dim: a [m][out_dim] residual (it may be
+//                   `out` itself) - the reference's f32out_add prefill pipelines (gemm_mm.metal:651)
+//   q4_k_gemm_swiglu_f16
+//                   (w_gate, w_up, xp, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32): out = silu(x W_gate^T) * (x W_up^T),
+//                   the reference's simd_mm_q4k_h16_b64_swiglu (gemm_q4k.metal:1233). A tile is 128 tokens x 96 rows of each
+//                   matrix; block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/96) / 8), no k split
+//   gemm_sum_splits_f32 (planes, bias|null, out, m*out_dim:u32, out_dim:u32, splits:u32, bias_stride:u32)   block 256, grid ceil(m*out_dim/1024)
 //
 // Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows, so 512 x 12288 gives 256
 // workgroups, one per CU. K is walked one 256-value super-block at a time = 16 MFMA k-steps of 16.
@@ -145,7 +151,7 @@ __shared__ uint4 gemm_wbuf5[32 * 64];
 // layout both share (kh = 0 writes into x buffer 0, kh = 1 into x buffer 1: 2 x 24 KiB each). Sum first, bias second.
 template <int KH>
 __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
-                                                   u32 mt, u32 nt, u32 nh, u32 j, u32 kg, u32 lane) {
+                                                   u32 mt, u32 nt, u32 nh, u32 j, u32 kg, u32 lane, u32 bias_stride) {
   float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * 24 * 64 + lane;
   const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * 24 * 64 + lane;
 #pragma unroll
@@ -192,9 +198,12 @@ __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][3], const
         const u32 n = nt * GEMM_BN + nh * 96 + 32 * c + 8 * g4 + 4 * kg;
         if (token < m && n < out_dim) {
           float* dst = out + (size_t)token * out_dim + n;
+          // what is added: element n of the bias, or element (token, n) of a residual (which may be `out`: a thread reads
+          // the values it is about to overwrite, nobody else's)
+          const float* b = bias ? bias + (size_t)token * bias_stride + n : nullptr;
           if (n + 4 <= out_dim) {
-            if (bias) {
-              o.x += bias[n]; o.y += bias[n + 1]; o.z += bias[n + 2]; o.w += bias[n + 3];
+            if (b) {
+              o.x += b[0]; o.y += b[1]; o.z += b[2]; o.w += b[3];
             }
             if (vec) {
               *reinterpret_cast<float4*>(dst) = o;
@@ -203,16 +212,90 @@ __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][3], const
             }
           } else {
             const float ov[4] = {o.x, o.y, o.z, o.w};
-            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (bias ? bias[n + e] : 0.0f);
+            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (b ? b[e] : 0.0f);
           }
         }
       }
   }
 }
 __device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
-                                              u32 mt, u32 nt, u32 nh, u32 kh, u32 j, u32 kg, u32 tid) {
-  if (kh == 0) gemm_epilogue_half<0>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63);
-  else gemm_epilogue_half<1>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63);
+                                              u32 mt, u32 nt, u32 nh, u32 kh, u32 j, u32 kg, u32 tid, u32 bias_stride = 0) {
+  if (kh == 0) gemm_epilogue_half<0>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
+  else gemm_epilogue_half<1>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
+}
+
+// Epilogue of the gate | up kernel: the nh = 0 wavefronts hold 96 gate rows, the nh = 1 wavefronts the same 96 rows of up,
+// in the same lane layout. First the two k halves are added as above, each wavefront finishing its two token tiles in
+// place; then the up wavefronts hand their sums to the gate wavefronts (same kh) through LDS, which store
+// silu(gate) * up: 128 tokens x 96 outputs per workgroup, four consecutive floats per register quad.
+template <int KH>
+__device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3], float* out, u32 out_dim, u32 m, u32 mt, u32 nt,
+                                                          u32 nh, u32 j, u32 kg, u32 lane) {
+  float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * 24 * 64 + lane;
+  const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * 24 * 64 + lane;
+#pragma unroll
+  for (int rr = 0; rr < 2; rr++)
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const float16_t& t = acc[2 * (1 - KH) + rr][c];
+        mine[((rr * 3 + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
+      }
+  __syncthreads();
+#pragma unroll
+  for (int rr = 0; rr < 2; rr++)
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        float16_t& t = acc[2 * KH + rr][c];
+        const float4 p = theirs[((rr * 3 + c) * 4 + g4) * 64];
+        // (k half 0) + (k half 1), in that order whichever of the two this wavefront holds
+        t[4 * g4] = KH ? p.x + t[4 * g4] : t[4 * g4] + p.x;
+        t[4 * g4 + 1] = KH ? p.y + t[4 * g4 + 1] : t[4 * g4 + 1] + p.y;
+        t[4 * g4 + 2] = KH ? p.z + t[4 * g4 + 2] : t[4 * g4 + 2] + p.z;
+        t[4 * g4 + 3] = KH ? p.w + t[4 * g4 + 3] : t[4 * g4 + 3] + p.w;
+      }
+  __syncthreads();   // the hand-over regions have been read: they carry the up sums next
+  float4* up = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + lane;
+  if (nh == 1) {
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++)
+#pragma unroll
+      for (int c = 0; c < 3; c++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const float16_t& t = acc[2 * KH + rr][c];
+          up[((rr * 3 + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
+        }
+  }
+  __syncthreads();
+  if (nh != 0) return;
+  const bool vec = (out_dim & 3u) == 0;
+#pragma unroll
+  for (int rr = 0; rr < 2; rr++) {
+    const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const float16_t& t = acc[2 * KH + rr][c];
+        const float4 u = up[((rr * 3 + c) * 4 + g4) * 64];
+        const float4 o = make_float4(swiglu_one(t[4 * g4], u.x), swiglu_one(t[4 * g4 + 1], u.y), swiglu_one(t[4 * g4 + 2], u.z),
+                                     swiglu_one(t[4 * g4 + 3], u.w));
+        const u32 n = nt * (GEMM_BN / 2) + 32 * c + 8 * g4 + 4 * kg;
+        if (token < m && n < out_dim) {
+          float* dst = out + (size_t)token * out_dim + n;
+          if (vec && n + 4 <= out_dim) {
+            *reinterpret_cast<float4*>(dst) = o;
+          } else {
+            const float ov[4] = {o.x, o.y, o.z, o.w};
+            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e];
+          }
+        }
+      }
+  }
 }
 
 // raw bytes of one group of one super-block of one weight row, as a lane sees them
@@ -227,9 +310,12 @@ struct GemmRawT<true> {   // Q5_K: plus the 32 bytes of fifth bits (bit 2g + hi 
 
 // Q5 = false: Q4_K (144-byte super-blocks, everything through gemm_wbuf); true: Q5_K (176 bytes; same nibbles, groups and
 // x order, one more bit per value).
-template <bool Q5>
+// SWIGLU (Q4_K): rows 0..95 of the tile are rows [96 nt, 96 nt + 96) of `w` (gate), rows 96..191 the same rows of `w_b` (up);
+// the epilogue stores silu(gate) * up. No k split and no bias then.
+template <bool Q5, bool SWIGLU = false>
 __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim,
-                                              u32 out_dim, u32 m) {
+                                              u32 out_dim, u32 m, u32 bias_stride = 0, const uint8_t* w_b = nullptr) {
+  static_assert(!(Q5 && SWIGLU), "the gate | up kernel is built for Q4_K");
   constexpr u32 BS = Q5 ? 176 : 144;      // bytes of a super-block
   constexpr u32 PPR = Q5 ? 10 : 9;        // 16-byte pieces of a row that go through LDS
   constexpr int NCOPY = Q5 ? 8 : 7;       // copies of 64 pieces a wavefront issues per super-block
@@ -246,7 +332,8 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   const u32 nkb_all = in_dim >> 8;
   const u32 kb0 = blockIdx.y * nkb_all / gridDim.y, nkb = (blockIdx.y + 1) * nkb_all / gridDim.y - kb0;
   out += (size_t)blockIdx.y * m * out_dim;
-  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_BN - 1) / GEMM_BN;
+  constexpr u32 TILE_ROWS = SWIGLU ? GEMM_BN / 2 : GEMM_BN;   // rows of a matrix a tile covers
+  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + TILE_ROWS - 1) / TILE_ROWS;
   // Workgroup -> tile, XCD-aware. Workgroups go to the 8 XCDs round-robin (id % 8) and each XCD has its own
   // L2, so the tiles are numbered token-tile-major and XCD x takes the contiguous run [x*per, (x+1)*per):
   // the workgroups that share an L2 then share one or two x tiles (1 MiB each at in_dim 4096), which stay
@@ -274,14 +361,21 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   // Weight copies: piece p = 64 i + lane of the tile's super-block, i = wave, wave + 4, ... (27 copies of 64 pieces per
   // workgroup and super-block; every wavefront issues 7, the 28th repeats the last piece into spare LDS so that no
   // copy is conditional). Piece p is bytes [16 (p % 9), +16) of row p / 9.
-  const u32 tile_row0 = min(nt * GEMM_BN, out_dim - 1);
+  const u32 tile_row0 = min(nt * TILE_ROWS, out_dim - 1);
   const uint8_t* wbase = w + (size_t)tile_row0 * row_bytes + (size_t)kb0 * BS;   // uniform
   u32 woff[NCOPY];
+  const uint8_t* wsrc[SWIGLU ? NCOPY : 1];   // gate | up: the two matrices are separate allocations, a piece has a full address
 #pragma unroll
   for (int i = 0; i < NCOPY; i++) {
     const u32 p = min((4u * i + wave) * 64u + lane, (u32)GEMM_BN * PPR - 1u);
     const u32 r = p / PPR, part = p - PPR * r;
-    woff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part + (Q5 ? 16u : 0u);
+    if constexpr (SWIGLU) {
+      const u32 row = min(nt * TILE_ROWS + (r < TILE_ROWS ? r : r - TILE_ROWS), out_dim - 1);
+      wsrc[i] = (r < TILE_ROWS ? w : w_b) + (size_t)row * row_bytes + 16u * part;
+      woff[i] = 0;
+    } else {
+      woff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part + (Q5 ? 16u : 0u);
+    }
   }
   // where this lane finds the raw bytes of its three rows in gemm_wbuf (in uint4 units): header, then the 32 bytes of
   // its group
@@ -303,8 +397,11 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
   auto copy_w = [&](u32 kb, int i) {   // copy i of this wavefront for super-block kb
-    __builtin_amdgcn_global_load_lds((gbl_void*)(wbase + (size_t)kb * BS + woff[i]),
-                                     (lds_void*)(wbuf + (4 * i + wave) * 64), 16, 0, 0);
+    if constexpr (SWIGLU)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(wsrc[i] + (size_t)kb * BS), (lds_void*)(wbuf + (4 * i + wave) * 64), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((gbl_void*)(wbase + (size_t)kb * BS + woff[i]),
+                                       (lds_void*)(wbuf + (4 * i + wave) * 64), 16, 0, 0);
   };
   uint4 nhdr[3];   // Q5_K: headers of the super-block being copied
   auto load_hdr = [&](u32 kb, int c) {
@@ -509,23 +606,34 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   }
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
-  gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid);
+  if constexpr (SWIGLU) {
+    if (kh == 0) gemm_epilogue_swiglu_half<0>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
+    else gemm_epilogue_swiglu_half<1>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
+  } else {
+    gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
+  }
 }
 
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_f16(
-    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
-  gemm_k45_core<false>(w, xp, bias, out, in_dim, out_dim, m);
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_k45_core<false>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }
 // Q5_K: x is packed by pack_x_f16_q4k (the values of a super-block sit where the Q4_K ones do).
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q5_k_gemm_f16(
-    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
-  gemm_k45_core<true>(w, xp, bias, out, in_dim, out_dim, m);
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_k45_core<true>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+}
+// gate | up of a feed-forward block against one packed x, silu(gate) * up stored: no gate and up matrices in memory.
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_f16(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<false, true>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up);
 }
 
-// Sum of the k-split planes: out[i] = (bias ? bias[i % out_dim] : 0) + partials[0][i] + partials[1][i] + ... in that order
+// Sum of the k-split planes: out[i] = (bias ? bias[bias_stride ? i : i % out_dim] : 0) + partials[0][i] + partials[1][i] + ... in that order
 // (the result does not depend on which workgroup finished first). block 256, grid ceil(total / 1024); 4 elements per lane.
-extern "C" __global__ __launch_bounds__(256) void gemm_sum_splits_f32(const float* __restrict__ partials, const float* __restrict__ bias,
-                                                                       float* __restrict__ out, u32 total, u32 out_dim, u32 splits) {
+// (bias and out are not __restrict__: a residual may be `out` itself; a thread reads only the elements it writes)
+extern "C" __global__ __launch_bounds__(256) void gemm_sum_splits_f32(const float* __restrict__ partials, const float* bias,
+                                                                       float* out, u32 total, u32 out_dim, u32 splits, u32 bias_stride) {
   const u32 i = (blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= total) return;
   if (i + 4 <= total && (total & 3u) == 0) {
@@ -535,14 +643,18 @@ extern "C" __global__ __launch_bounds__(256) void gemm_sum_splits_f32(const floa
       a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
     }
     if (bias) {
-      a.x += bias[i % out_dim]; a.y += bias[(i + 1) % out_dim]; a.z += bias[(i + 2) % out_dim]; a.w += bias[(i + 3) % out_dim];
+      if (bias_stride) {   // a [m][out_dim] residual: element for element
+        a.x += bias[i]; a.y += bias[i + 1]; a.z += bias[i + 2]; a.w += bias[i + 3];
+      } else {
+        a.x += bias[i % out_dim]; a.y += bias[(i + 1) % out_dim]; a.z += bias[(i + 2) % out_dim]; a.w += bias[(i + 3) % out_dim];
+      }
     }
     *reinterpret_cast<float4*>(out + i) = a;
   } else {
     for (u32 e = i; e < total && e < i + 4; e++) {
       float a = partials[e];
       for (u32 s = 1; s < splits; s++) a += partials[(size_t)s * total + e];
-      out[e] = a + (bias ? bias[e % out_dim] : 0.0f);
+      out[e] = a + (bias ? bias[bias_stride ? e : e % out_dim] : 0.0f);
     }
   }
 }

@@ -2,7 +2,7 @@
 // out[m][n] = (bias[n] +) sum_k x[m][k] * deq(W[n][k]) (src/ml/gguf/kernels/gemm_q4k.metal:615-776 is the reference's
 // prefill kernel; precision as there: x and the dequantized weights rounded to half, fp32 accumulation).
 //
-//   q4_k_gemm_wide_f16 (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
+//   q4_k_gemm_wide_f16 (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32, bias_stride:u32)
 //                      block 512, grid 8 * ceil(ceil(m/128) * ceil(out_dim/256) / 8), no dynamic LDS (136 KiB static)
 //   xp is the image pack_x_f16_q4k writes (gemm_q4k.hpp); bias as for q4_k_gemm_f16; no k split.
 //
@@ -36,7 +36,7 @@ __shared__ uint4 gemm_wide_wbuf[8 * 256];   // [wavefront][64 rows][4 pieces]
 // into x buffer 0, kh = 1 into x buffer 1: 4 x 16 KiB each). Sum first, bias second.
 template <int KH>
 __device__ __forceinline__ void gemm_wide_epilogue_half(float16_t (&acc)[4][2], const float* bias, float* out, u32 out_dim, u32 m,
-                                                        u32 mt, u32 nt, u32 nh, u32 j, u32 kg, u32 lane) {
+                                                        u32 mt, u32 nt, u32 nh, u32 j, u32 kg, u32 lane, u32 bias_stride) {
   float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * 16 * 64 + lane;
   const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * 16 * 64 + lane;
 #pragma unroll
@@ -65,9 +65,10 @@ __device__ __forceinline__ void gemm_wide_epilogue_half(float16_t (&acc)[4][2], 
         const u32 n = nt * GEMM_WIDE_BN + nh * 64 + 32 * c + 8 * g4 + 4 * kg;
         if (token < m && n < out_dim) {
           float* dst = out + (size_t)token * out_dim + n;
+          const float* b = bias ? bias + (size_t)token * bias_stride + n : nullptr;   // bias, or a residual (stride out_dim)
           if (n + 4 <= out_dim) {
-            if (bias) {
-              o.x += bias[n]; o.y += bias[n + 1]; o.z += bias[n + 2]; o.w += bias[n + 3];
+            if (b) {
+              o.x += b[0]; o.y += b[1]; o.z += b[2]; o.w += b[3];
             }
             if (vec) {
               *reinterpret_cast<float4*>(dst) = o;
@@ -76,7 +77,7 @@ __device__ __forceinline__ void gemm_wide_epilogue_half(float16_t (&acc)[4][2], 
             }
           } else {
             const float ov[4] = {o.x, o.y, o.z, o.w};
-            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (bias ? bias[n + e] : 0.0f);
+            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (b ? b[e] : 0.0f);
           }
         }
       }
@@ -84,7 +85,7 @@ __device__ __forceinline__ void gemm_wide_epilogue_half(float16_t (&acc)[4][2], 
 }
 
 extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void q4_k_gemm_wide_f16(
-    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
   constexpr u32 BS = 144;
   const u32 tid = threadIdx.x, lane = tid & 63;
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -292,6 +293,6 @@ extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(
   }
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
-  if (kh == 0) gemm_wide_epilogue_half<0>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, lane);
-  else gemm_wide_epilogue_half<1>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, lane);
+  if (kh == 0) gemm_wide_epilogue_half<0>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, lane, bias_stride);
+  else gemm_wide_epilogue_half<1>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, lane, bias_stride);
 }

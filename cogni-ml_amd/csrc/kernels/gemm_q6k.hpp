@@ -4,7 +4,7 @@
 // x as fp16 in LDS (two 64 KiB buffers filled by global_load_lds_dwordx4). What differs is the weight side:
 //
 //   pack_x_f16_q6k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 16 * in_dim/256
-//   q6_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32)
+//   q6_k_gemm_f16   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32, bias_stride:u32; as q4_k_gemm_f16)
 //                   block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), no dynamic LDS (128 KiB static)
 //
 // A Q6_K super-block (210 bytes, 2-byte aligned: ql[128], qh[64], scales:i8[16], d:f16; src/ml/gguf/dequant.cr:197-236)
@@ -55,7 +55,7 @@ __shared__ uint4 gemm_wbuf6[GEMM_BN * 9];
 __shared__ u32 gemm_wsc6[GEMM_BN * 6];
 
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_f16(
-    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m) {
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
   const u32 tid = threadIdx.x, lane = tid & 63;
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const u32 nh = wave & 1, kh = wave >> 1;
@@ -272,5 +272,5 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     iteration(kb + 1, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
   }
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
-  gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid);
+  gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
 }

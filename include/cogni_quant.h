@@ -327,7 +327,8 @@ int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uin
  * other tokens of the call are not affected. `workspace` is caller-owned device memory of at least
  * cogni_gemm_workspace_bytes(...) bytes (x repacked as fp16, in the k order of the weight type); nothing is allocated.
  * Kernels: pack_x_f16_q4k (Q4_K and Q5_K) | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
- *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens), block 256,
+ *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens,
+ *          bias_stride: 0 for a [out_dim] bias, out_dim for a [tokens][out_dim] residual), block 256,
  *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/192)/8), no dynamic shared memory; or, for Q4_K launches that fill
  *          whole rounds of 128 x 256 tiles (cogni_gemm_plan says which), q4_k_gemm_wide_f16 (same arguments), block 512,
  *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/256)/8).
@@ -336,7 +337,7 @@ size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tok
 /* The workspace size with which cogni_gemm_dev may also split the k range: a launch with fewer than 128 tiles of
  * 128 tokens x 192 rows (few tokens, or a short out_dim such as the 12288 -> 4096 down projection) would leave most
  * compute units idle, so up to 8 workgroups per tile each take a run of super-blocks (at least two), write their sums
- * to planes behind the packed activations, and gemm_sum_splits_f32 (planes, bias, out, tokens*out_dim, out_dim, splits;
+ * to planes behind the packed activations, and gemm_sum_splits_f32 (planes, bias, out, tokens*out_dim, out_dim, splits, bias_stride;
  * block 256, grid ceil(tokens*out_dim/1024)) adds the planes in a fixed order, so results repeat from run to run.
  * The GEMM kernels take the split as gridDim.y. Equal to cogni_gemm_workspace_bytes(...) where no split applies; with a
  * workspace smaller than this, cogni_gemm_dev runs unsplit. No counterpart in the reference (its Metal GEMM does not
@@ -355,6 +356,22 @@ int cogni_gemm_packed_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, s
                           uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
                    uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream);
+/* The prefill forms of the fused decode operators, for a feed-forward block at more tokens than the GEMV path takes
+ * (src/ml/gguf/qwen35_cpu.cr:1711-1722 is the sequence, src/ml/gguf/kernels/gemm_mm.metal:651 `simd_mm_q6k_f32out_add`
+ * and gemm_q4k.metal:1233 `simd_mm_q4k_h16_b64_swiglu` the reference's kernels), both against activations
+ * cogni_gemm_pack_dev has packed:
+ *   cogni_gemm_packed_add_dev     out[m][o] = residual[m][o] + sum_j x[m][j] * deq(W[o][j]); residual is [tokens][out_dim]
+ *                                 fp32 and may be `out` itself. The same kernels as cogni_gemm_packed_dev with their
+ *                                 last argument (bias_stride) set to out_dim instead of 0.
+ *   cogni_gemm_packed_swiglu_dev  out[m][o] = silu(g) * u, g = x[m] . W_gate[o], u = x[m] . W_up[o] (Q4_K; two matrices of
+ *                                 out_dim rows; the sums as cogni_gemm_packed_dev gives them, silu as swiglu_f32): the
+ *                                 gate and up matrices never exist in memory. Kernel q4_k_gemm_swiglu_f16 (w_gate, w_up,
+ *                                 workspace, out, in_dim, out_dim, tokens), block 256, grid
+ *                                 8*ceil(ceil(tokens/128)*ceil(out_dim/96)/8). Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
+int cogni_gemm_packed_add_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t residual, uint64_t out,
+                              uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
+int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
+                                 uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 /* The launch cogni_gemm_packed_dev makes for a shape and a workspace of `workspace_bytes`: kernel name, grid (x: tiles,
  * y: k splits; with y > 1 gemm_sum_splits_f32 follows) and block, for hosts that launch by name (level 1) and for
  * callers who want to know which of the two Q4_K tilings a shape gets. Any out pointer may be null. The counterpart of

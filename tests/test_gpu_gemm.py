@@ -141,6 +141,70 @@ def test_wide_tiles(gpu, oracle, tokens, out_dim, in_dim, with_bias):
         assert np.array_equal(part, got[:, rows]), r0
 
 
+@pytest.mark.parametrize("t,tokens,out_dim,in_dim", [(Q4_K, 130, 400, 768), (Q6_K, 64, 384, 4096), (Q5_K, 40, 100, 512),
+                                                     (Q4_K, 128, 65536, 256), (Q6_K, 512, 4096, 2048)])
+def test_residual_add_in_the_epilogue(gpu, oracle, t, tokens, out_dim, in_dim):
+    """cogni_gemm_packed_add_dev: the GEMM's sums plus a [tokens][out_dim] residual, unsplit, k-split (the plane sum adds it)
+    and on the wide tiles; the bits of the plain GEMM followed by an fp32 add, also when the residual is the output buffer."""
+    rng = np.random.default_rng(tokens + out_dim)
+    raw = synth.make_weights(rng, t, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = (rng.standard_normal(tokens * out_dim) * 30).astype(np.float32)
+    plain = run_gemm(raw, x, in_dim, out_dim, tokens, t=t)
+    wsb = quant.gemm_workspace_bytes(t, in_dim, tokens, out_dim)
+    w, xd, ws = DevArray(raw), DevArray(x), DevArray(nbytes=wsb)
+    rd, od = DevArray(res), DevArray(nbytes=4 * tokens * out_dim)
+    quant.gemm_pack_dev(xd.ptr, t, in_dim, tokens, ws.ptr, wsb)
+    quant.gemm_packed_add_dev(w.ptr, t, ws.ptr, wsb, rd.ptr, od.ptr, in_dim, out_dim, tokens)
+    got = od.read(np.float32, tokens * out_dim)
+    assert np.array_equal(got, plain + res)
+    quant.gemm_packed_add_dev(w.ptr, t, ws.ptr, wsb, rd.ptr, rd.ptr, in_dim, out_dim, tokens)      # in place
+    assert np.array_equal(rd.read(np.float32, tokens * out_dim), got)
+    sample = [0, 1, tokens // 2, tokens - 1]
+    xs = np.ascontiguousarray(x.reshape(tokens, in_dim)[sample].reshape(-1))
+    want = oracle.matmul_add(xs, len(sample), in_dim, raw, t, out_dim, np.zeros(out_dim, dtype=np.float32), threads=16).reshape(len(sample), out_dim)
+    want = want + res.reshape(tokens, out_dim)[sample]
+    assert np.max(np.abs(got.reshape(tokens, out_dim)[sample] - want)) <= 2e-3 * np.max(np.abs(want))
+    with pytest.raises(quant.QuantError, match="null device pointer"):
+        quant.gemm_packed_add_dev(w.ptr, t, ws.ptr, wsb, 0, od.ptr, in_dim, out_dim, tokens)
+    for a in (w, xd, ws, rd, od):
+        a.close()
+
+
+@pytest.mark.parametrize("tokens,out_dim,in_dim", [(130, 200, 512), (9, 96, 256), (64, 12288, 4096), (512, 12288, 4096), (257, 1000, 768)])
+def test_gate_up_swiglu_in_one_gemm(gpu, oracle, tokens, out_dim, in_dim):
+    """cogni_gemm_packed_swiglu_dev: silu(x W_gate^T) * (x W_up^T) without the two matrices in memory. The bits of the two
+    GEMMs followed by swiglu_f32 (same sums in the same order, the same device function), clipped tiles in both directions
+    and an odd number of super-blocks; against the oracle's CPU form on a sample of tokens."""
+    rng = np.random.default_rng(tokens * 7 + out_dim)
+    raw_g = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    raw_u = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    n = tokens * out_dim
+    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens)          # packed activations only: the two plain GEMMs run unsplit
+    wg, wu, xd, ws = DevArray(raw_g), DevArray(raw_u), DevArray(x), DevArray(nbytes=wsb)
+    og, ou, o2, of = (DevArray(nbytes=4 * n) for _ in range(4))
+    quant.gemm_pack_dev(xd.ptr, Q4_K, in_dim, tokens, ws.ptr, wsb)
+    quant.gemm_packed_dev(wg.ptr, Q4_K, ws.ptr, wsb, og.ptr, in_dim, out_dim, tokens)
+    quant.gemm_packed_dev(wu.ptr, Q4_K, ws.ptr, wsb, ou.ptr, in_dim, out_dim, tokens)
+    quant.swiglu_dev(og.ptr, ou.ptr, o2.ptr, n)
+    quant.gemm_packed_swiglu_dev(wg.ptr, wu.ptr, Q4_K, ws.ptr, wsb, of.ptr, in_dim, out_dim, tokens)
+    fused, two_step = of.read(np.float32, n), o2.read(np.float32, n)
+    assert np.array_equal(fused, two_step)
+    sample = sorted({t_ for t_ in (0, 1, 31, 32, tokens // 2, tokens - 1) if t_ < tokens})
+    xs = np.ascontiguousarray(x.reshape(tokens, in_dim)[sample].reshape(-1))
+    zero = np.zeros(out_dim, dtype=np.float32)
+    ref = oracle.swiglu(oracle.matmul_add(xs, len(sample), in_dim, raw_g, Q4_K, out_dim, zero, threads=16),
+                        oracle.matmul_add(xs, len(sample), in_dim, raw_u, Q4_K, out_dim, zero, threads=16))
+    got = fused.reshape(tokens, out_dim)[sample].reshape(-1)
+    assert cosine(got, ref) >= 0.9999
+    assert np.max(np.abs(got - ref)) <= 4e-3 * np.max(np.abs(ref))      # a product of two sums that each carry 2e-3
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for the fused gate/up SwiGLU GEMM: Q6_K"):
+        quant.gemm_packed_swiglu_dev(wg.ptr, wu.ptr, Q6_K, ws.ptr, wsb, of.ptr, in_dim, out_dim, tokens)
+    for a in (wg, wu, xd, ws, og, ou, o2, of):
+        a.close()
+
+
 def test_projections_share_one_packed_activation_block(gpu, oracle):
     """gemm_pack_dev once, then gemm_packed_dev for several matrices of one type family (Q4_K and Q5_K read the same packed
     layout; a k-split and an unsplit shape, with and without bias): the bits of gemm_dev on each matrix alone."""
