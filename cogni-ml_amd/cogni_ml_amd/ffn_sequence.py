@@ -6,6 +6,11 @@ ResidentSequenceRunner. Where the reference launches gate, up, the activation an
 a group of up to four tokens here is two launches (gate | up | SwiGLU fused, then down with the residual add); an FFN width
 that is not a multiple of 16 goes through the weight-stationary kernels for several tokens (gate | up pair, swiglu_f32, down).
 
+A sequence of more tokens than the GEMM threshold (quant.get_gemm_threshold()) is the prefill form of the same block, all
+tokens at once in four launches: the activations packed, gate | up as one GEMM with SwiGLU in its epilogue, the result
+packed in the down matrix's layout, the down GEMM with the residual added in its epilogue (src/ml/gguf/qwen35_cpu.cr:1711-1722;
+the reference's Metal kernels gemm_q4k.metal:1233 and gemm_mm.metal:651).
+
 With `norm` and `add` the sequence is the whole FFN half of a decoder layer (src/ml/gguf/qwen35_cpu.cr:1705-1725):
 r = x + add (the attention output joining the residual stream), h = rmsnorm(r, norm), out = r + down(silu(gate h) * up h).
 """
@@ -49,6 +54,13 @@ class FFNSequenceRunner:
         self._up = self._alloc(4 * tokens * ffn_dim)
         self._act = self._alloc(4 * tokens * ffn_dim)
         self._out = self._alloc(4 * tokens * hidden)
+        # prefill: workspaces for x (Q4_K layout) and for the SwiGLU output (the down matrix's layout, with its k-split planes)
+        self._ws_x = self._ws_act = None
+        gemm_types = (int(TensorType.Q4_K), int(TensorType.Q5_K), int(TensorType.Q6_K))
+        if tokens > quant.get_gemm_threshold() and hidden % 256 == 0 and ffn_dim % 256 == 0 and int(down_type) in gemm_types:
+            self._ws_x_bytes = quant.gemm_workspace_bytes(TensorType.Q4_K, hidden, tokens)
+            self._ws_act_bytes = quant.gemm_workspace_bytes(down_type, ffn_dim, tokens, hidden)
+            self._ws_x, self._ws_act = self._alloc(self._ws_x_bytes), self._alloc(self._ws_act_bytes)
         self.combined = self.out = None
         self._runner = hip.ResidentSequenceRunner(tokens, self._upload_weights, self._reset_sequence, self._run_token,
                                                   self._read_outputs, self._run_sequence)
@@ -99,10 +111,31 @@ class FFNSequenceRunner:
         res = self._res.ptr + 4 * tok0 * h if self._res is not None else 0
         quant.gemv_dev(self._w["down"].ptr, self.down_type, act, self._out.ptr + 4 * tok0 * h, f, h, count, res, st)
 
+    def _launch_prefill(self, count):
+        st = hip.current_stream_handle()
+        h, f = self.hidden, self.ffn_dim
+        x = self._x.ptr
+        if self._norm is not None:
+            quant.add_rmsnorm_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, self._normed.ptr, h, count, self._eps, st)
+            x = self._normed.ptr
+        quant.gemm_pack_dev(x, TensorType.Q4_K, h, count, self._ws_x.ptr, self._ws_x_bytes, st)
+        quant.gemm_packed_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, self._ws_x.ptr, self._ws_x_bytes,
+                                     self._act.ptr, h, f, count, st)
+        quant.gemm_pack_dev(self._act.ptr, self.down_type, f, count, self._ws_act.ptr, self._ws_act_bytes, st)
+        if self._res is not None:
+            quant.gemm_packed_add_dev(self._w["down"].ptr, self.down_type, self._ws_act.ptr, self._ws_act_bytes, self._res.ptr,
+                                      self._out.ptr, f, h, count, st)
+        else:
+            quant.gemm_packed_dev(self._w["down"].ptr, self.down_type, self._ws_act.ptr, self._ws_act_bytes, self._out.ptr, f, h,
+                                  count, 0, st)
+
     def _run_token(self, tok):
         self._launch(tok, 1)
 
     def _run_sequence(self, active_tokens):
+        if self._ws_x is not None and active_tokens > quant.get_gemm_threshold():
+            self._launch_prefill(active_tokens)
+            return
         for tok0 in range(0, active_tokens, quant.MAX_GEMV_TOKENS):
             self._launch(tok0, min(quant.MAX_GEMV_TOKENS, active_tokens - tok0))
 
@@ -131,9 +164,13 @@ class FFNSequenceRunner:
 
     def bytes_per_sequence(self):
         """Algorithmic bytes: the three matrices once per group of up to 8 tokens, x and residual in, out out."""
-        groups = -(-self.tokens // quant.MAX_GEMV_TOKENS)
+        groups = 1 if (self._ws_x is not None and self.tokens > quant.get_gemm_threshold()) else -(-self.tokens // quant.MAX_GEMV_TOKENS)
         vec = 4 * self.tokens * self.hidden * (4 if self._norm is not None else 3 if self._res is not None else 2)
         return groups * sum(r.size for r in self._raw.values()) + vec
+
+    def flops_per_sequence(self):
+        """Multiply-adds x 2 of the three projections for every token."""
+        return 2.0 * self.tokens * 3 * self.hidden * self.ffn_dim
 
     def close(self):
         for b in self._buffers:

@@ -8,7 +8,10 @@ launched back to back into the current stream, and the lifecycle goes through Re
 
 Where the reference runs either one launch per token or weight-stationary groups of 4 tokens
 (`tbatch4`, qwen_full_attn_projection_runner.cr:274-301), this runner hands groups of up to 8 tokens
-to one weight-stationary launch.
+to one weight-stationary launch. A sequence of more tokens than the GEMM threshold (quant.get_gemm_threshold(), 8 as
+in the reference's router) goes through the prefill GEMMs instead, all tokens at once: every distinct input is packed
+once (q | k | v and gate | up share x) and each projection is one GEMM against it - the reference's
+`qmatmul_nobias(qw, x, batch)` calls of a prefill layer (src/ml/gguf/qwen35_cpu.cr:1478-1490).
 """
 import numpy as np
 
@@ -65,6 +68,15 @@ class QwenProjectionStackRunner:
             nbytes = quant.gemv_image_bytes(t, in_dim, quant.MAX_GEMV_TOKENS)
             if nbytes and (src, int(t)) not in self._images:
                 self._images[(src, int(t))] = self._alloc(nbytes)
+        # prefill: one workspace per (input, packed layout) - Q4_K and Q5_K read one layout, Q6_K its own - large enough
+        # for the k-split planes of the projection that needs the most
+        self._prefill_ws = {}
+        if tokens > quant.get_gemm_threshold() and all(self._gemm_capable(e) for e in weights.entries):
+            need = {}
+            for name, src, t, out_dim, in_dim, raw in weights.entries:
+                key = (src, self._family(t))
+                need[key] = max(need.get(key, 0), quant.gemm_workspace_bytes(t, in_dim, tokens, out_dim))
+            self._prefill_ws = {k: (self._alloc(n), n) for k, n in need.items()}
         self.outputs = {}
         self._runner = hip.ResidentSequenceRunner(
             tokens, self._upload_weights, self._reset_sequence, self._run_token, self._read_outputs,
@@ -131,10 +143,33 @@ class QwenProjectionStackRunner:
                            self._act[name].ptr + 4 * tok0 * out_dim, in_dim, out_dim, count, 0, stream)
             i += 1
 
+    @staticmethod
+    def _family(t):
+        return "q6" if int(t) == int(TensorType.Q6_K) else "q45"
+
+    @staticmethod
+    def _gemm_capable(entry):
+        return int(entry[2]) in (int(TensorType.Q4_K), int(TensorType.Q5_K), int(TensorType.Q6_K)) and entry[4] % 256 == 0
+
+    def _launch_prefill(self, count):
+        """All `count` tokens through the GEMMs: one pack per (input, layout), one GEMM per projection."""
+        stream = hip.current_stream_handle()
+        packed = set()
+        for name, src, t, out_dim, in_dim, raw in self.weights.entries:
+            key = (src, self._family(t))
+            ws, nbytes = self._prefill_ws[key]
+            if key not in packed:
+                quant.gemm_pack_dev(self._act[src].ptr, t, in_dim, count, ws.ptr, nbytes, stream)
+                packed.add(key)
+            quant.gemm_packed_dev(self._w[name].ptr, t, ws.ptr, nbytes, self._act[name].ptr, in_dim, out_dim, count, 0, stream)
+
     def _run_token(self, tok):
         self._launch(tok, 1)
 
     def _run_sequence(self, active_tokens):
+        if self._prefill_ws and active_tokens > quant.get_gemm_threshold():
+            self._launch_prefill(active_tokens)
+            return
         for tok0 in range(0, active_tokens, quant.MAX_GEMV_TOKENS):
             self._launch(tok0, min(quant.MAX_GEMV_TOKENS, active_tokens - tok0))
 
@@ -183,7 +218,7 @@ class QwenProjectionStackRunner:
     def bytes_per_sequence(self, active_tokens=None):
         """Algorithmic bytes of one run_sequence: every weight once per group of up to 8 tokens, x in, out out."""
         m = self.tokens if active_tokens is None else active_tokens
-        groups = -(-m // quant.MAX_GEMV_TOKENS)
+        groups = 1 if (self._prefill_ws and m > quant.get_gemm_threshold()) else -(-m // quant.MAX_GEMV_TOKENS)
         total = 0
         for name, src, t, out_dim, in_dim, raw in self.weights.entries:
             total += groups * raw.size + 4 * m * (in_dim + out_dim)
