@@ -246,25 +246,34 @@ def gemv_record(r, bytes_per_step):
 
 
 def bench_gemm(hip, quant, synth, rng, stream, w_type, tokens, out_dim, in_dim, steps, warmup, graph=True):
-    """Prefill GEMM (x repack + MFMA kernel, every launch of the call) at `tokens`; returns the case record."""
+    """Prefill GEMM (x repack + MFMA kernel, every launch of the call) at `tokens`; returns the case record. Consecutive
+    steps read different copies of the weights, as the GEMV cases do, so that a step's weights come from HBM and not from
+    the last-level cache the previous step left them in."""
     raw = synth.make_weights(rng, w_type, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
     wsb = quant.gemm_workspace_bytes(w_type, in_dim, tokens, out_dim)
-    bufs = [hip.DeviceBuffer(n) for n in (raw.nbytes, x.nbytes, 4 * tokens * out_dim, wsb)]
-    hip.copy_htod(bufs[0].ptr, raw, raw.nbytes, "w")
-    hip.copy_htod(bufs[1].ptr, x, x.nbytes, "x")
+    copies = int(max(2, min(24, -(-int(1.2 * LLC_BYTES) // raw.nbytes))))
+    wbufs = []
+    for c in range(copies):
+        b = hip.DeviceBuffer(raw.nbytes)
+        hip.copy_htod(b.ptr, raw if c == 0 else np.roll(raw, 4096 * c + 17), raw.nbytes, "w")
+        wbufs.append(b)
+    bufs = [hip.DeviceBuffer(n) for n in (x.nbytes, 4 * tokens * out_dim, wsb)]
+    hip.copy_htod(bufs[0].ptr, x, x.nbytes, "x")
 
     def launch(copy, st):
-        quant.gemm_dev(bufs[0].ptr, w_type, bufs[1].ptr, bufs[2].ptr, in_dim, out_dim, tokens, bufs[3].ptr, wsb, 0,
+        quant.gemm_dev(wbufs[copy].ptr, w_type, bufs[0].ptr, bufs[1].ptr, in_dim, out_dim, tokens, bufs[2].ptr, wsb, 0,
                        st.handle)
-    r = measure(hip, stream, Rotating(launch, 1, raw.nbytes), steps, warmup, graph)
-    for b in bufs:
+    r = measure(hip, stream, Rotating(launch, copies, raw.nbytes), steps, warmup, graph)
+    kernel, grid_x, splits, block = quant.gemm_plan(w_type, in_dim, out_dim, tokens, wsb)
+    for b in bufs + wbufs:
         b.close()
     flops = 2.0 * tokens * out_dim * in_dim
     tf = flops / r["us"] / 1e6
     return {"us": round(r["us"], 2), "us_min": round(r["us_min"], 2), "us_max": round(r["us_max"], 2),
             "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
             "samples": r["samples"], "timed_region_ms": round(r["timed_region_ms"], 2),
+            "kernel": kernel, "grid": [grid_x, splits], "block": block, "weight_copies_rotated": r["buffers_rotated"],
             "includes": "activation repack + GEMM (+ plane sum where the k range is split)"}
 
 
@@ -462,6 +471,34 @@ def main():
         cases["cfg4 q4_k gemm 12288x4096 M=%d" % tokens] = rec
         log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
             tokens, gsteps, rec["us"], rec["tflops"], rec["frac_mfma_f16"]))
+    # the feed-forward block of a layer at M = 512 in its prefill form: add + RMSNorm, pack, gate | up GEMM with SwiGLU inside,
+    # pack, Q6_K down GEMM with the residual inside (three rotating sets of weights: 290 MB)
+    from cogni_ml_amd.ffn_sequence import FFNSequenceRunner as _FFN
+    ffn_tokens = 512
+    fx = rng.uniform(-0.1, 0.1, ffn_tokens * 4096).astype(np.float32)
+    fnorm = np.full(4096, 0.1, dtype=np.float32)
+    ffns = []
+    for _ in range(3):
+        fr = _FFN(synth.make_weights(rng, Q4_K, 12288, 4096), synth.make_weights(rng, Q4_K, 12288, 4096),
+                  synth.make_weights(rng, Q6_K, 4096, 12288), 4096, 12288, ffn_tokens, fx, norm=fnorm, add=fx.copy())
+        fr.upload_weights()
+        fr.reset_sequence()
+        ffns.append(fr)
+
+    def ffn_seq(copy, st, ffns=ffns):
+        with hip.with_stream(st):
+            ffns[copy].run_sequence()
+    r = measure(hip, stream, Rotating(ffn_seq, 3, 97 << 20), max(5, min(30, args.steps)), 3)
+    fflops = ffns[0].flops_per_sequence()
+    cases["cfg4 ffn block prefill M=512 (add+rmsnorm, gate|up|swiglu gemm, q6_k down gemm + residual)"] = {
+        "us": round(r["us"], 2), "tflops": round(fflops / r["us"] / 1e6, 1),
+        "frac_mfma_f16": round(fflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "flops": fflops,
+        "launches": "add_rmsnorm, pack, q4_k_gemm_swiglu_f16, pack, q6_k_gemm_f16 (k split) + plane sum with the residual"}
+    log("case=ffn block prefill M=512\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
+        r["us"], fflops / r["us"] / 1e6, fflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS))
+    for fr in ffns:
+        fr.close()
+
     if args.mode == "cases":
         for name, t, o, i in (("q6_k gemm down 4096x12288 M=512", Q6_K, 4096, 12288), ("q5_k gemm 12288x4096 M=512", Q5_K, 12288, 4096)):
             rec = bench_gemm(hip, quant, synth, rng, stream, t, 512, o, i, 50, 5)

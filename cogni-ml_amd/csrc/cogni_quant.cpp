@@ -1000,7 +1000,12 @@ static GemmPlan gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, ui
   // a workspace that holds the packed activations only: one workgroup per tile walks the whole row
   p.splits = gemm_splits(in_dim, out_dim, tokens);
   if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) p.splits = 1;
-  const bool wide = w_type == COGNI_TYPE_Q4_K && p.splits == 1 && gemm_q4k_use_wide(out_dim, tokens);
+  // COGNI_GEMM_WIDE=0 | 1 overrides the rule (a measurement knob: 1 takes the wide tiles for every unsplit Q4_K launch)
+  bool wide = w_type == COGNI_TYPE_Q4_K && p.splits == 1 && gemm_q4k_use_wide(out_dim, tokens);
+  if (const char* e = std::getenv("COGNI_GEMM_WIDE")) {
+    if (e[0] == '0') wide = false;
+    if (e[0] == '1') wide = w_type == COGNI_TYPE_Q4_K && p.splits == 1;
+  }
   p.kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : w_type == COGNI_TYPE_Q5_K ? "q5_k_gemm_f16" : wide ? "q4_k_gemm_wide_f16" : "q4_k_gemm_f16";
   const uint32_t ntiles = wide ? (out_dim + 255) / 256 : (out_dim + 191) / 192;
   p.grid_x = 8 * ((mtiles * ntiles + 7) / 8);

@@ -50,6 +50,32 @@ __device__ __forceinline__ void gemm_wide_epilogue_half(float16_t (&acc)[4][2], 
       }
   __syncthreads();
   const bool vec = (out_dim & 3u) == 0;
+  if (vec && mt * GEMM_BM + GEMM_BM <= m && nt * GEMM_WIDE_BN + GEMM_WIDE_BN <= out_dim) {
+    // a whole tile: one address per token row, the 8 stores of a row at constant offsets from it, 16 bytes each (kept
+    // apart from the general path below so that the compiler cannot merge the two into single-float stores)
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++) {
+      const size_t token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
+      const u32 col = nt * GEMM_WIDE_BN + nh * 64 + 4 * kg;
+      float* base = out + token * out_dim + col;
+      const float* bbase = bias ? bias + token * bias_stride + col : nullptr;
+#pragma unroll
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const float16_t& t = acc[2 * KH + rr][c];
+          const float4 p = theirs[((rr * 2 + c) * 4 + g4) * 64];
+          float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
+                        : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
+          if (bbase) {
+            const float* b = bbase + 32 * c + 8 * g4;
+            o.x += b[0]; o.y += b[1]; o.z += b[2]; o.w += b[3];
+          }
+          *reinterpret_cast<float4*>(base + 32 * c + 8 * g4) = o;
+        }
+    }
+    return;
+  }
 #pragma unroll
   for (int rr = 0; rr < 2; rr++) {
     const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
@@ -66,19 +92,8 @@ __device__ __forceinline__ void gemm_wide_epilogue_half(float16_t (&acc)[4][2], 
         if (token < m && n < out_dim) {
           float* dst = out + (size_t)token * out_dim + n;
           const float* b = bias ? bias + (size_t)token * bias_stride + n : nullptr;   // bias, or a residual (stride out_dim)
-          if (n + 4 <= out_dim) {
-            if (b) {
-              o.x += b[0]; o.y += b[1]; o.z += b[2]; o.w += b[3];
-            }
-            if (vec) {
-              *reinterpret_cast<float4*>(dst) = o;
-            } else {
-              dst[0] = o.x; dst[1] = o.y; dst[2] = o.z; dst[3] = o.w;
-            }
-          } else {
-            const float ov[4] = {o.x, o.y, o.z, o.w};
-            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (b ? b[e] : 0.0f);
-          }
+          const float ov[4] = {o.x, o.y, o.z, o.w};
+          for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (b ? b[e] : 0.0f);
         }
       }
   }
