@@ -22,9 +22,9 @@ only reads the same bytes takes.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
   python bench.py --mode cases      more shapes and fused sequences in the same line
-  python bench.py --mode pmc        plain launches of the dominant kernel and of a copy kernel of
-                                    known size, for rocprofv3 --pmc / --kernel-trace runs
-  python bench.py --mode pmc-gemm   plain launches of the M = 512 prefill GEMM for the same purpose
+  python bench.py --mode pmc        plain launches of the dominant kernels (one-token and one-pass GEMV, prefill GEMM)
+                                    and of a copy kernel of known size, for rocprofv3 --pmc / --kernel-trace runs
+  python bench.py --mode pmc-gemm   plain launches of the M = 512 prefill GEMM alone
   python bench.py --mode ceiling    empty launch, read-only stream, matrix-core-only loop
   python bench.py --launch direct   the same work without HIP graphs (for rocprofv3 --kernel-trace)
 """
@@ -277,6 +277,11 @@ def bench_gemm(hip, quant, synth, rng, stream, w_type, tokens, out_dim, in_dim, 
             "includes": "activation repack + GEMM (+ plane sum where the k range is split)"}
 
 
+def raw_gemm_bytes(tokens, out_dim, in_dim):
+    """Algorithmic bytes of the Q4_K GEMM kernel alone: weights once, packed fp16 x in, fp32 out."""
+    return out_dim * (in_dim // 256) * 144 + 2 * tokens * in_dim + 4 * tokens * out_dim
+
+
 def cpu_baseline(oracle, case, budget_s=10.0, threads=1):
     """The CPU oracle (C restatement of QuantMatmul.matmul_add, f64 accumulation) on the same matrix: one thread, or
     the output rows divided among `threads` host threads."""
@@ -292,15 +297,48 @@ def cpu_baseline(oracle, case, budget_s=10.0, threads=1):
     return ref, reps, el
 
 
-def recorded_traffic():
-    """HBM bytes per launch of the headline kernel as the profiler counted them, from profiles/traffic.json (written
-    from two rocprofv3 --pmc runs; the file names the commit and the command). None if there is no record."""
+def kernel_source_hash():
+    """sha256 (first 16 hex digits) over the kernel sources of the code object: a traffic record counted on other sources
+    is reported as stale."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    base = os.path.join(ROOT, "cogni-ml_amd", "csrc")
+    for path in sorted(glob.glob(os.path.join(base, "kernels", "*.h*")) + [os.path.join(base, "cogni_quant_kernels.hip")]):
+        h.update(open(path, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic(kernel):
+    """HBM bytes per launch of `kernel` as the profiler counted them: the record of that kernel in profiles/traffic.json
+    (written from two rocprofv3 --pmc runs of `bench.py --mode pmc`; the file names the commit and the commands). Returns
+    (bytes or None, record or None); the record carries "stale": true when the kernel sources have changed since."""
     try:
-        rec = json.load(open(TRAFFIC_JSON))
+        doc = json.load(open(TRAFFIC_JSON))
+        rec = dict(doc["kernels"][kernel])
+        rec["commit"] = doc.get("commit")
+        rec["stale"] = doc.get("kernel_source_hash") != kernel_source_hash()
         return int(rec["bytes_per_launch"]), rec
     except Exception as e:
-        log("no recorded traffic (%s)" % e)
+        log("no recorded traffic for %s (%s)" % (kernel, e))
         return None, None
+
+
+def traffic_field(kernel, algorithmic_bytes):
+    """The "traffic" entry of a case record."""
+    nbytes, rec = recorded_traffic(kernel)
+    if rec is None:
+        return None
+    return {"kernel": kernel, "bytes_per_launch": nbytes, "x_algorithmic": round(nbytes / max(1, algorithmic_bytes), 3),
+            "workload": rec.get("workload"), "commit": rec.get("commit"), "stale": rec["stale"]}
+
+
+def gemv_kernel_of(quant, w_type, tokens, in_dim, out_dim):
+    """The kernel that dominates a gemv_dev call of this shape."""
+    frm = quant.gemv_one_pass_from(w_type, in_dim, out_dim)
+    if frm and tokens >= frm:
+        return {Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}[w_type] + "_gemv_mt_f32"
+    return quant.gemv_plan(w_type, min(tokens, 4) if tokens > 1 else 1, in_dim, out_dim)[0]
 
 
 def steps_for(args, bytes_per_step, cap_bytes=6e9):
@@ -346,21 +384,35 @@ def main():
     head = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 1)
 
     if args.mode == "pmc":
-        # plain (uncaptured) launches so a profiler attributes counters per dispatch; the copy kernel moves a
-        # known number of bytes and calibrates the counters' units
+        # plain (uncaptured) launches so a profiler attributes counters per dispatch: the dominant kernel of the headline,
+        # of the Q6_K down projection, of the one-pass decode at 8 tokens and of the prefill GEMM at M = 512 and 2048, each
+        # over rotating weight copies, then a copy kernel that moves a known number of bytes and calibrates the counters' units
         mk = MeasureKernels(hip)
         copy_fn = mk.fn("copy_bytes_16")
         nbytes = 512 << 20
         src, dst = hip.DeviceBuffer(nbytes), hip.DeviceBuffer(nbytes)
         params = hip.KernelParams(ctypes.c_uint64(src.ptr), ctypes.c_uint64(dst.ptr), ctypes.c_uint64(nbytes))
+        n = args.warmup + args.steps
+        for i in range(n):
+            head.launch(i % head.copies, stream)
+        stream.synchronize()
+        for w_type, out_dim, in_dim, tokens in ((Q6_K, 4096, 12288, 1), (Q4_K, 12288, 4096, 8), (Q6_K, 4096, 12288, 8)):
+            c = GemvCase(hip, quant, synth, rng, w_type, out_dim, in_dim, tokens, min_total_bytes=LLC_BYTES + (64 << 20))
+            for i in range(n):
+                c.launch(i % c.copies, stream)
+            stream.synchronize()
+            log("pmc mode: %d x %s %dx%d M=%d -> %s over %d weight copies" % (
+                n, TYPE_NAME[w_type], in_dim, out_dim, tokens, gemv_kernel_of(quant, w_type, tokens, in_dim, out_dim), c.copies))
+            c.close()
+        for tokens in (512, 2048):
+            rec = bench_gemm(hip, quant, synth, rng, stream, Q4_K, tokens, 12288, 4096, max(4, n // 4), 2, graph=False)
+            log("pmc mode: prefill GEMM M=%d -> %s (pack_x_f16_q4k in front), %d weight copies" % (tokens, rec["kernel"], rec["weight_copies_rotated"]))
         with hip.with_stream(stream):
-            for i in range(args.warmup + args.steps):
-                head.launch(i % head.copies, stream)
             for i in range(8):
                 hip.launch(copy_fn, 8192, 1, 1, 256, 1, 1, params, "copy_bytes_16")
         stream.synchronize()
         log("pmc mode: %d x %s over %d weight copies, 8 x copy_bytes_16 of %d bytes" % (
-            args.warmup + args.steps, quant.gemv_kernel_name(Q4_K, 1), head.copies, nbytes))
+            n, quant.gemv_kernel_name(Q4_K, 1), head.copies, nbytes))
         return
 
     if args.mode == "ceiling":
@@ -432,6 +484,9 @@ def main():
         r = measure(hip, stream, c.rotating(), steps, min(args.warmup, steps))
         rec = gemv_record(r, c.bytes_per_step)
         rec["steps"] = steps
+        rec["kernel"] = gemv_kernel_of(quant, w_type, tokens, in_dim, out_dim)
+        rec["passes_over_weights"] = quant.gemv_passes(w_type, tokens, in_dim, out_dim)
+        rec["traffic"] = traffic_field(rec["kernel"], c.bytes_per_step)
         if floor if floor is not None else c.w_bytes < (16 << 20):
             fu, fg = mk.read_floor(stream, c, steps, min(args.warmup, steps))
             rec["read_only_us"] = round(fu, 3)
@@ -467,6 +522,7 @@ def main():
         gsteps = max(5, min(100, args.steps, int(4e12 // (2.0 * tokens * 12288 * 4096))))
         rec = bench_gemm(hip, quant, synth, rng, stream, Q4_K, tokens, 12288, 4096, gsteps, min(5, args.warmup))
         rec["steps"] = gsteps
+        rec["traffic"] = traffic_field(rec["kernel"], raw_gemm_bytes(tokens, 12288, 4096))
         gemm["M=%d" % tokens] = rec
         cases["cfg4 q4_k gemm 12288x4096 M=%d" % tokens] = rec
         log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
@@ -633,7 +689,7 @@ def main():
         "stands in for the reference's Crystal QuantMatmul\ncpu_ms=%.3f\ncos=%.8f\nmax_diff=%g\nok=%s" % (
             cpu_gbps, cpu_reps, cpu_s, mt_cores, mt_gbps, mt_reps, mt_s, cpu_s / cpu_reps * 1e3, cos, max_diff, str(ok).lower()))
 
-    traffic, traffic_rec = recorded_traffic()
+    traffic, traffic_rec = recorded_traffic("q4_k_gemv_f32")
     result = {
         "metric": "Q4_K GEMV GB/s 4096x12288 M=1",
         "value": round(gbps, 1),
@@ -664,8 +720,8 @@ def main():
         "roofline": {
             "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic,
-            "traffic_source": None if traffic_rec is None else "profiles/traffic.json: rocprofv3 --pmc record for %s at commit %s, not counted in this run" % (
-                traffic_rec.get("kernel"), traffic_rec.get("commit")),
+            "traffic_source": None if traffic_rec is None else "profiles/traffic.json: rocprofv3 --pmc record for q4_k_gemv_f32 at commit %s%s, not counted in this run" % (
+                traffic_rec.get("commit"), " (stale: the kernel sources have changed since)" if traffic_rec["stale"] else ""),
         },
         "cpu_baseline": {
             "value": round(cpu_gbps, 4), "unit": "GB/s", "cores": 1, "kind": "port",

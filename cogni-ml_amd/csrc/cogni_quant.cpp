@@ -1008,7 +1008,7 @@ static GemmPlan gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, ui
   }
   p.kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : w_type == COGNI_TYPE_Q5_K ? "q5_k_gemm_f16" : wide ? "q4_k_gemm_wide_f16" : "q4_k_gemm_f16";
   const uint32_t ntiles = wide ? (out_dim + 255) / 256 : (out_dim + 191) / 192;
-  p.grid_x = 8 * ((mtiles * ntiles + 7) / 8);
+  p.grid_x = gemm_grid_x(mtiles, ntiles);
   p.block = wide ? 512 : 256;
   return p;
 }
@@ -1071,7 +1071,7 @@ int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type
   // a tile is 128 tokens x 96 rows of each matrix
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 95) / 96;
   void* params[] = {&w_gate, &w_up, &workspace, &out, &in_dim, &out_dim, &tokens};
-  return launch("q4_k_gemm_swiglu_f16", 8 * ((mtiles * ntiles + 7) / 8), 256, 0, params, stream);
+  return launch("q4_k_gemm_swiglu_f16", gemm_grid_x(mtiles, ntiles), 256, 0, params, stream);
 }
 
 int cogni_set_gemm_threshold(int32_t tokens) {

@@ -8,14 +8,14 @@
 //   pack_x_f16_q4k  (x:f32 [m][in_dim], xp:f16, m:u32, in_dim:u32)           block 256, grid ceil(m/128) * 16 * in_dim/256
 //   q4_k_gemm_f16, q5_k_gemm_f16
 //                   (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32, bias_stride:u32)
-//                   block 256, grid (8 * ceil(ceil(m/128) * ceil(out_dim/192) / 8), k splits), no dynamic LDS
+//                   block 256, grid (gemm_grid_x(ceil(m/128), ceil(out_dim/192)) from gemv_config.h, k splits), no dynamic LDS
 //                   (156 / 160 KiB static); with k splits > 1 `out` is `splits` planes of [m][out_dim] and bias is null.
 //                   bias_stride 0: a [out_dim] bias added to every token; out_dim: a [m][out_dim] residual (it may be
 //                   `out` itself) - the reference's f32out_add prefill pipelines (gemm_mm.metal:651)
 //   q4_k_gemm_swiglu_f16
 //                   (w_gate, w_up, xp, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32): out = silu(x W_gate^T) * (x W_up^T),
 //                   the reference's simd_mm_q4k_h16_b64_swiglu (gemm_q4k.metal:1233). A tile is 128 tokens x 96 rows of each
-//                   matrix; block 256, grid 8 * ceil(ceil(m/128) * ceil(out_dim/96) / 8), no k split
+//                   matrix; block 256, grid gemm_grid_x(ceil(m/128), ceil(out_dim/96)), no k split
 //   gemm_sum_splits_f32 (planes, bias|null, out, m*out_dim:u32, out_dim:u32, splits:u32, bias_stride:u32)   block 256, grid ceil(m*out_dim/1024)
 //
 // Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows, so 512 x 12288 gives 256
@@ -44,6 +44,7 @@
 // buffer as soon as every wavefront has taken the current ones into registers.
 #pragma once
 #include "common.hpp"
+#include "gemv_config.h"
 
 #define GEMM_BM 128
 #define GEMM_BN 192
@@ -331,15 +332,11 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   out += (size_t)blockIdx.y * m * out_dim;
   constexpr u32 TILE_ROWS = SWIGLU ? GEMM_BN / 2 : GEMM_BN;   // rows of a matrix a tile covers
   const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + TILE_ROWS - 1) / TILE_ROWS;
-  // Workgroup -> tile, XCD-aware. Workgroups go to the 8 XCDs round-robin (id % 8) and each XCD has its own
-  // L2, so the tiles are numbered token-tile-major and XCD x takes the contiguous run [x*per, (x+1)*per):
-  // the workgroups that share an L2 then share one or two x tiles (1 MiB each at in_dim 4096), which stay
-  // resident while the weights stream through. Numbered the other way round every L2 sees every x tile,
-  // and at M = 512 the x tiles alone (4 MiB) fill it. The grid is 8 * per; the surplus workgroups leave.
-  const u32 per = (mtiles * ntiles + GEMM_XCDS - 1) / GEMM_XCDS;
-  const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
-  if (vt >= mtiles * ntiles) return;
-  const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
+  // Workgroup -> tile, XCD-aware (gemm_tile_of, gemv_config.h): the 32 workgroups that run side by side on an XCD take
+  // a block of neighbouring tiles, so that its L2 fills with a weight tile once for several token tiles and with an x
+  // tile once for several weight tiles. The grid is rounded up to whole blocks; the surplus workgroups leave.
+  u32 mt, nt;
+  if (!gemm_tile_of(blockIdx.x, mtiles, ntiles, &mt, &nt)) return;
   const size_t row_bytes = (size_t)nkb_all * BS;
   const u32 sh = 16u * kg;
   // Unpacking the 6-bit (scale, min) pairs takes one of two forms by g >= 2, i.e. by kh, which is the same for a whole

@@ -3,7 +3,7 @@
 // prefill kernel; precision as there: x and the dequantized weights rounded to half, fp32 accumulation).
 //
 //   q4_k_gemm_wide_f16 (w_raw, xp, bias|null, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32, bias_stride:u32)
-//                      block 512, grid 8 * ceil(ceil(m/128) * ceil(out_dim/256) / 8), no dynamic LDS (136 KiB static)
+//                      block 512, grid gemm_grid_x(ceil(m/128), ceil(out_dim/256)) from gemv_config.h, no dynamic LDS (136 KiB static)
 //   xp is the image pack_x_f16_q4k writes (gemm_q4k.hpp); bias as for q4_k_gemm_f16; no k split.
 //
 // Tiling. A workgroup owns 128 tokens x 256 weight rows. Its eight wavefronts are (row quarter nh) x (k-step half kh):
@@ -108,11 +108,9 @@ extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(
   const u32 j = lane & 31, kg = lane >> 5;
   const u32 nkb = in_dim >> 8;   // (no k split: the host takes this kernel only for launches of whole rounds of tiles)
   const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_WIDE_BN - 1) / GEMM_WIDE_BN;
-  // workgroup -> tile, XCD-aware (see q4_k_gemm_f16): the workgroups of one XCD share one or two x tiles
-  const u32 per = (mtiles * ntiles + GEMM_XCDS - 1) / GEMM_XCDS;
-  const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
-  if (vt >= mtiles * ntiles) return;
-  const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
+  // workgroup -> tile, XCD-aware (see q4_k_gemm_f16)
+  u32 mt, nt;
+  if (!gemm_tile_of(blockIdx.x, mtiles, ntiles, &mt, &nt)) return;
   const size_t row_bytes = (size_t)nkb * BS;
   const u32 sh = 16u * kg;
   // the two forms of the 6-bit unpacking folded into one through opaque masks (see gemm_k45_core)

@@ -66,10 +66,8 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   out += (size_t)blockIdx.y * m * out_dim;
   const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_BN - 1) / GEMM_BN;
   // workgroup -> tile as in q4_k_gemm_f16: XCD x takes a contiguous run of token-tile-major tiles
-  const u32 per = (mtiles * ntiles + GEMM_XCDS - 1) / GEMM_XCDS;
-  const u32 vt = (blockIdx.x % GEMM_XCDS) * per + blockIdx.x / GEMM_XCDS;
-  if (vt >= mtiles * ntiles) return;
-  const u32 mt = vt / ntiles, nt = vt - mt * ntiles;
+  u32 mt, nt;
+  if (!gemm_tile_of(blockIdx.x, mtiles, ntiles, &mt, &nt)) return;
   const u32 n0 = nt * GEMM_BN + nh * 96;             // first weight row of this wavefront
   const size_t row_bytes = (size_t)nkb_all * 210;
 

@@ -240,6 +240,38 @@ static inline int gemm_q4k_use_wide(unsigned out_dim, unsigned tokens) {
   return rw * GEMM_WIDE_ROUND_COST_X100 < rn * 100u;
 }
 
+// ---- prefill GEMM: which tile a workgroup takes. Workgroups go to the 8 XCDs round-robin (id % 8), each XCD has its own
+// L2 and 32 compute units, and a GEMM workgroup has a compute unit to itself, so the workgroups id = 8 l + x with the
+// same l / 32 run side by side on XCD x. They are given a block of bnt x bmt = 32 neighbouring tiles (bmt token tiles of
+// bnt weight tiles each): a weight tile is then fetched into that L2 once for bmt workgroups and an x tile once for bnt,
+// where one token tile per XCD (every workgroup of an XCD on the same x, each on weights of its own) made every L2 fill
+// with all the weights. One token tile: the blocks degenerate to that older numbering, which is kept as it is.
+#define GEMM_XCD_COUNT 8u
+#define GEMM_XCD_UNITS 32u
+static inline GEMV_HD unsigned gemm_block_mt(unsigned mtiles) { return mtiles >= 4u ? 4u : (mtiles >= 2u ? 2u : 1u); }
+static inline GEMV_HD unsigned gemm_grid_x(unsigned mtiles, unsigned ntiles) {
+  if (mtiles < 2u) return GEMM_XCD_COUNT * ((mtiles * ntiles + GEMM_XCD_COUNT - 1u) / GEMM_XCD_COUNT);
+  const unsigned bmt = gemm_block_mt(mtiles), bnt = GEMM_XCD_UNITS / bmt;
+  const unsigned nb = ((ntiles + bnt - 1u) / bnt) * ((mtiles + bmt - 1u) / bmt);
+  return GEMM_XCD_COUNT * GEMM_XCD_UNITS * ((nb + GEMM_XCD_COUNT - 1u) / GEMM_XCD_COUNT);
+}
+// false: this workgroup has no tile (the grid is rounded up to whole blocks)
+static inline GEMV_HD bool gemm_tile_of(unsigned id, unsigned mtiles, unsigned ntiles, unsigned* mt, unsigned* nt) {
+  const unsigned x = id % GEMM_XCD_COUNT, l = id / GEMM_XCD_COUNT;
+  if (mtiles < 2u) {
+    const unsigned per = (mtiles * ntiles + GEMM_XCD_COUNT - 1u) / GEMM_XCD_COUNT, vt = x * per + l;
+    *mt = vt / ntiles;
+    *nt = vt - *mt * ntiles;
+    return vt < mtiles * ntiles;
+  }
+  const unsigned bmt = gemm_block_mt(mtiles), bnt = GEMM_XCD_UNITS / bmt;
+  const unsigned nbn = (ntiles + bnt - 1u) / bnt, nb = nbn * ((mtiles + bmt - 1u) / bmt);
+  const unsigned b = (l / GEMM_XCD_UNITS) * GEMM_XCD_COUNT + x, i = l % GEMM_XCD_UNITS;
+  *nt = (b % nbn) * bnt + i / bmt;
+  *mt = (b / nbn) * bmt + i % bmt;
+  return b < nb && *nt < ntiles && *mt < mtiles;
+}
+
 // ---- one-pass kernel, rows above 4096 values: what a streamed unit waits for (gemv_mt.hpp)
 // vmcnt value that says "operand set i and unit i of a streamed row group have landed" (T = 1, S super-blocks per
 // k-slice, NSLOT units in LDS). Issue order: set 0, unit 0, set 1, unit 1, units 2 .. min(S, NSLOT) - 1 up front; behind unit

@@ -329,9 +329,9 @@ int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uin
  * Kernels: pack_x_f16_q4k (Q4_K and Q5_K) | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
  *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens,
  *          bias_stride: 0 for a [out_dim] bias, out_dim for a [tokens][out_dim] residual), block 256,
- *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/192)/8), no dynamic shared memory; or, for Q4_K launches that fill
+ *          grid from cogni_gemm_plan (whole blocks of 32 tiles of 128 x 192, 8 XCDs at a time), no dynamic shared memory; or, for Q4_K launches that fill
  *          whole rounds of 128 x 256 tiles (cogni_gemm_plan says which), q4_k_gemm_wide_f16 (same arguments), block 512,
- *          grid 8*ceil(ceil(tokens/128)*ceil(out_dim/256)/8).
+ *          grid from cogni_gemm_plan.
  * (pack_x_f16_*: block 256, grid ceil(tokens/128)*16*(in_dim/256).) Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 /* The workspace size with which cogni_gemm_dev may also split the k range: a launch with fewer than 128 tiles of
@@ -366,8 +366,8 @@ int cogni_gemm_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, u
  *   cogni_gemm_packed_swiglu_dev  out[m][o] = silu(g) * u, g = x[m] . W_gate[o], u = x[m] . W_up[o] (Q4_K; two matrices of
  *                                 out_dim rows; the sums as cogni_gemm_packed_dev gives them, silu as swiglu_f32): the
  *                                 gate and up matrices never exist in memory. Kernel q4_k_gemm_swiglu_f16 (w_gate, w_up,
- *                                 workspace, out, in_dim, out_dim, tokens), block 256, grid
- *                                 8*ceil(ceil(tokens/128)*ceil(out_dim/96)/8). Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
+ *                                 workspace, out, in_dim, out_dim, tokens), block 256, grid as cogni_gemm_plan gives it
+ *                                 for a matrix of 2 * out_dim rows. Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
 int cogni_gemm_packed_add_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t residual, uint64_t out,
                               uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,

@@ -146,6 +146,8 @@ def test_gemm_plan_picks_tile_and_split_for_the_shape():
     assert quant.gemm_plan(12, 4096, 12288, 2048, big) == ("q4_k_gemm_wide_f16", 768, 1, 512)
     assert quant.gemm_plan(12, 4096, 12288, 1024, big) == ("q4_k_gemm_f16", 512, 1, 256)       # two rounds either way
     assert quant.gemm_plan(12, 4096, 12288, 4096, big) == ("q4_k_gemm_wide_f16", 1536, 1, 512)  # 6 rounds instead of 8
+    # the grid is whole blocks of 32 tiles (8 weight tiles x 4 token tiles), 8 blocks at a time: a clipped shape rounds up
+    assert quant.gemm_plan(12, 4096, 12288 + 192, 512, big)[1] == 8 * 32 * 2 and quant.gemm_plan(12, 256, 400, 130, big)[1:3] == (256, 1)
     # few tiles: the k range is split when the workspace has room for the planes, else not
     name, gx, gy, block = quant.gemm_plan(12, 4096, 12288, 64, big)
     assert (name, gx, block) == ("q4_k_gemm_f16", 64, 256) and gy == 4
