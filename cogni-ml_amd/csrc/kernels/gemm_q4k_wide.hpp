@@ -76,27 +76,40 @@ __device__ __forceinline__ void gemm_wide_epilogue_half(float16_t (&acc)[4][2], 
     }
     return;
   }
+  // a clipped tile: a lane's four values go out as 16 bytes where the row allows it and they all exist, else one by one.
+  // (Two copies of the loop, chosen once, rather than one loop with the choice inside: there the compiler merges the
+  // two kinds of store into single floats for every tile.)
+  auto tail = [&](auto vec16) {
 #pragma unroll
-  for (int rr = 0; rr < 2; rr++) {
-    const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
+    for (int rr = 0; rr < 2; rr++) {
+      const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
 #pragma unroll
-    for (int c = 0; c < 2; c++)
+      for (int c = 0; c < 2; c++)
 #pragma unroll
-      for (int g4 = 0; g4 < 4; g4++) {
-        const float16_t& t = acc[2 * KH + rr][c];
-        const float4 p = theirs[((rr * 2 + c) * 4 + g4) * 64];
-        // (k half 0) + (k half 1) whichever of the two this wavefront holds
-        float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
-                      : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
-        const u32 n = nt * GEMM_WIDE_BN + nh * 64 + 32 * c + 8 * g4 + 4 * kg;
-        if (token < m && n < out_dim) {
+        for (int g4 = 0; g4 < 4; g4++) {
+          const float16_t& t = acc[2 * KH + rr][c];
+          const float4 p = theirs[((rr * 2 + c) * 4 + g4) * 64];
+          // (k half 0) + (k half 1) whichever of the two this wavefront holds
+          float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
+                        : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
+          const u32 n = nt * GEMM_WIDE_BN + nh * 64 + 32 * c + 8 * g4 + 4 * kg;
+          if (token >= m || n >= out_dim) continue;
           float* dst = out + (size_t)token * out_dim + n;
           const float* b = bias ? bias + (size_t)token * bias_stride + n : nullptr;   // bias, or a residual (stride out_dim)
-          const float ov[4] = {o.x, o.y, o.z, o.w};
-          for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (b ? b[e] : 0.0f);
+          if (decltype(vec16)::value && n + 4 <= out_dim) {
+            if (b) {
+              o.x += b[0]; o.y += b[1]; o.z += b[2]; o.w += b[3];
+            }
+            *reinterpret_cast<float4*>(dst) = o;
+          } else {
+            const float ov[4] = {o.x, o.y, o.z, o.w};
+            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e] + (b ? b[e] : 0.0f);
+          }
         }
-      }
-  }
+    }
+  };
+  if (vec) tail(std::true_type{});
+  else tail(std::false_type{});
 }
 
 extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void q4_k_gemm_wide_f16(

@@ -249,11 +249,20 @@ static inline int gemm_q4k_use_wide(unsigned out_dim, unsigned tokens) {
 #define GEMM_XCD_COUNT 8u
 #define GEMM_XCD_UNITS 32u
 static inline GEMV_HD unsigned gemm_block_mt(unsigned mtiles) { return mtiles >= 4u ? 4u : (mtiles >= 2u ? 2u : 1u); }
+// A block is bnt weight tiles x bmt token tiles: 32 tiles where there are enough of them, fewer when the launch has
+// fewer than 256 tiles, so that the blocks still go round all 8 XCDs.
+static inline GEMV_HD void gemm_block_shape(unsigned mtiles, unsigned ntiles, unsigned* bmt, unsigned* bnt) {
+  *bmt = gemm_block_mt(mtiles);
+  const unsigned per_xcd = (mtiles * ntiles + GEMM_XCD_COUNT - 1u) / GEMM_XCD_COUNT;   // tiles an XCD gets when they are dealt evenly
+  const unsigned want = (per_xcd + *bmt - 1u) / *bmt, cap = GEMM_XCD_UNITS / *bmt;
+  *bnt = want < 1u ? 1u : (want > cap ? cap : want);
+}
 static inline GEMV_HD unsigned gemm_grid_x(unsigned mtiles, unsigned ntiles) {
   if (mtiles < 2u) return GEMM_XCD_COUNT * ((mtiles * ntiles + GEMM_XCD_COUNT - 1u) / GEMM_XCD_COUNT);
-  const unsigned bmt = gemm_block_mt(mtiles), bnt = GEMM_XCD_UNITS / bmt;
+  unsigned bmt, bnt;
+  gemm_block_shape(mtiles, ntiles, &bmt, &bnt);
   const unsigned nb = ((ntiles + bnt - 1u) / bnt) * ((mtiles + bmt - 1u) / bmt);
-  return GEMM_XCD_COUNT * GEMM_XCD_UNITS * ((nb + GEMM_XCD_COUNT - 1u) / GEMM_XCD_COUNT);
+  return GEMM_XCD_COUNT * bmt * bnt * ((nb + GEMM_XCD_COUNT - 1u) / GEMM_XCD_COUNT);
 }
 // false: this workgroup has no tile (the grid is rounded up to whole blocks)
 static inline GEMV_HD bool gemm_tile_of(unsigned id, unsigned mtiles, unsigned ntiles, unsigned* mt, unsigned* nt) {
@@ -264,9 +273,10 @@ static inline GEMV_HD bool gemm_tile_of(unsigned id, unsigned mtiles, unsigned n
     *nt = vt - *mt * ntiles;
     return vt < mtiles * ntiles;
   }
-  const unsigned bmt = gemm_block_mt(mtiles), bnt = GEMM_XCD_UNITS / bmt;
-  const unsigned nbn = (ntiles + bnt - 1u) / bnt, nb = nbn * ((mtiles + bmt - 1u) / bmt);
-  const unsigned b = (l / GEMM_XCD_UNITS) * GEMM_XCD_COUNT + x, i = l % GEMM_XCD_UNITS;
+  unsigned bmt, bnt;
+  gemm_block_shape(mtiles, ntiles, &bmt, &bnt);
+  const unsigned units = bmt * bnt, nbn = (ntiles + bnt - 1u) / bnt, nb = nbn * ((mtiles + bmt - 1u) / bmt);
+  const unsigned b = (l / units) * GEMM_XCD_COUNT + x, i = l % units;
   *nt = (b % nbn) * bnt + i / bmt;
   *mt = (b / nbn) * bmt + i % bmt;
   return b < nb && *nt < ntiles && *mt < mtiles;

@@ -147,7 +147,9 @@ def test_gemm_plan_picks_tile_and_split_for_the_shape():
     assert quant.gemm_plan(12, 4096, 12288, 1024, big) == ("q4_k_gemm_f16", 512, 1, 256)       # two rounds either way
     assert quant.gemm_plan(12, 4096, 12288, 4096, big) == ("q4_k_gemm_wide_f16", 1536, 1, 512)  # 6 rounds instead of 8
     # the grid is whole blocks of 32 tiles (8 weight tiles x 4 token tiles), 8 blocks at a time: a clipped shape rounds up
-    assert quant.gemm_plan(12, 4096, 12288 + 192, 512, big)[1] == 8 * 32 * 2 and quant.gemm_plan(12, 256, 400, 130, big)[1:3] == (256, 1)
+    assert quant.gemm_plan(12, 4096, 12288 + 192, 512, big)[1] == 8 * 32 * 2 and quant.gemm_plan(12, 256, 400, 130, big)[1:3] == (16, 1)
+    # 88 tiles of the 12288 -> 4096 down projection at M = 512: blocks of 3 x 4 tiles, one per XCD, k split in two
+    assert quant.gemm_plan(14, 12288, 4096, 512, big) == ("q6_k_gemm_f16", 96, 2, 256)
     # few tiles: the k range is split when the workspace has room for the planes, else not
     name, gx, gy, block = quant.gemm_plan(12, 4096, 12288, 64, big)
     assert (name, gx, block) == ("q4_k_gemm_f16", 64, 256) and gy == 4
@@ -337,3 +339,42 @@ def test_matrix_core_gemv_grid_covers_every_row():
                 assert block == 512 and 0 < grid <= groups and lds <= 160 * 1024, (name, in_dim, out_dim, grid)
                 assert grid == groups or (grid == 256 and not chunked), (name, in_dim, out_dim, grid, groups)
     assert checked > 500
+
+
+def test_gemm_tile_numbering_covers_every_tile_once():
+    """gemm_tile_of / gemm_grid_x (gemv_config.h) through a small C++ program: every tile of a launch is taken by exactly
+    one workgroup, and the workgroups that share an XCD side by side hold a compact block of tiles."""
+    import subprocess
+    import tempfile
+    src = r'''
+#include <cstdio>
+#include <set>
+#include <utility>
+#include "gemv_config.h"
+int main() {
+  int bad = 0;
+  for (unsigned mt = 1; mt <= 40; mt++)
+    for (unsigned nt = 1; nt <= 130; nt += (nt < 70 ? 1 : 7)) {
+      const unsigned grid = gemm_grid_x(mt, nt);
+      std::set<std::pair<unsigned, unsigned>> seen;
+      for (unsigned id = 0; id < grid; id++) {
+        unsigned a, b;
+        if (!gemm_tile_of(id, mt, nt, &a, &b)) continue;
+        if (a >= mt || b >= nt || !seen.insert({a, b}).second) bad++;
+      }
+      if (seen.size() != (size_t)mt * nt || grid % 8 != 0 || grid > 8 * (mt * nt + 32 * 8)) bad++;
+    }
+  // 512 x 12288 in 128 x 192 tiles: the first 32 workgroups of XCD 0 hold 8 weight tiles x 4 token tiles
+  std::set<unsigned> ms, ns;
+  for (unsigned l = 0; l < 32; l++) { unsigned a, b; gemm_tile_of(8 * l, 4, 64, &a, &b); ms.insert(a); ns.insert(b); }
+  if (ms.size() != 4 || ns.size() != 8) bad++;
+  std::printf("bad=%d\n", bad);
+  return bad != 0;
+}
+'''
+    with tempfile.TemporaryDirectory() as d:
+        open(os.path.join(d, "t.cpp"), "w").write(src)
+        subprocess.run(["g++", "-O1", "-std=c++17", "-I", os.path.join(ROOT, "cogni-ml_amd", "csrc", "kernels"), "-o", os.path.join(d, "t"),
+                        os.path.join(d, "t.cpp")], check=True)
+        r = subprocess.run([os.path.join(d, "t")], capture_output=True, text=True)
+        assert r.returncode == 0 and "bad=0" in r.stdout, r.stdout + r.stderr
