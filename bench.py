@@ -455,6 +455,26 @@ def main():
                     flops = 2.0 * 32 * 32 * 16 * 12 * iters * (block // 64) * wgs
                     log("%s workgroups=%d iters=%d us=%.2f tflops=%.1f frac_of_published_peak=%.3f" % (
                         name, wgs, iters, r["us"], flops / r["us"] / 1e6, flops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS))
+        # the same twelve MFMAs per k-step with the prefill GEMM's other work added piece by piece: token-tile reads
+        # from LDS (all variants), global -> LDS copies of 1 KiB per wavefront, the 4-bit decode's vector instructions
+        region = hip.DeviceBuffer((1 << 20) + (1 << 17))
+        fill = (rng.standard_normal(region.bytesize // 2) * 0.25).astype(np.float16)
+        hip.copy_htod(region.ptr, fill, fill.nbytes, "probe operands")
+        iters, wgs = 256, 256
+        base = None
+        for name in ("bare", "decode", "copy1", "copy2", "copy3", "copy2_decode", "copy3_decode"):
+            fn = mk.fn("mfma_step_probe_" + name)
+            box = hip.KernelParams(ctypes.c_uint64(region.ptr), ctypes.c_uint64(res.ptr), ctypes.c_uint32(iters))
+
+            def pr(copy, st, fn=fn, box=box):
+                with hip.with_stream(st):
+                    hip.launch(fn, wgs, 1, 1, 256, 1, 1, box, "probe")
+            r = measure(hip, stream, Rotating(pr, 1, 1 << 30), 20, 3)
+            step_ns = r["us"] * 1e3 / (iters * 8)
+            base = step_ns if base is None else base
+            flops = 2.0 * 32 * 32 * 16 * 12 * 8 * iters * 4 * wgs
+            log("mfma_step_probe_%s k_step_ns=%.1f (+%.1f over bare) tflops=%.1f frac_of_published_peak=%.3f" % (
+                name, step_ns, step_ns - base, flops / r["us"] / 1e6, flops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS))
         return
 
     mk = MeasureKernels(hip)

@@ -77,3 +77,126 @@ extern "C" __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(
     const uint4* src, float* out, u32 iters) {
   mfma_ceiling_core(src, out, iters);
 }
+
+// What the other work of the prefill GEMM's k-step costs a wavefront that is issuing its twelve MFMAs (one wavefront per
+// SIMD, four ds_read_b128 of token tiles per k-step, as in q4_k_gemm_f16). COPIES: global -> LDS copies of 1 KiB per
+// wavefront and k-step (global_load_lds_dwordx4 out of a 1 MiB region that 32 workgroups share, so they hit in L2);
+// DECODE: the 54 vector instructions that turn twelve 4-bit words into fp16 weight operands. (src, out, iters): `src`
+// holds at least 1 MiB + 64 KiB; one iteration is eight k-steps, 2 * 32*32*16 * 12 * 8 flops per wavefront.
+typedef const __attribute__((address_space(1))) void probe_gbl_void;
+typedef __attribute__((address_space(3))) void probe_lds_void;
+__shared__ uint4 probe_tokens[4096];
+__shared__ uint4 probe_landing[4096];
+__device__ __forceinline__ u32 probe_q4_pair(u32 t, u32 scale, u32 negmin) {
+  const u32 off = 0xE400E400u;   // -1024 twice: takes the 0x6400 exponent trick's offset out again
+  const __half2 q = __hadd2(*reinterpret_cast<const __half2*>(&t), *reinterpret_cast<const __half2*>(&off));
+  const __half2 w = __hfma2(q, *reinterpret_cast<const __half2*>(&scale), *reinterpret_cast<const __half2*>(&negmin));
+  return *reinterpret_cast<const u32*>(&w);
+}
+template <int COPIES, bool DECODE>
+__device__ __forceinline__ void mfma_step_probe_core(const uint4* src, float* out, u32 iters) {
+  const u32 tid = threadIdx.x, lane = tid & 63;
+  const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const u32 j = lane & 31, kg = lane >> 5, kh = wave >> 1;
+  const uint4* region = src + (size_t)(blockIdx.x & 7) * 8192;   // 8 x 128 KiB windows of the first MiB
+  util_float16 acc[4][3];
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
+  util_half8 B[3], Bnext[3];
+  uint4 raw[3];
+  u32 sc[3], nm[3];
+#pragma unroll
+  for (int c = 0; c < 3; c++) {
+    uint4 v = src[tid + 256 * c];
+    B[c] = *reinterpret_cast<util_half8*>(&v);
+    Bnext[c] = B[c];
+    raw[c] = src[tid + 256 * c + 2048];
+    sc[c] = src[tid + 3000 + c].x;
+    nm[c] = src[tid + 3000 + c].y;
+  }
+  for (u32 i = tid; i < 4096; i += 256) {
+    probe_tokens[i] = src[i];
+    probe_landing[i] = src[i + 4096];
+  }
+  __syncthreads();
+  uint4 A[2][4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) A[0][r] = probe_tokens[(16 * kh + kg) * 128 + j + r * 32];
+  for (u32 it = 0; it < iters; it++) {
+    const uint4* xsrc = region + (size_t)(it & 1) * 4096;
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      const uint4* arow = probe_tokens + (16 * kh + kg) * 128 + j;
+#pragma unroll
+      for (int r = 0; r < 4; r++) A[(t + 1) & 1][r] = arow[((t + 1) & 7) * 256 + r * 32];
+#pragma unroll
+      for (int i = 0; i < COPIES; i++) {
+        const int ci = (t * COPIES + i) & 15;
+        __builtin_amdgcn_global_load_lds((probe_gbl_void*)(xsrc + 256 * ci + tid),
+                                         (probe_lds_void*)(probe_landing + 256 * ci + wave * 64), 16, 0, 0);
+      }
+      if (DECODE) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+          uint4 q = raw[c];
+          asm volatile("" : "+v"(q.x), "+v"(q.y), "+v"(q.z), "+v"(q.w));
+          uint4 bw;
+          bw.x = probe_q4_pair((q.x & 0x000F000Fu) | 0x64006400u, sc[c], nm[c]);
+          bw.y = probe_q4_pair(((q.x >> 8) & 0x000F000Fu) | 0x64006400u, sc[c], nm[c]);
+          bw.z = probe_q4_pair((q.y & 0x000F000Fu) | 0x64006400u, sc[c], nm[c]);
+          bw.w = probe_q4_pair(((q.y >> 8) & 0x000F000Fu) | 0x64006400u, sc[c], nm[c]);
+          Bnext[c] = *reinterpret_cast<util_half8*>(&bw);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const util_half8 Ar = *reinterpret_cast<const util_half8*>(&A[t & 1][r]);
+#pragma unroll
+        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[c], Ar, acc[r][c], 0, 0, 0);
+      }
+      if (DECODE) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+          asm volatile("" : "+v"(Bnext[c]));
+          B[c] = Bnext[c];
+        }
+      }
+      // one MFMA, the four LDS reads, then a copy behind every second MFMA: the placement the GEMM kernel uses
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+      for (int i = 0; i < COPIES; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (COPIES > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+  }
+  __syncthreads();
+  float s = __uint_as_float(probe_landing[tid].x);
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+#pragma unroll
+    for (int c = 0; c < 3; c++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) s += acc[r][c][v];
+  out[blockIdx.x * 256 + tid] = s;
+}
+#define MFMA_STEP_PROBE(name, copies, decode)                                                                        \
+  extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(                 \
+      const uint4* src, float* out, u32 iters) {                                                                     \
+    mfma_step_probe_core<copies, decode>(src, out, iters);                                                           \
+  }
+MFMA_STEP_PROBE(mfma_step_probe_bare, 0, false)
+MFMA_STEP_PROBE(mfma_step_probe_decode, 0, true)
+MFMA_STEP_PROBE(mfma_step_probe_copy1, 1, false)
+MFMA_STEP_PROBE(mfma_step_probe_copy2, 2, false)
+MFMA_STEP_PROBE(mfma_step_probe_copy3, 3, false)
+MFMA_STEP_PROBE(mfma_step_probe_copy2_decode, 2, true)
+MFMA_STEP_PROBE(mfma_step_probe_copy3_decode, 3, true)
