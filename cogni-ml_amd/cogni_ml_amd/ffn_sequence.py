@@ -50,6 +50,7 @@ class FFNSequenceRunner:
         # several tokens behind the norm: the norm itself writes the activation image gate | up read (no pack launch)
         image_bytes = quant.gemv_image_bytes(TensorType.Q4_K, hidden, quant.MAX_GEMV_TOKENS) if hidden <= 4096 else 0
         self._image = self._alloc(image_bytes) if norm is not None and image_bytes and ffn_dim % 16 == 0 else None
+        self._image_from = quant.gemv_one_pass_multi_from(TensorType.Q4_K, hidden)   # token count from which it is used
         self._gate = self._alloc(4 * tokens * ffn_dim)      # only used when several tokens run together
         self._up = self._alloc(4 * tokens * ffn_dim)
         self._act = self._alloc(4 * tokens * ffn_dim)
@@ -87,7 +88,7 @@ class FFNSequenceRunner:
         st = hip.current_stream_handle()
         h, f = self.hidden, self.ffn_dim
         x, act = self._x.ptr + 4 * tok0 * h, self._act.ptr + 4 * tok0 * f
-        fused_norm = self._image is not None and count >= 2
+        fused_norm = self._image is not None and count >= self._image_from
         if fused_norm:
             # r = x + add, and rmsnorm(r) written straight as the activation image gate | up | SwiGLU read
             quant.add_rmsnorm_pack_dev(x, self._add.ptr + 4 * tok0 * h, self._norm.ptr, self._res.ptr + 4 * tok0 * h, 0,

@@ -112,7 +112,7 @@ class QwenProjectionStackRunner:
             j = i + 1
             while j < len(ents) and j - i < 3 and (ents[j][1], ents[j][2], ents[j][4]) == (src, t, in_dim):
                 j += 1
-            if j - i >= 2 and count > 1 and quant.gemv_image_bytes(t, in_dim, min(count, quant.MAX_GEMV_TOKENS)) > 0:
+            if j - i >= 2 and 0 < quant.gemv_one_pass_multi_from(t, in_dim) <= count:
                 # several tokens of a shape the one-pass kernel takes: the input is packed once per sequence step and
                 # every list that reads it (q | k | v, then gate | up) goes against that one image
                 grp = ents[i:j]

@@ -92,6 +92,13 @@ def gemv_one_pass_from(w_type, in_dim, out_dim):
     return int(f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim)))
 
 
+def gemv_one_pass_multi_from(w_type, in_dim):
+    """The same for pairs, lists and the fused gate | up | SwiGLU (0: never for this row length)."""
+    f = hip.lib().cogni_gemv_one_pass_multi_from
+    f.restype = ctypes.c_uint32
+    return int(f(ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim)))
+
+
 def gemv_image_stats():
     """(slots, in use, pinned by a capture, multi-token calls that found no slot) of the library's activation images."""
     a, b, c, d = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint64()

@@ -333,6 +333,7 @@ size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens)
 }
 
 uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim, uint32_t out_dim) { return gemv_mt_from(w_type, in_dim, out_dim); }
+uint32_t cogni_gemv_one_pass_multi_from(uint32_t w_type, uint32_t in_dim) { return gemv_mt_multi_from(w_type, in_dim); }
 
 int cogni_gemv_release_stream(void* stream) {
   int slot = -1;
@@ -405,7 +406,7 @@ int cogni_gemv_pack_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t t
                                             "(cogni_gemv_image_bytes is 0)");
   if (!x || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack_dev: null device pointer");
   void* params[] = {&x, &image, &tokens, &in_dim};
-  return launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_mt_q6k_f16" : "pack_x_mt_q4k_f16", 2 * (in_dim >> 8), 256, 0, params, stream);
+  return launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_mt_q6k_f16" : "pack_x_mt_q4k_f16", 2 * gemv_mt_padded_sb(in_dim), 256, 0, params, stream);
 }
 
 int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,
@@ -577,11 +578,11 @@ int cogni_gemv_dual_dev(uint64_t w_raw_a, uint64_t w_raw_b, uint32_t w_type, uin
     return launch("q4_k_dual_gemv_f32", grid, block, shmem, params, stream);
   }
   // several tokens of a pair the one-pass kernel takes: the activations packed once, both matrices in one launch
-  if (tokens >= 2) {
+  if (const uint32_t from = gemv_mt_multi_from(w_type, in_dim); from && tokens >= from) {
     const uint64_t ws[2] = {w_raw_a, w_raw_b}, os[2] = {out_a, out_b};
     const uint32_t dims[2] = {out_dim, out_dim};
     int rc = 0;
-    if (try_one_pass(ws, w_type, x, 0, os, dims, 2, in_dim, tokens, 2, stream, &rc)) return rc;
+    if (try_one_pass(ws, w_type, x, 0, os, dims, 2, in_dim, tokens, from, stream, &rc)) return rc;
   }
   // several tokens of a Q4_K pair whose shape the matrix-core kernel takes: groups of up to four tokens, the two
   // matrices as one of 2 * out_dim rows (the activations are staged once for both); a last single token goes to the
@@ -630,9 +631,10 @@ int cogni_gemv_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t x, cons
     total += out_dims[i];
     aligned = aligned && (out_dims[i] % 16) == 0;
   }
-  if (count >= 2 && tokens >= 2) {   // the one-pass kernel: one image for all of them, up to three matrices per launch
+  if (const uint32_t from = gemv_mt_multi_from(w_type, in_dim); from && count >= 2 && tokens >= from) {
+    // the one-pass kernel: one image for all of them, up to three matrices per launch
     int rc = 0;
-    if (try_one_pass(w_raw, w_type, x, 0, out, out_dims, count, in_dim, tokens, 2, stream, &rc)) return rc;
+    if (try_one_pass(w_raw, w_type, x, 0, out, out_dims, count, in_dim, tokens, from, stream, &rc)) return rc;
   }
   if (count == 2 && out_dims[0] == out_dims[1])
     return cogni_gemv_dual_dev(w_raw[0], w_raw[1], w_type, x, out[0], out[1], in_dim, out_dims[0], tokens, stream);
@@ -712,7 +714,7 @@ int cogni_gemv_dual_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, 
     return fail(COGNI_ERR_INVALID_ARGUMENT, "Q4_K GEMV requires in_dim multiple of 256, got " + std::to_string(in_dim));
   // several tokens of a pair the one-pass kernel takes: the activations packed once per group of up to eight tokens, gate
   // tile and up tile side by side in a workgroup, which stores silu(gate) * up
-  if (tokens >= 2 && gemv_mt_supported(w_type, 2, in_dim) && out_dim <= 0x7FFFFFFFu) {
+  if (const uint32_t from = gemv_mt_multi_from(w_type, in_dim); from && tokens >= from && out_dim <= 0x7FFFFFFFu) {
     const uint64_t image = image_for_stream(stream);
     if (image) {
       for (uint32_t t0 = 0; t0 < tokens;) {
@@ -902,7 +904,7 @@ int cogni_add_rmsnorm_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t resi
 }
 
 // The norms with the activation image of the one-pass GEMV as a second output (norm.hpp): dim must be a shape those
-// kernels take with rows short enough for a thread to keep its values (a multiple of 2048 up to 4096).
+// kernels take with rows short enough for a thread to keep its values (a multiple of 256 up to 4096).
 static int norm_pack_check(const char* who, uint32_t w_type, uint32_t dim, uint32_t tokens) {
   if (!gemv_mt_supported(w_type, tokens < 2 ? 2 : (int)tokens, dim) || dim > 4096u || tokens == 0)
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": needs 1..8 tokens of a row length the one-pass GEMV takes, up to 4096 "

@@ -179,11 +179,14 @@ static inline unsigned gemv_mfma_lds_bytes(unsigned type, int tokens, unsigned i
 #define GEMV_MT_TMAX 3              // 16-row tiles a wavefront carries at most (Q4_K, Q5_K; Q6_K two)
 #define GEMV_MT_MAX_TOKENS 8
 #define GEMV_MT_MAX_IN_DIM 12288u
-// Shapes the kernels take: Q4_K, Q5_K or Q6_K, 2..8 tokens, in_dim a multiple of 2048 up to 12288 (1..6 super-blocks per k-slice).
+// Shapes the kernels take: Q4_K, Q5_K or Q6_K, 2..8 tokens, in_dim a multiple of 256 up to 12288 (1..6 super-blocks per
+// k-slice; a row whose super-blocks do not divide by 8 is worked on as if zeros filled it up, gemv_mt_padded_sb).
 static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned in_dim) {
-  return (type == 12 || type == 13 || type == 14) && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && in_dim != 0 && (in_dim & 2047u) == 0 &&
+  return (type == 12 || type == 13 || type == 14) && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && in_dim != 0 && (in_dim & 255u) == 0 &&
          in_dim <= GEMV_MT_MAX_IN_DIM;
 }
+// super-blocks of the activation image: the row's, rounded up to a multiple of the 8 k-slices
+static inline GEMV_HD unsigned gemv_mt_padded_sb(unsigned in_dim) { return ((in_dim >> 8) + 7u) & ~7u; }
 // Token count from which one matrix goes through pack + one pass rather than the per-token-group kernels (0: never): where
 // the pair measures faster. Q6_K from three tokens; Q4_K and Q5_K from four on rows of 4096 values and more, else from five.
 // Tall matrices of up to 4096 columns (an output head): the workgroups walk many row groups and pay their start once, which
@@ -193,8 +196,17 @@ static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned 
 #define GEMV_MT_VERY_TALL_ROWS 98304u
 static inline unsigned gemv_mt_from(unsigned type, unsigned in_dim, unsigned out_dim) {
   if (!gemv_mt_supported(type, 2, in_dim)) return 0;
+  // rows that fill less than three quarters of their eight k-slices (1024 values: half of them): from five tokens, where
+  // the per-token-group kernels start to read the weights twice
+  if (4u * (in_dim >> 8) < 3u * gemv_mt_padded_sb(in_dim)) return 5u;
   if (in_dim <= 4096u && out_dim >= GEMV_MT_TALL_ROWS) return (type == 14 || out_dim >= GEMV_MT_VERY_TALL_ROWS) ? 2u : 3u;
   return type == 14 ? 3u : (in_dim >= 4096u ? 4u : 5u);
+}
+// The same for a pair, a list of matrices or the fused gate | up | SwiGLU: from two tokens (one pack serves all of them and
+// the weights are read once), from five on rows that fill less than three quarters of their k-slices.
+static inline unsigned gemv_mt_multi_from(unsigned type, unsigned in_dim) {
+  if (!gemv_mt_supported(type, 2, in_dim)) return 0;
+  return 4u * (in_dim >> 8) < 3u * gemv_mt_padded_sb(in_dim) ? 5u : 2u;
 }
 // tiles per wavefront: rows of more than 4096 values one (the operands are streamed); else as many as keep 256 workgroups
 // busy, at most three (Q4_K) or two (Q6_K: its units are larger). Host and kernel use the same rule.
@@ -217,11 +229,11 @@ static inline unsigned gemv_mt_lds_bytes(unsigned type) {
   return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u +
          GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : (type == 13 ? 6u * 2816u : 6u * 2304u));
 }
-// bytes of the activation image: 8 KiB of operands per super-block, then 16 bytes per (super-block, lane) for the scales and
+// bytes of the activation image: per super-block (of the padded count) 8 KiB of operands, then 16 bytes per (super-block, lane) for the scales and
 // the sub-block sums (one more matrix-core operand). Q4_K and Q5_K share one image, Q6_K has its own.
 static inline unsigned long long gemv_mt_image_bytes(unsigned type, unsigned in_dim) {
   (void)type;
-  return (unsigned long long)(in_dim >> 8) * (8192u + 1024u);
+  return (unsigned long long)gemv_mt_padded_sb(in_dim) * (8192u + 1024u);
 }
 
 // ---- prefill GEMM: which Q4_K kernel an unsplit launch takes (gemm_q4k.hpp: 128 x 192 tiles, four wavefronts;

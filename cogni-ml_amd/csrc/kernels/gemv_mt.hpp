@@ -2,7 +2,7 @@
 //   out_i[m][o] = (residual[m][o] +) sum_j x[m][j] * deq(W_i[o][j])      for up to three matrices W_i of one in_dim.
 //
 // Kernels.
-//   pack_x_mt_q4k_f16 | pack_x_mt_q6k_f16 (x, image, tokens, in_dim)            block 256, grid 2 * in_dim / 256
+//   pack_x_mt_q4k_f16 | pack_x_mt_q6k_f16 (x, image, tokens, in_dim)            block 256, grid 2 * gemv_mt_padded_sb(in_dim)
 //     turn the activations x[tokens][in_dim] (fp32) into the image the GEMV kernel of that weight type reads: per
 //     super-block of 256 values the matrix-core operands of its instructions, laid out lane by lane, followed by the
 //     scale and the sub-block sums of every (token, super-block). Written once per activation block, whatever the number
@@ -11,8 +11,8 @@
 //     (Q5_K reads the image pack_x_mt_q4k_f16 writes)
 //     block 512 (8 wavefronts), grid and dynamic shared memory from gemv_config.h (gemv_mt_grid, gemv_mt_lds_bytes).
 //     rows1 / rows2 may be 0 (then w1 / w2 / out1 / out2 are not read); residual (may be null) belongs to the first
-//     matrix. Row counts of all but the last matrix present must be multiples of 16. in_dim must be a multiple of 2048
-//     up to 12288 (8 k-slices of 1..6 super-blocks). out_i rows at stride rows_i (the reference's multi-token kernel
+//     matrix. Row counts of all but the last matrix present must be multiples of 16. in_dim must be a multiple of 256
+//     up to 12288 (8 k-slices of 1..6 super-blocks; see "Rows that are not a multiple of 2048 values" below). out_i rows at stride rows_i (the reference's multi-token kernel
 //     contract, src/ml/cuda/kernels/q4k_gemv_probe.ptx:437-768, q5k_gemv_probe.ptx:237 and q6k_gemv_probe.ptx:977: x rows at stride in_dim, outs
 //     at stride out_dim; these kernels handle eight tokens where those handle four).
 //   q4_k_gemv_mt_swiglu_f32 (w_gate, w_up, image, out, in_dim, out_dim, tokens)
@@ -33,6 +33,13 @@
 // With one or two super-blocks per k-slice the activation operands stay in registers for the whole kernel and the next
 // row group's weights are requested while the current one is worked on; with three to six (rows of 6144..12288 values)
 // a wavefront carries one tile and streams the operands of its super-blocks through two register sets.
+//
+// Rows that are not a multiple of 2048 values. The eight k-slices take ceil(nsb / 8) super-blocks each, as if the row had
+// nsbp = 8 * ceil(nsb / 8) of them. The image has nsbp super-blocks, the ones past the row's end all zeros (operands, sums
+// and the tokens' scales), and a k-slice whose super-block does not exist copies the row's last block in its place: a
+// finite weight times zero, so such a unit adds exactly 0 to every sum and every wavefront issues the same loads and
+// waits as for a full row. (A 1024-value row keeps four of the eight wavefronts busy with zeros: still one pass over the
+// weights where the per-token-group kernels take two from five tokens on.)
 //
 // Memory. A tile's share of a super-block is 16 rows x one block at a stride of a whole row: fetched by the lanes that
 // use it (a few bytes each, 16 rows per instruction) it comes in at a third of the rate of a plain stream. So the weights
@@ -144,12 +151,13 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float*
                                                                     u32 tokens, u32 in_dim) {
   const u32 lane = threadIdx.x & 63;
   const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const u32 nsb = in_dim >> 8;
+  const u32 nsb = in_dim >> 8, nsbp = gemv_mt_padded_sb(in_dim);
   const u32 sb = unit >> 3, tok = unit & 7;
-  if (sb >= nsb) return;
+  if (sb >= nsbp) return;
+  const bool present = tok < tokens && sb < nsb;   // (super-blocks past the row's end: zeros, as for an absent token)
   float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (tok < tokens) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
-  mt_pack_store_q4k(image, nsb, sb, tok, lane, v, tok < tokens);
+  if (present) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  mt_pack_store_q4k(image, nsbp, sb, tok, lane, v, present);
 }
 
 // Q6_K image: [super-block][sub-block pair p][lane = 16 kg + row][2 x 4 halves]: the halves of lane (kg, row = 2 token +
@@ -182,12 +190,13 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q6k_f16(const float*
                                                                     u32 tokens, u32 in_dim) {
   const u32 lane = threadIdx.x & 63;
   const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const u32 nsb = in_dim >> 8;
+  const u32 nsb = in_dim >> 8, nsbp = gemv_mt_padded_sb(in_dim);
   const u32 sb = unit >> 3, tok = unit & 7;
-  if (sb >= nsb) return;
+  if (sb >= nsbp) return;
+  const bool present = tok < tokens && sb < nsb;   // (super-blocks past the row's end: zeros, as for an absent token)
   float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (tok < tokens) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
-  mt_pack_store_q6k(image, nsb, sb, tok, lane, v, tok < tokens);
+  if (present) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  mt_pack_store_q6k(image, nsbp, sb, tok, lane, v, present);
 }
 
 // ---- loads in assembly ---------------------------------------------------------------------------------------------------
@@ -431,7 +440,7 @@ struct MtArgs {
 
 // (mt_stream_wait, the number a streamed unit waits with, lives in gemv_config.h: host code can test it there)
 
-// SBW: super-blocks per k-slice (in_dim / 2048). SBW <= 2: operands resident in registers, T tiles per wavefront, the next
+// SBW: super-blocks per k-slice (ceil(in_dim / 2048)). SBW <= 2: operands resident in registers, T tiles per wavefront, the next
 // row group requested while this one is worked on. SBW >= 3: T = 1, operands streamed through two register sets.
 // SWIGLU (T = 2, or T = 1 with streamed operands: gate tile, then up tile): the two tiles of a row group are tile grp of
 // w[0] (gate) and tile grp of w[1] (up), rows[0] = rows[1] = out_dim, and the workgroup stores out[0][m][o] = silu(gate . x) * (up . x) (swiglu_one, the function of
@@ -454,7 +463,7 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
   char* lds = reinterpret_cast<char*>(mt_lds4);
   const int tid = threadIdx.x, lane = tid & 63;
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const u32 nsb = in_dim >> 8;
+  const u32 nsb = in_dim >> 8, nsbp = gemv_mt_padded_sb(in_dim);   // super-blocks of a row, and of the image
   const u32 total_rows = a.rows[0] + a.rows[1] + a.rows[2];
   const u32 ntiles = (total_rows + 15) >> 4;
   const u32 ngroups = SWIGLU ? (a.rows[0] + 15) >> 4 : (ntiles + T - 1) / T;
@@ -477,7 +486,7 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
 
   // ---- operand sets: the A operands of a super-block and its scales and sub-block sums ----
   mt_u32x4 breg[NSETS][8], auxr[NSETS][F::NAUX];
-  const uint8_t* aux = image + (size_t)nsb * 8192;
+  const uint8_t* aux = image + (size_t)nsbp * 8192;
   // (uniform bases and two lane offsets: no address registers per load)
   const u32 lane16 = lane * 16u, rg_off = F::aux_offset(lane);
   auto issue_set = [&](int i, int set) {
@@ -530,7 +539,8 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
     }
   };
   auto issue_unit = [&](int i, int t, int slot) {
-    const u32 off = (wave + 8u * i) * F::BB, dst = slots_lds + (u32)slot * F::UNIT_BYTES;
+    // (a super-block past the row's end: the row's last block stands in; its operands in the image are zeros)
+    const u32 off = min(wave + 8u * i, nsb - 1u) * F::BB, dst = slots_lds + (u32)slot * F::UNIT_BYTES;
 #pragma unroll
     for (int m = 0; m + 1 < NC; m++) mt_copy16(dst + 1024u * m, cptr[t][m] + off);
     if (lane < F::LAST) mt_copy16(dst + 1024u * (NC - 1), cptr[t][NC - 1] + off);
@@ -721,7 +731,7 @@ __device__ __forceinline__ void gemv_mt_dispatch(const MtArgs& a, const uint8_t*
                                                  u32* top_ids = nullptr) {
   const u32 ntiles = (a.rows[0] + a.rows[1] + a.rows[2] + 15) >> 4;
   const u32 t = gemv_mt_tiles(F::TYPE, in_dim, ntiles);
-  switch (in_dim >> 11) {
+  switch (gemv_mt_padded_sb(in_dim) >> 3) {
     case 1:
       if (t <= 1) gemv_mt_core<F, 1, 1, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
       else if (t == 2) gemv_mt_core<F, 1, 2, false, TOP1>(a, image, residual, in_dim, tokens, top_ids);
@@ -775,7 +785,7 @@ GEMV_MT_TOP1_ENTRY(q6_k_gemv_mt_top1_partial_f32, MtQ6K)
 extern "C" __global__ __launch_bounds__(GEMV_MT_WAVES * 64) void q4_k_gemv_mt_swiglu_f32(
     const uint8_t* w_gate, const uint8_t* w_up, const uint8_t* image, float* out, u32 in_dim, u32 out_dim, u32 tokens) {
   const MtArgs a = {{w_gate, w_up, nullptr}, {out, nullptr, nullptr}, {out_dim, out_dim, 0u}};
-  switch (in_dim >> 11) {
+  switch (gemv_mt_padded_sb(in_dim) >> 3) {
     case 1: gemv_mt_core<MtQ4K, 1, 2, true>(a, image, nullptr, in_dim, tokens); break;
     case 2: gemv_mt_core<MtQ4K, 2, 2, true>(a, image, nullptr, in_dim, tokens); break;
     case 3: gemv_mt_core<MtQ4K, 3, 1, true>(a, image, nullptr, in_dim, tokens); break;

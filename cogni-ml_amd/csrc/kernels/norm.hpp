@@ -15,7 +15,7 @@
 #define NORM_KEEP 4   // float4 a thread keeps across the reduction on the short-row path
 
 // IMG: 0 = no image, 12 = the Q4_K (and Q5_K) image, 14 = the Q6_K image. With an image the grid is the image's eight token
-// slots, the workgroups of slots at and above `tokens` write the zeros of an absent token, dim is a multiple of 1024 up to
+// slots, the workgroups of slots at and above `tokens` write the zeros of an absent token, dim is a multiple of 256 up to
 // 4096 (the short-row path), and `out` may be null (the normalised rows then exist only as the image).
 template <bool ADD, int IMG = 0>
 __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __restrict__ add,
@@ -23,13 +23,20 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
                                              float* __restrict__ out, u32 dim, float eps, uint8_t* __restrict__ image = nullptr,
                                              u32 tokens = 0) {
   __shared__ float part[NORM_BLOCK / WAVE];
+  // this token slot's share of the image from super-block `from` on: zeros (an absent token; the super-blocks past the
+  // row's end that fill the image up to a multiple of 8)
+  [[maybe_unused]] auto zero_image = [&](u32 from) {
+    if constexpr (IMG != 0) {
+      const u32 lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+      for (u32 sb = from + wave; sb < gemv_mt_padded_sb(dim); sb += NORM_BLOCK / WAVE) {
+        if constexpr (IMG == 14) mt_pack_store_q6k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
+        else mt_pack_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
+      }
+    }
+  };
   if constexpr (IMG != 0) {
     if (blockIdx.x >= tokens) {
-      const u32 lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-      for (u32 sb = wave; sb < (dim >> 8); sb += NORM_BLOCK / WAVE) {
-        if constexpr (IMG == 14) mt_pack_store_q6k(image, dim >> 8, sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
-        else mt_pack_store_q4k(image, dim >> 8, sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
-      }
+      zero_image(0);
       return;
     }
   }
@@ -77,13 +84,14 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
         o.x = (v[k].x * inv) * w[k].x, o.y = (v[k].y * inv) * w[k].y, o.z = (v[k].z * inv) * w[k].z, o.w = (v[k].w * inv) * w[k].w;
         if (IMG == 0 || out) *reinterpret_cast<float4*>(ot + i) = o;
         if constexpr (IMG != 0) {
-          // (i < dim holds for whole wavefronts: dim is a multiple of 1024)
+          // (i < dim holds for whole wavefronts: dim is a multiple of 256)
           const u32 sb = 4u * (u32)k + (tid >> 6);
-          if constexpr (IMG == 14) mt_pack_store_q6k(image, dim >> 8, sb, blockIdx.x, tid & 63, o, true);
-          else mt_pack_store_q4k(image, dim >> 8, sb, blockIdx.x, tid & 63, o, true);
+          if constexpr (IMG == 14) mt_pack_store_q6k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, tid & 63, o, true);
+          else mt_pack_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, tid & 63, o, true);
         }
       }
     }
+    zero_image(dim >> 8);
     return;
   }
   static_assert(IMG == 0 || IMG == 12 || IMG == 14, "image kinds");
@@ -148,7 +156,7 @@ extern "C" __global__ __launch_bounds__(NORM_BLOCK) void add_rmsnorm_f32(const f
 // The same with the normalised rows written as the activation image of the one-pass GEMV as well:
 //   rmsnorm_pack_q4k_f32 | rmsnorm_pack_q6k_f32 (x, norm, out | null, image, dim, tokens, eps)
 //   add_rmsnorm_pack_q4k_f32 | add_rmsnorm_pack_q6k_f32 (x, add, norm, residual_out, normed_out | null, image, dim, tokens, eps)
-// grid.x = 8 (the image's token slots; x, add and the outputs hold `tokens` rows), block 256, dim a multiple of 2048 up
+// grid.x = 8 (the image's token slots; x, add and the outputs hold `tokens` rows), block 256, dim a multiple of 256 up
 // to 4096. The image is that of pack_x_mt_q4k_f16 | pack_x_mt_q6k_f16 on the normalised rows, bit for bit.
 #define NORM_PACK_ENTRIES(SFX, IMG)                                                                                          \
   extern "C" __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_pack_##SFX##_f32(                                         \

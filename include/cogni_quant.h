@@ -125,7 +125,7 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
                    uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 
-/* Several tokens in ONE pass over the weights (Q4_K, Q5_K and Q6_K, in_dim a multiple of 2048 up to 12288, 2..8 tokens): the
+/* Several tokens in ONE pass over the weights (Q4_K, Q5_K and Q6_K, in_dim a multiple of 256 up to 12288, 2..8 tokens): the
  * activations are packed once into an image - per 256-value super-block the matrix-core operands of its instructions (x as
  * two binary16 terms, scaled per token and super-block), then the scales and sub-block sums - and every matrix that meets
  * those activations (q | k | v | gate | up of a layer) is one launch that reads its weights once for all the tokens. The
@@ -134,7 +134,8 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
  * sub-blocks differently; Q5_K reads the Q4_K image, so one pack serves matrices of both types).
  *   cogni_gemv_image_bytes  size of the image for (type, in_dim, tokens); 0 = no one-pass kernel for that combination.
  *   cogni_gemv_pack_dev     kernel "pack_x_mt_q4k_f16" | "pack_x_mt_q6k_f16" (x, image, tokens:u32, in_dim:u32), block 256,
- *                           grid 2 * in_dim / 256.
+ *                           grid 2 * S with S = in_dim / 256 rounded up to a multiple of 8 (the image holds S super-blocks:
+ *                           the eight k-slices of the GEMV take S / 8 each, the ones past the row's end are zeros).
  *   cogni_gemv_packed_dev   `count` (1..8) matrices of one type and in_dim against the image:
  *                           out[i][m*out_dims[i] + o] = (residual ? residual[m*out_dims[0] + o] : 0) + sum_j x[m][j] deq(W_i[o][j])
  *                           (a residual only with count == 1). Kernel "q4_k_gemv_mt_f32" | "q5_k_gemv_mt_f32" |
@@ -157,6 +158,12 @@ size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens)
  * earlier: Q6_K 2, Q4_K and Q5_K 3, and 2 from 98304 rows), 0 where they never do; below it the call runs the kernel
  * cogni_gemv_plan names. No GPU needed. */
 uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim, uint32_t out_dim);
+/* The same for the calls that take several matrices of one input (cogni_gemv_dual_dev, cogni_gemv_many_dev,
+ * cogni_gemv_dual_swiglu_dev): 2, or 5 where a row fills less than three quarters of the eight k-slices the kernel
+ * divides it into (in_dim / 256 rounded up to a multiple of 8: rows of 256..1280, 2304, 2560 values ...); 0 = never.
+ * Rows that are not a multiple of 2048 values also wait for 5 tokens in cogni_gemv_one_pass_from when they fill less
+ * than that. No GPU needed. */
+uint32_t cogni_gemv_one_pass_multi_from(uint32_t w_type, uint32_t in_dim);
 /* Gives back the image the library keeps for `stream` (waits for the stream's work first; nothing to do and no error if it
  * has none). Call it before destroying a stream that ran multi-token GEMVs: the eight slots are otherwise used up by the
  * first eight streams of the process, and later streams run the per-token-group kernels. A graph captured on the stream

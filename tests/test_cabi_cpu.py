@@ -251,20 +251,30 @@ def test_one_pass_geometry_and_thresholds():
     assert quant.gemv_image_bytes(12, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(14, 12288, 2) == 48 * (8192 + 1024)
     assert quant.gemv_image_bytes(13, 4096, 4) == quant.gemv_image_bytes(12, 4096, 4)      # Q5_K reads the Q4_K image
-    for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1024, 4), (12, 14336, 4), (13, 1024, 4), (8, 4096, 4), (12, 0, 4)):
+    # rows that are not a multiple of 2048 values: the image is filled up to a multiple of 8 super-blocks
+    assert quant.gemv_image_bytes(12, 1024, 4) == 8 * (8192 + 1024)
+    assert quant.gemv_image_bytes(14, 5120, 8) == 24 * (8192 + 1024)
+    assert quant.gemv_image_bytes(13, 256, 2) == 8 * (8192 + 1024)
+    for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1000, 4), (12, 14336, 4), (13, 12544, 4), (8, 4096, 4), (12, 0, 4)):
         assert quant.gemv_image_bytes(t, in_dim, tokens) == 0, (t, in_dim, tokens)
-    assert [quant.gemv_one_pass_from(12, d, 4096) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 0]
-    assert [quant.gemv_one_pass_from(13, d, 8192) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 0]
+    assert [quant.gemv_one_pass_from(12, d, 4096) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 5]
+    assert [quant.gemv_one_pass_from(13, d, 8192) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 5]
+    # rows that fill less than three quarters of their k-slices wait for five tokens, whatever the type and the height
+    assert [quant.gemv_one_pass_from(14, d, 4096) for d in (1024, 2560, 3584, 5120)] == [5, 5, 3, 3]
+    assert [quant.gemv_one_pass_from(12, d, 151936) for d in (1024, 2560, 3584)] == [5, 5, 2]
+    assert [quant.gemv_one_pass_multi_from(12, d) for d in (256, 1024, 1536, 2048, 2560, 3072, 4096, 5120, 12288, 12544, 1000)] == \
+        [5, 5, 2, 2, 5, 2, 2, 2, 2, 0, 0]
+    assert quant.gemv_one_pass_multi_from(8, 4096) == 0 and quant.gemv_one_pass_multi_from(14, 1024) == 5
     assert [quant.gemv_one_pass_from(t, 4096, 12288) for t in (14, 8, 2)] == [3, 0, 0]
     # tall matrices of up to 4096 columns (an output head) take the path earlier
     assert [quant.gemv_one_pass_from(14, 4096, r) for r in (40959, 40960, 151936)] == [3, 2, 2]
     assert [quant.gemv_one_pass_from(12, 4096, r) for r in (40959, 40960, 98303, 98304, 151936)] == [4, 3, 3, 2, 2]
     assert [quant.gemv_one_pass_from(13, 2048, r) for r in (40960, 98304)] == [3, 2]
-    assert [quant.gemv_one_pass_from(t, 12288, 151936) for t in (12, 14)] == [4, 3] and quant.gemv_one_pass_from(12, 1024, 151936) == 0
+    assert [quant.gemv_one_pass_from(t, 12288, 151936) for t in (12, 14)] == [4, 3] and quant.gemv_one_pass_from(12, 14336, 151936) == 0
     rng = np.random.default_rng(11)
     for t, tmax, lds in ((12, 3, 8 * 3 * 8 * 16 * 4 + 8 * 6 * 16 * 144), (13, 3, 8 * 3 * 8 * 16 * 4 + 8 * 6 * 16 * 176),
                          (14, 2, 8 * 3 * 8 * 16 * 4 + 8 * 4 * 16 * 240)):
-        for in_dim in (2048, 4096, 6144, 8192, 10240, 12288):
+        for in_dim in (256, 1024, 2048, 3584, 4096, 5120, 6144, 8192, 10240, 11008, 12288):
             for rows in [1, 15, 16, 17, 4096, 4097, 12288, 8 * 4096 - 16, 151936] + [int(r) for r in rng.integers(1, 400000, 40)]:
                 grid, block, shmem = quant.gemv_packed_launch_dims(t, in_dim, rows)
                 ntiles = -(-rows // 16)
@@ -272,7 +282,7 @@ def test_one_pass_geometry_and_thresholds():
                 groups = -(-ntiles // tiles)
                 assert (block, shmem) == (512, lds) and shmem <= 160 * 1024
                 assert grid == min(256, groups) and grid >= 1
-    for bad in ((12, 1024, 16), (8, 4096, 16), (12, 4096, 0)):
+    for bad in ((12, 1000, 16), (12, 12544, 16), (8, 4096, 16), (12, 4096, 0)):
         with pytest.raises(quant.QuantError):
             quant.gemv_packed_launch_dims(*bad)
 
@@ -280,7 +290,7 @@ def test_one_pass_geometry_and_thresholds():
 def test_one_pass_argument_errors_do_not_need_a_gpu():
     assert hip.lib().cogni_gemv_release_stream(None) == 0          # a stream without an image: nothing to do
     with pytest.raises(quant.QuantError, match="no one-pass kernel") as e:
-        quant.gemv_pack_dev(0x1000, 12, 1024, 4, 0x2000)
+        quant.gemv_pack_dev(0x1000, 12, 1000, 4, 0x2000)
     assert e.value.code == -1
     with pytest.raises(quant.QuantError, match="null device pointer"):
         quant.gemv_pack_dev(0, 12, 4096, 4, 0x2000)
@@ -301,7 +311,7 @@ def test_one_pass_argument_errors_do_not_need_a_gpu():
     with pytest.raises(quant.QuantError, match="null device pointer"):
         quant.gemv_packed_top1_dev(0x1000, 14, 0, 0x3000, 0x4000, 0x5000, 0x6000, 4096, 1000, 4)
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
-        quant.rmsnorm_pack_dev(0x1000, 0x2000, 0, 12, 0x3000, 1024, 4)
+        quant.rmsnorm_pack_dev(0x1000, 0x2000, 0, 12, 0x3000, 1000, 4)
     with pytest.raises(quant.QuantError, match="bad out_dim"):
         quant.gemv_packed_swiglu_dev(0x1000, 0x1100, 12, 0x2000, 0x3000, 4096, 0, 4)
 

@@ -173,9 +173,9 @@ def test_one_pass_element_order_and_scale_positions(gpu, oracle):
 
 def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
     """9 and 13 tokens: a group of eight in one pass, the rest as the token count decides (one token on the vector ALU,
-    five in one pass); in_dim 1024 and in_dim above 12288 have no one-pass kernel and keep their older paths."""
+    five in one pass); in_dim above 12288 has no one-pass kernel and keeps its older path (four tokens per pass)."""
     rng = np.random.default_rng(11)
-    for in_dim, out_dim, tokens in ((4096, 272, 9), (2048, 100, 13), (1024, 64, 8)):
+    for in_dim, out_dim, tokens in ((4096, 272, 9), (2048, 100, 13), (14336, 64, 8)):
         raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
         x = synth.make_activations(rng, tokens, in_dim)
         want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens)
@@ -184,11 +184,49 @@ def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
         assert_bars(od.read(np.float32, tokens * out_dim), want, tol, tokens, out_dim, "%dx%d M=%d" % (in_dim, out_dim, tokens))
         for a in (w, xd, od):
             a.close()
-    assert quant.gemv_image_bytes(Q4_K, 1024, 8) == 0 and quant.gemv_image_bytes(Q5_K, 4096, 8) == 16 * (8192 + 1024)
+    assert quant.gemv_image_bytes(Q4_K, 1000, 8) == 0 and quant.gemv_image_bytes(Q5_K, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(Q4_K, 14336, 8) == 0 and quant.gemv_image_bytes(Q6_K, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(Q4_K, 4096, 1) == 0 and quant.gemv_image_bytes(Q4_K, 4096, 9) == 0
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
-        quant.gemv_pack_dev(0x1000, Q4_K, 1024, 8, 0x1000)
+        quant.gemv_pack_dev(0x1000, Q4_K, 14336, 8, 0x1000)
+
+
+RAGGED_ROWS = [(Q4_K, 1024, 4096), (Q4_K, 256, 48), (Q4_K, 2560, 16 * 3 * 256 + 24), (Q4_K, 3584, 1040), (Q4_K, 5120, 5120),
+               (Q4_K, 6912, 530), (Q4_K, 11008, 4096), (Q4_K, 1792, 37),
+               (Q5_K, 1024, 1040), (Q5_K, 2560, 4096), (Q5_K, 5120, 530), (Q5_K, 11776, 50),
+               (Q6_K, 1024, 4096), (Q6_K, 768, 37), (Q6_K, 2560, 16 * 2 * 256 + 24), (Q6_K, 3584, 3584), (Q6_K, 5120, 1040),
+               (Q6_K, 9472, 530), (Q6_K, 11008, 16 * 257)]
+
+
+@pytest.mark.parametrize("type_id,in_dim,out_dim", RAGGED_ROWS)
+@pytest.mark.parametrize("tokens", [5, 8])
+def test_rows_that_do_not_fill_their_k_slices(gpu, oracle, type_id, in_dim, out_dim, tokens):
+    """in_dim any multiple of 256: the eight k-slices take ceil(super-blocks / 8) each, the image is filled up with zero
+    super-blocks and a k-slice without a super-block of its own re-reads the row's last block against those zeros. Rows of
+    1 (only one wavefront has real work), 3, 4, 7, 10, 14, 20, 27, 37, 43 and 46 super-blocks: resident and streamed
+    operands, one to three tiles per wavefront, partial tiles; with and without residual; the explicit image as well."""
+    print("case type=%d in_dim=%d out_dim=%d tokens=%d" % (type_id, in_dim, out_dim, tokens), flush=True)
+    nsbp = -(-(in_dim // 256) // 8) * 8
+    assert quant.gemv_image_bytes(type_id, in_dim, tokens) == nsbp * (8192 + 1024)
+    assert quant.gemv_passes(type_id, tokens, in_dim, out_dim) == 1
+    rng = np.random.default_rng(type_id * 1000003 + in_dim * 13 + out_dim * 7 + tokens)
+    raw = synth.make_weights(rng, type_id, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    res = rng.standard_normal(tokens * out_dim).astype(np.float32)
+    want, tol = oracle_rows(oracle, raw, x, in_dim, out_dim, tokens, type_id)
+    w, xd, od, rd = DevArray(raw), DevArray(x), DevArray(nbytes=4 * tokens * out_dim), DevArray(res)
+    quant.gemv_dev(w.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, tokens)
+    plain = od.read(np.float32, tokens * out_dim)
+    assert_bars(plain, want, tol, tokens, out_dim, "type %d %dx%d M=%d" % (type_id, in_dim, out_dim, tokens))
+    quant.gemv_dev(w.ptr, type_id, xd.ptr, od.ptr, in_dim, out_dim, tokens, rd.ptr)
+    assert np.array_equal(od.read(np.float32, tokens * out_dim), plain + res)
+    # the same through a caller-owned image that held other data before (the zero super-blocks are written by the pack)
+    image = DevArray(np.full(quant.gemv_image_bytes(type_id, in_dim, tokens), 0x7B, dtype=np.uint8))
+    quant.gemv_pack_dev(xd.ptr, type_id, in_dim, tokens, image.ptr)
+    quant.gemv_packed_dev([w.ptr], type_id, image.ptr, [od.ptr], [out_dim], in_dim, tokens)
+    assert np.array_equal(od.read(np.float32, tokens * out_dim), plain)
+    for a in (w, xd, od, rd, image):
+        a.close()
 
 
 LONG_AND_Q6K = [(Q4_K, 12288, 4096), (Q4_K, 6144, 530), (Q4_K, 8192, 16 * 300 + 5), (Q4_K, 10240, 33),

@@ -48,14 +48,15 @@ def test_rmsnorm_argument_errors(gpu):
 
 
 @pytest.mark.parametrize("w_type", [12, 13, 14])
-@pytest.mark.parametrize("dim,tokens", [(4096, 8), (4096, 3), (2048, 1), (2048, 6)])
+@pytest.mark.parametrize("dim,tokens", [(4096, 8), (4096, 3), (2048, 1), (2048, 6), (1024, 5), (2560, 8), (3584, 2), (256, 4)])
 def test_norms_that_also_write_the_activation_image(gpu, w_type, dim, tokens):
     """rmsnorm_pack / add_rmsnorm_pack: the normalised rows and residual stream of the plain kernels, bit for bit, and the
     image cogni_gemv_pack_dev writes from those rows, byte for byte (absent tokens' slots zeroed; the image buffer starts as
-    garbage). With the fp32 output left out the image is the same."""
+    garbage; rows that are not a multiple of 2048 values: the zero super-blocks that fill the image up as well). With the
+    fp32 output left out the image is the same."""
     rng = np.random.default_rng(dim + 17 * tokens + w_type)
     x = (rng.standard_normal(tokens * dim) * 2.5).astype(np.float32)
-    x[:300] *= np.float32(1e-20)                                   # a super-block far below the binary16 range
+    x[:min(300, dim)] *= np.float32(1e-20)                                   # a super-block far below the binary16 range
     add = rng.standard_normal(tokens * dim).astype(np.float32)
     w = (1.0 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
     eps = 1.0e-6
@@ -94,7 +95,7 @@ def test_norms_that_also_write_the_activation_image(gpu, w_type, dim, tokens):
 
 def test_norm_pack_argument_errors(gpu):
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
-        quant.rmsnorm_pack_dev(1, 1, 1, 12, 1, 1024, 4)            # no one-pass kernel for rows of 1024
+        quant.rmsnorm_pack_dev(1, 1, 1, 12, 1, 1000, 4)            # no one-pass kernel for rows of 1000
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
         quant.rmsnorm_pack_dev(1, 1, 1, 12, 1, 6144, 4)            # longer than a thread keeps
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
