@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
-"""Build-time check of the gfx950 code object for two instruction-spacing rules that the compiler keeps for the code it
-emits itself but cannot keep for instructions written inside asm statements:
+"""Build-time check of the gfx950 code object for rules that the compiler keeps for the code it emits itself but cannot
+keep for instructions written inside asm statements:
 
   * a vector instruction that writes a scalar register (v_readfirstlane_b32, v_readlane_b32, a compare with a scalar
     destination, a carry-out) must be five wait states ahead of a memory instruction that reads that register as its
@@ -9,6 +9,12 @@ emits itself but cannot keep for instructions written inside asm statements:
   * in the kernels whose copies to LDS set M0 inside asm statements (names with "_mt_"), the compiler does not know
     that M0 changes, so nothing may read a value of M0 that it assumes to have survived: every instruction that reads
     M0 must have a write of M0 within the two instructions in front of it, with no label in between.
+
+  * in the same kernels the loads into registers are written in asm statements too, so the compiler takes their
+    destinations for valid from the load on and does not know about the counted s_waitcnt vmcnt(N) that makes them
+    so: no instruction may read or write such a register between its load and the wait that covers it (vector memory
+    instructions retire in order: after vmcnt(N) all but the last N issued are done). Followed along the fall-through
+    path only: behind an unconditional branch nothing is taken to be pending.
 
 An instruction is one wait state, "s_nop N" is N + 1. The scan is linear over each kernel of the disassembly (this
 library's own code object, made by llvm-objdump); labels do not reset it, so a sequence that is only adjacent in the
@@ -74,9 +80,31 @@ def vmem_scalar_base(mnemonic, operands):
     return out
 
 
+VREG = re.compile(r"(?<![a-z0-9_])v(\d+)(?![0-9\[])|(?<![a-z0-9_])v\[(\d+):(\d+)\]")
+
+
+def vregs(text):
+    """The vector registers a piece of operand text names."""
+    out = set()
+    for m in VREG.finditer(text):
+        if m.group(1) is not None:
+            out.add(int(m.group(1)))
+        else:
+            out |= set(range(int(m.group(2)), int(m.group(3)) + 1))
+    return out
+
+
+def waited_vmcnt(operands_text):
+    """N of an s_waitcnt that has a vmcnt field, else None."""
+    m = re.search(r"vmcnt\((\d+)\)", operands_text)
+    return int(m.group(1)) if m else None
+
+
 def check(lines):
     problems = []
     kernel = "?"
+    vm_issued = 0    # vector memory instructions issued so far in this kernel
+    pending = []     # (issue number, destination vgprs, text) of loads into registers not yet covered by a wait
     recent = []      # (wait states since, written sgprs, text) of recent vector-writes-scalar instructions
     m0_age = None    # wait states since the last write of m0
     m0_dist = None   # instructions since the last write of m0 in this basic block
@@ -89,6 +117,7 @@ def check(lines):
             if not lab.group(1).startswith("L"):
                 kernel = lab.group(1)
                 recent, m0_age = [], None
+                vm_issued, pending = 0, []
             m0_dist = None
             continue
         if line.endswith(":") or line.startswith((".", "Disassembly", "/")) or "file format" in line:
@@ -96,6 +125,25 @@ def check(lines):
         parts = line.split(None, 1)
         mnemonic = parts[0]
         operands = [o.strip() for o in parts[1].split(",")] if len(parts) > 1 else []
+        if asm_m0_kernel(kernel):
+            if mnemonic == "s_waitcnt":
+                n = waited_vmcnt(parts[1] if len(parts) > 1 else "")
+                if n is not None:
+                    pending = [p for p in pending if p[0] > vm_issued - n]
+            elif pending:
+                touched = vregs(parts[1]) if len(parts) > 1 else set()
+                for num, regs, text in pending:
+                    if touched & regs:
+                        problems.append("%s: '%s' touches v%s, loaded by '%s' %d vector memory instruction(s) ago and not waited for" % (
+                            kernel, line, sorted(touched & regs)[:4], text, vm_issued - num))
+                        break
+            if mnemonic in ("s_branch", "s_endpgm", "s_setpc_b64"):
+                pending = []   # what follows is reached from elsewhere, not by falling through
+            if is_vmem(mnemonic):
+                vm_issued += 1
+                to_lds = "_lds_" in mnemonic or (operands and operands[-1].strip().endswith("lds"))
+                if "_load_" in mnemonic and not to_lds and operands:
+                    pending.append((vm_issued, vregs(operands[0]), line))
         if is_vmem(mnemonic):
             used = vmem_scalar_base(mnemonic, operands)
             for age, regs, text in recent:

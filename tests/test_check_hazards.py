@@ -60,6 +60,29 @@ def test_m0_readers_in_kernels_with_asm_copies():
     assert ch.check(lines("s_mov_b32 m0, s3\ns_nop 0\nglobal_load_lds_dwordx4 v[2:3], off\nv_mov_b32_e32 v1, v2\nv_mov_b32_e32 v1, v2\nglobal_load_lds_dwordx4 v[4:5], off")) == []
 
 
+def test_registers_of_asm_loads_are_left_alone_until_their_wait():
+    """Kernels whose loads are written in asm statements: nothing reads or writes a load's destination before the
+    s_waitcnt vmcnt(N) that covers it (in-order retirement: all but the last N issued are done)."""
+    def mt(text):
+        return ["0000000000001000 <q4_k_gemv_mt_f32>:"] + lines(text)[1:]
+    load = "global_load_dwordx4 v[4:7], v1, s[2:3]\n"
+    assert len(ch.check(mt(load + "v_add_f32_e32 v9, v5, v8"))) == 1                       # read before any wait
+    assert len(ch.check(mt(load + "v_mov_b32_e32 v6, v8"))) == 1                           # overwritten before it lands
+    assert ch.check(mt(load + "s_waitcnt vmcnt(0)\nv_add_f32_e32 v9, v5, v8")) == []
+    assert ch.check(mt(load + "v_add_f32_e32 v9, v10, v8\nv_mov_b32_e32 v3, v40")) == []    # other registers (v40 is not v4)
+    # two more memory instructions behind it: vmcnt(2) covers it, vmcnt(3) does not; a wait without a vmcnt field does not
+    two = load + "global_load_dwordx4 v[10:13], v1, s[2:3] offset:16\ns_mov_b32 m0, s9\ns_nop 0\nglobal_load_lds_dwordx4 v[20:21], off\n"
+    assert ch.check(mt(two + "s_waitcnt vmcnt(2)\nv_add_f32_e32 v9, v5, v8")) == []
+    assert len(ch.check(mt(two + "s_waitcnt vmcnt(3)\nv_add_f32_e32 v9, v5, v8"))) == 1
+    assert len(ch.check(mt(two + "s_waitcnt lgkmcnt(0)\nv_add_f32_e32 v9, v5, v8"))) == 1
+    assert len(ch.check(mt(two + "s_waitcnt vmcnt(2)\nv_add_f32_e32 v9, v11, v8"))) == 1     # the second load is still out
+    # a store that takes its data from a pending register, and the code behind an unconditional branch (reached from elsewhere)
+    assert len(ch.check(mt(load + "global_store_dword v1, v4, s[2:3]"))) == 1
+    assert ch.check(mt(load + "s_branch 12\nv_add_f32_e32 v9, v5, v8")) == []
+    # kernels the compiler writes the loads of: its own business
+    assert ch.check(lines(load + "v_add_f32_e32 v9, v5, v8")) == []
+
+
 def test_a_new_kernel_starts_clean():
     two = lines("v_readfirstlane_b32 s6, v147") + ["0000000000002000 <k2>:", "\tglobal_load_dword v3, v1, s[6:7]    // 0: 0"]
     assert ch.check(two) == []
