@@ -292,7 +292,7 @@ int cogni_quant_init(int32_t ordinal) {
     g_rt.image_pool = nullptr;
     return undo(hip_fail(he, "hipMalloc(activation images)"));
   }
-  for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q5_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32",
+  for (const char* name : {"pack_x_mt_q4k_f16", "pack_x_mt_q6k_f16", "q4_k_gemv_mt_f32", "q5_k_gemv_mt_f32", "q6_k_gemv_mt_f32", "q8_0_gemv_mt_f32", "q4_k_gemv_mt_swiglu_f32",
                            "q4_k_gemv_mt_top1_partial_f32", "q6_k_gemv_mt_top1_partial_f32", "rmsnorm_pack_q4k_f32",
                            "rmsnorm_pack_q6k_f32", "add_rmsnorm_pack_q4k_f32", "add_rmsnorm_pack_q6k_f32"})
     if (int rc = resolve(name, true)) return undo(rc);
@@ -433,7 +433,8 @@ int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image
     if (total > 0x7FFFFFFFull) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_dev: too many rows");
     uint64_t res = i0 == 0 ? residual : 0;
     void* params[] = {&w[0], &w[1], &w[2], &image, &res, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2], &tokens};
-    const int rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt_f32" : (w_type == COGNI_TYPE_Q5_K ? "q5_k_gemv_mt_f32" : "q4_k_gemv_mt_f32"), gemv_mt_grid(w_type, in_dim, (uint32_t)total),
+    const char* kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt_f32" : (w_type == COGNI_TYPE_Q5_K ? "q5_k_gemv_mt_f32" : (w_type == COGNI_TYPE_Q8_0 ? "q8_0_gemv_mt_f32" : "q4_k_gemv_mt_f32"));
+    const int rc = launch(kernel, gemv_mt_grid(w_type, in_dim, (uint32_t)total),
                           GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type), params, stream);
     if (rc != 0) return rc;
     i0 += n;

@@ -179,11 +179,11 @@ static inline unsigned gemv_mfma_lds_bytes(unsigned type, int tokens, unsigned i
 #define GEMV_MT_TMAX 3              // 16-row tiles a wavefront carries at most (Q4_K, Q5_K; Q6_K two)
 #define GEMV_MT_MAX_TOKENS 8
 #define GEMV_MT_MAX_IN_DIM 12288u
-// Shapes the kernels take: Q4_K, Q5_K or Q6_K, 2..8 tokens, in_dim a multiple of 256 up to 12288 (1..6 super-blocks per
+// Shapes the kernels take: Q4_K, Q5_K, Q6_K or Q8_0 (eight blocks at a time), 2..8 tokens, in_dim a multiple of 256 up to 12288 (1..6 super-blocks per
 // k-slice; a row whose super-blocks do not divide by 8 is worked on as if zeros filled it up, gemv_mt_padded_sb).
 static inline GEMV_HD int gemv_mt_supported(unsigned type, int tokens, unsigned in_dim) {
-  return (type == 12 || type == 13 || type == 14) && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && in_dim != 0 && (in_dim & 255u) == 0 &&
-         in_dim <= GEMV_MT_MAX_IN_DIM;
+  return (type == 12 || type == 13 || type == 14 || type == 8) && tokens >= 2 && tokens <= GEMV_MT_MAX_TOKENS && in_dim != 0 &&
+         (in_dim & 255u) == 0 && in_dim <= GEMV_MT_MAX_IN_DIM;
 }
 // super-blocks of the activation image: the row's, rounded up to a multiple of the 8 k-slices
 static inline GEMV_HD unsigned gemv_mt_padded_sb(unsigned in_dim) { return ((in_dim >> 8) + 7u) & ~7u; }
@@ -191,14 +191,21 @@ static inline GEMV_HD unsigned gemv_mt_padded_sb(unsigned in_dim) { return ((in_
 // the pair measures faster. Q6_K from three tokens; Q4_K and Q5_K from four on rows of 4096 values and more, else from five.
 // Tall matrices of up to 4096 columns (an output head): the workgroups walk many row groups and pay their start once, which
 // puts the kernel ahead earlier - Q6_K from two tokens at GEMV_MT_TALL_ROWS rows, Q4_K and Q5_K from three there and from
-// two at GEMV_MT_VERY_TALL_ROWS.
+// two at GEMV_MT_VERY_TALL_ROWS. Q8_0 (the other way is one launch on the vector ALU for up to eight tokens, whose time
+// grows with every token: 3584 -> 1024 takes 9.0 / 13.6 / 21.3 us at 2 / 4 / 8 tokens against 7.3 in one pass): from two
+// tokens on rows of 3584 values and more and on tall matrices, else from three; half-filled rows (1024 values) from five.
 #define GEMV_MT_TALL_ROWS 40960u
 #define GEMV_MT_VERY_TALL_ROWS 98304u
 static inline unsigned gemv_mt_from(unsigned type, unsigned in_dim, unsigned out_dim) {
   if (!gemv_mt_supported(type, 2, in_dim)) return 0;
   // rows that fill less than three quarters of their eight k-slices (1024 values: half of them): from five tokens, where
   // the per-token-group kernels start to read the weights twice
-  if (4u * (in_dim >> 8) < 3u * gemv_mt_padded_sb(in_dim)) return 5u;
+  const int sparse = 4u * (in_dim >> 8) < 3u * gemv_mt_padded_sb(in_dim);
+  if (type == 8) {
+    if (out_dim >= GEMV_MT_TALL_ROWS) return 2u;
+    return sparse ? 5u : (in_dim >= 3584u ? 2u : 3u);
+  }
+  if (sparse) return 5u;
   if (in_dim <= 4096u && out_dim >= GEMV_MT_TALL_ROWS) return (type == 14 || out_dim >= GEMV_MT_VERY_TALL_ROWS) ? 2u : 3u;
   return type == 14 ? 3u : (in_dim >= 4096u ? 4u : 5u);
 }
@@ -212,7 +219,7 @@ static inline unsigned gemv_mt_multi_from(unsigned type, unsigned in_dim) {
 // busy, at most three (Q4_K) or two (Q6_K: its units are larger). Host and kernel use the same rule.
 static inline GEMV_HD unsigned gemv_mt_tiles(unsigned type, unsigned in_dim, unsigned ntiles) {
   if (in_dim > 4096u) return 1;
-  const unsigned tmax = type == 14 ? 2u : (unsigned)GEMV_MT_TMAX;
+  const unsigned tmax = (type == 14 || type == 8) ? 2u : (unsigned)GEMV_MT_TMAX;
   unsigned t = ntiles / 256u;
   if (t < 1) t = 1;
   if (t > tmax) t = tmax;
@@ -224,10 +231,10 @@ static inline unsigned gemv_mt_grid(unsigned type, unsigned in_dim, unsigned tot
   return groups < 256u ? groups : 256u;   // more groups than compute units: the workgroups walk them
 }
 // the k-slices' partial sums, then per wavefront the slots of its units: 6 x (16 rows x 144 B) for Q4_K, 6 x (16 rows x
-// 176 B) for Q5_K, 4 x (16 rows x 240 B) for Q6_K
+// 176 B) for Q5_K, 4 x (16 rows x 240 B) for Q6_K, 4 x (16 rows x 272 B) for Q8_0
 static inline unsigned gemv_mt_lds_bytes(unsigned type) {
   return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u +
-         GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : (type == 13 ? 6u * 2816u : 6u * 2304u));
+         GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : (type == 8 ? 4u * 4352u : (type == 13 ? 6u * 2816u : 6u * 2304u)));
 }
 // bytes of the activation image: per super-block (of the padded count) 8 KiB of operands, then 16 bytes per (super-block, lane) for the scales and
 // the sub-block sums (one more matrix-core operand). Q4_K and Q5_K share one image, Q6_K has its own.

@@ -1,4 +1,4 @@
-// Decode GEMV for 2..8 tokens in ONE pass over the weights, Q4_K, Q5_K and Q6_K, on the matrix cores:
+// Decode GEMV for 2..8 tokens in ONE pass over the weights, Q4_K, Q5_K, Q6_K and Q8_0, on the matrix cores:
 //   out_i[m][o] = (residual[m][o] +) sum_j x[m][j] * deq(W_i[o][j])      for up to three matrices W_i of one in_dim.
 //
 // Kernels.
@@ -7,8 +7,8 @@
 //     super-block of 256 values the matrix-core operands of its instructions, laid out lane by lane, followed by the
 //     scale and the sub-block sums of every (token, super-block). Written once per activation block, whatever the number
 //     of matrices that block then meets (q | k | v | gate | up of a decoder layer share one).
-//   q4_k_gemv_mt_f32 | q5_k_gemv_mt_f32 | q6_k_gemv_mt_f32 (w0, w1, w2, image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens)
-//     (Q5_K reads the image pack_x_mt_q4k_f16 writes)
+//   q4_k_gemv_mt_f32 | q5_k_gemv_mt_f32 | q6_k_gemv_mt_f32 | q8_0_gemv_mt_f32 (w0, w1, w2, image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens)
+//     (Q5_K and Q8_0 read the image pack_x_mt_q4k_f16 writes)
 //     block 512 (8 wavefronts), grid and dynamic shared memory from gemv_config.h (gemv_mt_grid, gemv_mt_lds_bytes).
 //     rows1 / rows2 may be 0 (then w1 / w2 / out1 / out2 are not read); residual (may be null) belongs to the first
 //     matrix. Row counts of all but the last matrix present must be multiples of 16. in_dim must be a multiple of 256
@@ -350,6 +350,73 @@ struct MtK45 {
 };
 typedef MtK45<false> MtQ4K;
 typedef MtK45<true> MtQ5K;
+
+// Q8_0 (34 B per 32 values: d, qs:i8[32]). Eight blocks are taken together as one 272-byte "super-block" of 256 values
+// (17 pieces of 16 bytes; in_dim a multiple of 256 makes every row a whole number of them, 16-byte aligned when the matrix
+// is). Block j of the eight is instruction j: a lane supplies bytes 8 kg .. 8 kg + 7 of its 32 codes, which the masks
+// deliver in the order (0, 2, 1, 3, 4, 6, 5, 7) - the order of the Q4_K image, so Q8_0 reads the image pack_x_mt_q4k_f16
+// writes. A code goes in as the unsigned byte q + 128 (q ^ 0x80 read as a binary16 subnormal, (q + 128) * 2^-24); the 128
+// comes out again through the sub-block sums: sum_j d_j * (sum(x u) - 128 sum(x)), with sum_j d_j * sum_j(x) as one more
+// instruction (the image's sums operand against the eight d as they are: binary16 numbers).
+// In LDS a row is its 272 bytes as they are: d of block j at 34 j, its codes at 34 j + 2. The codes of the odd blocks start
+// on a multiple of 4 (two dword reads); the even blocks' are 2 bytes off and come out of three dwords through
+// v_alignbyte_b32.
+struct MtQ80 {
+  static constexpr unsigned TYPE = 8;
+  static constexpr int BB = 272, P = 17, NCOPY = 5, LAST = 16, NAUX = 1, NSLOT = 4, TMAX = 2;
+  static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 64 * 16;
+  static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece * 16; }
+  static __device__ __forceinline__ u32 aux_offset(u32 lane) { return lane * 16; }
+  typedef MtK45<false>::Aux Aux;
+  static __device__ __forceinline__ Aux aux(const mt_u32x4 (&r)[NAUX]) { return MtK45<false>::aux(r); }
+  struct Raw { u32 q[8][2]; u32 d[8]; u32 kg; };   // (d: binary16 bits)
+  static __device__ __forceinline__ Raw read(const char* row, u32 kg) {
+    Raw w;
+    w.kg = kg;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      w.d[j] = *reinterpret_cast<const unsigned short*>(row + 34 * j);
+      const char* c = row + 34 * j + 2 + 8 * kg;
+      if (j & 1) {
+        w.q[j][0] = *reinterpret_cast<const u32*>(c);
+        w.q[j][1] = *reinterpret_cast<const u32*>(c + 4);
+      } else {
+        const u32 a = *reinterpret_cast<const u32*>(c - 2), b = *reinterpret_cast<const u32*>(c + 2), e = *reinterpret_cast<const u32*>(c + 6);
+        w.q[j][0] = __builtin_amdgcn_alignbyte(b, a, 2);
+        w.q[j][1] = __builtin_amdgcn_alignbyte(e, b, 2);
+      }
+    }
+    return w;
+  }
+  static __device__ __forceinline__ void unit(const Raw& w, const mt_u32x4 (&b)[8], const Aux& ax, float (&acc)[4]) {
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const u32 u0 = w.q[j][0] ^ 0x80808080u, u1 = w.q[j][1] ^ 0x80808080u;
+      uint4 a4;
+      a4.x = u0 & 0x00FF00FFu;          // bytes 0, 2
+      a4.y = (u0 >> 8) & 0x00FF00FFu;   // bytes 1, 3
+      a4.z = u1 & 0x00FF00FFu;
+      a4.w = (u1 >> 8) & 0x00FF00FFu;
+      const mt_float4 r = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(mt_half8, b[j]), __builtin_bit_cast(mt_half8, a4),
+                                                                 (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      const float dj = h2f(w.d[j]);
+#pragma unroll
+      for (int k = 0; k < 4; k++) sum[k] = fmaf(dj, r[k], sum[k]);
+    }
+    // sum_j d_j * sum_j(x): the image's sums (times 2^(e-5), hi and lo; sub-blocks 4 kg + (0, 2, 1, 3) for kg < 2) against d
+    const u32 dA = w.kg == 0 ? (w.d[0] | (w.d[2] << 16)) : (w.d[4] | (w.d[6] << 16));
+    const u32 dB = w.kg == 0 ? (w.d[1] | (w.d[3] << 16)) : (w.d[5] | (w.d[7] << 16));
+    const mt_u32x2 db = w.kg < 2 ? (mt_u32x2){dA, dB} : (mt_u32x2){0u, 0u};
+    const mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), __builtin_bit_cast(mt_half4, db),
+                                                                (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const float in = fmaf(MT_TWO_P24, sum[k], -4096.0f * off[k]);   // 128 * 2^5
+      acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
+    }
+  }
+};
 
 
 // Q6_K (210 B: ql[128], qh[64], scales:i8[16], d). Element 128 n + 32 k + l (half n, quarter k, l < 32) has its low four bits
@@ -767,6 +834,7 @@ __device__ __forceinline__ void gemv_mt_dispatch(const MtArgs& a, const uint8_t*
 GEMV_MT_ENTRY(q4_k_gemv_mt_f32, MtQ4K)
 GEMV_MT_ENTRY(q5_k_gemv_mt_f32, MtQ5K)
 GEMV_MT_ENTRY(q6_k_gemv_mt_f32, MtQ6K)
+GEMV_MT_ENTRY(q8_0_gemv_mt_f32, MtQ80)
 
 // (w, image, partial_ids, partial_values, in_dim, out_dim, tokens): the output head's arg-max for 2..8 tokens in one pass
 // over the weights. Grid, block and dynamic shared memory as q4_k_gemv_mt_f32 | q6_k_gemv_mt_f32 for out_dim rows;

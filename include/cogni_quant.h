@@ -125,13 +125,14 @@ int cogni_dequantize_dev(uint64_t w_raw, uint32_t w_type, uint64_t n_elements, u
 int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residual, uint64_t out,
                    uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 
-/* Several tokens in ONE pass over the weights (Q4_K, Q5_K and Q6_K, in_dim a multiple of 256 up to 12288, 2..8 tokens): the
+/* Several tokens in ONE pass over the weights (Q4_K, Q5_K, Q6_K and Q8_0, in_dim a multiple of 256 up to 12288, 2..8 tokens): the
  * activations are packed once into an image - per 256-value super-block the matrix-core operands of its instructions (x as
  * two binary16 terms, scaled per token and super-block), then the scales and sub-block sums - and every matrix that meets
  * those activations (q | k | v | gate | up of a layer) is one launch that reads its weights once for all the tokens. The
  * reference's multi-token kernels stop at four tokens per pass (tbatch4, src/ml/cuda/kernels/q4k_gemv_probe.ptx:437-768,
  * q6k_gemv_probe.ptx:977; q5k_gemv_probe.ptx:237). The image depends on the weight type (Q4_K and Q6_K order their
- * sub-blocks differently; Q5_K reads the Q4_K image, so one pack serves matrices of both types).
+ * sub-blocks differently; Q5_K and Q8_0 - eight of its blocks at a time - read the Q4_K image, so one pack serves matrices
+ * of the three types).
  *   cogni_gemv_image_bytes  size of the image for (type, in_dim, tokens); 0 = no one-pass kernel for that combination.
  *   cogni_gemv_pack_dev     kernel "pack_x_mt_q4k_f16" | "pack_x_mt_q6k_f16" (x, image, tokens:u32, in_dim:u32), block 256,
  *                           grid 2 * S with S = in_dim / 256 rounded up to a multiple of 8 (the image holds S super-blocks:
@@ -139,7 +140,7 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
  *   cogni_gemv_packed_dev   `count` (1..8) matrices of one type and in_dim against the image:
  *                           out[i][m*out_dims[i] + o] = (residual ? residual[m*out_dims[0] + o] : 0) + sum_j x[m][j] deq(W_i[o][j])
  *                           (a residual only with count == 1). Kernel "q4_k_gemv_mt_f32" | "q5_k_gemv_mt_f32" |
- *                           "q6_k_gemv_mt_f32" (w0, w1, w2,
+ *                           "q6_k_gemv_mt_f32" | "q8_0_gemv_mt_f32" (w0, w1, w2,
  *                           image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens), block 512, up to three
  *                           matrices per launch as one matrix of all their rows (a matrix whose row count is not a multiple
  *                           of 16 ends its launch), geometry from cogni_gemv_packed_launch_dims.
@@ -155,8 +156,8 @@ int cogni_gemv_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t residua
 size_t cogni_gemv_image_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 /* The token count from which cogni_gemv_dev and cogni_gemv_top1_dev take this path for one matrix (Q6_K 3; Q4_K and Q5_K 4
  * on rows of 4096 values and more, else 5; a tall matrix of up to 4096 columns - 40960 rows and more, an output head -
- * earlier: Q6_K 2, Q4_K and Q5_K 3, and 2 from 98304 rows), 0 where they never do; below it the call runs the kernel
- * cogni_gemv_plan names. No GPU needed. */
+ * earlier: Q6_K 2, Q4_K and Q5_K 3, and 2 from 98304 rows; Q8_0 2 on rows of 3584 values and more and on tall matrices,
+ * else 3), 0 where they never do; below it the call runs the kernel cogni_gemv_plan names. No GPU needed. */
 uint32_t cogni_gemv_one_pass_from(uint32_t w_type, uint32_t in_dim, uint32_t out_dim);
 /* The same for the calls that take several matrices of one input (cogni_gemv_dual_dev, cogni_gemv_many_dev,
  * cogni_gemv_dual_swiglu_dev): 2, or 5 where a row fills less than three quarters of the eight k-slices the kernel

@@ -175,7 +175,7 @@ static int gpu_probe() {
 static void stream_wait_spec() {
   struct Fmt { int slots, nc; };
   for (int S = 3; S <= 6; S++)
-    for (Fmt f : {Fmt{6, 3}, Fmt{4, 4}})
+    for (Fmt f : {Fmt{6, 3}, Fmt{4, 4}, Fmt{4, 5}})   // Q4_K | Q5_K, Q6_K, Q8_0
       for (int NS = 2; NS <= 3; NS++)
         for (int NA : {9, 13}) {
           const int NSLOT = f.slots < S ? f.slots : S, NC = f.nc;

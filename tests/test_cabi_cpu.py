@@ -255,7 +255,8 @@ def test_one_pass_geometry_and_thresholds():
     assert quant.gemv_image_bytes(12, 1024, 4) == 8 * (8192 + 1024)
     assert quant.gemv_image_bytes(14, 5120, 8) == 24 * (8192 + 1024)
     assert quant.gemv_image_bytes(13, 256, 2) == 8 * (8192 + 1024)
-    for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1000, 4), (12, 14336, 4), (13, 12544, 4), (8, 4096, 4), (12, 0, 4)):
+    assert quant.gemv_image_bytes(8, 4096, 4) == quant.gemv_image_bytes(12, 4096, 4)       # so does Q8_0, eight blocks at a time
+    for t, in_dim, tokens in ((12, 4096, 1), (12, 4096, 9), (12, 1000, 4), (12, 14336, 4), (13, 12544, 4), (8, 4128, 4), (2, 4096, 4), (12, 0, 4)):
         assert quant.gemv_image_bytes(t, in_dim, tokens) == 0, (t, in_dim, tokens)
     assert [quant.gemv_one_pass_from(12, d, 4096) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 5]
     assert [quant.gemv_one_pass_from(13, d, 8192) for d in (2048, 4096, 6144, 12288, 14336, 1024)] == [5, 4, 4, 4, 0, 5]
@@ -264,8 +265,11 @@ def test_one_pass_geometry_and_thresholds():
     assert [quant.gemv_one_pass_from(12, d, 151936) for d in (1024, 2560, 3584)] == [5, 5, 2]
     assert [quant.gemv_one_pass_multi_from(12, d) for d in (256, 1024, 1536, 2048, 2560, 3072, 4096, 5120, 12288, 12544, 1000)] == \
         [5, 5, 2, 2, 5, 2, 2, 2, 2, 0, 0]
-    assert quant.gemv_one_pass_multi_from(8, 4096) == 0 and quant.gemv_one_pass_multi_from(14, 1024) == 5
-    assert [quant.gemv_one_pass_from(t, 4096, 12288) for t in (14, 8, 2)] == [3, 0, 0]
+    assert quant.gemv_one_pass_multi_from(8, 4096) == 2 and quant.gemv_one_pass_multi_from(14, 1024) == 5 and quant.gemv_one_pass_multi_from(2, 4096) == 0
+    # Q8_0: from two tokens on long rows and on tall matrices, from three on shorter rows, from five on half-filled ones
+    assert [quant.gemv_one_pass_from(8, d, 4096) for d in (1024, 2048, 3584, 4096, 12288, 12320)] == [5, 3, 2, 2, 2, 0]
+    assert quant.gemv_one_pass_from(8, 1024, 248320) == 2
+    assert [quant.gemv_one_pass_from(t, 4096, 12288) for t in (14, 8, 2)] == [3, 2, 0]
     # tall matrices of up to 4096 columns (an output head) take the path earlier
     assert [quant.gemv_one_pass_from(14, 4096, r) for r in (40959, 40960, 151936)] == [3, 2, 2]
     assert [quant.gemv_one_pass_from(12, 4096, r) for r in (40959, 40960, 98303, 98304, 151936)] == [4, 3, 3, 2, 2]
@@ -282,7 +286,7 @@ def test_one_pass_geometry_and_thresholds():
                 groups = -(-ntiles // tiles)
                 assert (block, shmem) == (512, lds) and shmem <= 160 * 1024
                 assert grid == min(256, groups) and grid >= 1
-    for bad in ((12, 1000, 16), (12, 12544, 16), (8, 4096, 16), (12, 4096, 0)):
+    for bad in ((12, 1000, 16), (12, 12544, 16), (8, 4128, 16), (2, 4096, 16), (12, 4096, 0)):
         with pytest.raises(quant.QuantError):
             quant.gemv_packed_launch_dims(*bad)
 
@@ -297,7 +301,7 @@ def test_one_pass_argument_errors_do_not_need_a_gpu():
     with pytest.raises(quant.QuantError, match="count must be 1..8"):
         quant.gemv_packed_dev([], 12, 0x2000, [], [], 4096, 4)
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
-        quant.gemv_packed_dev([0x1000], 8, 0x2000, [0x3000], [16], 4096, 4)
+        quant.gemv_packed_dev([0x1000], 2, 0x2000, [0x3000], [16], 4096, 4)
     with pytest.raises(quant.QuantError, match="a residual goes with a single matrix"):
         quant.gemv_packed_dev([0x1000, 0x1100], 12, 0x2000, [0x3000, 0x3100], [16, 16], 4096, 4, residual_ptr=0x4000)
     with pytest.raises(quant.QuantError, match="null pointer or zero rows"):

@@ -467,7 +467,9 @@ def test_swiglu_kernel_and_fused_gate_up(gpu, oracle):
         for d in (wg, wu, xd, og, ou, o2, of):
             d.close()
     with pytest.raises(quant.QuantError, match="Unsupported quant type for the fused gate/up SwiGLU: Q6_K"):
-        quant.gemv_dual_swiglu_dev(1, 1, Q6_K, 1, 1, 256, 16, 1)
+        big = DevArray(nbytes=1 << 20)   # (real memory behind the pointers: a call accepted by mistake would stay inside it)
+        quant.gemv_dual_swiglu_dev(big.ptr, big.ptr, Q6_K, big.ptr, big.ptr, 256, 16, 1)
+    big.close()
     for d in (gd, ud, od):
         d.close()
 

@@ -10,7 +10,7 @@ import pytest
 
 from cogni_ml_amd import hip, quant, synth
 from gpu_common import DevArray, gpu  # noqa: F401
-from helpers import Q4_K, Q5_K, Q6_K, cosine, gemv_tolerance
+from helpers import Q4_K, Q5_K, Q6_K, Q8_0, cosine, gemv_tolerance
 
 pytestmark = pytest.mark.gpu
 
@@ -187,21 +187,26 @@ def test_token_counts_above_eight_and_other_shapes_fall_back(gpu, oracle):
     assert quant.gemv_image_bytes(Q4_K, 1000, 8) == 0 and quant.gemv_image_bytes(Q5_K, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(Q4_K, 14336, 8) == 0 and quant.gemv_image_bytes(Q6_K, 4096, 8) == 16 * (8192 + 1024)
     assert quant.gemv_image_bytes(Q4_K, 4096, 1) == 0 and quant.gemv_image_bytes(Q4_K, 4096, 9) == 0
+    big = DevArray(nbytes=4 << 20)
     with pytest.raises(quant.QuantError, match="no one-pass kernel"):
-        quant.gemv_pack_dev(0x1000, Q4_K, 14336, 8, 0x1000)
+        quant.gemv_pack_dev(big.ptr, Q4_K, 14336, 8, big.ptr)   # (real memory of sufficient size behind the pointers)
+    big.close()
 
 
 RAGGED_ROWS = [(Q4_K, 1024, 4096), (Q4_K, 256, 48), (Q4_K, 2560, 16 * 3 * 256 + 24), (Q4_K, 3584, 1040), (Q4_K, 5120, 5120),
                (Q4_K, 6912, 530), (Q4_K, 11008, 4096), (Q4_K, 1792, 37),
                (Q5_K, 1024, 1040), (Q5_K, 2560, 4096), (Q5_K, 5120, 530), (Q5_K, 11776, 50),
                (Q6_K, 1024, 4096), (Q6_K, 768, 37), (Q6_K, 2560, 16 * 2 * 256 + 24), (Q6_K, 3584, 3584), (Q6_K, 5120, 1040),
-               (Q6_K, 9472, 530), (Q6_K, 11008, 16 * 257)]
+               (Q6_K, 9472, 530), (Q6_K, 11008, 16 * 257),
+               (Q8_0, 1024, 3584), (Q8_0, 3584, 1024), (Q8_0, 256, 37), (Q8_0, 2048, 16 * 2 * 256 + 24), (Q8_0, 4096, 1040),
+               (Q8_0, 5120, 530), (Q8_0, 12288, 50), (Q8_0, 7936, 16 * 257), (Q8_0, 2560, 16 * 600)]
 
 
 @pytest.mark.parametrize("type_id,in_dim,out_dim", RAGGED_ROWS)
 @pytest.mark.parametrize("tokens", [5, 8])
 def test_rows_that_do_not_fill_their_k_slices(gpu, oracle, type_id, in_dim, out_dim, tokens):
-    """in_dim any multiple of 256: the eight k-slices take ceil(super-blocks / 8) each, the image is filled up with zero
+    """(Q8_0 as well, at full and at ragged row lengths: eight of its 34-byte blocks stand for a super-block, the codes of
+    every second block sit 2 bytes off a dword in LDS.) in_dim any multiple of 256: the eight k-slices take ceil(super-blocks / 8) each, the image is filled up with zero
     super-blocks and a k-slice without a super-block of its own re-reads the row's last block against those zeros. Rows of
     1 (only one wavefront has real work), 3, 4, 7, 10, 14, 20, 27, 37, 43 and 46 super-blocks: resident and streamed
     operands, one to three tiles per wavefront, partial tiles; with and without residual; the explicit image as well."""
@@ -233,7 +238,9 @@ LONG_AND_Q6K = [(Q4_K, 12288, 4096), (Q4_K, 6144, 530), (Q4_K, 8192, 16 * 300 + 
                 (Q5_K, 4096, 8192), (Q5_K, 2048, 1040), (Q5_K, 4096, 16 * 3 * 256 * 2 + 24), (Q5_K, 2048, 37), (Q5_K, 4096, 16 * 600),
                 (Q5_K, 12288, 530), (Q5_K, 6144, 16 * 257), (Q5_K, 10240, 50),
                 (Q6_K, 12288, 4096), (Q6_K, 4096, 4096), (Q6_K, 2048, 1040), (Q6_K, 4096, 16 * 2 * 256 * 2 + 24), (Q6_K, 6144, 50),
-                (Q6_K, 8192, 16 * 257), (Q6_K, 2048, 37)]
+                (Q6_K, 8192, 16 * 257), (Q6_K, 2048, 37),
+                (Q8_0, 4096, 4096), (Q8_0, 2048, 1040), (Q8_0, 4096, 16 * 2 * 256 * 2 + 24), (Q8_0, 6144, 50), (Q8_0, 8192, 16 * 257),
+                (Q8_0, 10240, 530), (Q8_0, 12288, 4096)]
 
 
 @pytest.mark.parametrize("type_id,in_dim,out_dim", LONG_AND_Q6K)

@@ -40,11 +40,16 @@ def test_rmsnorm_and_add_rmsnorm(gpu, oracle, dim, tokens):
 
 
 def test_rmsnorm_argument_errors(gpu):
+    # (real device memory behind every pointer, large enough for the shapes named: a call that were accepted by mistake
+    # would stay inside it)
+    buf = DevArray(nbytes=4 << 20)
+    p = buf.ptr
     with pytest.raises(quant.QuantError, match="zero dimension"):
-        quant.rmsnorm_dev(1, 1, 1, 0, 1)
+        quant.rmsnorm_dev(p, p, p, 0, 1)
     with pytest.raises(quant.QuantError, match="null device pointer"):
-        quant.add_rmsnorm_dev(1, 0, 1, 1, 1, 16, 1)
-    quant.rmsnorm_dev(1, 1, 1, 16, 0)       # no tokens: nothing is launched
+        quant.add_rmsnorm_dev(p, 0, p, p, p, 16, 1)
+    quant.rmsnorm_dev(p, p, p, 16, 0)       # no tokens: nothing is launched
+    buf.close()
 
 
 @pytest.mark.parametrize("w_type", [12, 13, 14])
@@ -94,13 +99,18 @@ def test_norms_that_also_write_the_activation_image(gpu, w_type, dim, tokens):
 
 
 def test_norm_pack_argument_errors(gpu):
+    # (real device memory behind every pointer, large enough for the shapes named: a call that were accepted by mistake
+    # would stay inside it)
+    buf = DevArray(nbytes=4 << 20)
+    p = buf.ptr
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
-        quant.rmsnorm_pack_dev(1, 1, 1, 12, 1, 1000, 4)            # no one-pass kernel for rows of 1000
+        quant.rmsnorm_pack_dev(p, p, p, 12, p, 1000, 4)            # no one-pass kernel for rows of 1000
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
-        quant.rmsnorm_pack_dev(1, 1, 1, 12, 1, 6144, 4)            # longer than a thread keeps
+        quant.rmsnorm_pack_dev(p, p, p, 12, p, 6144, 4)            # longer than a thread keeps
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
-        quant.add_rmsnorm_pack_dev(1, 1, 1, 1, 1, 8, 1, 4096, 4)   # Q8_0 has no image
+        quant.add_rmsnorm_pack_dev(p, p, p, p, p, 2, p, 4096, 4)   # Q4_0 has no image
     with pytest.raises(quant.QuantError, match="one-pass GEMV takes"):
-        quant.rmsnorm_pack_dev(1, 1, 1, 14, 1, 4096, 9)
+        quant.rmsnorm_pack_dev(p, p, p, 14, p, 4096, 9)
     with pytest.raises(quant.QuantError, match="null device pointer"):
-        quant.add_rmsnorm_pack_dev(1, 1, 1, 0, 1, 12, 1, 4096, 4)
+        quant.add_rmsnorm_pack_dev(p, p, p, 0, p, 12, p, 4096, 4)
+    buf.close()

@@ -78,17 +78,17 @@ def test_random_gemm_shapes(gpu, oracle, seed):
 @pytest.mark.parametrize("seed", range(4))
 def test_random_one_pass_shapes(gpu, oracle, seed):
     """Shapes the one-pass kernels take (in_dim a multiple of 256 up to 12288, half of the draws a multiple of 2048; Q4_K,
-    Q5_K, Q6_K), drawn: 2..17 tokens (a
+    Q5_K, Q6_K, Q8_0), drawn: 2..17 tokens (a
     group of eight and what is left), single matrices with and without residual, lists of two to five matrices with row
     counts that are and are not multiples of 16, top-1, activations scaled far out of the binary16 range."""
     from test_gpu_gemv_one_pass import assert_bars, oracle_rows
     rng = np.random.default_rng(9100 + seed)
     for case in range(12):
-        t = [Q4_K, Q5_K, Q6_K][int(rng.integers(0, 3))]
+        t = [Q4_K, Q5_K, Q6_K, Q8_0][int(rng.integers(0, 4))]
         in_dim = 2048 * int(rng.integers(1, 7)) if rng.integers(0, 2) else 256 * int(rng.integers(1, 49))
         tokens = int(rng.integers(2, 18))
         kind = ["single", "residual", "list", "top1"][int(rng.integers(0, 4))]
-        if kind == "top1" and t == Q5_K:
+        if kind == "top1" and t in (Q5_K, Q8_0):
             kind = "single"
         count = int(rng.integers(2, 6)) if kind == "list" else 1
         dims = [int(rng.integers(1, 1500)) if rng.integers(0, 3) else 16 * int(rng.integers(1, 90)) for _ in range(count)]

@@ -113,9 +113,13 @@ def test_noalloc_top1_rejects_what_does_not_fit_the_static_array(gpu):
     fail before it launches anything (the pointers are never dereferenced)."""
     out_dim = 151936
     assert 8 * quant.gemv_top1_partials(Q8_0, out_dim) > quant.TOP1_NOALLOC_MAX_PARTIALS
+    # (real device memory behind every pointer, as large as the matrix named: a call accepted by mistake would stay inside it)
+    big = DevArray(nbytes=out_dim * (1024 // 32) * 34)
+    p = big.ptr
     with pytest.raises(quant.QuantError, match="exceed the static scratch of 65536") as e:
-        quant.gemv_top1_noalloc_dev(0x1000, Q8_0, 0x1000, 0x1000, 0x1000, 1024, out_dim, 8)
+        quant.gemv_top1_noalloc_dev(p, Q8_0, p, p, p, 1024, out_dim, 8)
     assert e.value.code == -1
     # the operator's own argument checks still apply
     with pytest.raises(quant.QuantError, match="Unsupported quant type"):
-        quant.gemv_top1_noalloc_dev(0x1000, 20, 0x1000, 0x1000, 0x1000, 1024, 64, 1)
+        quant.gemv_top1_noalloc_dev(p, 20, p, p, p, 1024, 64, 1)
+    big.close()
