@@ -337,7 +337,7 @@ def gemv_kernel_of(quant, w_type, tokens, in_dim, out_dim):
     """The kernel that dominates a gemv_dev call of this shape."""
     frm = quant.gemv_one_pass_from(w_type, in_dim, out_dim)
     if frm and tokens >= frm:
-        return {Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k"}[w_type] + "_gemv_mt_f32"
+        return {Q4_K: "q4_k", Q5_K: "q5_k", Q6_K: "q6_k", Q8_0: "q8_0"}[w_type] + "_gemv_mt_f32"
     return quant.gemv_plan(w_type, min(tokens, 4) if tokens > 1 else 1, in_dim, out_dim)[0]
 
 
@@ -526,6 +526,26 @@ def main():
     # several tokens against one pass over the weights (what config 5's row batches are made of)
     gemv_case("q4_k gemv 12288x4096 M=4", Q4_K, 12288, 4096, 4)
     gemv_case("q4_k gemv 12288x4096 M=8", Q4_K, 12288, 4096, 8)
+    # the same GEMV against an activation image that is already there (the norm in front wrote it, or an earlier matrix of the
+    # same input paid for the pack): what a projection costs inside a runner
+    img_case = GemvCase(hip, quant, synth, rng, Q4_K, 12288, 4096, 8)
+    image = hip.DeviceBuffer(quant.gemv_image_bytes(Q4_K, 4096, 8))
+    quant.gemv_pack_dev(img_case.x.ptr, Q4_K, 4096, 8, image.ptr, stream.handle)
+
+    def packed_only(copy, st):
+        quant.gemv_packed_dev([img_case.w[copy].ptr], Q4_K, image.ptr, [img_case.out.ptr], [12288], 4096, 8, 0, st.handle)
+    steps = steps_for(args, img_case.bytes_per_step)
+    r = measure(hip, stream, Rotating(packed_only, img_case.copies, img_case.w_bytes), steps, min(args.warmup, steps))
+    rec = gemv_record(r, img_case.bytes_per_step)
+    rec.update({"steps": steps, "kernel": "q4_k_gemv_mt_f32", "passes_over_weights": 1,
+                "traffic": traffic_field("q4_k_gemv_mt_f32", img_case.bytes_per_step)})
+    cases["q4_k gemv 12288x4096 M=8, image kept by the caller (no pack launch)"] = rec
+    log("case=q4_k gemv M=8 against a kept image\nhip_us=%.3f\ngbps_hbm=%.1f\n" % (r["us"], rec["gbps"]))
+    image.close()
+    img_case.close()
+    # Q8_0 at eight tokens: the draft model's ffn_up and ffn_down shapes, one pass on the matrix cores
+    gemv_case("q8_0 gemv 3584x1024 M=8", Q8_0, 3584, 1024, 8)
+    gemv_case("q8_0 gemv 1024x3584 M=8", Q8_0, 1024, 3584, 8)
     if args.mode == "cases":
         gemv_case("q4_k gemv 4096x12288 M=4", Q4_K, 4096, 12288, 4)
         gemv_case("q4_k gemv 4096x12288 M=8", Q4_K, 4096, 12288, 8)
