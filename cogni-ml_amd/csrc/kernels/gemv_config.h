@@ -216,7 +216,7 @@ static inline unsigned gemv_mt_multi_from(unsigned type, unsigned in_dim) {
   return 4u * (in_dim >> 8) < 3u * gemv_mt_padded_sb(in_dim) ? 5u : 2u;
 }
 // tiles per wavefront: rows of more than 4096 values one (the operands are streamed); else as many as keep 256 workgroups
-// busy, at most three (Q4_K) or two (Q6_K: its units are larger). Host and kernel use the same rule.
+// busy, at most three (Q4_K, Q5_K) or two (Q6_K, Q8_0: their units are larger). Host and kernel use the same rule.
 static inline GEMV_HD unsigned gemv_mt_tiles(unsigned type, unsigned in_dim, unsigned ntiles) {
   if (in_dim > 4096u) return 1;
   const unsigned tmax = (type == 14 || type == 8) ? 2u : (unsigned)GEMV_MT_TMAX;
