@@ -497,6 +497,18 @@ int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, ui
     *shared_mem_bytes = gemv_mfma_lds_bytes(type, (int)tokens, in_dim);
     return 0;
   }
+  // one token of a matrix of few rows: the variant with fewer rows per wavefront, so that 256 workgroups share the matrix
+  if (tokens == 1) {
+    const int r = gemv_rows_m1(type, out_dim);
+    if (r * GEMV_WAVES != gemv_rows_per_block(type, 1)) {
+      std::snprintf(buf, sizeof buf, "%s_gemv_%sf32_r%d", type_prefix(type), add ? "add_" : "", r);
+      *kernel = buf;
+      *grid_x = (out_dim + (uint32_t)(GEMV_WAVES * r) - 1) / (uint32_t)(GEMV_WAVES * r);
+      *block_x = GEMV_BLOCK;
+      *shared_mem_bytes = gemv_lds_bytes(type, 1, in_dim);
+      return 0;
+    }
+  }
   *kernel = cogni_gemv_kernel_name(type, tokens, add);
   return cogni_gemv_launch_dims(type, tokens, in_dim, out_dim, grid_x, block_x, shared_mem_bytes);
 }

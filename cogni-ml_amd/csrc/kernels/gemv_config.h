@@ -35,6 +35,15 @@ static inline int gemv_rows_per_block(unsigned type, int tokens) {
   }
 }
 
+// One token of a matrix of few rows: halve the rows per wavefront until at least 256 workgroups share the matrix
+// (kernels NAME_r1, Q8_0 also NAME_r2). Returns rows per wavefront; the value for many rows is the kernel's own.
+#define GEMV_SHORT_MIN_GROUPS 256u
+static inline int gemv_rows_m1(unsigned type, unsigned out_dim) {
+  int r = gemv_rows_per_block(type, 1) / GEMV_WAVES;
+  while (r > 1 && (out_dim + (unsigned)(GEMV_WAVES * r) - 1) / (unsigned)(GEMV_WAVES * r) < GEMV_SHORT_MIN_GROUPS) r >>= 1;
+  return r;
+}
+
 // ---- staged activations ------------------------------------------------------------------------
 // A workgroup keeps the activations of up to GEMV_LDS_BYTES in LDS: `chunk` whole column sets for the
 // token group it is working on. per_set_f4 = float4 count of one column set for that token group.

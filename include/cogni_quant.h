@@ -85,7 +85,10 @@ int cogni_gemv_launch_dims(uint32_t type, uint32_t tokens, uint32_t in_dim, uint
  * cogni_gemv_one_pass_from), with its geometry: for 2..4 tokens of a Q4_K matrix and
  * 3 or 4 tokens of a Q5_K or Q6_K matrix whose activations fit the staging buffer (tokens * in_dim / 256 <= 96, or 64 from
  * 3 tokens) or whose in_dim is a multiple of 2048 (staged a chunk at a time) that is the matrix-core variant
- * "q4_k_gemv_mfma_[add_]f32_tbatchM" / "q5_k_..." / "q6_k_gemv_mfma_[add_]f32_tbatchM" (same parameter list, block 512), otherwise the kernel
+ * "q4_k_gemv_mfma_[add_]f32_tbatchM" / "q5_k_..." / "q6_k_gemv_mfma_[add_]f32_tbatchM" (same parameter list, block 512); for one
+ * token of a matrix with so few rows that the plain kernel would run on fewer than 256 workgroups (Q4_K, Q5_K, Q6_K below
+ * 2048 rows, Q8_0 below 4096) the variant of the plain kernel with fewer rows per wavefront, "<type>_gemv_[add_]f32_r1" (Q8_0
+ * from 2048 rows: "_r2"; same parameter list and block, grid ceil(out_dim / (4 R))); otherwise the kernel
  * cogni_gemv_kernel_name / cogni_gemv_launch_dims describe. *kernel points at thread-local storage that the
  * next call on the thread overwrites. tokens in 1..COGNI_MAX_GEMV_TOKENS. No GPU needed. */
 int cogni_gemv_plan(uint32_t type, uint32_t tokens, int add, uint32_t in_dim, uint32_t out_dim, const char** kernel,

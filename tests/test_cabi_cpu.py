@@ -97,6 +97,27 @@ def test_gemv_launch_dims():
         quant.gemv_launch_dims(12, 9, 256, 16)
 
 
+def test_one_token_of_a_short_matrix_gets_fewer_rows_per_wavefront():
+    """Matrices whose rows would fill fewer than 256 workgroups of the plain one-token kernel: the plan names the variant with
+    one row per wavefront (Q8_0, whose kernel has four: two from 2048 rows), and its grid still covers every row."""
+    assert quant.gemv_plan(12, 1, 4096, 1024) == ("q4_k_gemv_f32_r1", 256, 256, quant.gemv_launch_dims(12, 1, 4096, 1024)[2])
+    assert quant.gemv_plan(12, 1, 4096, 1024, add=True)[0] == "q4_k_gemv_add_f32_r1"
+    assert quant.gemv_plan(13, 1, 4096, 2040)[:2] == ("q5_k_gemv_f32_r1", 510) and quant.gemv_plan(13, 1, 4096, 2041)[0] == "q5_k_gemv_f32"
+    assert quant.gemv_plan(14, 1, 4096, 37)[:2] == ("q6_k_gemv_f32_r1", 10)
+    assert quant.gemv_plan(8, 1, 1024, 3584)[:2] == ("q8_0_gemv_f32_r2", 448)          # config 1's shape
+    assert quant.gemv_plan(8, 1, 3584, 1024)[:2] == ("q8_0_gemv_f32_r1", 256)
+    assert quant.gemv_plan(8, 1, 1024, 2040)[:2] == ("q8_0_gemv_f32_r1", 510) and quant.gemv_plan(8, 1, 1024, 2041)[:2] == ("q8_0_gemv_f32_r2", 256)
+    assert quant.gemv_plan(8, 1, 1024, 4080)[0] == "q8_0_gemv_f32_r2" and quant.gemv_plan(8, 1, 1024, 4081)[0] == "q8_0_gemv_f32"
+    for t, rows_default in ((12, 2), (13, 2), (14, 2), (8, 4)):
+        for out_dim in (1, 3, 4, 5, 255, 1023, 1024, 1025, 2047, 2048, 4095, 4096, 12288):
+            name, grid, block, lds = quant.gemv_plan(t, 1, 1024, out_dim)
+            r = int(name.rsplit("_r", 1)[1]) if "_r" in name.rsplit("f32", 1)[1] else rows_default
+            assert block == 256 and grid * 4 * r >= out_dim > (grid - 1) * 4 * r or grid < -(-out_dim // (4 * r)), (t, out_dim, name, grid)
+            assert r == rows_default or -(-out_dim // (8 * r)) < 256      # halved only while the larger size gave fewer than 256 groups
+    # the names by token count and their launch geometry stay those of the plain kernels (hosts that launch by name)
+    assert quant.gemv_kernel_name(12, 1) == "q4_k_gemv_f32" and quant.gemv_launch_dims(12, 1, 4096, 1024)[0] == 128
+
+
 def test_gemv_plan_picks_the_kernel_for_the_shape():
     # one token: the vector-ALU kernel and its geometry
     assert quant.gemv_plan(12, 1, 4096, 12288) == ("q4_k_gemv_f32",) + quant.gemv_launch_dims(12, 1, 4096, 12288)

@@ -62,6 +62,30 @@ def test_small_shapes_all_token_counts(gpu, oracle, type_id, tokens, add):
     check(oracle, raw, type_id, x, in_dim, out_dim, tokens, res, "type %d M=%d add=%s" % (type_id, tokens, add))
 
 
+@pytest.mark.parametrize("type_id,in_dim,short_rows", [(Q4_K, 4096, 1024), (Q4_K, 1024, 37), (Q5_K, 4096, 2040), (Q6_K, 4096, 1024),
+                                                        (Q6_K, 12288, 130), (Q4_K, 12288, 64), (Q5_K, 8192, 300), (Q4_K, 26624, 33), (Q8_0, 1024, 3584), (Q8_0, 3584, 1024), (Q8_0, 1000, 2041),
+                                                        (Q8_0, 4096, 5)])
+@pytest.mark.parametrize("add", [False, True])
+def test_one_token_of_a_short_matrix(gpu, oracle, type_id, in_dim, short_rows, add):
+    """Matrices of few rows run the one-token kernel's variant with fewer rows per wavefront (one; Q8_0 two from 2041 rows):
+    within the bars against the oracle, and - a row's arithmetic does not depend on how many rows its wavefront carries -
+    bit for bit the values the plain kernel gives the same rows as the head of a matrix tall enough to be taken by it."""
+    name = quant.gemv_plan(type_id, 1, in_dim, short_rows, add=add)[0]
+    assert name.endswith("_r1") or name.endswith("_r2"), name
+    tall_rows = 4096 + 16
+    assert "_r" not in quant.gemv_plan(type_id, 1, in_dim, tall_rows)[0].rsplit("f32", 1)[1]
+    rng = np.random.default_rng(type_id * 7919 + in_dim + short_rows)
+    raw_tall = synth.make_weights(rng, type_id, tall_rows, in_dim)
+    row_bytes = raw_tall.size // tall_rows
+    raw_short = np.ascontiguousarray(raw_tall[:short_rows * row_bytes])
+    x = synth.make_activations(rng, 1, in_dim)
+    res_tall = rng.standard_normal(tall_rows).astype(np.float32) if add else None
+    res_short = res_tall[:short_rows].copy() if add else None
+    short = check(oracle, raw_short, type_id, x, in_dim, short_rows, 1, res_short, "%s %dx%d" % (name, short_rows, in_dim))[0]
+    tall = run_gemv(raw_tall, type_id, x, in_dim, tall_rows, 1, res_tall)
+    assert np.array_equal(short, tall[:short_rows])
+
+
 @pytest.mark.parametrize("in_dim", [32, 80, 1000, 1024, 2048 + 32])
 def test_q8_0_row_lengths_including_clipped_tail(gpu, oracle, in_dim):
     rng = np.random.default_rng(in_dim)
