@@ -396,7 +396,7 @@ def main():
         for i in range(n):
             head.launch(i % head.copies, stream)
         stream.synchronize()
-        for w_type, out_dim, in_dim, tokens in ((Q6_K, 4096, 12288, 1), (Q4_K, 12288, 4096, 8), (Q6_K, 4096, 12288, 8)):
+        for w_type, out_dim, in_dim, tokens in ((Q6_K, 4096, 12288, 1), (Q4_K, 12288, 4096, 8), (Q6_K, 4096, 12288, 8), (Q8_0, 4096, 4096, 8)):
             c = GemvCase(hip, quant, synth, rng, w_type, out_dim, in_dim, tokens, min_total_bytes=LLC_BYTES + (64 << 20))
             for i in range(n):
                 c.launch(i % c.copies, stream)
