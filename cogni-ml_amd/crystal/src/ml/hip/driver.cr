@@ -57,6 +57,9 @@ lib LibCogniHIP
   fun cogni_gemv_plan(type : UInt32, tokens : UInt32, add : Int32, in_dim : UInt32, out_dim : UInt32, kernel : UInt8**,
                       grid_x : UInt32*, block_x : UInt32*, shared_mem_bytes : UInt32*) : Int32
   fun cogni_gemv_one_pass_from(w_type : UInt32, in_dim : UInt32, out_dim : UInt32) : UInt32
+  fun cogni_gemv_one_pass_multi_from(w_type : UInt32, in_dim : UInt32) : UInt32
+  fun cogni_gemv_passes(w_type : UInt32, tokens : UInt32, in_dim : UInt32, out_dim : UInt32) : Int32
+  fun cogni_gemv_image_stats(slots : UInt32*, in_use : UInt32*, pinned : UInt32*, calls_without_image : UInt64*) : Int32
   fun cogni_gemv_release_stream(stream : Void*) : Int32
   fun cogni_gemv_image_bytes(w_type : UInt32, in_dim : UInt32, tokens : UInt32) : LibC::SizeT
   fun cogni_gemv_packed_launch_dims(w_type : UInt32, in_dim : UInt32, total_rows : UInt32,
@@ -102,6 +105,18 @@ lib LibCogniHIP
                           workspace : UInt64, workspace_bytes : LibC::SizeT, stream : Void*) : Int32
   fun cogni_gemm_packed_dev(w_raw : UInt64, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT, bias : UInt64,
                             out : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemm_packed_add_dev(w_raw : UInt64, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT, residual : UInt64,
+                                out : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemm_packed_swiglu_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT,
+                                   out : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemm_plan(w_type : UInt32, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, workspace_bytes : LibC::SizeT,
+                      kernel : UInt8**, grid_x : UInt32*, grid_y : UInt32*, block_x : UInt32*) : Int32
+  fun cogni_set_gemm_threshold(tokens : Int32) : Int32
+  fun cogni_get_gemm_threshold : Int32
+  fun cogni_block_bytes(type : UInt32) : Int32
+  fun cogni_block_elements(type : UInt32) : Int32
+  fun cogni_data_bytes(type : UInt32, n_elements : Int64) : Int64
+  fun cogni_quant_shutdown : Int32
   fun cogni_matmul_dev(w_raw : UInt64, w_type : UInt32, x : UInt64, bias : UInt64, out : UInt64,
                        in_dim : UInt32, out_dim : UInt32, tokens : UInt32,
                        workspace : UInt64, workspace_bytes : LibC::SizeT, stream : Void*) : Int32

@@ -29,6 +29,14 @@ def test_every_declared_symbol_is_exported(header):
         assert hasattr(L, n), "%s declared in %s but not exported" % (n, header)
 
 
+def test_the_crystal_binding_names_every_operator():
+    """The `lib` block a cogni-ml maintainer would use (crystal/src/ml/hip/driver.cr) declares every function of cogni_quant.h."""
+    src = open(os.path.join(ROOT, "cogni-ml_amd", "crystal", "src", "ml", "hip", "driver.cr")).read()
+    bound = set(re.findall(r"^\s*fun (\w+)", src, re.M))
+    missing = [n for n in declared_functions("cogni_quant.h") if n not in bound]
+    assert not missing, missing
+
+
 def test_geometry_matches_reference_table():
     L = hip.lib()
     for t in TensorType:
