@@ -951,21 +951,59 @@ size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tok
   return mtiles * 128 * (size_t)in_dim * 2;
 }
 
-// k splits of the prefill GEMM: a launch of fewer than half as many 128 x 192 tiles as there are compute units (256)
-// leaves most of them idle, so the super-blocks of a row are divided among up to 8 workgroups per tile, each with at
-// least two super-blocks; the partial sums go through the workspace.
-static uint32_t gemm_splits(uint32_t in_dim, uint32_t out_dim, uint32_t tokens) {
-  const uint32_t tiles = ((tokens + 127) / 128) * ((out_dim + 191) / 192), nkb = in_dim / 256;
+// k splits of the prefill GEMM: a launch of fewer than half as many tiles as there are compute units (256) leaves most
+// of them idle, so the super-blocks of a row are divided among up to 8 workgroups per tile, each with at least two
+// super-blocks; the partial sums go through the workspace.
+static uint32_t gemm_splits_of(uint32_t tiles, uint32_t in_dim) {
+  const uint32_t nkb = in_dim / 256;
   uint32_t s = 256u / tiles;
   if (s > 8) s = 8;
   if (s > nkb / 2) s = nkb / 2;
   return s < 2 ? 1 : s;
 }
+// Rows of the workgroup tile and k splits of a launch. Every type has two tile heights, 192 and 128 rows (<type>_gemm_f16 and
+// <type>_gemm_n128_f16), Q4_K also the 256-row tile of the eight-wavefront kernel (no k split). A launch runs in rounds of
+// 256 workgroups and a workgroup walks ceil(super-blocks / splits) super-blocks; per super-block a 128-row tile costs
+// GEMM_N128_COST_X100 per cent of a 192-row one and a 256-row tile GEMM_WIDE_ROUND_COST_X100 per cent; the cheapest plan wins
+// (the 4096-row projections at 512 tokens: 88 tiles x 2 splits = 176 workgroups of 192 rows, or 128 x 2 = 256 of the
+// smaller ones). `split` false: the plan for a workspace without planes. COGNI_GEMM_N128=0 | 1 and COGNI_GEMM_WIDE=0 | 1
+// override the choice (measurement knobs: 1 takes that tile wherever its kernel can run).
+#define GEMM_N128_COST_X100 75u
+struct GemmShape {
+  uint32_t bn, splits;
+};
+static GemmShape gemm_shape(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens, bool split = true) {
+  const uint32_t mtiles = (tokens + 127) / 128, nkb = in_dim / 256;
+  auto eval = [&](uint32_t bn, uint32_t cost_x100, uint32_t* cost) {
+    const uint32_t tiles = mtiles * ((out_dim + bn - 1) / bn), s = split && bn != 256 ? gemm_splits_of(tiles, in_dim) : 1u;
+    *cost = ((tiles * s + 255u) / 256u) * ((nkb + s - 1) / s) * cost_x100;
+    return s;
+  };
+  uint32_t cost192 = 0, cost128 = 0, cost256 = 0;
+  const uint32_t s192 = eval(192, 100u, &cost192), s128 = eval(128, GEMM_N128_COST_X100, &cost128);
+  bool n128 = cost128 < cost192;
+  if (const char* e = std::getenv("COGNI_GEMM_N128")) {
+    if (e[0] == '0') n128 = false;
+    if (e[0] == '1') n128 = true;
+  }
+  GemmShape best = n128 ? GemmShape{128, s128} : GemmShape{192, s192};
+  // the eight-wavefront kernel: Q4_K launches that are not split and fill whole rounds of its tiles
+  if (w_type == COGNI_TYPE_Q4_K && best.splits == 1) {
+    (void)eval(256, GEMM_WIDE_ROUND_COST_X100, &cost256);
+    bool wide = gemm_q4k_use_wide(out_dim, tokens) && cost256 < (n128 ? cost128 : cost192);
+    if (const char* e = std::getenv("COGNI_GEMM_WIDE")) {
+      if (e[0] == '0') wide = false;
+      if (e[0] == '1') wide = true;
+    }
+    if (wide) best = GemmShape{256, 1};
+  }
+  return best;
+}
 
 size_t cogni_gemm_workspace_bytes_split(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, uint32_t tokens) {
   const size_t pack = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
   if (pack == 0 || out_dim == 0 || (in_dim % 256) != 0) return pack;
-  const uint32_t s = gemm_splits(in_dim, out_dim, tokens);
+  const uint32_t s = gemm_shape(w_type, in_dim, out_dim, tokens).splits;
   return s == 1 ? pack : pack + (size_t)s * tokens * out_dim * sizeof(float);
 }
 
@@ -1013,16 +1051,14 @@ static GemmPlan gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, ui
   const uint32_t mtiles = (tokens + 127) / 128;
   GemmPlan p;
   // a workspace that holds the packed activations only: one workgroup per tile walks the whole row
-  p.splits = gemm_splits(in_dim, out_dim, tokens);
-  if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) p.splits = 1;
-  // COGNI_GEMM_WIDE=0 | 1 overrides the rule (a measurement knob: 1 takes the wide tiles for every unsplit Q4_K launch)
-  bool wide = w_type == COGNI_TYPE_Q4_K && p.splits == 1 && gemm_q4k_use_wide(out_dim, tokens);
-  if (const char* e = std::getenv("COGNI_GEMM_WIDE")) {
-    if (e[0] == '0') wide = false;
-    if (e[0] == '1') wide = w_type == COGNI_TYPE_Q4_K && p.splits == 1;
-  }
-  p.kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemm_f16" : w_type == COGNI_TYPE_Q5_K ? "q5_k_gemm_f16" : wide ? "q4_k_gemm_wide_f16" : "q4_k_gemm_f16";
-  const uint32_t ntiles = wide ? (out_dim + 255) / 256 : (out_dim + 191) / 192;
+  GemmShape shape = gemm_shape(w_type, in_dim, out_dim, tokens);
+  if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) shape = gemm_shape(w_type, in_dim, out_dim, tokens, false);
+  p.splits = shape.splits;
+  const bool wide = shape.bn == 256, n128 = shape.bn == 128;
+  p.kernel = w_type == COGNI_TYPE_Q6_K ? (n128 ? "q6_k_gemm_n128_f16" : "q6_k_gemm_f16")
+             : w_type == COGNI_TYPE_Q5_K ? (n128 ? "q5_k_gemm_n128_f16" : "q5_k_gemm_f16")
+             : wide ? "q4_k_gemm_wide_f16" : (n128 ? "q4_k_gemm_n128_f16" : "q4_k_gemm_f16");
+  const uint32_t ntiles = (out_dim + shape.bn - 1) / shape.bn;
   p.grid_x = gemm_grid_x(mtiles, ntiles);
   p.block = wide ? 512 : 256;
   return p;

@@ -146,43 +146,45 @@ __shared__ uint4 gemm_wbuf5[32 * 64];
 
 // Epilogue shared by the GEMM kernels. The MFMAs are issued as (weights, x), so an accumulator tile is laid out with the
 // weight rows along the register index: acc[r][c][v] of lane (j, kg) belongs to token 32 r + j and weight row
-// nh * 96 + 32 c + 8 (v / 4) + 4 kg + v % 4 - four consecutive output floats per register quad, which leave as one
+// nh * 32 NT + 32 c + 8 (v / 4) + 4 kg + v % 4 (NT = 3 tiles of 32 rows per wavefront, two with the 128-row workgroup tile) - four
+// consecutive output floats per register quad, which leave as one
 // 16-byte store without passing through LDS. What does pass through LDS is the other k half: a kh wavefront finishes the
 // token tiles r = 2 kh, 2 kh + 1 and hands the other two to its partner (same nh) as 24 float4 per lane in the lane
 // layout both share (kh = 0 writes into x buffer 0, kh = 1 into x buffer 1: 2 x 24 KiB each). Sum first, bias second.
-template <int KH>
-__device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
+template <int KH, int NT = 3>
+__device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][NT], const float* bias, float* out, u32 out_dim, u32 m,
                                                    u32 mt, u32 nt, u32 nh, u32 j, u32 kg, u32 lane, u32 bias_stride) {
-  float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * 24 * 64 + lane;
-  const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * 24 * 64 + lane;
+  constexpr u32 BN = 64 * NT;   // weight rows of the workgroup tile: NT tiles of 32 rows per wavefront, two row halves
+  float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * (8 * NT) * 64 + lane;
+  const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * (8 * NT) * 64 + lane;
 #pragma unroll
   for (int rr = 0; rr < 2; rr++)
 #pragma unroll
-    for (int c = 0; c < 3; c++)
+    for (int c = 0; c < NT; c++)
 #pragma unroll
       for (int g4 = 0; g4 < 4; g4++) {
         const float16_t& t = acc[2 * (1 - KH) + rr][c];
-        mine[((rr * 3 + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
+        mine[((rr * NT + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
       }
   __syncthreads();
   const bool vec = (out_dim & 3u) == 0;
-  if (vec && mt * GEMM_BM + GEMM_BM <= m && nt * GEMM_BN + GEMM_BN <= out_dim) {
+  if (vec && mt * GEMM_BM + GEMM_BM <= m && nt * BN + BN <= out_dim) {
     // a whole tile: one address per token row, the 12 stores of a row at constant offsets from it, 16 bytes each (kept
     // apart from the general path below so that the compiler cannot merge the two into single-float stores)
 #pragma unroll
     for (int rr = 0; rr < 2; rr++) {
       const size_t token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
-      const u32 col = nt * GEMM_BN + nh * 96 + 4 * kg;
+      const u32 col = nt * BN + nh * (32 * NT) + 4 * kg;
       float* base = out + token * out_dim + col;
       // what is added: a [out_dim] bias, or row `token` of a residual (which may be `out`: a thread reads the values it
       // is about to overwrite, nobody else's)
       const float* bbase = bias ? bias + token * bias_stride + col : nullptr;
 #pragma unroll
-      for (int c = 0; c < 3; c++)
+      for (int c = 0; c < NT; c++)
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++) {
           const float16_t& t = acc[2 * KH + rr][c];
-          const float4 p = theirs[((rr * 3 + c) * 4 + g4) * 64];
+          const float4 p = theirs[((rr * NT + c) * 4 + g4) * 64];
           float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
                         : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
           if (bbase) {
@@ -202,15 +204,15 @@ __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][3], const
     for (int rr = 0; rr < 2; rr++) {
       const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
 #pragma unroll
-      for (int c = 0; c < 3; c++)
+      for (int c = 0; c < NT; c++)
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++) {
           const float16_t& t = acc[2 * KH + rr][c];
-          const float4 p = theirs[((rr * 3 + c) * 4 + g4) * 64];
+          const float4 p = theirs[((rr * NT + c) * 4 + g4) * 64];
           // (k half 0) + (k half 1) whichever of the two this wavefront holds
           float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
                         : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
-          const u32 n = nt * GEMM_BN + nh * 96 + 32 * c + 8 * g4 + 4 * kg;
+          const u32 n = nt * BN + nh * (32 * NT) + 32 * c + 8 * g4 + 4 * kg;
           if (token >= m || n >= out_dim) continue;
           float* dst = out + (size_t)token * out_dim + n;
           const float* b = bias ? bias + (size_t)token * bias_stride + n : nullptr;   // bias, or a residual (stride out_dim)
@@ -229,10 +231,11 @@ __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][3], const
   if (vec) tail(std::true_type{});
   else tail(std::false_type{});
 }
-__device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][3], const float* bias, float* out, u32 out_dim, u32 m,
+template <int NT>
+__device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][NT], const float* bias, float* out, u32 out_dim, u32 m,
                                               u32 mt, u32 nt, u32 nh, u32 kh, u32 j, u32 kg, u32 tid, u32 bias_stride = 0) {
-  if (kh == 0) gemm_epilogue_half<0>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
-  else gemm_epilogue_half<1>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
+  if (kh == 0) gemm_epilogue_half<0, NT>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
+  else gemm_epilogue_half<1, NT>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
 }
 
 // Epilogue of the gate | up kernel: the nh = 0 wavefronts hold 96 gate rows, the nh = 1 wavefronts the same 96 rows of up,
@@ -323,13 +326,17 @@ struct GemmRawT<true> {   // Q5_K: plus the 32 bytes of fifth bits (bit 2g + hi 
 // x order, one more bit per value).
 // SWIGLU (Q4_K): rows 0..95 of the tile are rows [96 nt, 96 nt + 96) of `w` (gate), rows 96..191 the same rows of `w_b` (up);
 // the epilogue stores silu(gate) * up. No k split and no bias then.
-template <bool Q5, bool SWIGLU = false>
+// NT: tiles of 32 weight rows per wavefront - 3 (workgroup tile 128 tokens x 192 rows) or 2 (128 x 128, for launches whose
+// 192-row tiles, times the k split, leave compute units idle: q4_k_gemm_n128_f16, q5_k_gemm_n128_f16).
+template <bool Q5, bool SWIGLU = false, int NT = 3>
 __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim,
                                               u32 out_dim, u32 m, u32 bias_stride = 0, const uint8_t* w_b = nullptr) {
   static_assert(!(Q5 && SWIGLU), "the gate | up kernel is built for Q4_K");
+  static_assert(NT == 3 || (NT == 2 && !SWIGLU), "tile heights");
+  constexpr u32 BN = 64 * NT;             // weight rows of the workgroup tile
   constexpr u32 BS = Q5 ? 176 : 144;      // bytes of a super-block
   constexpr u32 PPR = Q5 ? 10 : 9;        // 16-byte pieces of a row that go through LDS
-  constexpr int NCOPY = Q5 ? 8 : 7;       // copies of 64 pieces a wavefront issues per super-block
+  constexpr int NCOPY = (int)((BN * PPR + 255) / 256);   // copies of 64 pieces a wavefront issues per super-block (192 rows: 7, Q5_K 8)
   uint4* const wbuf = Q5 ? gemm_wbuf5 : gemm_wbuf;
   // (no __restrict__ on w / xp: loads the compiler knows to be invariant are rematerialised next to
   // their use, which would undo the prefetch distance set up below)
@@ -343,7 +350,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   const u32 nkb_all = in_dim >> 8;
   const u32 kb0 = blockIdx.y * nkb_all / gridDim.y, nkb = (blockIdx.y + 1) * nkb_all / gridDim.y - kb0;
   out += (size_t)blockIdx.y * m * out_dim;
-  constexpr u32 TILE_ROWS = SWIGLU ? GEMM_BN / 2 : GEMM_BN;   // rows of a matrix a tile covers
+  constexpr u32 TILE_ROWS = SWIGLU ? BN / 2 : BN;   // rows of a matrix a tile covers
   const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + TILE_ROWS - 1) / TILE_ROWS;
   // Workgroup -> tile, XCD-aware (gemm_tile_of, gemv_config.h): the 32 workgroups that run side by side on an XCD take
   // a block of neighbouring tiles, so that its L2 fills with a weight tile once for several token tiles and with an x
@@ -374,32 +381,32 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   const uint8_t* wsrc[SWIGLU ? NCOPY : 1];   // gate | up: the two matrices are separate allocations, a piece has a full address
 #pragma unroll
   for (int i = 0; i < NCOPY; i++) {
-    const u32 p = min((4u * i + wave) * 64u + lane, (u32)GEMM_BN * PPR - 1u);
+    const u32 p = min((4u * i + wave) * 64u + lane, BN * PPR - 1u);
     const u32 r = p / PPR, part = p - PPR * r;
     if constexpr (SWIGLU) {
       const u32 row = min(nt * TILE_ROWS + (r < TILE_ROWS ? r : r - TILE_ROWS), out_dim - 1);
       wsrc[i] = (r < TILE_ROWS ? w : w_b) + (size_t)row * row_bytes + 16u * part;
       woff[i] = 0;
     } else {
-      woff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part + (Q5 ? 16u : 0u);
+      woff[i] = (min(nt * BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part + (Q5 ? 16u : 0u);
     }
   }
   // where this lane finds the raw bytes of its three rows in gemm_wbuf (in uint4 units): header, then the 32 bytes of
   // its group
-  u32 wrow[3];
+  u32 wrow[NT];
 #pragma unroll
-  for (int c = 0; c < 3; c++) wrow[c] = (nh * 96 + 32 * c + j) * PPR;
+  for (int c = 0; c < NT; c++) wrow[c] = (nh * (32 * NT) + 32 * c + j) * PPR;
   // Q5_K: where this lane's three rows start relative to wbase (their headers are read from there)
-  u32 hoff[3];
+  u32 hoff[NT];
 #pragma unroll
-  for (int c = 0; c < 3; c++) hoff[c] = (min(nt * GEMM_BN + nh * 96 + 32 * c + j, out_dim - 1) - tile_row0) * (u32)row_bytes;
+  for (int c = 0; c < NT; c++) hoff[c] = (min(nt * BN + nh * (32 * NT) + 32 * c + j, out_dim - 1) - tile_row0) * (u32)row_bytes;
   const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
-  float16_t acc[4][3];
+  float16_t acc[4][NT];
 #pragma unroll
   for (int r = 0; r < 4; r++)
 #pragma unroll
-    for (int c = 0; c < 3; c++)
+    for (int c = 0; c < NT; c++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
@@ -410,7 +417,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       __builtin_amdgcn_global_load_lds((gbl_void*)(wbase + (size_t)kb * BS + woff[i]),
                                        (lds_void*)(wbuf + (4 * i + wave) * 64), 16, 0, 0);
   };
-  uint4 nhdr[3];   // Q5_K: headers of the super-block being copied
+  uint4 nhdr[NT];   // Q5_K: headers of the super-block being copied
   auto load_hdr = [&](u32 kb, int c) {
     if constexpr (Q5) nhdr[c] = ld16(wbase + (size_t)kb * BS + hoff[c]);
   };
@@ -422,7 +429,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
 #pragma unroll
   for (int i = 0; i < NCOPY; i++) copy_w(0, i);
 #pragma unroll
-  for (int c = 0; c < 3; c++) load_hdr(0, c);
+  for (int c = 0; c < NT; c++) load_hdr(0, c);
   if (odd) {
 #pragma unroll
     for (int i = 0; i < 16; i++)
@@ -438,14 +445,14 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
 
   // State that lives across super-blocks: the raw bytes and the decoded (scale, -min) pairs of the current one, and
   // the two operand sets of the k-step pipeline.
-  GemmRawT<Q5> cur[3];
-  u32 S[3][4];
+  GemmRawT<Q5> cur[NT];
+  u32 S[NT][4];
   uint4 A[2][4];
-  half8_t B[2][3];
+  half8_t B[2][NT];
   // The raw bytes of a super-block, out of gemm_wbuf into the registers of the lanes that decode them.
   auto take_raw = [&]() {
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
+    for (int c = 0; c < NT; c++) {
       if constexpr (Q5) {
         cur[c].hdr = nhdr[c];
         cur[c].qh0 = wbuf[wrow[c]];
@@ -462,7 +469,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   // (scale, -min) of sub-blocks 2g (low nibbles) and 2g+1 (high nibbles) as duplicated half2
   auto decode_scales = [&]() {
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
+    for (int c = 0; c < NT; c++) {
       const float d = h2f(cur[c].hdr.x), dm = h2f(cur[c].hdr.x >> 16);
       const u32 a0 = cur[c].hdr.y >> sh, a1 = cur[c].hdr.z >> sh, a2 = cur[c].hdr.w >> sh;
       // kh = 0: a0 & 0x3F3F, a1 & 0x3F3F; kh = 1: (a2 & 0x0F0F) | ((a0 >> 2) & 0x3030), ((a2 >> 4) & 0x0F0F) | ((a1 >> 2) & 0x3030)
@@ -475,10 +482,10 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       S[c][3] = h2_dup(-(dm * ubyte_f<1>(mp)));
     }
   };
-  auto build_b = [&](half8_t (&Bd)[3], int t) {
+  auto build_b = [&](half8_t (&Bd)[NT], int t) {
     const int h = t >> 2, op = t & 3, hi = op >> 1;
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
+    for (int c = 0; c < NT; c++) {
       const uint4 Q = h ? cur[c].qb : cur[c].qa;
       const u32 qa = (op & 1) ? Q.z : Q.x, qb = (op & 1) ? Q.w : Q.y;
       const u32 mask = hi ? 0x00F000F0u : 0x000F000Fu;
@@ -536,13 +543,14 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       // Copies for the next super-block, a few per k-step rather than all up front: a wavefront issues in order and
       // a vector memory instruction costs it some 50 clocks, so 23 of them in a row stall the (only) wavefront of the
       // SIMD with nothing to overlap. All of them are out by k-step 5; they are waited for behind k-step 6.
+      // (copy 2 t and 2 t + 1 in k-steps 0..2, the seventh in k-step 3, the eighth in k-step 4, as far as the tile has them)
       if (t < 3) {
-        copy_w(kn, 2 * t);
-        copy_w(kn, 2 * t + 1);
-        load_hdr(kn, t);
+        if (2 * t < NCOPY) copy_w(kn, 2 * t);
+        if (2 * t + 1 < NCOPY) copy_w(kn, 2 * t + 1);
+        if (t < NT) load_hdr(kn, t);
       }
-      if (t == 3) copy_w(kn, 6);
-      if (Q5 && t == 4) copy_w(kn, 7);
+      if (t == 3 && NCOPY > 6) copy_w(kn, 6);
+      if (t == 4 && NCOPY > 7) copy_w(kn, 7);
       if (t < 6) {
 #pragma unroll
         for (int i = (t < 2 ? 2 * t : 3 * t - 2); i < (t < 2 ? 2 * t + 2 : 3 * t + 1); i++) copy_x(i);
@@ -563,7 +571,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       for (int r = 0; r < 4; r++) {
         const half8_t Ar = *reinterpret_cast<const half8_t*>(&A[p][r]);
 #pragma unroll
-        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[p][c], Ar, acc[r][c], 0, 0, 0);
+        for (int c = 0; c < NT; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[p][c], Ar, acc[r][c], 0, 0, 0);
       }
       // Scheduling window = one k-step. Left alone the scheduler emits the twelve MFMAs back to back and the
       // operand preparation of the next step behind them, so the matrix pipe and the vector ALU take turns;
@@ -573,21 +581,21 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       // keep the operands built above inside this window (otherwise they sink next to their first use,
       // behind the window's MFMAs)
 #pragma unroll
-      for (int c = 0; c < 3; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
+      for (int c = 0; c < NT; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
       if (t < 7) {
         __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);   // VMEM reads (LDS-direct copies) of this step
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
 #pragma unroll
-        for (int i = 0; i < 12; i++) {
+        for (int i = 0; i < 4 * NT; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
           __builtin_amdgcn_sched_group_barrier(0x002, Q5 ? 8 : 5, 0);   // five VALU (eight with the fifth bits)
         }
       } else {
         __builtin_amdgcn_sched_group_barrier(0x100, Q5 ? 16 : 13, 0);  // LDS reads: raw bytes and first A operands of the next super-block
 #pragma unroll
-        for (int i = 0; i < 3; i++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // three MFMAs while they arrive
+        for (int i = 0; i < NT; i++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // a few MFMAs while they arrive
 #pragma unroll
-        for (int i = 0; i < 9; i++) {
+        for (int i = 0; i < 3 * NT; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
         }
@@ -617,13 +625,22 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
     if (kh == 0) gemm_epilogue_swiglu_half<0>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
     else gemm_epilogue_swiglu_half<1>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
   } else {
-    gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
+    gemm_epilogue<NT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
   }
 }
 
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_f16(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
   gemm_k45_core<false>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+}
+// the same with a workgroup tile of 128 tokens x 128 rows; grid from gemm_grid_x(ceil(m/128), ceil(out_dim/128))
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_n128_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_k45_core<false, false, 2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+}
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q5_k_gemm_n128_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_k45_core<true, false, 2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }
 // Q5_K: x is packed by pack_x_f16_q4k (the values of a super-block sit where the Q4_K ones do).
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q5_k_gemm_f16(

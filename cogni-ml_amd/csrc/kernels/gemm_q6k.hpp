@@ -54,8 +54,13 @@ __shared__ uint4 gemm_wbuf6[GEMM_BN * 9];
 // the 16 scale bytes and d of the same rows, [row][6 dwords]: staged one row per thread by the first three wavefronts
 __shared__ u32 gemm_wsc6[GEMM_BN * 6];
 
-extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_f16(
-    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+// NT: tiles of 32 weight rows per wavefront - 3 (a workgroup tile of 128 tokens x 192 rows) or 2 (128 x 128: a third less
+// work per workgroup for shapes whose 192-row tiles, times the k split, leave compute units idle - 4096 rows at 512 tokens
+// are 88 tiles x 2 splits = 176 workgroups, but 128 x 2 = 256 of the smaller ones).
+template <int NT>
+__device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim,
+                                              u32 m, u32 bias_stride) {
+  constexpr u32 BN = 64 * NT, NSTG = 2 * NT;   // rows of the workgroup tile; 16-byte pieces of ql a thread stages per super-block
   const u32 tid = threadIdx.x, lane = tid & 63;
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const u32 nh = wave & 1, kh = wave >> 1;
@@ -64,65 +69,65 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   const u32 nkb_all = in_dim >> 8;
   const u32 kb0 = blockIdx.y * nkb_all / gridDim.y, nkb = (blockIdx.y + 1) * nkb_all / gridDim.y - kb0;
   out += (size_t)blockIdx.y * m * out_dim;
-  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + GEMM_BN - 1) / GEMM_BN;
+  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + BN - 1) / BN;
   // workgroup -> tile as in q4_k_gemm_f16: XCD x takes a contiguous run of token-tile-major tiles
   u32 mt, nt;
   if (!gemm_tile_of(blockIdx.x, mtiles, ntiles, &mt, &nt)) return;
-  const u32 n0 = nt * GEMM_BN + nh * 96;             // first weight row of this wavefront
+  const u32 n0 = nt * BN + nh * (32 * NT);           // first weight row of this wavefront
   const size_t row_bytes = (size_t)nkb_all * 210;
 
   // uniform base of the wavefront's rows + a 32-bit per-lane offset (96 rows are far below 4 GiB) to the lane's
   // piece of qh at 128 + 32 kh + 16 kg
   const u32 base_row = min(n0, out_dim - 1);
   const uint8_t* wbase = w + (size_t)base_row * row_bytes + (size_t)kb0 * 210;
-  u32 rowoff[3];
+  u32 rowoff[NT];
 #pragma unroll
-  for (int c = 0; c < 3; c++) rowoff[c] = (min(n0 + 32 * c + j, out_dim - 1) - base_row) * (u32)row_bytes;
+  for (int c = 0; c < NT; c++) rowoff[c] = (min(n0 + 32 * c + j, out_dim - 1) - base_row) * (u32)row_bytes;
   const u32 o_qh = 128 + 32 * kh + 16 * kg;
   const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
-  float16_t acc[4][3];
+  float16_t acc[4][NT];
 #pragma unroll
   for (int r = 0; r < 4; r++)
 #pragma unroll
-    for (int c = 0; c < 3; c++)
+    for (int c = 0; c < NT; c++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
-  // staging of ql: piece p = 64 (4 i + wave) + lane, i < 6, is bytes [16 (p % 8), +16) of row p / 8 of the tile
-  const u32 tile_row0 = min(nt * GEMM_BN, out_dim - 1);
+  // staging of ql: piece p = 64 (4 i + wave) + lane, i < NSTG, is bytes [16 (p % 8), +16) of row p / 8 of the tile
+  const u32 tile_row0 = min(nt * BN, out_dim - 1);
   const uint8_t* tbase = w + (size_t)tile_row0 * row_bytes + (size_t)kb0 * 210;   // uniform
-  u32 soff[6], sdst[6];
+  u32 soff[NSTG], sdst[NSTG];
 #pragma unroll
-  for (int i = 0; i < 6; i++) {
+  for (int i = 0; i < (int)NSTG; i++) {
     const u32 p = (4u * i + wave) * 64u + lane, r = p >> 3, part = p & 7u;
-    soff[i] = (min(nt * GEMM_BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part;
+    soff[i] = (min(nt * BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part;
     sdst[i] = r * 9u + part;
   }
-  const u32 take0 = (nh * 96 + j) * 9 + 4 * kh + kg;   // the lane's first ql piece of its row c = 0; the second is 2 further
-  const u32 srow = (min(nt * GEMM_BN + min(tid, (u32)GEMM_BN - 1), out_dim - 1) - tile_row0) * (u32)row_bytes + 192u;
-  const u32 tsc = (nh * 96 + j) * 6;                   // the lane's row c = 0 in gemm_wsc6
-  uint4 stg[6], stg_sc;
+  const u32 take0 = (nh * (32 * NT) + j) * 9 + 4 * kh + kg;   // the lane's first ql piece of its row c = 0; the second is 2 further
+  const u32 srow = (min(nt * BN + min(tid, BN - 1), out_dim - 1) - tile_row0) * (u32)row_bytes + 192u;
+  const u32 tsc = (nh * (32 * NT) + j) * 6;                   // the lane's row c = 0 in gemm_wsc6
+  uint4 stg[NSTG], stg_sc;
   u32 stg_d;
   auto stage_load = [&](const uint8_t* kbase, int i) { stg[i] = ld16(kbase + soff[i]); };
   auto stage_load_sc = [&](const uint8_t* kbase) {
-    if (wave < 3) {
+    if (wave < (u32)NT) {   // one row per thread: the first BN threads
       stg_sc = ld16(kbase + srow);
       stg_d = ld2(kbase + (srow + 16));
     }
   };
   auto stage_store = [&]() {
 #pragma unroll
-    for (int i = 0; i < 6; i++) gemm_wbuf6[sdst[i]] = stg[i];
-    if (wave < 3) {
+    for (int i = 0; i < (int)NSTG; i++) gemm_wbuf6[sdst[i]] = stg[i];
+    if (wave < (u32)NT) {
       *reinterpret_cast<uint2*>(&gemm_wsc6[tid * 6]) = make_uint2(stg_sc.x, stg_sc.y);
       *reinterpret_cast<uint2*>(&gemm_wsc6[tid * 6 + 2]) = make_uint2(stg_sc.z, stg_sc.w);
       gemm_wsc6[tid * 6 + 4] = stg_d;
     }
   };
-  auto take_ql = [&](GemmRaw6 (&raw)[3]) {
+  auto take_ql = [&](GemmRaw6 (&raw)[NT]) {
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
+    for (int c = 0; c < NT; c++) {
       raw[c].qa = gemm_wbuf6[take0 + 288 * c];
       raw[c].qb = gemm_wbuf6[take0 + 288 * c + 2];
       raw[c].sc = *reinterpret_cast<const uint2*>(&gemm_wsc6[tsc + 192 * c + 2 * kh]);
@@ -138,20 +143,20 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   // buffer 0 then 1, weight registers A then B); with an odd number of super-blocks the first one is taken alone
   // out of buffer 1 / registers B.
   const bool odd = nkb & 1;
-  GemmRaw6 rawA[3], rawB[3];
+  GemmRaw6 rawA[NT], rawB[NT];
 #pragma unroll
-  for (int i = 0; i < 6; i++) stage_load(tbase, i);
+  for (int i = 0; i < (int)NSTG; i++) stage_load(tbase, i);
   stage_load_sc(tbase);
   if (odd) {
 #pragma unroll
-    for (int c = 0; c < 3; c++) load_row(rawB[c], wbase, c);
+    for (int c = 0; c < NT; c++) load_row(rawB[c], wbase, c);
 #pragma unroll
     for (int i = 0; i < 16; i++)
       __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf1 + 256 * i + wave * 64),
                                        16, 0, 0);
   } else {
 #pragma unroll
-    for (int c = 0; c < 3; c++) load_row(rawA[c], wbase, c);
+    for (int c = 0; c < NT; c++) load_row(rawA[c], wbase, c);
 #pragma unroll
     for (int i = 0; i < 16; i++)
       __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
@@ -164,12 +169,12 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
   __builtin_amdgcn_s_barrier();   // gemm_wbuf6 is free for the next super-block
   asm volatile("" ::: "memory");
 
-  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt, const GemmRaw6 (&cur)[3], GemmRaw6 (&nxt)[3]) {
+  auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt, const GemmRaw6 (&cur)[NT], GemmRaw6 (&nxt)[NT]) {
     // d * sc of the four 16-value sub-blocks of the lane's group (scale bytes kg, kg + 2, kg + 4, kg + 6 of the
     // half's eight), as duplicated half2
-    u32 S[3][4];
+    u32 S[NT][4];
 #pragma unroll
-    for (int c = 0; c < 3; c++) {
+    for (int c = 0; c < NT; c++) {
       const float d = h2f(cur[c].d);
       const u32 lo = cur[c].sc.x >> (8 * kg), hi = cur[c].sc.y >> (8 * kg);
       S[c][0] = h2_dup(d * (float)(int)(signed char)(lo & 0xFFu));
@@ -183,10 +188,10 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     const uint8_t* tnext = tbase + (size_t)kn * 210;  // uniform
 
     const uint4* arow = xcur + (16 * kh + kg) * 128 + j;   // k-steps 8*kh .. 8*kh+7; 32 lanes read 512 contiguous bytes
-    auto build_b = [&](half8_t (&B)[3], int t) {
+    auto build_b = [&](half8_t (&B)[NT], int t) {
       const int qd = t >> 1, h8 = t & 1, hi = qd >> 1;
 #pragma unroll
-      for (int c = 0; c < 3; c++) {
+      for (int c = 0; c < NT; c++) {
         const uint4 Q = (qd & 1) ? cur[c].qb : cur[c].qa;
         const u32 qa = h8 ? Q.z : Q.x, qb = h8 ? Q.w : Q.y;
         const u32 ha = (h8 ? cur[c].qh.z : cur[c].qh.x) >> (2 * qd), hb = (h8 ? cur[c].qh.w : cur[c].qh.y) >> (2 * qd);
@@ -205,7 +210,7 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     // software pipeline over the wavefront's eight k-steps: while the MFMAs of step t run, the A operands
     // of step t+1 are read from LDS and its B operands are built
     uint4 A[2][4];
-    half8_t B[2][3];
+    half8_t B[2][NT];
 #pragma unroll
     for (int r = 0; r < 4; r++) A[0][r] = arow[r * 32];
     build_b(B[0], 0);
@@ -213,8 +218,8 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     for (int t = 0; t < 8; t++) {
       const int p = t & 1;
       // prefetches for the next super-block, a few per k-step: the raw weights of one row tile (5 loads) in each of
-      // the first three steps, the x tile global -> LDS spread over the first six
-      if (t < 3) {
+      // the first NT steps, the x tile global -> LDS spread over the first six
+      if (t < NT) {
         stage_load(tnext, 2 * t);
         stage_load(tnext, 2 * t + 1);
         load_row(nxt[t], knbase, t);
@@ -237,16 +242,16 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
       for (int r = 0; r < 4; r++) {
         const half8_t Ar = *reinterpret_cast<const half8_t*>(&A[p][r]);
 #pragma unroll
-        for (int c = 0; c < 3; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[p][c], Ar, acc[r][c], 0, 0, 0);
+        for (int c = 0; c < NT; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[p][c], Ar, acc[r][c], 0, 0, 0);
       }
       if (t < 7) {
 #pragma unroll
-        for (int c = 0; c < 3; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
+        for (int c = 0; c < NT; c++) asm volatile("" : "+v"(B[p ^ 1][c]));
       }
       __builtin_amdgcn_sched_group_barrier(0x020, 10, 0);  // VMEM reads (weights, LDS-direct x) of this step
       __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
 #pragma unroll
-      for (int i = 0; i < 12; i++) {
+      for (int i = 0; i < 4 * NT; i++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
         __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);   // eight VALU (a Q6_K operand takes more than a Q4_K one)
       }
@@ -270,5 +275,15 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     iteration(kb + 1, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
   }
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
-  gemm_epilogue(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
+  gemm_epilogue<NT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
+}
+
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_q6k_core<3>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+}
+// the same with a workgroup tile of 128 tokens x 128 rows; grid from gemm_grid_x(ceil(m/128), ceil(out_dim/128))
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_n128_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_q6k_core<2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }

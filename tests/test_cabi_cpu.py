@@ -166,7 +166,8 @@ def test_gemv_plan_picks_the_kernel_for_the_shape():
 
 def test_gemm_plan_picks_tile_and_split_for_the_shape():
     blob = code_object()
-    for k in ("q4_k_gemm_f16", "q4_k_gemm_wide_f16", "q5_k_gemm_f16", "q6_k_gemm_f16", "gemm_sum_splits_f32", "pack_x_f16_q4k", "pack_x_f16_q6k"):
+    for k in ("q4_k_gemm_f16", "q4_k_gemm_wide_f16", "q5_k_gemm_f16", "q6_k_gemm_f16", "q4_k_gemm_n128_f16", "q5_k_gemm_n128_f16",
+              "q6_k_gemm_n128_f16", "gemm_sum_splits_f32", "pack_x_f16_q4k", "pack_x_f16_q6k"):
         assert (k.encode() + b"\x00") in blob, k
     big = 1 << 40
     # 512 x 12288: 256 tiles of 128 x 192, one per compute unit; 192 wide tiles would leave a quarter of them idle
@@ -177,13 +178,24 @@ def test_gemm_plan_picks_tile_and_split_for_the_shape():
     assert quant.gemm_plan(12, 4096, 12288, 4096, big) == ("q4_k_gemm_wide_f16", 1536, 1, 512)  # 6 rounds instead of 8
     # the grid is whole blocks of 32 tiles (8 weight tiles x 4 token tiles), 8 blocks at a time: a clipped shape rounds up
     assert quant.gemm_plan(12, 4096, 12288 + 192, 512, big)[1] == 8 * 32 * 2 and quant.gemm_plan(12, 256, 400, 130, big)[1:3] == (16, 1)
-    # 88 tiles of the 12288 -> 4096 down projection at M = 512: blocks of 3 x 4 tiles, one per XCD, k split in two
-    assert quant.gemm_plan(14, 12288, 4096, 512, big) == ("q6_k_gemm_f16", 96, 2, 256)
+    # the 12288 -> 4096 down projection at M = 512: 88 tiles of 192 rows with the k range split in two are 176 workgroups,
+    # 128 tiles of 128 rows are 256 (blocks of 4 x 4 tiles, one per XCD) - every type has the smaller tile for such shapes
+    for t, pfx in ((12, "q4_k"), (13, "q5_k"), (14, "q6_k")):
+        assert quant.gemm_plan(t, 12288, 4096, 512, big) == (pfx + "_gemm_n128_f16", 128, 2, 256)
+        assert quant.gemm_plan(t, 4096, 4096, 512, big) == (pfx + "_gemm_n128_f16", 128, 2, 256)
+        assert quant.gemm_plan(t, 12288, 4096, 64, big) == (pfx + "_gemm_n128_f16", 32, 8, 256)
+        assert quant.gemm_plan(t, 4096, 12288, 512, big)[0] == pfx + "_gemm_f16"            # 256 tiles of 192 rows fill the chip exactly
+        assert quant.gemm_plan(t, 4096, 12288, 1024, big)[0] == pfx + "_gemm_f16"           # two rounds of 192 rows against three of 128
+        # the planes of a split launch are sized by the same plan
+        assert quant.gemm_workspace_bytes(t, 12288, 512, 4096) == quant.gemm_workspace_bytes(t, 12288, 512) + 2 * 512 * 4096 * 4
+    assert quant.gemm_plan(13, 12288, 4096, 2048, big) == ("q5_k_gemm_n128_f16", 512, 1, 256)   # two rounds either way, of less work each
+    assert quant.gemm_plan(12, 12288, 4096, 2048, big)[0] == "q4_k_gemm_wide_f16"              # one round of the 256-row tiles
     # few tiles: the k range is split when the workspace has room for the planes, else not
     name, gx, gy, block = quant.gemm_plan(12, 4096, 12288, 64, big)
     assert (name, gx, block) == ("q4_k_gemm_f16", 64, 256) and gy == 4
-    assert quant.gemm_plan(12, 4096, 12288, 64, quant.gemm_workspace_bytes(12, 4096, 64)) == ("q4_k_gemm_f16", 64, 1, 256)
-    # the other types have one tiling
+    # (unsplit, 96 tiles of 128 rows spread over more compute units than 64 of 192)
+    assert quant.gemm_plan(12, 4096, 12288, 64, quant.gemm_workspace_bytes(12, 4096, 64)) == ("q4_k_gemm_n128_f16", 96, 1, 256)
+    # the eight-wavefront kernel is Q4_K's alone
     assert quant.gemm_plan(13, 4096, 12288, 2048, big)[0] == "q5_k_gemm_f16" and quant.gemm_plan(14, 4096, 12288, 2048, big)[0] == "q6_k_gemm_f16"
     with pytest.raises(quant.QuantError, match="Unsupported quant type"):
         quant.gemm_plan(8, 4096, 12288, 512, big)

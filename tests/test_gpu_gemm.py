@@ -121,7 +121,7 @@ def test_k_split_matches_unsplit(gpu, oracle, tokens, out_dim, in_dim, t):
 def test_wide_tiles(gpu, oracle, tokens, out_dim, in_dim, with_bias):
     """Launches of whole rounds of 128 x 256 tiles go to the eight-wavefront kernel: a clipped last tile with an out_dim that
     is no multiple of 4, an odd number of super-blocks, a partial token tile and a bias, against the oracle on a sample of
-    tokens; and every output against the four-wavefront kernel's, which adds in the same order (bit for bit)."""
+    tokens; and every output against a four-wavefront kernel's, which adds in the same order (bit for bit)."""
     rng = np.random.default_rng(out_dim + tokens)
     raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
@@ -134,10 +134,33 @@ def test_wide_tiles(gpu, oracle, tokens, out_dim, in_dim, with_bias):
     # the same rows through the narrow kernel: 8192 rows at a time are fewer than a round of wide tiles
     for r0 in (0, 8192 * 3, out_dim - 8192):
         rows = slice(r0, r0 + 8192)
-        assert quant.gemm_plan(Q4_K, in_dim, 8192, tokens, 0)[0] == "q4_k_gemm_f16"
+        assert quant.gemm_plan(Q4_K, in_dim, 8192, tokens, 0)[0] in ("q4_k_gemm_f16", "q4_k_gemm_n128_f16")
         part = run_gemm(raw[r0 * (in_dim // 256) * 144:(r0 + 8192) * (in_dim // 256) * 144], x, in_dim, 8192, tokens,
                         None if bias is None else bias[rows], split=False).reshape(tokens, 8192)
         assert np.array_equal(part, got[:, rows]), r0
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("tokens,out_dim,in_dim", [(512, 4096, 2048), (130, 4096 + 37, 768), (64, 250, 4096), (300, 1024, 256)])
+def test_tile_heights_agree(gpu, oracle, t, tokens, out_dim, in_dim, monkeypatch):
+    """Every type has a 128-row and a 192-row workgroup tile and the library picks by launch shape; forced either way
+    (COGNI_GEMM_N128, read per call) the results are the same bits - clipped tiles, k splits, a bias - and within the bar."""
+    rng = np.random.default_rng(t * 31 + tokens + out_dim)
+    raw = synth.make_weights(rng, t, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    bias = rng.standard_normal(out_dim).astype(np.float32)
+    outs, splits = {}, {}
+    for mode in ("0", "1"):
+        monkeypatch.setenv("COGNI_GEMM_N128", mode)
+        wsb = quant.gemm_workspace_bytes(t, in_dim, tokens, out_dim)
+        name, _, splits[mode], _ = quant.gemm_plan(t, in_dim, out_dim, tokens, wsb)
+        assert name.endswith("_n128_f16") == (mode == "1") or name == "q4_k_gemm_wide_f16", name
+        outs[mode] = run_gemm(raw, x, in_dim, out_dim, tokens, bias, t=t)
+    monkeypatch.delenv("COGNI_GEMM_N128")
+    assert splits["0"] == splits["1"]       # (the k split, which these shapes share, is what fixes the order of the sums)
+    assert np.array_equal(outs["0"], outs["1"])
+    check(oracle, raw, x, in_dim, out_dim, tokens, bias, "type %d M=%d N=%d K=%d" % (t, tokens, out_dim, in_dim), t=t,
+          sample_tokens=[i for i in (0, 1, 63, 64, 127, 128, tokens - 1) if i < tokens])
 
 
 @pytest.mark.parametrize("t,tokens,out_dim,in_dim", [(Q4_K, 130, 400, 768), (Q6_K, 64, 384, 4096), (Q5_K, 40, 100, 512),
