@@ -340,9 +340,11 @@ int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uin
  * Kernels: pack_x_f16_q4k (Q4_K and Q5_K) | pack_x_f16_q6k (x, workspace, tokens, in_dim) then
  *          q4_k_gemm_f16 | q5_k_gemm_f16 | q6_k_gemm_f16 (w_raw, workspace, bias, out, in_dim, out_dim, tokens,
  *          bias_stride: 0 for a [out_dim] bias, out_dim for a [tokens][out_dim] residual), block 256,
- *          grid from cogni_gemm_plan (whole blocks of 32 tiles of 128 x 192, 8 XCDs at a time), no dynamic shared memory; or, for Q4_K launches that fill
- *          whole rounds of 128 x 256 tiles (cogni_gemm_plan says which), q4_k_gemm_wide_f16 (same arguments), block 512,
- *          grid from cogni_gemm_plan.
+ *          grid from cogni_gemm_plan (whole blocks of 32 tiles of 128 x 192, 8 XCDs at a time), no dynamic shared memory; or, where
+ *          tiles of 128 x 192 times the k split would leave compute units idle (the 4096-row projections at 512 tokens),
+ *          q4_k_gemm_n128_f16 | q5_k_gemm_n128_f16 | q6_k_gemm_n128_f16 (same arguments and block, tiles of 128 x 128); or,
+ *          for Q4_K launches that fill whole rounds of 128 x 256 tiles, q4_k_gemm_wide_f16 (same arguments), block 512.
+ *          cogni_gemm_plan says which, with the grid; all of them give the same bits for the same k split.
  * (pack_x_f16_*: block 256, grid ceil(tokens/128)*16*(in_dim/256).) Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);
 /* The workspace size with which cogni_gemm_dev may also split the k range: a launch with fewer than 128 tiles of
