@@ -1055,9 +1055,16 @@ static GemmPlan gemm_plan(uint32_t w_type, uint32_t in_dim, uint32_t out_dim, ui
   if (workspace_bytes < cogni_gemm_workspace_bytes_split(w_type, in_dim, out_dim, tokens)) shape = gemm_shape(w_type, in_dim, out_dim, tokens, false);
   p.splits = shape.splits;
   const bool wide = shape.bn == 256, n128 = shape.bn == 128;
-  p.kernel = w_type == COGNI_TYPE_Q6_K ? (n128 ? "q6_k_gemm_n128_f16" : "q6_k_gemm_f16")
-             : w_type == COGNI_TYPE_Q5_K ? (n128 ? "q5_k_gemm_n128_f16" : "q5_k_gemm_f16")
-             : wide ? "q4_k_gemm_wide_f16" : (n128 ? "q4_k_gemm_n128_f16" : "q4_k_gemm_f16");
+  // up to 64 tokens: the kernels that work on the first 64 tokens of the (one) token tile (COGNI_GEMM_M64=0 keeps the
+  // 128-token tiles, a measurement knob)
+  bool m64 = tokens <= 64 && !wide;
+  if (const char* e = std::getenv("COGNI_GEMM_M64"))
+    if (e[0] == '0') m64 = false;
+  static const char* const names[3][2][2] = {
+      {{"q4_k_gemm_f16", "q4_k_gemm_n128_f16"}, {"q4_k_gemm_m64_f16", "q4_k_gemm_m64_n128_f16"}},
+      {{"q5_k_gemm_f16", "q5_k_gemm_n128_f16"}, {"q5_k_gemm_m64_f16", "q5_k_gemm_m64_n128_f16"}},
+      {{"q6_k_gemm_f16", "q6_k_gemm_n128_f16"}, {"q6_k_gemm_m64_f16", "q6_k_gemm_m64_n128_f16"}}};
+  p.kernel = wide ? "q4_k_gemm_wide_f16" : names[w_type == COGNI_TYPE_Q6_K ? 2 : (w_type == COGNI_TYPE_Q5_K ? 1 : 0)][m64][n128];
   const uint32_t ntiles = (out_dim + shape.bn - 1) / shape.bn;
   p.grid_x = gemm_grid_x(mtiles, ntiles);
   p.block = wide ? 512 : 256;

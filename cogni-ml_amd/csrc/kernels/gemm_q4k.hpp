@@ -149,31 +149,32 @@ __shared__ uint4 gemm_wbuf5[32 * 64];
 // nh * 32 NT + 32 c + 8 (v / 4) + 4 kg + v % 4 (NT = 3 tiles of 32 rows per wavefront, two with the 128-row workgroup tile) - four
 // consecutive output floats per register quad, which leave as one
 // 16-byte store without passing through LDS. What does pass through LDS is the other k half: a kh wavefront finishes the
-// token tiles r = 2 kh, 2 kh + 1 and hands the other two to its partner (same nh) as 24 float4 per lane in the lane
+// token tiles r = 2 kh, 2 kh + 1 (r = kh with the 64-token tile, MT = 2) and hands the others to its partner (same nh) as 24 float4 per lane in the lane
 // layout both share (kh = 0 writes into x buffer 0, kh = 1 into x buffer 1: 2 x 24 KiB each). Sum first, bias second.
-template <int KH, int NT = 3>
-__device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][NT], const float* bias, float* out, u32 out_dim, u32 m,
+template <int KH, int NT = 3, int MT = 4>
+__device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[MT][NT], const float* bias, float* out, u32 out_dim, u32 m,
                                                    u32 mt, u32 nt, u32 nh, u32 j, u32 kg, u32 lane, u32 bias_stride) {
   constexpr u32 BN = 64 * NT;   // weight rows of the workgroup tile: NT tiles of 32 rows per wavefront, two row halves
+  constexpr int RH = MT / 2;    // token tiles of 32 a wavefront finishes (MT = 4: tokens 0..127 of the tile; 2: 0..63)
   float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * (8 * NT) * 64 + lane;
   const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * (8 * NT) * 64 + lane;
 #pragma unroll
-  for (int rr = 0; rr < 2; rr++)
+  for (int rr = 0; rr < RH; rr++)
 #pragma unroll
     for (int c = 0; c < NT; c++)
 #pragma unroll
       for (int g4 = 0; g4 < 4; g4++) {
-        const float16_t& t = acc[2 * (1 - KH) + rr][c];
+        const float16_t& t = acc[RH * (1 - KH) + rr][c];
         mine[((rr * NT + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
       }
   __syncthreads();
   const bool vec = (out_dim & 3u) == 0;
-  if (vec && mt * GEMM_BM + GEMM_BM <= m && nt * BN + BN <= out_dim) {
+  if (vec && mt * GEMM_BM + 32 * MT <= m && nt * BN + BN <= out_dim) {
     // a whole tile: one address per token row, the 12 stores of a row at constant offsets from it, 16 bytes each (kept
     // apart from the general path below so that the compiler cannot merge the two into single-float stores)
 #pragma unroll
-    for (int rr = 0; rr < 2; rr++) {
-      const size_t token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
+    for (int rr = 0; rr < RH; rr++) {
+      const size_t token = mt * GEMM_BM + 32 * (RH * KH + rr) + j;
       const u32 col = nt * BN + nh * (32 * NT) + 4 * kg;
       float* base = out + token * out_dim + col;
       // what is added: a [out_dim] bias, or row `token` of a residual (which may be `out`: a thread reads the values it
@@ -183,7 +184,7 @@ __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][NT], cons
       for (int c = 0; c < NT; c++)
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++) {
-          const float16_t& t = acc[2 * KH + rr][c];
+          const float16_t& t = acc[RH * KH + rr][c];
           const float4 p = theirs[((rr * NT + c) * 4 + g4) * 64];
           float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
                         : make_float4(t[4 * g4] + p.x, t[4 * g4 + 1] + p.y, t[4 * g4 + 2] + p.z, t[4 * g4 + 3] + p.w);
@@ -201,13 +202,13 @@ __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][NT], cons
   // two kinds of store into single floats for every tile.)
   auto tail = [&](auto vec16) {
 #pragma unroll
-    for (int rr = 0; rr < 2; rr++) {
-      const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
+    for (int rr = 0; rr < RH; rr++) {
+      const u32 token = mt * GEMM_BM + 32 * (RH * KH + rr) + j;
 #pragma unroll
       for (int c = 0; c < NT; c++)
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++) {
-          const float16_t& t = acc[2 * KH + rr][c];
+          const float16_t& t = acc[RH * KH + rr][c];
           const float4 p = theirs[((rr * NT + c) * 4 + g4) * 64];
           // (k half 0) + (k half 1) whichever of the two this wavefront holds
           float4 o = KH ? make_float4(p.x + t[4 * g4], p.y + t[4 * g4 + 1], p.z + t[4 * g4 + 2], p.w + t[4 * g4 + 3])
@@ -231,11 +232,11 @@ __device__ __forceinline__ void gemm_epilogue_half(float16_t (&acc)[4][NT], cons
   if (vec) tail(std::true_type{});
   else tail(std::false_type{});
 }
-template <int NT>
-__device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[4][NT], const float* bias, float* out, u32 out_dim, u32 m,
+template <int NT, int MT>
+__device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[MT][NT], const float* bias, float* out, u32 out_dim, u32 m,
                                               u32 mt, u32 nt, u32 nh, u32 kh, u32 j, u32 kg, u32 tid, u32 bias_stride = 0) {
-  if (kh == 0) gemm_epilogue_half<0, NT>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
-  else gemm_epilogue_half<1, NT>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
+  if (kh == 0) gemm_epilogue_half<0, NT, MT>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
+  else gemm_epilogue_half<1, NT, MT>(acc, bias, out, out_dim, m, mt, nt, nh, j, kg, tid & 63, bias_stride);
 }
 
 // Epilogue of the gate | up kernel: the nh = 0 wavefronts hold 96 gate rows, the nh = 1 wavefronts the same 96 rows of up,
@@ -328,11 +329,15 @@ struct GemmRawT<true> {   // Q5_K: plus the 32 bytes of fifth bits (bit 2g + hi 
 // the epilogue stores silu(gate) * up. No k split and no bias then.
 // NT: tiles of 32 weight rows per wavefront - 3 (workgroup tile 128 tokens x 192 rows) or 2 (128 x 128, for launches whose
 // 192-row tiles, times the k split, leave compute units idle: q4_k_gemm_n128_f16, q5_k_gemm_n128_f16).
-template <bool Q5, bool SWIGLU = false, int NT = 3>
+// MT: tiles of 32 tokens - 4 (128 tokens) or 2: launches of up to 64 tokens, where the upper half of a 128-token tile would
+// be MFMAs on padding and copies of nothing (<type>_gemm_m64[_n128]_f16; the packed x is the same, its first 64 tokens are used).
+template <bool Q5, bool SWIGLU = false, int NT = 3, int MT = 4>
 __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim,
                                               u32 out_dim, u32 m, u32 bias_stride = 0, const uint8_t* w_b = nullptr) {
   static_assert(!(Q5 && SWIGLU), "the gate | up kernel is built for Q4_K");
   static_assert(NT == 3 || (NT == 2 && !SWIGLU), "tile heights");
+  static_assert(MT == 4 || (MT == 2 && !SWIGLU), "tokens per tile");
+  constexpr int NX = 4 * MT;              // copies of x per thread and super-block: 32 chunks of 128 tokens x 16 bytes, or of the first 64 tokens of each
   constexpr u32 BN = 64 * NT;             // weight rows of the workgroup tile
   constexpr u32 BS = Q5 ? 176 : 144;      // bytes of a super-block
   constexpr u32 PPR = Q5 ? 10 : 9;        // 16-byte pieces of a row that go through LDS
@@ -402,14 +407,22 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   for (int c = 0; c < NT; c++) hoff[c] = (min(nt * BN + nh * (32 * NT) + 32 * c + j, out_dim - 1) - tile_row0) * (u32)row_bytes;
   const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
-  float16_t acc[4][NT];
+  float16_t acc[MT][NT];
 #pragma unroll
-  for (int r = 0; r < 4; r++)
+  for (int r = 0; r < MT; r++)
 #pragma unroll
     for (int c = 0; c < NT; c++)
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[r][c][v] = 0.0f;
 
+  // copy i of a super-block's x tile: 128 tokens - 4 KiB of the image per instruction and workgroup; 64 tokens - the
+  // wavefront takes the first KiB (tokens 0..63) of the 2 KiB chunk 4 i + wave
+  auto x_copy = [&](const uint4* src, uint4* dst, int i) {
+    if constexpr (MT == 4)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(src + 256 * i + tid), (lds_void*)(dst + 256 * i + wave * 64), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((gbl_void*)(src + (4 * i + wave) * 128 + lane), (lds_void*)(dst + (4 * i + wave) * 128), 16, 0, 0);
+  };
   auto copy_w = [&](u32 kb, int i) {   // copy i of this wavefront for super-block kb
     if constexpr (SWIGLU)
       __builtin_amdgcn_global_load_lds((gbl_void*)(wsrc[i] + (size_t)kb * BS), (lds_void*)(wbuf + (4 * i + wave) * 64), 16, 0, 0);
@@ -432,14 +445,10 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   for (int c = 0; c < NT; c++) load_hdr(0, c);
   if (odd) {
 #pragma unroll
-    for (int i = 0; i < 16; i++)
-      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf1 + 256 * i + wave * 64),
-                                       16, 0, 0);
+    for (int i = 0; i < NX; i++) x_copy(xtile, gemm_xbuf1, i);
   } else {
 #pragma unroll
-    for (int i = 0; i < 16; i++)
-      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
-                                       16, 0, 0);
+    for (int i = 0; i < NX; i++) x_copy(xtile, gemm_xbuf0, i);
   }
   __syncthreads();
 
@@ -447,7 +456,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   // the two operand sets of the k-step pipeline.
   GemmRawT<Q5> cur[NT];
   u32 S[NT][4];
-  uint4 A[2][4];
+  uint4 A[2][MT];
   half8_t B[2][NT];
   // The raw bytes of a super-block, out of gemm_wbuf into the registers of the lanes that decode them.
   auto take_raw = [&]() {
@@ -513,10 +522,10 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
     }
   };
   // A operands of k-step t of the wavefront (k-steps 8*kh .. 8*kh+7 of the tile; 32 lanes read 512 contiguous bytes)
-  auto read_a = [&](uint4 (&Ad)[4], const uint4* xbuf, int t) {
+  auto read_a = [&](uint4 (&Ad)[MT], const uint4* xbuf, int t) {
     const uint4* arow = xbuf + (16 * kh + kg) * 128 + j;
 #pragma unroll
-    for (int r = 0; r < 4; r++) Ad[r] = arow[t * 256 + r * 32];
+    for (int r = 0; r < MT; r++) Ad[r] = arow[t * 256 + r * 32];
   };
 
   // Operands of k-step 0 of the first super-block; after that every super-block prepares the first k-step of the
@@ -532,9 +541,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   auto iteration = [&](u32 kb, const uint4* xcur, uint4* xnxt) {
     const u32 kn = min(kb + 1, nkb - 1);   // the last iteration re-reads its own tile; the copy is not used
     const uint4* xnext = xtile + (size_t)kn * 4096;   // uniform
-    auto copy_x = [&](int i) {
-      __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64), 16, 0, 0);
-    };
+    auto copy_x = [&](int i) { x_copy(xnext, xnxt, i); };
     // software pipeline over the wavefront's eight k-steps: while the MFMAs of step t run, the A operands
     // of step t+1 are read from LDS and its B operands are built
 #pragma unroll
@@ -553,7 +560,8 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
       if (t == 4 && NCOPY > 7) copy_w(kn, 7);
       if (t < 6) {
 #pragma unroll
-        for (int i = (t < 2 ? 2 * t : 3 * t - 2); i < (t < 2 ? 2 * t + 2 : 3 * t + 1); i++) copy_x(i);
+        for (int i = (t < 2 ? 2 * t : 3 * t - 2); i < (t < 2 ? 2 * t + 2 : 3 * t + 1); i++)
+          if (i < NX) copy_x(i);   // (64 tokens: eight copies, out by k-step 3)
       }
       if (t < 7) {
         read_a(A[p ^ 1], xcur, t + 1);
@@ -568,7 +576,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
         build_b(B[0], 0);
       }
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
+      for (int r = 0; r < MT; r++) {
         const half8_t Ar = *reinterpret_cast<const half8_t*>(&A[p][r]);
 #pragma unroll
         for (int c = 0; c < NT; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[p][c], Ar, acc[r][c], 0, 0, 0);
@@ -586,7 +594,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
         __builtin_amdgcn_sched_group_barrier(0x020, 8, 0);   // VMEM reads (LDS-direct copies) of this step
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
 #pragma unroll
-        for (int i = 0; i < 4 * NT; i++) {
+        for (int i = 0; i < MT * NT; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            // one MFMA
           __builtin_amdgcn_sched_group_barrier(0x002, Q5 ? 8 : 5, 0);   // five VALU (eight with the fifth bits)
         }
@@ -595,7 +603,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
 #pragma unroll
         for (int i = 0; i < NT; i++) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // a few MFMAs while they arrive
 #pragma unroll
-        for (int i = 0; i < 3 * NT; i++) {
+        for (int i = 0; i < (MT - 1) * NT; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
         }
@@ -625,7 +633,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
     if (kh == 0) gemm_epilogue_swiglu_half<0>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
     else gemm_epilogue_swiglu_half<1>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
   } else {
-    gemm_epilogue<NT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
+    gemm_epilogue<NT, MT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
   }
 }
 
@@ -642,6 +650,16 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
   gemm_k45_core<true, false, 2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }
+// up to 64 tokens: the first 64 tokens of the (one) token tile only; grid from gemm_grid_x(1, ceil(out_dim / 192 | 128))
+#define GEMM_K45_M64_ENTRY(NAME, Q5, NT)                                                                                  \
+  extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void NAME(                       \
+      const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) { \
+    gemm_k45_core<Q5, false, NT, 2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);                                   \
+  }
+GEMM_K45_M64_ENTRY(q4_k_gemm_m64_f16, false, 3)
+GEMM_K45_M64_ENTRY(q4_k_gemm_m64_n128_f16, false, 2)
+GEMM_K45_M64_ENTRY(q5_k_gemm_m64_f16, true, 3)
+GEMM_K45_M64_ENTRY(q5_k_gemm_m64_n128_f16, true, 2)
 // Q5_K: x is packed by pack_x_f16_q4k (the values of a super-block sit where the Q4_K ones do).
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q5_k_gemm_f16(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {

@@ -57,9 +57,11 @@ __shared__ u32 gemm_wsc6[GEMM_BN * 6];
 // NT: tiles of 32 weight rows per wavefront - 3 (a workgroup tile of 128 tokens x 192 rows) or 2 (128 x 128: a third less
 // work per workgroup for shapes whose 192-row tiles, times the k split, leave compute units idle - 4096 rows at 512 tokens
 // are 88 tiles x 2 splits = 176 workgroups, but 128 x 2 = 256 of the smaller ones).
-template <int NT>
+// MT: tiles of 32 tokens, 4 or 2 (launches of up to 64 tokens: q6_k_gemm_m64[_n128]_f16), as in gemm_k45_core.
+template <int NT, int MT = 4>
 __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim,
                                               u32 m, u32 bias_stride) {
+  constexpr int NX = 4 * MT;   // copies of x per thread and super-block
   constexpr u32 BN = 64 * NT, NSTG = 2 * NT;   // rows of the workgroup tile; 16-byte pieces of ql a thread stages per super-block
   const u32 tid = threadIdx.x, lane = tid & 63;
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -86,9 +88,9 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
   const u32 o_qh = 128 + 32 * kh + 16 * kg;
   const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
-  float16_t acc[4][NT];
+  float16_t acc[MT][NT];
 #pragma unroll
-  for (int r = 0; r < 4; r++)
+  for (int r = 0; r < MT; r++)
 #pragma unroll
     for (int c = 0; c < NT; c++)
 #pragma unroll
@@ -135,6 +137,13 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
     }
   };
 
+  // copy i of a super-block's x tile (as in gemm_k45_core: 128 tokens, or the first 64 of every chunk)
+  auto x_copy = [&](const uint4* src, uint4* dst, int i) {
+    if constexpr (MT == 4)
+      __builtin_amdgcn_global_load_lds((gbl_void*)(src + 256 * i + tid), (lds_void*)(dst + 256 * i + wave * 64), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((gbl_void*)(src + (4 * i + wave) * 128 + lane), (lds_void*)(dst + (4 * i + wave) * 128), 16, 0, 0);
+  };
   auto load_row = [&](GemmRaw6& raw, const uint8_t* kbase, int c) {
     raw.qh = ld16(kbase + (rowoff[c] + o_qh));
   };
@@ -151,16 +160,12 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
 #pragma unroll
     for (int c = 0; c < NT; c++) load_row(rawB[c], wbase, c);
 #pragma unroll
-    for (int i = 0; i < 16; i++)
-      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf1 + 256 * i + wave * 64),
-                                       16, 0, 0);
+    for (int i = 0; i < NX; i++) x_copy(xtile, gemm_xbuf1, i);
   } else {
 #pragma unroll
     for (int c = 0; c < NT; c++) load_row(rawA[c], wbase, c);
 #pragma unroll
-    for (int i = 0; i < 16; i++)
-      __builtin_amdgcn_global_load_lds((gbl_void*)(xtile + 256 * i + tid), (lds_void*)(gemm_xbuf0 + 256 * i + wave * 64),
-                                       16, 0, 0);
+    for (int i = 0; i < NX; i++) x_copy(xtile, gemm_xbuf0, i);
   }
   stage_store();
   __syncthreads();
@@ -209,10 +214,10 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
 
     // software pipeline over the wavefront's eight k-steps: while the MFMAs of step t run, the A operands
     // of step t+1 are read from LDS and its B operands are built
-    uint4 A[2][4];
+    uint4 A[2][MT];
     half8_t B[2][NT];
 #pragma unroll
-    for (int r = 0; r < 4; r++) A[0][r] = arow[r * 32];
+    for (int r = 0; r < MT; r++) A[0][r] = arow[r * 32];
     build_b(B[0], 0);
 #pragma unroll
     for (int t = 0; t < 8; t++) {
@@ -230,16 +235,15 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
       if (t < 6) {
 #pragma unroll
         for (int i = (t < 3 ? 2 * t : 3 * t - 3); i < (t < 3 ? 2 * t + 2 : (t < 5 ? 3 * t : 16)); i++)
-          __builtin_amdgcn_global_load_lds((gbl_void*)(xnext + 256 * i + tid), (lds_void*)(xnxt + 256 * i + wave * 64),
-                                           16, 0, 0);
+          if (i < NX) x_copy(xnext, xnxt, i);
       }
       if (t < 7) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) A[p ^ 1][r] = arow[(t + 1) * 256 + r * 32];
+        for (int r = 0; r < MT; r++) A[p ^ 1][r] = arow[(t + 1) * 256 + r * 32];
         build_b(B[p ^ 1], t + 1);
       }
 #pragma unroll
-      for (int r = 0; r < 4; r++) {
+      for (int r = 0; r < MT; r++) {
         const half8_t Ar = *reinterpret_cast<const half8_t*>(&A[p][r]);
 #pragma unroll
         for (int c = 0; c < NT; c++) acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(B[p][c], Ar, acc[r][c], 0, 0, 0);
@@ -251,7 +255,7 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
       __builtin_amdgcn_sched_group_barrier(0x020, 10, 0);  // VMEM reads (weights, LDS-direct x) of this step
       __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);   // LDS reads: A operands of the next step
 #pragma unroll
-      for (int i = 0; i < 4 * NT; i++) {
+      for (int i = 0; i < MT * NT; i++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
         __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);   // eight VALU (a Q6_K operand takes more than a Q4_K one)
       }
@@ -275,12 +279,21 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
     iteration(kb + 1, gemm_xbuf1, gemm_xbuf0, rawB, rawA);
   }
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
-  gemm_epilogue<NT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
+  gemm_epilogue<NT, MT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
 }
 
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_f16(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
   gemm_q6k_core<3>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+}
+// up to 64 tokens, tiles of 64 x 192 and 64 x 128
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_m64_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_q6k_core<3, 2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+}
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_m64_n128_f16(
+    const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
+  gemm_q6k_core<2, 2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }
 // the same with a workgroup tile of 128 tokens x 128 rows; grid from gemm_grid_x(ceil(m/128), ceil(out_dim/128))
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_n128_f16(

@@ -344,6 +344,8 @@ int cogni_gemv_top1_noalloc_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uin
  *          tiles of 128 x 192 times the k split would leave compute units idle (the 4096-row projections at 512 tokens),
  *          q4_k_gemm_n128_f16 | q5_k_gemm_n128_f16 | q6_k_gemm_n128_f16 (same arguments and block, tiles of 128 x 128); or,
  *          for Q4_K launches that fill whole rounds of 128 x 256 tiles, q4_k_gemm_wide_f16 (same arguments), block 512.
+ *          Launches of up to 64 tokens take the forms of the 192- and 128-row kernels that work on the first 64 tokens of
+ *          the token tile, <type>_gemm_m64_f16 | <type>_gemm_m64_n128_f16 (same arguments and block).
  *          cogni_gemm_plan says which, with the grid; all of them give the same bits for the same k split.
  * (pack_x_f16_*: block 256, grid ceil(tokens/128)*16*(in_dim/256).) Other types: COGNI_ERR_UNSUPPORTED_TYPE. */
 size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tokens);

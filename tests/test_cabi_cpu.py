@@ -167,7 +167,7 @@ def test_gemv_plan_picks_the_kernel_for_the_shape():
 def test_gemm_plan_picks_tile_and_split_for_the_shape():
     blob = code_object()
     for k in ("q4_k_gemm_f16", "q4_k_gemm_wide_f16", "q5_k_gemm_f16", "q6_k_gemm_f16", "q4_k_gemm_n128_f16", "q5_k_gemm_n128_f16",
-              "q6_k_gemm_n128_f16", "gemm_sum_splits_f32", "pack_x_f16_q4k", "pack_x_f16_q6k"):
+              "q6_k_gemm_n128_f16", "q4_k_gemm_m64_f16", "q5_k_gemm_m64_n128_f16", "q6_k_gemm_m64_f16", "q6_k_gemm_m64_n128_f16", "gemm_sum_splits_f32", "pack_x_f16_q4k", "pack_x_f16_q6k"):
         assert (k.encode() + b"\x00") in blob, k
     big = 1 << 40
     # 512 x 12288: 256 tiles of 128 x 192, one per compute unit; 192 wide tiles would leave a quarter of them idle
@@ -183,7 +183,8 @@ def test_gemm_plan_picks_tile_and_split_for_the_shape():
     for t, pfx in ((12, "q4_k"), (13, "q5_k"), (14, "q6_k")):
         assert quant.gemm_plan(t, 12288, 4096, 512, big) == (pfx + "_gemm_n128_f16", 128, 2, 256)
         assert quant.gemm_plan(t, 4096, 4096, 512, big) == (pfx + "_gemm_n128_f16", 128, 2, 256)
-        assert quant.gemm_plan(t, 12288, 4096, 64, big) == (pfx + "_gemm_n128_f16", 32, 8, 256)
+        assert quant.gemm_plan(t, 12288, 4096, 64, big) == (pfx + "_gemm_m64_n128_f16", 32, 8, 256)   # up to 64 tokens: half a token tile
+        assert quant.gemm_plan(t, 12288, 4096, 65, big)[0] == pfx + "_gemm_n128_f16" and quant.gemm_plan(t, 4096, 12288, 9, big)[0] == pfx + "_gemm_m64_f16"
         assert quant.gemm_plan(t, 4096, 12288, 512, big)[0] == pfx + "_gemm_f16"            # 256 tiles of 192 rows fill the chip exactly
         assert quant.gemm_plan(t, 4096, 12288, 1024, big)[0] == pfx + "_gemm_f16"           # two rounds of 192 rows against three of 128
         # the planes of a split launch are sized by the same plan
@@ -192,9 +193,9 @@ def test_gemm_plan_picks_tile_and_split_for_the_shape():
     assert quant.gemm_plan(12, 12288, 4096, 2048, big)[0] == "q4_k_gemm_wide_f16"              # one round of the 256-row tiles
     # few tiles: the k range is split when the workspace has room for the planes, else not
     name, gx, gy, block = quant.gemm_plan(12, 4096, 12288, 64, big)
-    assert (name, gx, block) == ("q4_k_gemm_f16", 64, 256) and gy == 4
+    assert (name, gx, block) == ("q4_k_gemm_m64_f16", 64, 256) and gy == 4
     # (unsplit, 96 tiles of 128 rows spread over more compute units than 64 of 192)
-    assert quant.gemm_plan(12, 4096, 12288, 64, quant.gemm_workspace_bytes(12, 4096, 64)) == ("q4_k_gemm_n128_f16", 96, 1, 256)
+    assert quant.gemm_plan(12, 4096, 12288, 64, quant.gemm_workspace_bytes(12, 4096, 64)) == ("q4_k_gemm_m64_n128_f16", 96, 1, 256)
     # the eight-wavefront kernel is Q4_K's alone
     assert quant.gemm_plan(13, 4096, 12288, 2048, big)[0] == "q5_k_gemm_f16" and quant.gemm_plan(14, 4096, 12288, 2048, big)[0] == "q6_k_gemm_f16"
     with pytest.raises(quant.QuantError, match="Unsupported quant type"):

@@ -163,6 +163,26 @@ def test_tile_heights_agree(gpu, oracle, t, tokens, out_dim, in_dim, monkeypatch
           sample_tokens=[i for i in (0, 1, 63, 64, 127, 128, tokens - 1) if i < tokens])
 
 
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("tokens,out_dim,in_dim", [(64, 12288, 1024), (9, 4096 + 37, 768), (33, 250, 4096), (64, 1024, 256)])
+def test_launches_of_up_to_64_tokens(gpu, oracle, t, tokens, out_dim, in_dim, monkeypatch):
+    """Up to 64 tokens run the kernels that work on the first 64 tokens of the token tile (<type>_gemm_m64[_n128]_f16): the
+    bits of the 128-token kernels (COGNI_GEMM_M64=0), whole and clipped tiles, k splits, a bias; and the bar."""
+    rng = np.random.default_rng(t * 37 + tokens + out_dim)
+    raw = synth.make_weights(rng, t, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    bias = rng.standard_normal(out_dim).astype(np.float32)
+    wsb = quant.gemm_workspace_bytes(t, in_dim, tokens, out_dim)
+    assert "_m64" in quant.gemm_plan(t, in_dim, out_dim, tokens, wsb)[0]
+    half = run_gemm(raw, x, in_dim, out_dim, tokens, bias, t=t)
+    monkeypatch.setenv("COGNI_GEMM_M64", "0")
+    assert "_m64" not in quant.gemm_plan(t, in_dim, out_dim, tokens, wsb)[0]
+    full = run_gemm(raw, x, in_dim, out_dim, tokens, bias, t=t)
+    monkeypatch.delenv("COGNI_GEMM_M64")
+    assert np.array_equal(half, full)
+    check(oracle, raw, x, in_dim, out_dim, tokens, bias, "type %d M=%d N=%d K=%d" % (t, tokens, out_dim, in_dim), t=t)
+
+
 @pytest.mark.parametrize("t,tokens,out_dim,in_dim", [(Q4_K, 130, 400, 768), (Q6_K, 64, 384, 4096), (Q5_K, 40, 100, 512),
                                                      (Q4_K, 128, 65536, 256), (Q6_K, 512, 4096, 2048)])
 def test_residual_add_in_the_epilogue(gpu, oracle, t, tokens, out_dim, in_dim):
