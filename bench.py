@@ -567,8 +567,9 @@ def main():
         cases["cfg4 q4_k gemm 12288x4096 M=%d" % tokens] = rec
         log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
             tokens, gsteps, rec["us"], rec["tflops"], rec["frac_mfma_f16"]))
-    # the feed-forward block of a layer at M = 512 in its prefill form: add + RMSNorm, pack, gate | up GEMM with SwiGLU inside,
-    # pack, Q6_K down GEMM with the residual inside (three rotating sets of weights: 290 MB)
+    # the feed-forward block of a layer at M = 512 in its prefill form: add + RMSNorm, pack, gate | up GEMM with SwiGLU inside
+    # (its epilogue writes the down GEMM's packed input), Q6_K down GEMM with the residual inside (three rotating sets of
+    # weights: 290 MB)
     from cogni_ml_amd.ffn_sequence import FFNSequenceRunner as _FFN
     ffn_tokens = 512
     fx = rng.uniform(-0.1, 0.1, ffn_tokens * 4096).astype(np.float32)
@@ -576,7 +577,7 @@ def main():
     ffns = []
     for _ in range(3):
         fr = _FFN(synth.make_weights(rng, Q4_K, 12288, 4096), synth.make_weights(rng, Q4_K, 12288, 4096),
-                  synth.make_weights(rng, Q6_K, 4096, 12288), 4096, 12288, ffn_tokens, fx, norm=fnorm, add=fx.copy())
+                  synth.make_weights(rng, Q6_K, 4096, 12288), 4096, 12288, ffn_tokens, fx, norm=fnorm, add=fx.copy(), keep_combined=False)
         fr.upload_weights()
         fr.reset_sequence()
         ffns.append(fr)
@@ -589,7 +590,7 @@ def main():
     cases["cfg4 ffn block prefill M=512 (add+rmsnorm, gate|up|swiglu gemm, q6_k down gemm + residual)"] = {
         "us": round(r["us"], 2), "tflops": round(fflops / r["us"] / 1e6, 1),
         "frac_mfma_f16": round(fflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "flops": fflops,
-        "launches": "add_rmsnorm, pack, q4_k_gemm_swiglu_f16, pack, q6_k_gemm_f16 (k split) + plane sum with the residual"}
+        "launches": "add_rmsnorm, pack, q4_k_gemm_swiglu_pack_q6k_f16, q6_k_gemm_n128_f16 (k split) + plane sum with the residual"}
     log("case=ffn block prefill M=512\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
         r["us"], fflops / r["us"] / 1e6, fflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS))
     for fr in ffns:

@@ -7,9 +7,11 @@ a group of up to four tokens here is two launches (gate | up | SwiGLU fused, the
 that is not a multiple of 16 goes through the weight-stationary kernels for several tokens (gate | up pair, swiglu_f32, down).
 
 A sequence of more tokens than the GEMM threshold (quant.get_gemm_threshold()) is the prefill form of the same block, all
-tokens at once in four launches: the activations packed, gate | up as one GEMM with SwiGLU in its epilogue, the result
-packed in the down matrix's layout, the down GEMM with the residual added in its epilogue (src/ml/gguf/qwen35_cpu.cr:1711-1722;
-the reference's Metal kernels gemm_q4k.metal:1233 and gemm_mm.metal:651).
+tokens at once in three launches: the activations packed (by the add + RMSNorm in front, where there is one), gate | up as
+one GEMM with SwiGLU in its epilogue, which also writes its products as the packed fp16 activations of the down matrix's
+layout, and the down GEMM with the residual added in its epilogue (src/ml/gguf/qwen35_cpu.cr:1711-1722; the reference's Metal kernels gemm_q4k.metal:1233 and gemm_mm.metal:651).
+`keep_combined=False` leaves the fp32 products (`combined`, the probe's second output) unwritten on that route: they then
+exist only as the down GEMM's input.
 
 With `norm` and `add` the sequence is the whole FFN half of a decoder layer (src/ml/gguf/qwen35_cpu.cr:1705-1725):
 r = x + add (the attention output joining the residual stream), h = rmsnorm(r, norm), out = r + down(silu(gate h) * up h).
@@ -22,7 +24,7 @@ from .types import TensorType
 
 class FFNSequenceRunner:
     def __init__(self, gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, residual=None, down_type=TensorType.Q6_K,
-                 norm=None, add=None, eps=1.0e-6):
+                 norm=None, add=None, eps=1.0e-6, keep_combined=True):
         if not tokens > 0:
             raise ValueError("tokens must be positive")
         if len(xs) != tokens * hidden:
@@ -34,6 +36,7 @@ class FFNSequenceRunner:
         if norm is not None and (residual is not None or len(norm) != hidden or len(add) != tokens * hidden):
             raise ValueError("norm/add size mismatch, or a residual given besides them")
         self.hidden, self.ffn_dim, self.tokens, self.down_type = hidden, ffn_dim, tokens, down_type
+        self.keep_combined = keep_combined
         self._raw = {"gate": gate_raw, "up": up_raw, "down": down_raw}
         self._xs = np.ascontiguousarray(xs, dtype=np.float32)
         self._residual = None if residual is None else np.ascontiguousarray(residual, dtype=np.float32)
@@ -116,13 +119,19 @@ class FFNSequenceRunner:
         st = hip.current_stream_handle()
         h, f = self.hidden, self.ffn_dim
         x = self._x.ptr
-        if self._norm is not None:
-            quant.add_rmsnorm_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, self._normed.ptr, h, count, self._eps, st)
-            x = self._normed.ptr
-        quant.gemm_pack_dev(x, TensorType.Q4_K, h, count, self._ws_x.ptr, self._ws_x_bytes, st)
-        quant.gemm_packed_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, self._ws_x.ptr, self._ws_x_bytes,
-                                     self._act.ptr, h, f, count, st)
-        quant.gemm_pack_dev(self._act.ptr, self.down_type, f, count, self._ws_act.ptr, self._ws_act_bytes, st)
+        if self._norm is not None and h <= 4096:
+            # r = x + add, and rmsnorm(r) written straight as the packed activations gate | up read
+            quant.add_rmsnorm_gemm_pack_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, 0, TensorType.Q4_K, self._ws_x.ptr,
+                                            self._ws_x_bytes, h, count, self._eps, st)
+        else:
+            if self._norm is not None:
+                quant.add_rmsnorm_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, self._normed.ptr, h, count, self._eps, st)
+                x = self._normed.ptr
+            quant.gemm_pack_dev(x, TensorType.Q4_K, h, count, self._ws_x.ptr, self._ws_x_bytes, st)
+        # silu(gate) * up leaves the GEMM as the down GEMM's packed input (and as fp32 only when `combined` is wanted)
+        quant.gemm_packed_swiglu_pack_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, self._ws_x.ptr, self._ws_x_bytes,
+                                          self._act.ptr if self.keep_combined else 0, self.down_type, self._ws_act.ptr,
+                                          self._ws_act_bytes, h, f, count, st)
         if self._res is not None:
             quant.gemm_packed_add_dev(self._w["down"].ptr, self.down_type, self._ws_act.ptr, self._ws_act_bytes, self._res.ptr,
                                       self._out.ptr, f, h, count, st)
@@ -142,9 +151,12 @@ class FFNSequenceRunner:
 
     def _read_outputs(self):
         hip.synchronize("hipDeviceSynchronize(read_outputs)")
-        self.combined = np.empty(self.tokens * self.ffn_dim, dtype=np.float32)
+        prefill = self._ws_x is not None and self._runner.active_tokens > quant.get_gemm_threshold()
+        self.combined = None
+        if self.keep_combined or not prefill:
+            self.combined = np.empty(self.tokens * self.ffn_dim, dtype=np.float32)
+            hip.copy_dtoh(self.combined, self._act.ptr, self.combined.nbytes, "combined")
         self.out = np.empty(self.tokens * self.hidden, dtype=np.float32)
-        hip.copy_dtoh(self.combined, self._act.ptr, self.combined.nbytes, "combined")
         hip.copy_dtoh(self.out, self._out.ptr, self.out.nbytes, "out")
 
     # lifecycle

@@ -244,6 +244,21 @@ def add_rmsnorm_pack_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_
                                                 ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
 
 
+def rmsnorm_gemm_pack_dev(x_ptr, norm_ptr, out_ptr, w_type, workspace_ptr, workspace_bytes, dim, tokens, eps=1.0e-6, stream=None):
+    """rmsnorm_dev whose rows leave as the packed activations of the prefill GEMMs (what gemm_pack_dev would write); out_ptr may be 0."""
+    _check(hip.lib().cogni_rmsnorm_gemm_pack_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(out_ptr),
+                                                 ctypes.c_uint32(int(w_type)), ctypes.c_uint64(workspace_ptr), ctypes.c_size_t(workspace_bytes),
+                                                 ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
+
+def add_rmsnorm_gemm_pack_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_ptr, w_type, workspace_ptr, workspace_bytes, dim,
+                              tokens, eps=1.0e-6, stream=None):
+    """add_rmsnorm_dev whose normalised rows leave as the packed activations of the prefill GEMMs; normed_out_ptr may be 0."""
+    _check(hip.lib().cogni_add_rmsnorm_gemm_pack_dev(
+        ctypes.c_uint64(x_ptr), ctypes.c_uint64(add_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(residual_out_ptr),
+        ctypes.c_uint64(normed_out_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(workspace_ptr), ctypes.c_size_t(workspace_bytes),
+        ctypes.c_uint32(dim), ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
 def gemm_workspace_bytes(w_type, in_dim, tokens, out_dim=None):
     """Bytes of caller-owned scratch for gemm_dev: the packed activations, and with `out_dim` given also the planes of
     a k-split launch (few tiles), which gemm_dev uses when the workspace has room for them."""
@@ -301,6 +316,15 @@ def gemm_packed_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, workspace_ptr, workspac
     _check(hip.lib().cogni_gemm_packed_swiglu_dev(ctypes.c_uint64(w_gate_ptr), ctypes.c_uint64(w_up_ptr), ctypes.c_uint32(int(w_type)),
                                                   ctypes.c_uint64(workspace_ptr), ctypes.c_size_t(workspace_bytes), ctypes.c_uint64(out_ptr),
                                                   ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
+def gemm_packed_swiglu_pack_dev(w_gate_ptr, w_up_ptr, w_type, workspace_ptr, workspace_bytes, out_ptr, next_type, next_workspace_ptr,
+                                next_workspace_bytes, in_dim, out_dim, tokens, stream=None):
+    """gemm_packed_swiglu_dev whose products also (out_ptr 0: only) leave as the packed activations of the next GEMM."""
+    _check(hip.lib().cogni_gemm_packed_swiglu_pack_dev(
+        ctypes.c_uint64(w_gate_ptr), ctypes.c_uint64(w_up_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(workspace_ptr),
+        ctypes.c_size_t(workspace_bytes), ctypes.c_uint64(out_ptr), ctypes.c_uint32(int(next_type)), ctypes.c_uint64(next_workspace_ptr),
+        ctypes.c_size_t(next_workspace_bytes), ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
 def matmul_dev(w_ptr, w_type, x_ptr, out_ptr, in_dim, out_dim, tokens, workspace_ptr=0, workspace_bytes=0, bias_ptr=0,

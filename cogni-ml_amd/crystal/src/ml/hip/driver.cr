@@ -87,6 +87,11 @@ lib LibCogniHIP
   fun cogni_add_rmsnorm_pack_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,
                                  w_type : UInt32, image : UInt64, dim : UInt32, tokens : UInt32, eps : Float32,
                                  stream : Void*) : Int32
+  fun cogni_rmsnorm_gemm_pack_dev(x : UInt64, norm : UInt64, out : UInt64, w_type : UInt32, workspace : UInt64,
+                                  workspace_bytes : LibC::SizeT, dim : UInt32, tokens : UInt32, eps : Float32, stream : Void*) : Int32
+  fun cogni_add_rmsnorm_gemm_pack_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,
+                                      w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT, dim : UInt32,
+                                      tokens : UInt32, eps : Float32, stream : Void*) : Int32
   fun cogni_embed_dev(w_raw : UInt64, w_type : UInt32, token_ids : UInt64, output : UInt64, history : UInt64,
                       token_index : UInt32, hidden_dim : UInt32, vocab_size : UInt32, stream : Void*) : Int32
   fun cogni_gemv_top1_partials(w_type : UInt32, out_dim : UInt32) : UInt32
@@ -109,6 +114,9 @@ lib LibCogniHIP
                                 out : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemm_packed_swiglu_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT,
                                    out : UInt64, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemm_packed_swiglu_pack_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT,
+                                        out : UInt64, next_type : UInt32, next_workspace : UInt64, next_workspace_bytes : LibC::SizeT,
+                                        in_dim : UInt32, out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemm_plan(w_type : UInt32, in_dim : UInt32, out_dim : UInt32, tokens : UInt32, workspace_bytes : LibC::SizeT,
                       kernel : UInt8**, grid_x : UInt32*, grid_y : UInt32*, block_x : UInt32*) : Int32
   fun cogni_set_gemm_threshold(tokens : Int32) : Int32

@@ -951,6 +951,36 @@ size_t cogni_gemm_workspace_bytes(uint32_t w_type, uint32_t in_dim, uint32_t tok
   return mtiles * 128 * (size_t)in_dim * 2;
 }
 
+// The norms that write the packed activations of the prefill GEMMs (kernels/norm.hpp): one workgroup per token of whole
+// 128-token tiles, rows of the short-row path.
+static int norm_gemm_pack_check(const char* who, uint32_t w_type, uint32_t dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes) {
+  if (!gemm_type(w_type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the prefill GEMM: ") + type_name(w_type));
+  if (dim == 0 || tokens == 0 || (dim % 256) != 0 || dim > 4096)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": dim must be a multiple of 256 up to 4096, tokens at least 1");
+  const size_t need = cogni_gemm_workspace_bytes(w_type, dim, tokens);
+  if (!workspace || workspace_bytes < need)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": workspace has " + std::to_string(workspace_bytes) + " bytes, needs " + std::to_string(need));
+  return 0;
+}
+int cogni_rmsnorm_gemm_pack_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t w_type, uint64_t workspace, size_t workspace_bytes,
+                                uint32_t dim, uint32_t tokens, float eps, void* stream) {
+  if (!x || !norm) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_gemm_pack_dev: null device pointer");
+  if (int rc = norm_gemm_pack_check("cogni_rmsnorm_gemm_pack_dev", w_type, dim, tokens, workspace, workspace_bytes)) return rc;
+  void* params[] = {&x, &norm, &out, &workspace, &dim, &tokens, &eps};
+  return launch(w_type == COGNI_TYPE_Q6_K ? "rmsnorm_gemm_pack_q6k_f32" : "rmsnorm_gemm_pack_q4k_f32", 128 * ((tokens + 127) / 128), 256, 0,
+                params, stream);
+}
+int cogni_add_rmsnorm_gemm_pack_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t w_type,
+                                    uint64_t workspace, size_t workspace_bytes, uint32_t dim, uint32_t tokens, float eps, void* stream) {
+  if (!x || !add || !norm || !residual_out)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_add_rmsnorm_gemm_pack_dev: null device pointer");
+  if (int rc = norm_gemm_pack_check("cogni_add_rmsnorm_gemm_pack_dev", w_type, dim, tokens, workspace, workspace_bytes)) return rc;
+  void* params[] = {&x, &add, &norm, &residual_out, &normed_out, &workspace, &dim, &tokens, &eps};
+  return launch(w_type == COGNI_TYPE_Q6_K ? "add_rmsnorm_gemm_pack_q6k_f32" : "add_rmsnorm_gemm_pack_q4k_f32", 128 * ((tokens + 127) / 128),
+                256, 0, params, stream);
+}
+
 // k splits of the prefill GEMM: a launch of fewer than half as many tiles as there are compute units (256) leaves most
 // of them idle, so the super-blocks of a row are divided among up to 8 workgroups per tile, each with at least two
 // super-blocks; the partial sums go through the workspace.
@@ -1130,6 +1160,26 @@ int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 95) / 96;
   void* params[] = {&w_gate, &w_up, &workspace, &out, &in_dim, &out_dim, &tokens};
   return launch("q4_k_gemm_swiglu_f16", gemm_grid_x(mtiles, ntiles), 256, 0, params, stream);
+}
+
+int cogni_gemm_packed_swiglu_pack_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
+                                      uint32_t next_type, uint64_t next_workspace, size_t next_workspace_bytes, uint32_t in_dim,
+                                      uint32_t out_dim, uint32_t tokens, void* stream) {
+  const char* who = "cogni_gemm_packed_swiglu_pack_dev";
+  if (w_type != COGNI_TYPE_Q4_K)
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the fused gate/up SwiGLU GEMM: ") + type_name(w_type));
+  if (!gemm_type(next_type))
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the prefill GEMM: ") + type_name(next_type));
+  if (!w_gate || !w_up || !next_workspace) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null device pointer");
+  if (int rc = gemm_check(who, w_type, in_dim, out_dim, tokens, workspace, workspace_bytes)) return rc;
+  // the products are the activations of a matrix with rows of out_dim values
+  if ((out_dim % 256) != 0) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": out_dim must be a multiple of 256");
+  if (next_workspace_bytes < cogni_gemm_workspace_bytes(next_type, out_dim, tokens))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": next_workspace too small (cogni_gemm_workspace_bytes)");
+  const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 95) / 96;
+  void* params[] = {&w_gate, &w_up, &workspace, &out, &next_workspace, &in_dim, &out_dim, &tokens};
+  return launch(next_type == COGNI_TYPE_Q6_K ? "q4_k_gemm_swiglu_pack_q6k_f16" : "q4_k_gemm_swiglu_pack_q4k_f16", gemm_grid_x(mtiles, ntiles),
+                256, 0, params, stream);
 }
 
 int cogni_set_gemm_threshold(int32_t tokens) {

@@ -16,6 +16,9 @@
 //                   (w_gate, w_up, xp, out:f32 [m][out_dim], in_dim:u32, out_dim:u32, m:u32): out = silu(x W_gate^T) * (x W_up^T),
 //                   the reference's simd_mm_q4k_h16_b64_swiglu (gemm_q4k.metal:1233). A tile is 128 tokens x 96 rows of each
 //                   matrix; block 256, grid gemm_grid_x(ceil(m/128), ceil(out_dim/96)), no k split
+//   q4_k_gemm_swiglu_pack_q4k_f16, q4_k_gemm_swiglu_pack_q6k_f16
+//                   (w_gate, w_up, xp, out | null, xq, in_dim, out_dim, m): the same, and the products written as the packed
+//                   activations of the next GEMM (the down projection) as pack_x_f16_q4k | pack_x_f16_q6k would write them
 //   gemm_sum_splits_f32 (planes, bias|null, out, m*out_dim:u32, out_dim:u32, splits:u32, bias_stride:u32)   block 256, grid ceil(m*out_dim/1024)
 //
 // Tiling. A workgroup (4 wavefronts) owns 128 tokens x 192 weight rows, so 512 x 12288 gives 256
@@ -243,9 +246,14 @@ __device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[MT][NT], const fl
 // in the same lane layout. First the two k halves are added as above, each wavefront finishing its two token tiles in
 // place; then the up wavefronts hand their sums to the gate wavefronts (same kh) through LDS, which store
 // silu(gate) * up: 128 tokens x 96 outputs per workgroup, four consecutive floats per register quad.
-template <int KH>
+// PACK (12: the Q4_K / Q5_K order, 14: the Q6_K order): the products also leave as fp16 in the packed layout the GEMM
+// kernels read their activations from (what pack_x_f16_q4k | pack_x_f16_q6k would make of `out`, bit for bit), so that the
+// GEMM behind this one - the down projection - needs no pack launch and `out` may be null. A lane's four consecutive
+// products are one 8-byte half of a 16-byte cell of that layout, and the lane pair (kg = 0, 1) fills the cell: a wavefront
+// stores 512 contiguous bytes. out_dim is a multiple of 256 then (it is the row length of the next matrix).
+template <int KH, int PACK = 0>
 __device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3], float* out, u32 out_dim, u32 m, u32 mt, u32 nt,
-                                                          u32 nh, u32 j, u32 kg, u32 lane) {
+                                                          u32 nh, u32 j, u32 kg, u32 lane, uint2* xq = nullptr) {
   float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * 24 * 64 + lane;
   const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * 24 * 64 + lane;
 #pragma unroll
@@ -300,13 +308,37 @@ __device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3]
         const float4 o = make_float4(swiglu_one(t[4 * g4], u.x), swiglu_one(t[4 * g4 + 1], u.y), swiglu_one(t[4 * g4 + 2], u.z),
                                      swiglu_one(t[4 * g4 + 3], u.w));
         const u32 n = nt * (GEMM_BN / 2) + 32 * c + 8 * g4 + 4 * kg;
-        if (token < m && n < out_dim) {
+        if ((PACK == 0 || out) && token < m && n < out_dim) {
           float* dst = out + (size_t)token * out_dim + n;
           if (vec && n + 4 <= out_dim) {
             *reinterpret_cast<float4*>(dst) = o;
           } else {
             const float ov[4] = {o.x, o.y, o.z, o.w};
             for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e];
+          }
+        }
+        if constexpr (PACK != 0) {
+          // the eight consecutive rows n8 .. n8 + 7 of the lane pair are k values of the next GEMM: super-block n8 / 256,
+          // cell (k-step, k-group) by the inverse of gemm_k_element | gemm_k_element_q6k (as in pack_x_core), all
+          // uniform over the wavefront; the absent tokens of the last tile are zeros, as the pack kernel writes them
+          const u32 n8 = nt * (GEMM_BN / 2) + 32 * c + 8 * g4;
+          if (n8 < out_dim) {
+            const u32 kb = n8 >> 8, k = n8 & 255u;
+            u32 ks, kgr;
+            if (PACK == 14) {
+              ks = 8 * (k >> 7) + 2 * ((k >> 5) & 3) + ((k >> 3) & 1);
+              kgr = (k >> 4) & 1;
+            } else {
+              const u32 g = k >> 6;
+              ks = 8 * (g >> 1) + 4 * ((k >> 4) & 1) + 2 * ((k >> 5) & 1) + ((k >> 3) & 1);
+              kgr = g & 1;
+            }
+            const float4 z = token < m ? o : make_float4(0.f, 0.f, 0.f, 0.f);
+            const __half2 p0 = __floats2half2_rn(z.x, z.z), p1 = __floats2half2_rn(z.y, z.w);   // slot order 0,2,1,3
+            uint2 q;
+            q.x = *reinterpret_cast<const u32*>(&p0);
+            q.y = *reinterpret_cast<const u32*>(&p1);
+            xq[(((size_t)mt * (out_dim >> 8) + kb) * 4096 + (ks * 2 + kgr) * 128 + 32 * (2 * KH + rr) + j) * 2 + kg] = q;
           }
         }
       }
@@ -331,9 +363,12 @@ struct GemmRawT<true> {   // Q5_K: plus the 32 bytes of fifth bits (bit 2g + hi 
 // 192-row tiles, times the k split, leave compute units idle: q4_k_gemm_n128_f16, q5_k_gemm_n128_f16).
 // MT: tiles of 32 tokens - 4 (128 tokens) or 2: launches of up to 64 tokens, where the upper half of a 128-token tile would
 // be MFMAs on padding and copies of nothing (<type>_gemm_m64[_n128]_f16; the packed x is the same, its first 64 tokens are used).
-template <bool Q5, bool SWIGLU = false, int NT = 3, int MT = 4>
+// PACK (SWIGLU only): the epilogue also writes the products as the packed fp16 activations of the next GEMM, to `xq`.
+template <bool Q5, bool SWIGLU = false, int NT = 3, int MT = 4, int PACK = 0>
 __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim,
-                                              u32 out_dim, u32 m, u32 bias_stride = 0, const uint8_t* w_b = nullptr) {
+                                              u32 out_dim, u32 m, u32 bias_stride = 0, const uint8_t* w_b = nullptr,
+                                              uint4* xq = nullptr) {
+  static_assert(PACK == 0 || SWIGLU, "only the gate | up kernel writes packed activations");
   static_assert(!(Q5 && SWIGLU), "the gate | up kernel is built for Q4_K");
   static_assert(NT == 3 || (NT == 2 && !SWIGLU), "tile heights");
   static_assert(MT == 4 || (MT == 2 && !SWIGLU), "tokens per tile");
@@ -630,8 +665,8 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
   if constexpr (SWIGLU) {
-    if (kh == 0) gemm_epilogue_swiglu_half<0>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
-    else gemm_epilogue_swiglu_half<1>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane);
+    if (kh == 0) gemm_epilogue_swiglu_half<0, PACK>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane, reinterpret_cast<uint2*>(xq));
+    else gemm_epilogue_swiglu_half<1, PACK>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane, reinterpret_cast<uint2*>(xq));
   } else {
     gemm_epilogue<NT, MT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
   }
@@ -669,6 +704,17 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_f16(
     const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, u32 in_dim, u32 out_dim, u32 m) {
   gemm_k45_core<false, true>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up);
+}
+// The same with silu(gate) * up also (out null: only) written as the packed fp16 activations of the GEMM that follows, in
+// the order of its weight type - q4k: Q4_K and Q5_K, q6k: Q6_K; (w_gate, w_up, xp, out | null, xq, in_dim, out_dim, m),
+// out_dim a multiple of 256, xq as large as pack_x_f16_* needs for [m][out_dim].
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_pack_q4k_f16(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, uint4* xq, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<false, true, 3, 4, 12>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up, xq);
+}
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_pack_q6k_f16(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, uint4* xq, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<false, true, 3, 4, 14>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up, xq);
 }
 
 // Sum of the k-split planes: out[i] = (bias ? bias[bias_stride ? i : i % out_dim] : 0) + partials[0][i] + partials[1][i] + ... in that order

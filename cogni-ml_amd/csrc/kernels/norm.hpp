@@ -7,6 +7,10 @@
 // that the projections behind a norm (q | k | v, gate | up) need no pack launch of their own: a thread of the short-row
 // path holds elements 4 (tid % 64) .. + 3 of super-block 4 k + tid / 64, which is exactly one wavefront per (token,
 // super-block) with the lane order of pack_x_mt_*, and the image comes out bit for bit as from that kernel.
+// The gemm-pack forms write the normalised rows as the packed fp16 activations of the prefill GEMMs instead (the block
+// pack_x_f16_q4k | pack_x_f16_q6k makes of them, bit for bit): the same thread holds the four consecutive values that are
+// one 8-byte half of a 16-byte cell of that layout. Eight consecutive tokens share a 128-byte line of it, so the workgroups
+// of such a run are numbered onto one XCD (workgroups go to the eight XCDs round-robin) and its L2 sees the whole line.
 #pragma once
 #include "common.hpp"
 #include "gemv_mt.hpp"
@@ -17,12 +21,47 @@
 // IMG: 0 = no image, 12 = the Q4_K (and Q5_K) image, 14 = the Q6_K image. With an image the grid is the image's eight token
 // slots, the workgroups of slots at and above `tokens` write the zeros of an absent token, dim is a multiple of 256 up to
 // 4096 (the short-row path), and `out` may be null (the normalised rows then exist only as the image).
-template <bool ADD, int IMG = 0>
+// GP: 0, or the packed GEMM activations in the Q4_K / Q5_K order (12) or the Q6_K order (14) behind `image`: the grid is the
+// token count rounded up to whole tiles of 128, the workgroups of absent tokens write the zeros of the last tile, dim is a
+// multiple of 256 up to 4096, `out` may be null.
+template <int GP>
+__device__ __forceinline__ void gemm_pack_store(uint8_t* xq, u32 nkb, u32 tok, u32 kb, u32 lane, float4 o) {
+  // the lane's values are k0 .. k0 + 3 of super-block kb; their cell by the inverse of gemm_k_element | gemm_k_element_q6k
+  // (gemm_q4k.hpp, gemm_q6k.hpp), as in pack_x_core
+  const u32 k0 = 4 * lane;
+  u32 ks, kg;
+  if (GP == 14) {
+    ks = 8 * (k0 >> 7) + 2 * ((k0 >> 5) & 3) + ((k0 >> 3) & 1);
+    kg = (k0 >> 4) & 1;
+  } else {
+    const u32 g = k0 >> 6;
+    ks = 8 * (g >> 1) + 4 * ((k0 >> 4) & 1) + 2 * ((k0 >> 5) & 1) + ((k0 >> 3) & 1);
+    kg = g & 1;
+  }
+  const __half2 p0 = __floats2half2_rn(o.x, o.z), p1 = __floats2half2_rn(o.y, o.w);   // slot order 0,2,1,3
+  uint2 q;
+  q.x = *reinterpret_cast<const u32*>(&p0);
+  q.y = *reinterpret_cast<const u32*>(&p1);
+  reinterpret_cast<uint2*>(xq)[((((size_t)(tok >> 7) * nkb + kb) * 4096) + (ks * 2 + kg) * 128 + (tok & 127u)) * 2 + (lane & 1u)] = q;
+}
+
+template <bool ADD, int IMG = 0, int GP = 0>
 __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __restrict__ add,
                                              const float* __restrict__ norm, float* residual_out,
                                              float* __restrict__ out, u32 dim, float eps, uint8_t* __restrict__ image = nullptr,
                                              u32 tokens = 0) {
+  static_assert(IMG == 0 || GP == 0, "one image per launch");
   __shared__ float part[NORM_BLOCK / WAVE];
+  // the row of this workgroup; with the packed GEMM activations, workgroups b, b + 8, .., b + 56 (one XCD) take tokens
+  // 8 b .. 8 b + 7 of every run of 64
+  const u32 row = GP ? 64u * (blockIdx.x >> 6) + 8u * (blockIdx.x & 7u) + ((blockIdx.x >> 3) & 7u) : blockIdx.x;
+  if constexpr (GP != 0) {
+    if (row >= tokens) {
+      for (u32 i = threadIdx.x * 4; i < dim; i += NORM_BLOCK * 4)
+        gemm_pack_store<GP>(image, dim >> 8, row, i >> 8, threadIdx.x & 63, make_float4(0.f, 0.f, 0.f, 0.f));
+      return;
+    }
+  }
   // this token slot's share of the image from super-block `from` on: zeros (an absent token; the super-blocks past the
   // row's end that fill the image up to a multiple of 8)
   [[maybe_unused]] auto zero_image = [&](u32 from) {
@@ -40,7 +79,7 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
       return;
     }
   }
-  const u64 base = (u64)blockIdx.x * dim;
+  const u64 base = (u64)row * dim;
   const float* xt = x + base;
   const float* at = ADD ? add + base : nullptr;
   float* rt = ADD ? residual_out + base : nullptr;
@@ -82,7 +121,8 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
       if (i < dim) {
         float4 o;
         o.x = (v[k].x * inv) * w[k].x, o.y = (v[k].y * inv) * w[k].y, o.z = (v[k].z * inv) * w[k].z, o.w = (v[k].w * inv) * w[k].w;
-        if (IMG == 0 || out) *reinterpret_cast<float4*>(ot + i) = o;
+        if ((IMG == 0 && GP == 0) || out) *reinterpret_cast<float4*>(ot + i) = o;
+        if constexpr (GP != 0) gemm_pack_store<GP>(image, dim >> 8, row, 4u * (u32)k + (tid >> 6), tid & 63, o);
         if constexpr (IMG != 0) {
           // (i < dim holds for whole wavefronts: dim is a multiple of 256)
           const u32 sb = 4u * (u32)k + (tid >> 6);
@@ -95,7 +135,8 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
     return;
   }
   static_assert(IMG == 0 || IMG == 12 || IMG == 14, "image kinds");
-  if constexpr (IMG != 0) return;   // (the host launches the pack forms for the short-row shapes only)
+  static_assert(GP == 0 || GP == 12 || GP == 14, "packed layouts");
+  if constexpr (IMG != 0 || GP != 0) return;   // (the host launches the pack forms for the short-row shapes only)
   if (vec) {
     for (u32 i = tid * 4; i < dim; i += NORM_BLOCK * 4) {
       float4 v = *reinterpret_cast<const float4*>(xt + i);
@@ -170,3 +211,21 @@ extern "C" __global__ __launch_bounds__(NORM_BLOCK) void add_rmsnorm_f32(const f
   }
 NORM_PACK_ENTRIES(q4k, 12)
 NORM_PACK_ENTRIES(q6k, 14)
+
+// The same with the normalised rows written as the packed fp16 activations of the prefill GEMMs:
+//   rmsnorm_gemm_pack_q4k_f32 | rmsnorm_gemm_pack_q6k_f32 (x, norm, out | null, xp, dim, tokens, eps)
+//   add_rmsnorm_gemm_pack_q4k_f32 | add_rmsnorm_gemm_pack_q6k_f32 (x, add, norm, residual_out, normed_out | null, xp, dim, tokens, eps)
+// grid.x = 128 * ceil(tokens / 128), block 256, dim a multiple of 256 up to 4096. xp is what pack_x_f16_q4k | pack_x_f16_q6k
+// writes from the normalised rows, bit for bit.
+#define NORM_GEMM_PACK_ENTRIES(SFX, GP)                                                                                      \
+  extern "C" __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_gemm_pack_##SFX##_f32(                                    \
+      const float* x, const float* norm, float* out, uint8_t* xp, u32 dim, u32 tokens, float eps) {                          \
+    rmsnorm_core<false, 0, GP>(x, nullptr, norm, nullptr, out, dim, eps, xp, tokens);                                        \
+  }                                                                                                                          \
+  extern "C" __global__ __launch_bounds__(NORM_BLOCK) void add_rmsnorm_gemm_pack_##SFX##_f32(                                \
+      const float* x, const float* add, const float* norm, float* residual_out, float* normed_out, uint8_t* xp, u32 dim,     \
+      u32 tokens, float eps) {                                                                                               \
+    rmsnorm_core<true, 0, GP>(x, add, norm, residual_out, normed_out, dim, eps, xp, tokens);                                 \
+  }
+NORM_GEMM_PACK_ENTRIES(q4k, 12)
+NORM_GEMM_PACK_ENTRIES(q6k, 14)

@@ -271,6 +271,18 @@ int cogni_rmsnorm_pack_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t w_t
                            float eps, void* stream);
 int cogni_add_rmsnorm_pack_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t w_type,
                                uint64_t image, uint32_t dim, uint32_t tokens, float eps, void* stream);
+/* The norms in front of the prefill GEMMs (src/ml/gguf/qwen35_cpu.cr:1705-1722: the rms_norm that feeds the
+ * qmatmul_nobias calls of a prefill layer): the normalised rows leave as the packed fp16 activations cogni_gemm_pack_dev
+ * would make of them, bit for bit, in the layout of `w_type` (Q4_K and Q5_K share one, Q6_K has its own), so that
+ * cogni_gemm_packed_dev and its siblings follow with no pack launch. `out` / `normed_out` may be 0 (the normalised rows then
+ * exist only packed). dim a multiple of 256 up to 4096; workspace_bytes >= cogni_gemm_workspace_bytes(w_type, dim, tokens).
+ * Kernels "rmsnorm_gemm_pack_q4k_f32" | "rmsnorm_gemm_pack_q6k_f32" (x, norm, out, workspace, dim:u32, tokens:u32, eps:f32)
+ * and "add_rmsnorm_gemm_pack_q4k_f32" | "add_rmsnorm_gemm_pack_q6k_f32" (x, add, norm, residual_out, normed_out, workspace,
+ * dim:u32, tokens:u32, eps:f32), block 256, grid 128 * ceil(tokens / 128). */
+int cogni_rmsnorm_gemm_pack_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t w_type, uint64_t workspace, size_t workspace_bytes,
+                                uint32_t dim, uint32_t tokens, float eps, void* stream);
+int cogni_add_rmsnorm_gemm_pack_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t w_type,
+                                    uint64_t workspace, size_t workspace_bytes, uint32_t dim, uint32_t tokens, float eps, void* stream);
 
 /* One row of a Q4_K or Q6_K embedding matrix chosen by a token id that lives on the device: output[0..hidden_dim) =
  * dequantized row token_ids[0] (zeros if the id is not below vocab_size) and history[token_index] = token_ids[0].
@@ -387,6 +399,18 @@ int cogni_gemm_packed_add_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspac
                               uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
                                  uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
+/* cogni_gemm_packed_swiglu_dev that also hands its products on as the packed activations of the GEMM behind it - the down
+ * projection of the same feed-forward block (qwen35_cpu.cr:1711-1722: `act` goes nowhere else): the epilogue writes
+ * silu(g) * u as fp16 into `next_workspace` in the layout cogni_gemm_pack_dev gives a [tokens][out_dim] input of a matrix of
+ * `next_type` (Q4_K, Q5_K or Q6_K), bit for bit what that call would write from `out`, so cogni_gemm_packed_dev /
+ * cogni_gemm_packed_add_dev can follow with in_dim = out_dim and no pack launch. `out` may be 0: the fp32 products are then
+ * not stored at all. out_dim a multiple of 256; next_workspace_bytes >= cogni_gemm_workspace_bytes(next_type, out_dim,
+ * tokens) (with the k-split planes behind it if the next GEMM is to split: cogni_gemm_workspace_bytes_split); the two
+ * workspaces must not overlap. Kernels q4_k_gemm_swiglu_pack_q4k_f16 | q4_k_gemm_swiglu_pack_q6k_f16 (w_gate, w_up,
+ * workspace, out | 0, next_workspace, in_dim, out_dim, tokens), launched as q4_k_gemm_swiglu_f16. */
+int cogni_gemm_packed_swiglu_pack_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
+                                      uint32_t next_type, uint64_t next_workspace, size_t next_workspace_bytes, uint32_t in_dim,
+                                      uint32_t out_dim, uint32_t tokens, void* stream);
 /* The launch cogni_gemm_packed_dev makes for a shape and a workspace of `workspace_bytes`: kernel name, grid (x: tiles,
  * y: k splits; with y > 1 gemm_sum_splits_f32 follows) and block, for hosts that launch by name (level 1) and for
  * callers who want to know which of the two Q4_K tilings a shape gets. Any out pointer may be null. The counterpart of

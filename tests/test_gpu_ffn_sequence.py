@@ -124,6 +124,17 @@ def test_prefill_form_of_the_ffn_block(gpu, oracle, hidden, ffn_dim, tokens, blo
             assert np.max(np.abs(got - want)) <= 4e-3 * np.max(np.abs(want)), tok
         a, b = runner.out[:8 * hidden], small.out
         assert np.max(np.abs(a - b)) <= 4e-3 * np.max(np.abs(b))
+        # without the fp32 products stored (they leave the gate | up GEMM as the down GEMM's packed input only): same bits
+        lean = FFNSequenceRunner(gate_raw, up_raw, down_raw, hidden, ffn_dim, tokens, xs, keep_combined=False, **kw)
+        try:
+            lean.upload_weights()
+            lean.reset_sequence()
+            lean.run_sequence()
+            lean.read_outputs()
+            assert lean.combined is None and runner.combined is not None
+            assert np.array_equal(lean.out, runner.out)
+        finally:
+            lean.close()
     finally:
         runner.close()
         small.close()

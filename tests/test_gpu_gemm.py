@@ -247,6 +247,44 @@ def test_gate_up_swiglu_in_one_gemm(gpu, oracle, tokens, out_dim, in_dim):
         a.close()
 
 
+@pytest.mark.parametrize("next_type", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("tokens,out_dim,in_dim", [(130, 256, 512), (9, 768, 256), (64, 1024, 768), (300, 2560, 512), (512, 12288, 4096)])
+def test_gate_up_swiglu_hands_on_packed_activations(gpu, tokens, out_dim, in_dim, next_type):
+    """cogni_gemm_packed_swiglu_pack_dev: the products of the gate | up GEMM written by its epilogue as the packed fp16
+    activations of the next GEMM - every byte of what cogni_gemm_pack_dev writes from the fp32 products, for the three weight
+    types' layouts, last token tiles that are not full (zeros for the absent tokens), a row count that is not a multiple of
+    the 96-row tile (1024, 2560: the last tile is clipped), with and without the fp32 products stored as well."""
+    rng = np.random.default_rng(tokens * 11 + out_dim + int(next_type))
+    raw_g = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    raw_u = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    n = tokens * out_dim
+    wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens)
+    nxb = quant.gemm_workspace_bytes(next_type, out_dim, tokens)
+    wg, wu, xd, ws = DevArray(raw_g), DevArray(raw_u), DevArray(x), DevArray(nbytes=wsb)
+    # the buffers the fused launch writes start as 0xFF bytes: every byte of the packed block has to be written by it
+    ff = np.full(nxb, 0xFF, dtype=np.uint8)
+    of, o2 = DevArray(nbytes=4 * n), DevArray(np.full(n, np.float32(-7.0)))
+    p_ref, p_a, p_b = DevArray(nbytes=nxb), DevArray(ff), DevArray(ff)
+    quant.gemm_pack_dev(xd.ptr, Q4_K, in_dim, tokens, ws.ptr, wsb)
+    quant.gemm_packed_swiglu_dev(wg.ptr, wu.ptr, Q4_K, ws.ptr, wsb, of.ptr, in_dim, out_dim, tokens)
+    quant.gemm_pack_dev(of.ptr, next_type, out_dim, tokens, p_ref.ptr, nxb)
+    quant.gemm_packed_swiglu_pack_dev(wg.ptr, wu.ptr, Q4_K, ws.ptr, wsb, o2.ptr, next_type, p_a.ptr, nxb, in_dim, out_dim, tokens)
+    quant.gemm_packed_swiglu_pack_dev(wg.ptr, wu.ptr, Q4_K, ws.ptr, wsb, 0, next_type, p_b.ptr, nxb, in_dim, out_dim, tokens)
+    want = p_ref.read(np.uint8, nxb)
+    assert np.array_equal(p_a.read(np.uint8, nxb), want)
+    assert np.array_equal(p_b.read(np.uint8, nxb), want)
+    assert np.array_equal(o2.read(np.float32, n), of.read(np.float32, n))
+    with pytest.raises(quant.QuantError, match="out_dim must be a multiple of 256"):
+        quant.gemm_packed_swiglu_pack_dev(wg.ptr, wu.ptr, Q4_K, ws.ptr, wsb, 0, next_type, p_b.ptr, nxb, in_dim, out_dim - 64, tokens)
+    with pytest.raises(quant.QuantError, match="next_workspace too small"):
+        quant.gemm_packed_swiglu_pack_dev(wg.ptr, wu.ptr, Q4_K, ws.ptr, wsb, 0, next_type, p_b.ptr, nxb - 1, in_dim, out_dim, tokens)
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for the prefill GEMM"):
+        quant.gemm_packed_swiglu_pack_dev(wg.ptr, wu.ptr, Q4_K, ws.ptr, wsb, 0, Q8_0, p_b.ptr, nxb, in_dim, out_dim, tokens)
+    for a in (wg, wu, xd, ws, of, o2, p_ref, p_a, p_b):
+        a.close()
+
+
 def test_projections_share_one_packed_activation_block(gpu, oracle):
     """gemm_pack_dev once, then gemm_packed_dev for several matrices of one type family (Q4_K and Q5_K read the same packed
     layout; a k-split and an unsplit shape, with and without bias): the bits of gemm_dev on each matrix alone."""

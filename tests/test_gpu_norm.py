@@ -114,3 +114,62 @@ def test_norm_pack_argument_errors(gpu):
     with pytest.raises(quant.QuantError, match="null device pointer"):
         quant.add_rmsnorm_pack_dev(p, p, p, 0, p, 12, p, 4096, 4)
     buf.close()
+
+
+@pytest.mark.parametrize("w_type", [12, 13, 14])
+@pytest.mark.parametrize("dim,tokens", [(4096, 512), (4096, 9), (2048, 130), (1024, 64), (2560, 200), (256, 129), (3584, 65)])
+def test_norms_that_write_the_packed_gemm_activations(gpu, w_type, dim, tokens):
+    """cogni_rmsnorm_gemm_pack_dev / cogni_add_rmsnorm_gemm_pack_dev: every byte of the block cogni_gemm_pack_dev writes from
+    the plain norm's output (the layouts of the three GEMM weight types; last token tiles that are not full carry zeros for
+    the absent tokens), the residual stream and, when asked for, the normalised rows bit for bit the plain kernels'."""
+    rng = np.random.default_rng(dim + 13 * tokens + w_type)
+    x = (rng.standard_normal(tokens * dim) * 2.5).astype(np.float32)
+    add = rng.standard_normal(tokens * dim).astype(np.float32)
+    w = (1.0 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    eps = 1.0e-6
+    nbytes = quant.gemm_workspace_bytes(w_type, dim, tokens)
+    ff = np.full(nbytes, 0xFF, dtype=np.uint8)     # every byte of the packed block has to be written by the norm
+    xd, ad, wd = DevArray(x), DevArray(add), DevArray(w)
+    od, rd, nd, od2, rd2, nd2 = (DevArray(nbytes=x.nbytes) for _ in range(6))
+    p_ref, p_a, p_b, p_c = DevArray(nbytes=nbytes), DevArray(ff), DevArray(ff), DevArray(ff)
+    try:
+        quant.rmsnorm_dev(xd.ptr, wd.ptr, od.ptr, dim, tokens, eps)
+        quant.gemm_pack_dev(od.ptr, w_type, dim, tokens, p_ref.ptr, nbytes)
+        want = p_ref.read(np.uint8, nbytes)
+        quant.rmsnorm_gemm_pack_dev(xd.ptr, wd.ptr, od2.ptr, w_type, p_a.ptr, nbytes, dim, tokens, eps)
+        assert np.array_equal(p_a.read(np.uint8, nbytes), want)
+        assert np.array_equal(od2.read(np.float32, x.size), od.read(np.float32, x.size))
+        quant.rmsnorm_gemm_pack_dev(xd.ptr, wd.ptr, 0, w_type, p_b.ptr, nbytes, dim, tokens, eps)
+        assert np.array_equal(p_b.read(np.uint8, nbytes), want)
+
+        quant.add_rmsnorm_dev(xd.ptr, ad.ptr, wd.ptr, rd.ptr, nd.ptr, dim, tokens, eps)
+        quant.gemm_pack_dev(nd.ptr, w_type, dim, tokens, p_ref.ptr, nbytes)
+        want = p_ref.read(np.uint8, nbytes)
+        quant.add_rmsnorm_gemm_pack_dev(xd.ptr, ad.ptr, wd.ptr, rd2.ptr, nd2.ptr, w_type, p_c.ptr, nbytes, dim, tokens, eps)
+        assert np.array_equal(p_c.read(np.uint8, nbytes), want)
+        assert np.array_equal(rd2.read(np.float32, x.size), rd.read(np.float32, x.size))
+        assert np.array_equal(nd2.read(np.float32, x.size), nd.read(np.float32, x.size))
+        # the residual stream written in place (residual_out = x), no normalised rows
+        quant.add_rmsnorm_gemm_pack_dev(xd.ptr, ad.ptr, wd.ptr, xd.ptr, 0, w_type, p_a.ptr, nbytes, dim, tokens, eps)
+        assert np.array_equal(p_a.read(np.uint8, nbytes), want)
+        assert np.array_equal(xd.read(np.float32, x.size), rd.read(np.float32, x.size))
+    finally:
+        for d in (xd, ad, wd, od, rd, nd, od2, rd2, nd2, p_ref, p_a, p_b, p_c):
+            d.close()
+
+
+def test_norm_gemm_pack_argument_errors(gpu):
+    # (real device memory behind every pointer, as above)
+    buf = DevArray(nbytes=8 << 20)
+    p, n = buf.ptr, 8 << 20
+    with pytest.raises(quant.QuantError, match="dim must be a multiple of 256 up to 4096"):
+        quant.rmsnorm_gemm_pack_dev(p, p, p, 12, p, n, 1000, 16)
+    with pytest.raises(quant.QuantError, match="dim must be a multiple of 256 up to 4096"):
+        quant.add_rmsnorm_gemm_pack_dev(p, p, p, p, p, 14, p, n, 6144, 16)
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for the prefill GEMM: Q8_0"):
+        quant.rmsnorm_gemm_pack_dev(p, p, p, 8, p, n, 1024, 16)
+    with pytest.raises(quant.QuantError, match="workspace has 1000 bytes"):
+        quant.rmsnorm_gemm_pack_dev(p, p, p, 12, p, 1000, 1024, 16)
+    with pytest.raises(quant.QuantError, match="null device pointer"):
+        quant.add_rmsnorm_gemm_pack_dev(p, p, p, 0, p, 12, p, n, 1024, 16)
+    buf.close()
