@@ -245,10 +245,11 @@ def gemv_record(r, bytes_per_step):
             "samples": r["samples"], "timed_region_ms": round(r["timed_region_ms"], 2)}
 
 
-def bench_gemm(hip, quant, synth, rng, stream, w_type, tokens, out_dim, in_dim, steps, warmup, graph=True):
+def bench_gemm(hip, quant, synth, rng, stream, w_type, tokens, out_dim, in_dim, steps, warmup, graph=True, packed=False):
     """Prefill GEMM (x repack + MFMA kernel, every launch of the call) at `tokens`; returns the case record. Consecutive
     steps read different copies of the weights, as the GEMV cases do, so that a step's weights come from HBM and not from
-    the last-level cache the previous step left them in."""
+    the last-level cache the previous step left them in. packed: the activations are packed once, outside the timed
+    region - the GEMM as it runs behind a producer that writes them packed (cogni_rmsnorm_gemm_pack_dev, the SwiGLU GEMM)."""
     raw = synth.make_weights(rng, w_type, out_dim, in_dim)
     x = synth.make_activations(rng, tokens, in_dim)
     wsb = quant.gemm_workspace_bytes(w_type, in_dim, tokens, out_dim)
@@ -261,9 +262,16 @@ def bench_gemm(hip, quant, synth, rng, stream, w_type, tokens, out_dim, in_dim, 
     bufs = [hip.DeviceBuffer(n) for n in (x.nbytes, 4 * tokens * out_dim, wsb)]
     hip.copy_htod(bufs[0].ptr, x, x.nbytes, "x")
 
+    if packed:
+        quant.gemm_pack_dev(bufs[0].ptr, w_type, in_dim, tokens, bufs[2].ptr, wsb, stream.handle)
+        stream.synchronize()
+
     def launch(copy, st):
-        quant.gemm_dev(wbufs[copy].ptr, w_type, bufs[0].ptr, bufs[1].ptr, in_dim, out_dim, tokens, bufs[2].ptr, wsb, 0,
-                       st.handle)
+        if packed:
+            quant.gemm_packed_dev(wbufs[copy].ptr, w_type, bufs[2].ptr, wsb, bufs[1].ptr, in_dim, out_dim, tokens, 0, st.handle)
+        else:
+            quant.gemm_dev(wbufs[copy].ptr, w_type, bufs[0].ptr, bufs[1].ptr, in_dim, out_dim, tokens, bufs[2].ptr, wsb, 0,
+                           st.handle)
     r = measure(hip, stream, Rotating(launch, copies, raw.nbytes), steps, warmup, graph)
     kernel, grid_x, splits, block = quant.gemm_plan(w_type, in_dim, out_dim, tokens, wsb)
     for b in bufs + wbufs:
@@ -274,7 +282,8 @@ def bench_gemm(hip, quant, synth, rng, stream, w_type, tokens, out_dim, in_dim, 
             "tflops": round(tf, 1), "frac_mfma_f16": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
             "samples": r["samples"], "timed_region_ms": round(r["timed_region_ms"], 2),
             "kernel": kernel, "grid": [grid_x, splits], "block": block, "weight_copies_rotated": r["buffers_rotated"],
-            "includes": "activation repack + GEMM (+ plane sum where the k range is split)"}
+            "includes": ("GEMM against activations packed by their producer" if packed else "activation repack + GEMM") +
+                        " (+ plane sum where the k range is split)"}
 
 
 def raw_gemm_bytes(tokens, out_dim, in_dim):
@@ -567,6 +576,12 @@ def main():
         cases["cfg4 q4_k gemm 12288x4096 M=%d" % tokens] = rec
         log("case=q4_k_gemm prefill\ntype=Q4_K\nshape=4096x12288\ntokens=%d\nreps=%d\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
             tokens, gsteps, rec["us"], rec["tflops"], rec["frac_mfma_f16"]))
+    # the same GEMM behind a producer that hands it packed activations (the norm, the SwiGLU GEMM): no pack launch in the step
+    rec = bench_gemm(hip, quant, synth, rng, stream, Q4_K, 512, 12288, 4096, max(5, min(100, args.steps)), min(5, args.warmup), packed=True)
+    rec["traffic"] = traffic_field(rec["kernel"], raw_gemm_bytes(512, 12288, 4096))
+    cases["cfg4 q4_k gemm 12288x4096 M=512, activations packed by the producer (no pack launch)"] = rec
+    log("case=q4_k_gemm prefill, packed activations\ntokens=512\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
+        rec["us"], rec["tflops"], rec["frac_mfma_f16"]))
     # the feed-forward block of a layer at M = 512 in its prefill form: add + RMSNorm, pack, gate | up GEMM with SwiGLU inside
     # (its epilogue writes the down GEMM's packed input), Q6_K down GEMM with the residual inside (three rotating sets of
     # weights: 290 MB)

@@ -17,7 +17,9 @@
 // k-step 6 and picked up during k-step 7) and the 18 bytes of scales and d (gemm_wsc6, one row per thread); qh is read
 // from global memory straight into the registers of the lane that decodes it, also one super-block ahead. Rows are only 2-byte aligned, and a 16-byte load
 // from an odd multiple of 2 costs about twice an aligned one; the one-row-per-lane loads cost more again because a
-// wavefront instruction touches 32 rows. k-step t of the wavefront is quadrant
+// wavefront instruction touches 32 rows. The raw blocks of the 128-row tile (q6_k_gemm_n128_f16, q6_k_gemm_m64_n128_f16) do
+// fit, and there they are copied whole, global -> LDS, without passing through registers (template parameter DMA below).
+// k-step t of the wavefront is quadrant
 // t / 2, bytes 8 (t % 2) .. +8 of the pieces: 8 values with one scale. A code is put together in the low bits of a
 // half, (ql nibble) | (qh bits << 4) | 0x6400 = 1024 + q as binary16; subtracting 1056 gives q - 32 exactly and one
 // packed multiply gives fp16((q - 32) * (d * sc)). The 8 values come in byte order 0,2,1,3,4,6,5,7;
@@ -58,11 +60,18 @@ __shared__ u32 gemm_wsc6[GEMM_BN * 6];
 // work per workgroup for shapes whose 192-row tiles, times the k split, leave compute units idle - 4096 rows at 512 tokens
 // are 88 tiles x 2 splits = 176 workgroups, but 128 x 2 = 256 of the smaller ones).
 // MT: tiles of 32 tokens, 4 or 2 (launches of up to 64 tokens: q6_k_gemm_m64[_n128]_f16), as in gemm_k45_core.
-template <int NT, int MT = 4>
+// DMA (NT = 2 only): the whole 210-byte blocks of the 128 rows go global -> LDS without passing through registers, as the
+// Q4_K kernel's do (global_load_lds_dwordx4 from the blocks' 2-byte-aligned addresses): a row is 15 pieces of 16 bytes in
+// gemm_wbuf5 - bytes [16 p, 16 p + 16) for p < 13 (ql, qh, scales), bytes [194, 210) as piece 13 (d is its last two bytes)
+// and a 15th that repeats piece 12, there so that a row is 60 dwords and the 16-byte reads of 16 consecutive rows fall on
+// different banks. 1920 pieces = 30 copies of 64; every wavefront issues 8 (the last two repeat the tile's last piece into
+// spare LDS), which with the two x buffers is all of the 160 KiB. With three row tiles (2880 pieces) this does not fit.
+template <int NT, int MT = 4, bool DMA = false>
 __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim,
                                               u32 m, u32 bias_stride) {
+  static_assert(!DMA || NT == 2, "the raw blocks of 128 rows are what fits beside the x buffers");
   constexpr int NX = 4 * MT;   // copies of x per thread and super-block
-  constexpr u32 BN = 64 * NT, NSTG = 2 * NT;   // rows of the workgroup tile; 16-byte pieces of ql a thread stages per super-block
+  constexpr u32 BN = 64 * NT, NSTG = DMA ? 8 : 2 * NT;   // rows of the workgroup tile; 16-byte pieces a thread stages (DMA: copies) per super-block
   const u32 tid = threadIdx.x, lane = tid & 63;
   const u32 wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const u32 nh = wave & 1, kh = wave >> 1;
@@ -102,10 +111,32 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
   u32 soff[NSTG], sdst[NSTG];
 #pragma unroll
   for (int i = 0; i < (int)NSTG; i++) {
-    const u32 p = (4u * i + wave) * 64u + lane, r = p >> 3, part = p & 7u;
-    soff[i] = (min(nt * BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part;
-    sdst[i] = r * 9u + part;
+    if constexpr (DMA) {
+      const u32 p = min((4u * i + wave) * 64u + lane, BN * 15u - 1u), r = p / 15u, part = p - 15u * r;
+      soff[i] = (min(nt * BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + (part < 13u ? 16u * part : (part == 13u ? 194u : 192u));
+      sdst[i] = (4u * i + wave) * 64u;   // (the copy's LDS address is uniform: lane l lands 16 l bytes further)
+    } else {
+      const u32 p = (4u * i + wave) * 64u + lane, r = p >> 3, part = p & 7u;
+      soff[i] = (min(nt * BN + r, out_dim - 1) - tile_row0) * (u32)row_bytes + 16u * part;
+      sdst[i] = r * 9u + part;
+    }
   }
+  // DMA: piece 0 of the lane's row c = 0 in gemm_wbuf5 (row c is 32 * 15 pieces further)
+  const u32 dbase = (nh * (32 * NT) + j) * 15;
+  auto copy_w = [&](const uint8_t* kbase, int i) {
+    __builtin_amdgcn_global_load_lds((gbl_void*)(kbase + soff[i]), (lds_void*)(gemm_wbuf5 + sdst[i]), 16, 0, 0);
+  };
+  auto take_raw = [&](GemmRaw6 (&raw)[NT]) {
+#pragma unroll
+    for (int c = 0; c < NT; c++) {
+      const u32 b = dbase + 480 * c;
+      raw[c].qa = gemm_wbuf5[b + 4 * kh + kg];
+      raw[c].qb = gemm_wbuf5[b + 4 * kh + 2 + kg];
+      raw[c].qh = gemm_wbuf5[b + 8 + 2 * kh + kg];
+      raw[c].sc = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(gemm_wbuf5 + b + 12) + 8 * kh);
+      raw[c].d = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(gemm_wbuf5 + b + 13) + 14);
+    }
+  };
   const u32 take0 = (nh * (32 * NT) + j) * 9 + 4 * kh + kg;   // the lane's first ql piece of its row c = 0; the second is 2 further
   const u32 srow = (min(nt * BN + min(tid, BN - 1), out_dim - 1) - tile_row0) * (u32)row_bytes + 192u;
   const u32 tsc = (nh * (32 * NT) + j) * 6;                   // the lane's row c = 0 in gemm_wsc6
@@ -153,23 +184,36 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
   // out of buffer 1 / registers B.
   const bool odd = nkb & 1;
   GemmRaw6 rawA[NT], rawB[NT];
+  if constexpr (DMA) {
 #pragma unroll
-  for (int i = 0; i < (int)NSTG; i++) stage_load(tbase, i);
-  stage_load_sc(tbase);
+    for (int i = 0; i < (int)NSTG; i++) copy_w(tbase, i);
+  } else {
+#pragma unroll
+    for (int i = 0; i < (int)NSTG; i++) stage_load(tbase, i);
+    stage_load_sc(tbase);
+  }
   if (odd) {
+    if constexpr (!DMA) {
 #pragma unroll
-    for (int c = 0; c < NT; c++) load_row(rawB[c], wbase, c);
+      for (int c = 0; c < NT; c++) load_row(rawB[c], wbase, c);
+    }
 #pragma unroll
     for (int i = 0; i < NX; i++) x_copy(xtile, gemm_xbuf1, i);
   } else {
+    if constexpr (!DMA) {
 #pragma unroll
-    for (int c = 0; c < NT; c++) load_row(rawA[c], wbase, c);
+      for (int c = 0; c < NT; c++) load_row(rawA[c], wbase, c);
+    }
 #pragma unroll
     for (int i = 0; i < NX; i++) x_copy(xtile, gemm_xbuf0, i);
   }
-  stage_store();
+  if constexpr (!DMA) stage_store();
   __syncthreads();
-  if (odd) take_ql(rawB); else take_ql(rawA);
+  if constexpr (DMA) {
+    if (odd) take_raw(rawB); else take_raw(rawA);
+  } else {
+    if (odd) take_ql(rawB); else take_ql(rawA);
+  }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();   // gemm_wbuf6 is free for the next super-block
   asm volatile("" ::: "memory");
@@ -224,14 +268,24 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
       const int p = t & 1;
       // prefetches for the next super-block, a few per k-step: the raw weights of one row tile (5 loads) in each of
       // the first NT steps, the x tile global -> LDS spread over the first six
-      if (t < NT) {
-        stage_load(tnext, 2 * t);
-        stage_load(tnext, 2 * t + 1);
-        load_row(nxt[t], knbase, t);
+      if constexpr (DMA) {
+        // the eight copies of the next super-block's raw blocks, two per k-step; they and the x copies are waited for
+        // behind k-step 6, the lanes that decode them pick them up during k-step 7
+        if (t < 4) {
+          copy_w(tnext, 2 * t);
+          copy_w(tnext, 2 * t + 1);
+        }
+        if (t == 7) take_raw(nxt);
+      } else {
+        if (t < NT) {
+          stage_load(tnext, 2 * t);
+          stage_load(tnext, 2 * t + 1);
+          load_row(nxt[t], knbase, t);
+        }
+        if (t == 3) stage_load_sc(tnext);
+        if (t == 6) stage_store();
+        if (t == 7) take_ql(nxt);
       }
-      if (t == 3) stage_load_sc(tnext);
-      if (t == 6) stage_store();
-      if (t == 7) take_ql(nxt);
       if (t < 6) {
 #pragma unroll
         for (int i = (t < 3 ? 2 * t : 3 * t - 3); i < (t < 3 ? 2 * t + 2 : (t < 5 ? 3 * t : 16)); i++)
@@ -261,14 +315,16 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
       }
       __builtin_amdgcn_sched_barrier(0);
       if (t == 6) {
-        // the staged ql of the next super-block is complete once every wavefront's stores have landed
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // the staged ql of the next super-block is complete once every wavefront's stores have landed (DMA: once every
+        // wavefront's copies have)
+        if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
       }
     }
     // End of the iteration: everything this wavefront requested has to be there (the x tile for everybody, the
-    // weights for its own next iteration) and its reads of gemm_wbuf6 have to be done, then everybody meets.
+    // weights for its own next iteration) and its reads of the raw-weight buffer have to be done, then everybody meets.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -293,10 +349,11 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 }
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_m64_n128_f16(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
-  gemm_q6k_core<2, 2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+  gemm_q6k_core<2, 2, true>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }
-// the same with a workgroup tile of 128 tokens x 128 rows; grid from gemm_grid_x(ceil(m/128), ceil(out_dim/128))
+// the same with a workgroup tile of 128 tokens x 128 rows (whole blocks copied global -> LDS); grid from
+// gemm_grid_x(ceil(m/128), ceil(out_dim/128))
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q6_k_gemm_n128_f16(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
-  gemm_q6k_core<2>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
+  gemm_q6k_core<2, 4, true>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }
