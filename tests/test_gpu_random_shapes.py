@@ -118,3 +118,53 @@ def test_random_one_pass_shapes(gpu, oracle, seed):
             assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, what + " member %d" % d)
         for a in ws + outs + [xd]:
             a.close()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_prefill_ffn_blocks(gpu, oracle, seed):
+    """The feed-forward block of a prefill layer at drawn sizes (hidden and FFN width multiples of 256, 9..300 tokens, the down
+    matrix of any GEMM type), once with its producers packing - the norm writes the packed input of gate | up, the SwiGLU GEMM
+    that of the down GEMM - and once as five launches with the two pack launches: the same bits. Two tokens of it against the
+    CPU form."""
+    rng = np.random.default_rng(9500 + seed)
+    for case in range(4):
+        hidden, ffn = 256 * int(rng.integers(1, 9)), 256 * int(rng.integers(1, 13))
+        tokens = int(rng.integers(9, 301))
+        dt = [Q4_K, Q5_K, Q6_K][int(rng.integers(0, 3))]
+        what = "seed %d case %d: hidden=%d ffn=%d M=%d down type %d" % (seed, case, hidden, ffn, tokens, dt)
+        print(what, flush=True)
+        gate_raw, up_raw = synth.make_weights(rng, Q4_K, ffn, hidden), synth.make_weights(rng, Q4_K, ffn, hidden)
+        down_raw = synth.make_weights(rng, dt, hidden, ffn)
+        x = rng.uniform(-0.1, 0.1, tokens * hidden).astype(np.float32)
+        add = rng.uniform(-1.0, 1.0, tokens * hidden).astype(np.float32)
+        norm = (0.1 + 0.01 * rng.standard_normal(hidden)).astype(np.float32)
+        wsx, wsa = quant.gemm_workspace_bytes(Q4_K, hidden, tokens), quant.gemm_workspace_bytes(dt, ffn, tokens, hidden)
+        wg, wu, wd, xd, ad, nd = (DevArray(a) for a in (gate_raw, up_raw, down_raw, x, add, norm))
+        outs = []
+        for fused in (False, True):
+            res, normed, out = (DevArray(nbytes=x.nbytes) for _ in range(3))
+            act, ws_x, ws_a = DevArray(nbytes=4 * tokens * ffn), DevArray(nbytes=wsx), DevArray(nbytes=wsa)
+            if fused:
+                quant.add_rmsnorm_gemm_pack_dev(xd.ptr, ad.ptr, nd.ptr, res.ptr, 0, Q4_K, ws_x.ptr, wsx, hidden, tokens, 1e-6)
+                quant.gemm_packed_swiglu_pack_dev(wg.ptr, wu.ptr, Q4_K, ws_x.ptr, wsx, 0, dt, ws_a.ptr, wsa, hidden, ffn, tokens)
+            else:
+                quant.add_rmsnorm_dev(xd.ptr, ad.ptr, nd.ptr, res.ptr, normed.ptr, hidden, tokens, 1e-6)
+                quant.gemm_pack_dev(normed.ptr, Q4_K, hidden, tokens, ws_x.ptr, wsx)
+                quant.gemm_packed_swiglu_dev(wg.ptr, wu.ptr, Q4_K, ws_x.ptr, wsx, act.ptr, hidden, ffn, tokens)
+                quant.gemm_pack_dev(act.ptr, dt, ffn, tokens, ws_a.ptr, wsa)
+            quant.gemm_packed_add_dev(wd.ptr, dt, ws_a.ptr, wsa, res.ptr, out.ptr, ffn, hidden, tokens)
+            outs.append(out.read(np.float32, tokens * hidden))
+            for a in (res, normed, out, act, ws_x, ws_a):
+                a.close()
+        assert np.array_equal(outs[0], outs[1]), what
+        zero_f = np.zeros(ffn, dtype=np.float32)
+        for tok in (0, tokens - 1):
+            r = x[tok * hidden:(tok + 1) * hidden] + add[tok * hidden:(tok + 1) * hidden]
+            h = oracle.rms_norm(r, norm, 1e-6)
+            g = oracle.matmul_add(h, 1, hidden, gate_raw, Q4_K, ffn, zero_f, threads=8)
+            u = oracle.matmul_add(h, 1, hidden, up_raw, Q4_K, ffn, zero_f, threads=8)
+            want = oracle.matmul_add(oracle.swiglu(g, u), 1, ffn, down_raw, dt, hidden, r, threads=8)
+            got = outs[1][tok * hidden:(tok + 1) * hidden]
+            assert np.max(np.abs(got - want)) <= 4e-3 * np.max(np.abs(want)), what + " token %d" % tok
+        for a in (wg, wu, wd, xd, ad, nd):
+            a.close()
