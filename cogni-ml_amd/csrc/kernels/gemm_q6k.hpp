@@ -21,7 +21,8 @@
 // fit, and there they are copied whole, global -> LDS, without passing through registers (template parameter DMA below).
 // k-step t of the wavefront is quadrant
 // t / 2, bytes 8 (t % 2) .. +8 of the pieces: 8 values with one scale. A code is put together in the low bits of a
-// half, (ql nibble) | (qh bits << 4) | 0x6400 = 1024 + q as binary16; subtracting 1056 gives q - 32 exactly and one
+// half, (ql nibble) | (qh bits << 4) | 0x6400 = 1024 + q as binary16 (high nibbles are left in place, four bits up, beside
+// 0x5400: 64 + q); subtracting 1056 (96) gives q - 32 exactly and one
 // packed multiply gives fp16((q - 32) * (d * sc)). The 8 values come in byte order 0,2,1,3,4,6,5,7;
 // pack_x_f16_q6k writes x accordingly (gemm_k_element_q6k).
 #pragma once
@@ -95,6 +96,9 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
 #pragma unroll
   for (int c = 0; c < NT; c++) rowoff[c] = (min(n0 + 32 * c + j, out_dim - 1) - base_row) * (u32)row_bytes;
   const u32 o_qh = 128 + 32 * kh + 16 * kg;
+  // constants of the code assembly, kept in registers (as literals each (a & mask) | b would be two instructions)
+  u32 mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u, m3_lo = 0x00300030u, m3_hi = 0x03000300u;
+  asm volatile("" : "+v"(mask_lo), "+v"(mask_hi), "+v"(magic_lo), "+v"(magic_hi), "+v"(m3_lo), "+v"(m3_hi));
   const uint4* xtile = xp + ((size_t)mt * nkb_all + kb0) * 4096;
 
   float16_t acc[MT][NT];
@@ -243,15 +247,25 @@ __device__ __forceinline__ void gemm_q6k_core(const uint8_t* w, const uint4* xp,
       for (int c = 0; c < NT; c++) {
         const uint4 Q = (qd & 1) ? cur[c].qb : cur[c].qa;
         const u32 qa = h8 ? Q.z : Q.x, qb = h8 ? Q.w : Q.y;
-        const u32 ha = (h8 ? cur[c].qh.z : cur[c].qh.x) >> (2 * qd), hb = (h8 ? cur[c].qh.w : cur[c].qh.y) >> (2 * qd);
-        const u32 qsa = hi ? (qa >> 4) : qa, qsb = hi ? (qb >> 4) : qb;
-        const u32 off = 0xE420E420u;   // half2(-1056): 1024 + q - 1056 = q - 32
+        const u32 ha = h8 ? cur[c].qh.z : cur[c].qh.x, hb = h8 ? cur[c].qh.w : cur[c].qh.y;
+        // low nibbles: 1024 + q with the code in mantissa bits 0..5, minus 1056; high nibbles stay where they are: 64 + q with
+        // the code in mantissa bits 4..9 (one step is 1/16 there), minus 96 - q - 32 exactly either way. The two bits of qh
+        // go beside the nibble (bits 4..5, or 8..9): for bytes 0 and 2 of a dword a left shift by 4 (quadrants 0, 2) or 2
+        // (1, 3) puts them there, for bytes 1 and 3 a right shift by 4 or 6 - four shifted forms of a qh dword, each used by
+        // two quadrants. Masks and offsets sit in registers so that (a & mask) | b is one v_and_or_b32.
+        const u32 mask = hi ? mask_hi : mask_lo, magic = hi ? magic_hi : magic_lo, m3 = hi ? m3_hi : m3_lo;
+        const u32 off = hi ? 0xD600D600u : 0xE420E420u;   // half2(-96) : half2(-1056)
+        const int sl = (qd & 1) ? 2 : 4, sr = (qd & 1) ? 6 : 4;
         const u32 sc = S[c][qd];
         uint4 bw;
-        bw.x = h2_sub_mul((qsa & 0x000F000Fu) | ((ha & 0x00030003u) << 4) | 0x64006400u, off, sc);
-        bw.y = h2_sub_mul(((qsa >> 8) & 0x000F000Fu) | (((ha >> 8) & 0x00030003u) << 4) | 0x64006400u, off, sc);
-        bw.z = h2_sub_mul((qsb & 0x000F000Fu) | ((hb & 0x00030003u) << 4) | 0x64006400u, off, sc);
-        bw.w = h2_sub_mul(((qsb >> 8) & 0x000F000Fu) | (((hb >> 8) & 0x00030003u) << 4) | 0x64006400u, off, sc);
+        // (the nibble halves are held as values of their own: left to itself the compiler merges the two steps into two
+        // ands and a three-way or)
+        u32 n0 = (qa & mask) | magic, n1 = ((qa >> 8) & mask) | magic, n2 = (qb & mask) | magic, n3 = ((qb >> 8) & mask) | magic;
+        asm("" : "+v"(n0), "+v"(n1), "+v"(n2), "+v"(n3));
+        bw.x = h2_sub_mul(((ha << sl) & m3) | n0, off, sc);
+        bw.y = h2_sub_mul(((ha >> sr) & m3) | n1, off, sc);
+        bw.z = h2_sub_mul(((hb << sl) & m3) | n2, off, sc);
+        bw.w = h2_sub_mul(((hb >> sr) & m3) | n3, off, sc);
         B[c] = *reinterpret_cast<const half8_t*>(&bw);
       }
     };
