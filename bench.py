@@ -671,6 +671,29 @@ def main():
                 tokens, layers[0].raw_bytes, steps, r["us"], rec["gbps"], rec["frac_hbm"], r1["us"]))
         for r_ in runners:
             r_.close()
+    # the same stack beyond the GEMM threshold (its prefill route): x packed once, q | k | v | gate | up as one list GEMM, o and
+    # the Q6_K down projection behind their own packs
+    for tokens in (64, 512):
+        xs = rng.uniform(-1.0, 1.0, tokens * layers[0].hidden).astype(np.float32)
+        runners = [QwenProjectionStackRunner.from_weights(w, tokens, xs) for w in layers]
+        for r_ in runners:
+            r_.upload_weights()
+            r_.reset_sequence()
+
+        def pseq(copy, st, runners=runners):
+            with hip.with_stream(st):
+                runners[copy].run_sequence()
+        steps = max(5, min(args.steps, 30))
+        r = measure(hip, stream, Rotating(pseq, 3, layers[0].raw_bytes), steps, 3)
+        pflops = 2.0 * tokens * sum(e[3] * e[4] for e in layers[0].entries)
+        cases["cfg5 projection stack prefill M=%d" % tokens] = {
+            "us": round(r["us"], 2), "tflops": round(pflops / r["us"] / 1e6, 1),
+            "frac_mfma_f16": round(pflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "flops": pflops, "steps": steps,
+            "launches": "pack x, list GEMM q|k|v|gate|up, pack q, o GEMM, pack gate, Q6_K down GEMM (+ plane sums where the k range is split)"}
+        log("case=projection stack prefill\ntokens=%d\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
+            tokens, r["us"], pflops / r["us"] / 1e6, pflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS))
+        for r_ in runners:
+            r_.close()
 
     if args.mode == "cases":
         # output head without the logits: RMSNorm -> Q6_K vocabulary projection with arg-max -> top-1 reduce (510 MB)

@@ -152,16 +152,30 @@ class QwenProjectionStackRunner:
         return int(entry[2]) in (int(TensorType.Q4_K), int(TensorType.Q5_K), int(TensorType.Q6_K)) and entry[4] % 256 == 0
 
     def _launch_prefill(self, count):
-        """All `count` tokens through the GEMMs: one pack per (input, layout), one GEMM per projection."""
+        """All `count` tokens through the GEMMs: one pack per (input, layout), one GEMM per list of projections that share
+        their input, type and row length (or per projection)."""
         stream = hip.current_stream_handle()
-        packed = set()
-        for name, src, t, out_dim, in_dim, raw in self.weights.entries:
+        ents = self.weights.entries
+        packed, done = set(), set()
+        list_types = (int(TensorType.Q4_K), int(TensorType.Q5_K))
+        for idx, (name, src, t, out_dim, in_dim, raw) in enumerate(ents):
+            if name in done:
+                continue
             key = (src, self._family(t))
             ws, nbytes = self._prefill_ws[key]
             if key not in packed:
                 quant.gemm_pack_dev(self._act[src].ptr, t, in_dim, count, ws.ptr, nbytes, stream)
                 packed.add(key)
-            quant.gemm_packed_dev(self._w[name].ptr, t, ws.ptr, nbytes, self._act[name].ptr, in_dim, out_dim, count, 0, stream)
+            # every projection still to come of the same input, type and row length joins this launch (q | k | v | gate | up:
+            # their input is this one's, so it exists already) - the prefill counterpart of the qmatvec_many seam
+            grp = [e for e in ents[idx:] if e[0] not in done and (e[1], int(e[2]), e[4]) == (src, int(t), in_dim)][:6]
+            if len(grp) >= 2 and int(t) in list_types:
+                quant.gemm_packed_many_dev([self._w[e[0]].ptr for e in grp], t, ws.ptr, nbytes, [self._act[e[0]].ptr for e in grp],
+                                           [e[3] for e in grp], in_dim, count, stream)
+                done.update(e[0] for e in grp)
+            else:
+                quant.gemm_packed_dev(self._w[name].ptr, t, ws.ptr, nbytes, self._act[name].ptr, in_dim, out_dim, count, 0, stream)
+                done.add(name)
 
     def _run_token(self, tok):
         self._launch(tok, 1)

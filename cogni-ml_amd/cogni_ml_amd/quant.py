@@ -318,6 +318,17 @@ def gemm_packed_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, workspace_ptr, workspac
                                                   ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+def gemm_packed_many_dev(w_ptrs, w_type, workspace_ptr, workspace_bytes, out_ptrs, out_dims, in_dim, tokens, stream=None):
+    """One GEMM launch for up to six matrices of one type and row length against the same packed activations (no k split)."""
+    n = len(w_ptrs)
+    if not (n == len(out_ptrs) == len(out_dims)):
+        raise ValueError("w_ptrs, out_ptrs and out_dims must have one entry per matrix")
+    _check(hip.lib().cogni_gemm_packed_many_dev((ctypes.c_uint64 * n)(*w_ptrs), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(workspace_ptr),
+                                                ctypes.c_size_t(workspace_bytes), (ctypes.c_uint64 * n)(*out_ptrs),
+                                                (ctypes.c_uint32 * n)(*out_dims), ctypes.c_uint32(n), ctypes.c_uint32(in_dim),
+                                                ctypes.c_uint32(tokens), stream))
+
+
 def gemm_packed_swiglu_pack_dev(w_gate_ptr, w_up_ptr, w_type, workspace_ptr, workspace_bytes, out_ptr, next_type, next_workspace_ptr,
                                 next_workspace_bytes, in_dim, out_dim, tokens, stream=None):
     """gemm_packed_swiglu_dev whose products also (out_ptr 0: only) leave as the packed activations of the next GEMM."""

@@ -1162,6 +1162,70 @@ int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type
   return launch("q4_k_gemm_swiglu_f16", gemm_grid_x(mtiles, ntiles), 256, 0, params, stream);
 }
 
+// Several matrices of one type and row length against one block of packed activations, as one launch: no k split (the list
+// is what fills the chip), the tile height that needs fewer rounds of 256 workgroups (a 128-row tile costs
+// GEMM_N128_COST_X100 per cent of a 192-row one), the 64-token kernels for up to 64 tokens.
+namespace {
+struct GemmManyArgs {   // the kernels' first parameter (kernels/gemm_q4k.hpp)
+  uint64_t w[6];
+  uint64_t out[6];
+  uint32_t out_dim[6];
+  uint32_t tile_end[6];
+  uint32_t count;
+};
+}   // namespace
+int cogni_gemm_packed_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, const uint64_t* outs,
+                               const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream) {
+  const char* who = "cogni_gemm_packed_many_dev";
+  if (w_type != COGNI_TYPE_Q4_K && w_type != COGNI_TYPE_Q5_K)
+    return fail(COGNI_ERR_UNSUPPORTED_TYPE, std::string("Unsupported quant type for the list GEMM: ") + type_name(w_type));
+  if (!w_raw || !outs || !out_dims || count == 0 || count > 6) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": one to six matrices");
+  for (uint32_t i = 0; i < count; i++) {
+    if (!w_raw[i] || !outs[i]) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null device pointer");
+    if (int rc = gemm_check(who, w_type, in_dim, out_dims[i], tokens, workspace, workspace_bytes)) return rc;
+  }
+  const uint32_t mtiles = (tokens + 127) / 128, nkb = in_dim / 256;
+  const size_t packed_bytes = cogni_gemm_workspace_bytes(w_type, in_dim, tokens);
+  // a matrix that alone gets the 256-row tiles of the eight-wavefront kernel (many tokens, many rows) keeps them: it is
+  // launched by itself, unsplit as the list is; the others form the list
+  uint32_t listed[6], nlisted = 0;
+  for (uint32_t i = 0; i < count; i++) {
+    if (gemm_shape(w_type, in_dim, out_dims[i], tokens, false).bn == 256) {
+      if (int rc = gemm_packed_launch(who, w_raw[i], w_type, workspace, packed_bytes, 0, 0, outs[i], in_dim, out_dims[i], tokens, stream)) return rc;
+    } else {
+      listed[nlisted++] = i;
+    }
+  }
+  if (nlisted == 0) return 0;
+  if (nlisted == 1) {
+    const uint32_t i = listed[0];
+    return gemm_packed_launch(who, w_raw[i], w_type, workspace, packed_bytes, 0, 0, outs[i], in_dim, out_dims[i], tokens, stream);
+  }
+  uint64_t tiles[2] = {0, 0};   // 192-row, 128-row
+  for (uint32_t k = 0; k < nlisted; k++) {
+    tiles[0] += (out_dims[listed[k]] + 191) / 192;
+    tiles[1] += (out_dims[listed[k]] + 127) / 128;
+  }
+  const uint64_t cost192 = ((mtiles * tiles[0] + 255) / 256) * nkb * 100, cost128 = ((mtiles * tiles[1] + 255) / 256) * nkb * GEMM_N128_COST_X100;
+  const bool n128 = cost128 < cost192, m64 = tokens <= 64;
+  const uint32_t bn = n128 ? 128 : 192;
+  GemmManyArgs list{};
+  uint32_t end = 0;
+  for (uint32_t k = 0; k < nlisted; k++) {
+    const uint32_t i = listed[k];
+    list.w[k] = w_raw[i];
+    list.out[k] = outs[i];
+    list.out_dim[k] = out_dims[i];
+    list.tile_end[k] = end += (out_dims[i] + bn - 1) / bn;
+  }
+  list.count = nlisted;
+  static const char* const names[2][2][2] = {
+      {{"q4_k_gemm_many_f16", "q4_k_gemm_many_n128_f16"}, {"q4_k_gemm_many_m64_f16", "q4_k_gemm_many_m64_n128_f16"}},
+      {{"q5_k_gemm_many_f16", "q5_k_gemm_many_n128_f16"}, {"q5_k_gemm_many_m64_f16", "q5_k_gemm_many_m64_n128_f16"}}};
+  void* params[] = {&list, &workspace, &in_dim, &tokens};
+  return launch(names[w_type == COGNI_TYPE_Q5_K][m64][n128], gemm_grid_x(mtiles, end), 256, 0, params, stream);
+}
+
 int cogni_gemm_packed_swiglu_pack_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
                                       uint32_t next_type, uint64_t next_workspace, size_t next_workspace_bytes, uint32_t in_dim,
                                       uint32_t out_dim, uint32_t tokens, void* stream) {

@@ -345,6 +345,18 @@ __device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3]
   }
 }
 
+// Up to GEMM_MANY_MAX matrices of one type and row length against the same packed activations, as one launch: the tiles of
+// the launch are the tiles of matrix 0, then of matrix 1, ... (tile_end[i]: tiles of matrices 0..i), every matrix with its
+// own output [m][out_dim[i]]. A workgroup looks its matrix up once; everything behind that is the single-matrix kernel.
+#define GEMM_MANY_MAX 6
+struct GemmManyArgs {
+  const uint8_t* w[GEMM_MANY_MAX];
+  float* out[GEMM_MANY_MAX];
+  u32 out_dim[GEMM_MANY_MAX];
+  u32 tile_end[GEMM_MANY_MAX];
+  u32 count;
+};
+
 // raw bytes of one group of one super-block of one weight row, as a lane sees them
 template <bool Q5>
 struct GemmRawT {
@@ -367,7 +379,7 @@ struct GemmRawT<true> {   // Q5_K: plus the 32 bytes of fifth bits (bit 2g + hi 
 template <bool Q5, bool SWIGLU = false, int NT = 3, int MT = 4, int PACK = 0>
 __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim,
                                               u32 out_dim, u32 m, u32 bias_stride = 0, const uint8_t* w_b = nullptr,
-                                              uint4* xq = nullptr) {
+                                              uint4* xq = nullptr, const GemmManyArgs* many = nullptr) {
   static_assert(PACK == 0 || SWIGLU, "only the gate | up kernel writes packed activations");
   static_assert(!(Q5 && SWIGLU), "the gate | up kernel is built for Q4_K");
   static_assert(NT == 3 || (NT == 2 && !SWIGLU), "tile heights");
@@ -391,12 +403,22 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   const u32 kb0 = blockIdx.y * nkb_all / gridDim.y, nkb = (blockIdx.y + 1) * nkb_all / gridDim.y - kb0;
   out += (size_t)blockIdx.y * m * out_dim;
   constexpr u32 TILE_ROWS = SWIGLU ? BN / 2 : BN;   // rows of a matrix a tile covers
-  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM, ntiles = (out_dim + TILE_ROWS - 1) / TILE_ROWS;
+  const u32 mtiles = (m + GEMM_BM - 1) / GEMM_BM;
+  const u32 ntiles = many ? many->tile_end[many->count - 1] : (out_dim + TILE_ROWS - 1) / TILE_ROWS;
   // Workgroup -> tile, XCD-aware (gemm_tile_of, gemv_config.h): the 32 workgroups that run side by side on an XCD take
   // a block of neighbouring tiles, so that its L2 fills with a weight tile once for several token tiles and with an x
   // tile once for several weight tiles. The grid is rounded up to whole blocks; the surplus workgroups leave.
   u32 mt, nt;
   if (!gemm_tile_of(blockIdx.x, mtiles, ntiles, &mt, &nt)) return;
+  if (many) {
+    // a list of matrices: the tile's matrix (uniform over the workgroup), its weights, output and row count
+    u32 i = 0, first = 0;
+    while (i + 1 < many->count && nt >= many->tile_end[i]) first = many->tile_end[i++];
+    nt -= first;
+    w = many->w[i];
+    out = many->out[i];
+    out_dim = many->out_dim[i];
+  }
   const size_t row_bytes = (size_t)nkb_all * BS;
   const u32 sh = 16u * kg;
   // Unpacking the 6-bit (scale, min) pairs takes one of two forms by g >= 2, i.e. by kh, which is the same for a whole
@@ -700,6 +722,23 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
     const uint8_t* w, const uint4* xp, const float* bias, float* out, u32 in_dim, u32 out_dim, u32 m, u32 bias_stride) {
   gemm_k45_core<true>(w, xp, bias, out, in_dim, out_dim, m, bias_stride);
 }
+// Lists of matrices (q | k | v | gate | up of a prefill layer against one packed x): (list: GemmManyArgs by value, xp, in_dim, m),
+// block 256, grid gemm_grid_x(ceil(m/128), sum of the matrices' tiles), no k split, no bias; 192- and 128-row tiles, 128 and
+// up to 64 tokens, as the single-matrix kernels of the same suffixes, and every output bit for bit theirs.
+#define GEMM_K45_MANY_ENTRY(NAME, Q5, NT, MT)                                                                                \
+  extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void NAME(                       \
+      const GemmManyArgs list, const uint4* xp, u32 in_dim, u32 m) {                                                         \
+    gemm_k45_core<Q5, false, NT, MT>(nullptr, xp, nullptr, nullptr, in_dim, 0, m, 0, nullptr, nullptr, &list);              \
+  }
+GEMM_K45_MANY_ENTRY(q4_k_gemm_many_f16, false, 3, 4)
+GEMM_K45_MANY_ENTRY(q4_k_gemm_many_n128_f16, false, 2, 4)
+GEMM_K45_MANY_ENTRY(q4_k_gemm_many_m64_f16, false, 3, 2)
+GEMM_K45_MANY_ENTRY(q4_k_gemm_many_m64_n128_f16, false, 2, 2)
+GEMM_K45_MANY_ENTRY(q5_k_gemm_many_f16, true, 3, 4)
+GEMM_K45_MANY_ENTRY(q5_k_gemm_many_n128_f16, true, 2, 4)
+GEMM_K45_MANY_ENTRY(q5_k_gemm_many_m64_f16, true, 3, 2)
+GEMM_K45_MANY_ENTRY(q5_k_gemm_many_m64_n128_f16, true, 2, 2)
+
 // gate | up of a feed-forward block against one packed x, silu(gate) * up stored: no gate and up matrices in memory.
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_f16(
     const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, u32 in_dim, u32 out_dim, u32 m) {

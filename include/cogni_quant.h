@@ -399,6 +399,16 @@ int cogni_gemm_packed_add_dev(uint64_t w_raw, uint32_t w_type, uint64_t workspac
                               uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
                                  uint32_t in_dim, uint32_t out_dim, uint32_t tokens, void* stream);
+/* Several matrices of one type and row length against the same packed activations in one launch - q | k | v | gate | up of
+ * a prefill layer, the counterpart for M > 8 of cogni_gemv_many_dev (the reference issues one qmatmul_nobias per weight,
+ * src/ml/gguf/qwen35_cpu.cr:1478-1490): out_i[m][o] = sum_j x[m][j] * deq(W_i[o][j]), every output bit for bit what
+ * cogni_gemm_packed_dev gives for that matrix with a workspace that holds the packed activations only (no k split). One to
+ * six matrices, Q4_K or Q5_K, no bias. A matrix that alone gets the 256-row tiles of q4_k_gemm_wide_f16 (cogni_gemm_plan)
+ * keeps them and is launched by itself; the others form the list. Kernels "<type>_gemm_many[_m64][_n128]_f16" (list by value: six weight pointers, six
+ * output pointers, six row counts, six cumulative tile counts, the count; workspace; in_dim:u32; tokens:u32), block 256,
+ * grid as cogni_gemm_plan gives it for a matrix of all the tiles. */
+int cogni_gemm_packed_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, const uint64_t* outs,
+                               const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream);
 /* cogni_gemm_packed_swiglu_dev that also hands its products on as the packed activations of the GEMM behind it - the down
  * projection of the same feed-forward block (qwen35_cpu.cr:1711-1722: `act` goes nowhere else): the epilogue writes
  * silu(g) * u as fp16 into `next_workspace` in the layout cogni_gemm_pack_dev gives a [tokens][out_dim] input of a matrix of

@@ -285,6 +285,37 @@ def test_gate_up_swiglu_hands_on_packed_activations(gpu, tokens, out_dim, in_dim
         a.close()
 
 
+@pytest.mark.parametrize("t,tokens,in_dim,dims", [
+    (Q4_K, 130, 512, [200, 96, 1000]), (Q4_K, 64, 4096, [4096, 1024, 1024, 12288, 12288]), (Q5_K, 9, 256, [7]),
+    (Q5_K, 300, 768, [129, 128, 192, 193, 5, 640]), (Q4_K, 512, 4096, [4096, 1024, 1024]), (Q4_K, 33, 1024, [191, 385]),
+    (Q4_K, 2048, 512, [1024, 12288, 1024])])          # (the 12288-row member gets the eight-wavefront kernel, by itself)
+def test_lists_of_matrices_in_one_gemm(gpu, t, tokens, in_dim, dims):
+    """cogni_gemm_packed_many_dev: up to six matrices of one type and row length against one packed activation block in one
+    launch; every output bit for bit what cogni_gemm_packed_dev gives for that matrix alone without a k split (row counts that
+    are and are not multiples of either tile height, a single matrix, up to 64 tokens and more, the shapes of a layer)."""
+    rng = np.random.default_rng(tokens + in_dim + len(dims))
+    raws = [synth.make_weights(rng, t, d, in_dim) for d in dims]
+    x = synth.make_activations(rng, tokens, in_dim)
+    wsb = quant.gemm_workspace_bytes(t, in_dim, tokens)              # packed activations only: the single launches run unsplit
+    ws, xd, wd = DevArray(nbytes=wsb), DevArray(x), [DevArray(r) for r in raws]
+    singles = [DevArray(nbytes=4 * tokens * d) for d in dims]
+    lists = [DevArray(np.full(tokens * d, np.float32(-3.0))) for d in dims]
+    quant.gemm_pack_dev(xd.ptr, t, in_dim, tokens, ws.ptr, wsb)
+    for w, o, d in zip(wd, singles, dims):
+        quant.gemm_packed_dev(w.ptr, t, ws.ptr, wsb, o.ptr, in_dim, d, tokens)
+    quant.gemm_packed_many_dev([w.ptr for w in wd], t, ws.ptr, wsb, [o.ptr for o in lists], dims, in_dim, tokens)
+    for o1, o2, d in zip(singles, lists, dims):
+        assert np.array_equal(o2.read(np.float32, tokens * d), o1.read(np.float32, tokens * d)), d
+    with pytest.raises(quant.QuantError, match="Unsupported quant type for the list GEMM: Q6_K"):
+        quant.gemm_packed_many_dev([w.ptr for w in wd], Q6_K, ws.ptr, wsb, [o.ptr for o in lists], dims, in_dim, tokens)
+    with pytest.raises(quant.QuantError, match="one to six matrices"):
+        quant.gemm_packed_many_dev([wd[0].ptr] * 7, t, ws.ptr, wsb, [lists[0].ptr] * 7, [dims[0]] * 7, in_dim, tokens)
+    with pytest.raises(quant.QuantError, match="null device pointer"):
+        quant.gemm_packed_many_dev([0], t, ws.ptr, wsb, [lists[0].ptr], [dims[0]], in_dim, tokens)
+    for a in [ws, xd] + wd + singles + lists:
+        a.close()
+
+
 def test_projections_share_one_packed_activation_block(gpu, oracle):
     """gemm_pack_dev once, then gemm_packed_dev for several matrices of one type family (Q4_K and Q5_K read the same packed
     layout; a k-split and an unsplit shape, with and without bias): the bits of gemm_dev on each matrix alone."""
