@@ -168,3 +168,30 @@ def test_random_prefill_ffn_blocks(gpu, oracle, seed):
             assert np.max(np.abs(got - want)) <= 4e-3 * np.max(np.abs(want)), what + " token %d" % tok
         for a in (wg, wu, wd, xd, ad, nd):
             a.close()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_gemm_lists(gpu, seed):
+    """cogni_gemm_packed_many_dev at drawn sizes: one to six Q4_K or Q5_K matrices of 1..1500 rows, rows of 256..3072 values,
+    9..300 tokens; every output bit for bit the single launch's (no k split: the workspace holds the packed activations only)."""
+    rng = np.random.default_rng(9700 + seed)
+    for case in range(5):
+        t = [Q4_K, Q5_K][int(rng.integers(0, 2))]
+        count, in_dim, tokens = int(rng.integers(1, 7)), 256 * int(rng.integers(1, 13)), int(rng.integers(9, 301))
+        dims = [int(rng.integers(1, 1501)) if rng.integers(0, 2) else 64 * int(rng.integers(1, 24)) for _ in range(count)]
+        what = "seed %d case %d: type %d in=%d M=%d dims=%s" % (seed, case, t, in_dim, tokens, dims)
+        print(what, flush=True)
+        raws = [synth.make_weights(rng, t, d, in_dim) for d in dims]
+        x = synth.make_activations(rng, tokens, in_dim)
+        wsb = quant.gemm_workspace_bytes(t, in_dim, tokens)
+        ws, xd, wd = DevArray(nbytes=wsb), DevArray(x), [DevArray(r) for r in raws]
+        singles = [DevArray(nbytes=4 * tokens * d) for d in dims]
+        lists = [DevArray(np.full(tokens * d, np.float32(7.0))) for d in dims]
+        quant.gemm_pack_dev(xd.ptr, t, in_dim, tokens, ws.ptr, wsb)
+        for w, o, d in zip(wd, singles, dims):
+            quant.gemm_packed_dev(w.ptr, t, ws.ptr, wsb, o.ptr, in_dim, d, tokens)
+        quant.gemm_packed_many_dev([w.ptr for w in wd], t, ws.ptr, wsb, [o.ptr for o in lists], dims, in_dim, tokens)
+        for o1, o2, d in zip(singles, lists, dims):
+            assert np.array_equal(o2.read(np.float32, tokens * d), o1.read(np.float32, tokens * d)), what + " member %d" % d
+        for a in [ws, xd] + wd + singles + lists:
+            a.close()
