@@ -1159,7 +1159,7 @@ int cogni_gemm_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type
   // a tile is 128 tokens x 96 rows of each matrix
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 95) / 96;
   void* params[] = {&w_gate, &w_up, &workspace, &out, &in_dim, &out_dim, &tokens};
-  return launch("q4_k_gemm_swiglu_f16", gemm_grid_x(mtiles, ntiles), 256, 0, params, stream);
+  return launch(tokens <= 64 ? "q4_k_gemm_swiglu_m64_f16" : "q4_k_gemm_swiglu_f16", gemm_grid_x(mtiles, ntiles), 256, 0, params, stream);
 }
 
 // Several matrices of one type and row length against one block of packed activations, as one launch: no k split (the list
@@ -1242,8 +1242,9 @@ int cogni_gemm_packed_swiglu_pack_dev(uint64_t w_gate, uint64_t w_up, uint32_t w
     return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": next_workspace too small (cogni_gemm_workspace_bytes)");
   const uint32_t mtiles = (tokens + 127) / 128, ntiles = (out_dim + 95) / 96;
   void* params[] = {&w_gate, &w_up, &workspace, &out, &next_workspace, &in_dim, &out_dim, &tokens};
-  return launch(next_type == COGNI_TYPE_Q6_K ? "q4_k_gemm_swiglu_pack_q6k_f16" : "q4_k_gemm_swiglu_pack_q4k_f16", gemm_grid_x(mtiles, ntiles),
-                256, 0, params, stream);
+  static const char* const names[2][2] = {{"q4_k_gemm_swiglu_pack_q4k_f16", "q4_k_gemm_swiglu_pack_q4k_m64_f16"},
+                                          {"q4_k_gemm_swiglu_pack_q6k_f16", "q4_k_gemm_swiglu_pack_q6k_m64_f16"}};
+  return launch(names[next_type == COGNI_TYPE_Q6_K][tokens <= 64], gemm_grid_x(mtiles, ntiles), 256, 0, params, stream);
 }
 
 int cogni_set_gemm_threshold(int32_t tokens) {

@@ -251,28 +251,29 @@ __device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[MT][NT], const fl
 // GEMM behind this one - the down projection - needs no pack launch and `out` may be null. A lane's four consecutive
 // products are one 8-byte half of a 16-byte cell of that layout, and the lane pair (kg = 0, 1) fills the cell: a wavefront
 // stores 512 contiguous bytes. out_dim is a multiple of 256 then (it is the row length of the next matrix).
-template <int KH, int PACK = 0>
-__device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3], float* out, u32 out_dim, u32 m, u32 mt, u32 nt,
+template <int KH, int PACK = 0, int MT = 4>
+__device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[MT][3], float* out, u32 out_dim, u32 m, u32 mt, u32 nt,
                                                           u32 nh, u32 j, u32 kg, u32 lane, uint2* xq = nullptr) {
-  float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * 24 * 64 + lane;
-  const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * 24 * 64 + lane;
+  constexpr int RH = MT / 2;   // token tiles of 32 a wavefront finishes (MT = 2: the 64-token kernels)
+  float4* mine = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + nh * (12 * RH) * 64 + lane;
+  const float4* theirs = reinterpret_cast<const float4*>(KH ? gemm_xbuf0 : gemm_xbuf1) + nh * (12 * RH) * 64 + lane;
 #pragma unroll
-  for (int rr = 0; rr < 2; rr++)
+  for (int rr = 0; rr < RH; rr++)
 #pragma unroll
     for (int c = 0; c < 3; c++)
 #pragma unroll
       for (int g4 = 0; g4 < 4; g4++) {
-        const float16_t& t = acc[2 * (1 - KH) + rr][c];
+        const float16_t& t = acc[RH * (1 - KH) + rr][c];
         mine[((rr * 3 + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
       }
   __syncthreads();
 #pragma unroll
-  for (int rr = 0; rr < 2; rr++)
+  for (int rr = 0; rr < RH; rr++)
 #pragma unroll
     for (int c = 0; c < 3; c++)
 #pragma unroll
       for (int g4 = 0; g4 < 4; g4++) {
-        float16_t& t = acc[2 * KH + rr][c];
+        float16_t& t = acc[RH * KH + rr][c];
         const float4 p = theirs[((rr * 3 + c) * 4 + g4) * 64];
         // (k half 0) + (k half 1), in that order whichever of the two this wavefront holds
         t[4 * g4] = KH ? p.x + t[4 * g4] : t[4 * g4] + p.x;
@@ -284,12 +285,12 @@ __device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3]
   float4* up = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + lane;
   if (nh == 1) {
 #pragma unroll
-    for (int rr = 0; rr < 2; rr++)
+    for (int rr = 0; rr < RH; rr++)
 #pragma unroll
       for (int c = 0; c < 3; c++)
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++) {
-          const float16_t& t = acc[2 * KH + rr][c];
+          const float16_t& t = acc[RH * KH + rr][c];
           up[((rr * 3 + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
         }
   }
@@ -297,13 +298,13 @@ __device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3]
   if (nh != 0) return;
   const bool vec = (out_dim & 3u) == 0;
 #pragma unroll
-  for (int rr = 0; rr < 2; rr++) {
-    const u32 token = mt * GEMM_BM + 32 * (2 * KH + rr) + j;
+  for (int rr = 0; rr < RH; rr++) {
+    const u32 token = mt * GEMM_BM + 32 * (RH * KH + rr) + j;
 #pragma unroll
     for (int c = 0; c < 3; c++)
 #pragma unroll
       for (int g4 = 0; g4 < 4; g4++) {
-        const float16_t& t = acc[2 * KH + rr][c];
+        const float16_t& t = acc[RH * KH + rr][c];
         const float4 u = up[((rr * 3 + c) * 4 + g4) * 64];
         const float4 o = make_float4(swiglu_one(t[4 * g4], u.x), swiglu_one(t[4 * g4 + 1], u.y), swiglu_one(t[4 * g4 + 2], u.z),
                                      swiglu_one(t[4 * g4 + 3], u.w));
@@ -338,7 +339,10 @@ __device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[4][3]
             uint2 q;
             q.x = *reinterpret_cast<const u32*>(&p0);
             q.y = *reinterpret_cast<const u32*>(&p1);
-            xq[(((size_t)mt * (out_dim >> 8) + kb) * 4096 + (ks * 2 + kgr) * 128 + 32 * (2 * KH + rr) + j) * 2 + kg] = q;
+            uint2* cell = xq + (((size_t)mt * (out_dim >> 8) + kb) * 4096 + (ks * 2 + kgr) * 128 + 32 * (RH * KH + rr) + j) * 2 + kg;
+            *cell = q;
+            // (64 tokens: the upper half of the token tile is nobody's; it gets the zeros the pack kernel writes there)
+            if constexpr (MT == 2) cell[2 * 64] = make_uint2(0u, 0u);
           }
         }
       }
@@ -383,7 +387,7 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   static_assert(PACK == 0 || SWIGLU, "only the gate | up kernel writes packed activations");
   static_assert(!(Q5 && SWIGLU), "the gate | up kernel is built for Q4_K");
   static_assert(NT == 3 || (NT == 2 && !SWIGLU), "tile heights");
-  static_assert(MT == 4 || (MT == 2 && !SWIGLU), "tokens per tile");
+  static_assert(MT == 4 || MT == 2, "tokens per tile");
   constexpr int NX = 4 * MT;              // copies of x per thread and super-block: 32 chunks of 128 tokens x 16 bytes, or of the first 64 tokens of each
   constexpr u32 BN = 64 * NT;             // weight rows of the workgroup tile
   constexpr u32 BS = Q5 ? 176 : 144;      // bytes of a super-block
@@ -687,8 +691,8 @@ __device__ __forceinline__ void gemm_k45_core(const uint8_t* w, const uint4* xp,
   __syncthreads();   // drains the last (unused) prefetches before the buffers are reused below
 
   if constexpr (SWIGLU) {
-    if (kh == 0) gemm_epilogue_swiglu_half<0, PACK>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane, reinterpret_cast<uint2*>(xq));
-    else gemm_epilogue_swiglu_half<1, PACK>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane, reinterpret_cast<uint2*>(xq));
+    if (kh == 0) gemm_epilogue_swiglu_half<0, PACK, MT>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane, reinterpret_cast<uint2*>(xq));
+    else gemm_epilogue_swiglu_half<1, PACK, MT>(acc, out, out_dim, m, mt, nt, nh, j, kg, lane, reinterpret_cast<uint2*>(xq));
   } else {
     gemm_epilogue<NT, MT>(acc, bias, out, out_dim, m, mt, nt, nh, kh, j, kg, tid, bias_stride);
   }
@@ -754,6 +758,19 @@ extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(
 extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_pack_q6k_f16(
     const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, uint4* xq, u32 in_dim, u32 out_dim, u32 m) {
   gemm_k45_core<false, true, 3, 4, 14>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up, xq);
+}
+// the three for up to 64 tokens (two tiles of 32 tokens per wavefront, as <type>_gemm_m64_f16)
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_m64_f16(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<false, true, 3, 2>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up);
+}
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_pack_q4k_m64_f16(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, uint4* xq, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<false, true, 3, 2, 12>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up, xq);
+}
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void q4_k_gemm_swiglu_pack_q6k_m64_f16(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint4* xp, float* out, uint4* xq, u32 in_dim, u32 out_dim, u32 m) {
+  gemm_k45_core<false, true, 3, 2, 14>(w_gate, xp, nullptr, out, in_dim, out_dim, m, 0, w_up, xq);
 }
 
 // Sum of the k-split planes: out[i] = (bias ? bias[bias_stride ? i : i % out_dim] : 0) + partials[0][i] + partials[1][i] + ... in that order

@@ -417,7 +417,9 @@ int cogni_gemm_packed_many_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t 
  * not stored at all. out_dim a multiple of 256; next_workspace_bytes >= cogni_gemm_workspace_bytes(next_type, out_dim,
  * tokens) (with the k-split planes behind it if the next GEMM is to split: cogni_gemm_workspace_bytes_split); the two
  * workspaces must not overlap. Kernels q4_k_gemm_swiglu_pack_q4k_f16 | q4_k_gemm_swiglu_pack_q6k_f16 (w_gate, w_up,
- * workspace, out | 0, next_workspace, in_dim, out_dim, tokens), launched as q4_k_gemm_swiglu_f16. */
+ * workspace, out | 0, next_workspace, in_dim, out_dim, tokens), launched as q4_k_gemm_swiglu_f16. Up to 64 tokens go to the
+ * kernels of the same names with `_m64` in front of `_f16` (q4_k_gemm_swiglu_m64_f16, q4_k_gemm_swiglu_pack_q4k_m64_f16, ...:
+ * two tiles of 32 tokens per wavefront, the same parameters and bits). */
 int cogni_gemm_packed_swiglu_pack_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t workspace, size_t workspace_bytes, uint64_t out,
                                       uint32_t next_type, uint64_t next_workspace, size_t next_workspace_bytes, uint32_t in_dim,
                                       uint32_t out_dim, uint32_t tokens, void* stream);
