@@ -10,6 +10,8 @@ A sequence of more tokens than the GEMM threshold (quant.get_gemm_threshold()) i
 tokens at once in three launches: the activations packed (by the add + RMSNorm in front, where there is one), gate | up as
 one GEMM with SwiGLU in its epilogue, which also writes its products as the packed fp16 activations of the down matrix's
 layout, and the down GEMM with the residual added in its epilogue (src/ml/gguf/qwen35_cpu.cr:1711-1722; the reference's Metal kernels gemm_q4k.metal:1233 and gemm_mm.metal:651).
+Up to sixteen tokens take the one-pass decode kernels with sixteen single-term tokens instead (gate | up as one list, SwiGLU,
+down with the residual: every matrix read once, at the GEMM's precision class).
 `keep_combined=False` leaves the fp32 products (`combined`, the probe's second output) unwritten on that route: they then
 exist only as the down GEMM's input.
 
@@ -65,6 +67,14 @@ class FFNSequenceRunner:
             self._ws_x_bytes = quant.gemm_workspace_bytes(TensorType.Q4_K, hidden, tokens)
             self._ws_act_bytes = quant.gemm_workspace_bytes(down_type, ffn_dim, tokens, hidden)
             self._ws_x, self._ws_act = self._alloc(self._ws_x_bytes), self._alloc(self._ws_act_bytes)
+        # up to sixteen tokens: the images of the one-pass kernels with sixteen single-term tokens (x for gate | up, the
+        # SwiGLU products for down)
+        self._img16_x = self._img16_act = None
+        if self._ws_x is not None:
+            nx = quant.gemv_image_bytes(TensorType.Q4_K, hidden, quant.MAX_GEMV_TOKENS)
+            na = quant.gemv_image_bytes(down_type, ffn_dim, quant.MAX_GEMV_TOKENS)
+            if nx and na:
+                self._img16_x, self._img16_act = self._alloc(nx), self._alloc(na)
         self.combined = self.out = None
         self._runner = hip.ResidentSequenceRunner(tokens, self._upload_weights, self._reset_sequence, self._run_token,
                                                   self._read_outputs, self._run_sequence)
@@ -115,7 +125,27 @@ class FFNSequenceRunner:
         res = self._res.ptr + 4 * tok0 * h if self._res is not None else 0
         quant.gemv_dev(self._w["down"].ptr, self.down_type, act, self._out.ptr + 4 * tok0 * h, f, h, count, res, st)
 
+    def _launch_prefill16(self, count):
+        """9..16 tokens: every projection in one pass over its weights on the decode kernels with sixteen single-term tokens
+        (the GEMM's precision class at half its time): norm, image of x, gate | up as one list, SwiGLU, image of the products
+        in the down matrix's order, down with the residual."""
+        st = hip.current_stream_handle()
+        h, f = self.hidden, self.ffn_dim
+        x = self._x.ptr
+        if self._norm is not None:
+            quant.add_rmsnorm_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, self._normed.ptr, h, count, self._eps, st)
+            x = self._normed.ptr
+        quant.gemv_pack16_dev(x, TensorType.Q4_K, h, count, self._img16_x.ptr, st)
+        quant.gemv_packed16_dev([self._w["gate"].ptr, self._w["up"].ptr], TensorType.Q4_K, self._img16_x.ptr,
+                                [self._gate.ptr, self._up.ptr], [f, f], h, count, 0, st)
+        quant.swiglu_dev(self._gate.ptr, self._up.ptr, self._act.ptr, count * f, st)
+        quant.gemv_pack16_dev(self._act.ptr, self.down_type, f, count, self._img16_act.ptr, st)
+        quant.gemv_packed16_dev([self._w["down"].ptr], self.down_type, self._img16_act.ptr, [self._out.ptr], [h], f, count,
+                                self._res.ptr if self._res is not None else 0, st)
+
     def _launch_prefill(self, count):
+        if count <= 16 and self._img16_x is not None:
+            return self._launch_prefill16(count)
         st = hip.current_stream_handle()
         h, f = self.hidden, self.ffn_dim
         x = self._x.ptr
@@ -151,7 +181,8 @@ class FFNSequenceRunner:
 
     def _read_outputs(self):
         hip.synchronize("hipDeviceSynchronize(read_outputs)")
-        prefill = self._ws_x is not None and self._runner.active_tokens > quant.get_gemm_threshold()
+        active = self._runner.active_tokens
+        prefill = self._ws_x is not None and active > quant.get_gemm_threshold() and not (active <= 16 and self._img16_x is not None)
         self.combined = None
         if self.keep_combined or not prefill:
             self.combined = np.empty(self.tokens * self.ffn_dim, dtype=np.float32)

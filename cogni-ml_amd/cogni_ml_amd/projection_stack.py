@@ -71,11 +71,14 @@ class QwenProjectionStackRunner:
         # prefill: one workspace per (input, packed layout) - Q4_K and Q5_K read one layout, Q6_K its own - large enough
         # for the k-split planes of the projection that needs the most
         self._prefill_ws = {}
+        self._images16 = {}   # input name -> the image of the sixteen-token one-pass kernels (Q4_K / Q5_K projections, 9..16 tokens)
         if tokens > quant.get_gemm_threshold() and all(self._gemm_capable(e) for e in weights.entries):
             need = {}
             for name, src, t, out_dim, in_dim, raw in weights.entries:
                 key = (src, self._family(t))
                 need[key] = max(need.get(key, 0), quant.gemm_workspace_bytes(t, in_dim, tokens, out_dim))
+                if self._one_pass16(t, in_dim) and key not in self._images16:
+                    self._images16[key] = self._alloc(quant.gemv_image_bytes(t, in_dim, quant.MAX_GEMV_TOKENS))
             self._prefill_ws = {k: (self._alloc(n), n) for k, n in need.items()}
         self.outputs = {}
         self._runner = hip.ResidentSequenceRunner(
@@ -151,6 +154,11 @@ class QwenProjectionStackRunner:
     def _gemm_capable(entry):
         return int(entry[2]) in (int(TensorType.Q4_K), int(TensorType.Q5_K), int(TensorType.Q6_K)) and entry[4] % 256 == 0
 
+    @staticmethod
+    def _one_pass16(t, in_dim):
+        return int(t) in (int(TensorType.Q4_K), int(TensorType.Q5_K), int(TensorType.Q6_K)) and \
+            quant.gemv_image_bytes(t, in_dim, quant.MAX_GEMV_TOKENS) > 0
+
     def _launch_prefill(self, count):
         """All `count` tokens through the GEMMs: one pack per (input, layout), one GEMM per list of projections that share
         their input, type and row length (or per projection)."""
@@ -160,6 +168,19 @@ class QwenProjectionStackRunner:
         list_types = (int(TensorType.Q4_K), int(TensorType.Q5_K))
         for idx, (name, src, t, out_dim, in_dim, raw) in enumerate(ents):
             if name in done:
+                continue
+            if count <= 16 and self._one_pass16(t, in_dim):
+                # up to sixteen tokens: the one-pass decode kernels with sixteen single-term tokens, one image per input,
+                # every projection of that input, type and row length in the same call
+                key16 = (src, self._family(t))
+                img = self._images16[key16]
+                if key16 + ("x16",) not in packed:
+                    quant.gemv_pack16_dev(self._act[src].ptr, t, in_dim, count, img.ptr, stream)
+                    packed.add(key16 + ("x16",))
+                grp = [e for e in ents[idx:] if e[0] not in done and (e[1], int(e[2]), e[4]) == (src, int(t), in_dim)][:8]
+                quant.gemv_packed16_dev([self._w[e[0]].ptr for e in grp], t, img.ptr, [self._act[e[0]].ptr for e in grp],
+                                        [e[3] for e in grp], in_dim, count, 0, stream)
+                done.update(e[0] for e in grp)
                 continue
             key = (src, self._family(t))
             ws, nbytes = self._prefill_ws[key]

@@ -318,6 +318,23 @@ def gemm_packed_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, workspace_ptr, workspac
                                                   ctypes.c_uint32(in_dim), ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
 
 
+def gemv_pack16_dev(x_ptr, w_type, in_dim, tokens, image_ptr, stream=None):
+    """The activation image of the sixteen-token one-pass kernels (one binary16 term per token), gemv_image_bytes(type, in_dim, 8) bytes."""
+    _check(hip.lib().cogni_gemv_pack16_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint32(int(w_type)), ctypes.c_uint32(in_dim),
+                                           ctypes.c_uint32(tokens), ctypes.c_uint64(image_ptr), stream))
+
+
+def gemv_packed16_dev(w_ptrs, w_type, image_ptr, out_ptrs, out_dims, in_dim, tokens, residual_ptr=0, stream=None):
+    """Up to eight Q4_K, Q5_K or Q6_K matrices against a sixteen-token image, 1..16 tokens in one pass over the weights (a
+    [tokens][out_dim] residual with a single matrix)."""
+    n = len(w_ptrs)
+    if not (n == len(out_ptrs) == len(out_dims)):
+        raise ValueError("w_ptrs, out_ptrs and out_dims must have one entry per matrix")
+    _check(hip.lib().cogni_gemv_packed16_dev((ctypes.c_uint64 * n)(*w_ptrs), ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr),
+                                             ctypes.c_uint64(residual_ptr), (ctypes.c_uint64 * n)(*out_ptrs), (ctypes.c_uint32 * n)(*out_dims), ctypes.c_uint32(n),
+                                             ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens), stream))
+
+
 def gemm_packed_many_dev(w_ptrs, w_type, workspace_ptr, workspace_bytes, out_ptrs, out_dims, in_dim, tokens, stream=None):
     """One GEMM launch for up to six matrices of one type and row length against the same packed activations (no k split)."""
     n = len(w_ptrs)

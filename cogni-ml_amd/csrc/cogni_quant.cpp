@@ -442,6 +442,50 @@ int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image
   return 0;
 }
 
+// Nine to sixteen tokens in one pass over the weights: the one-pass kernels with their sixteen activation rows as sixteen
+// tokens in one binary16 term each (the precision class of the prefill GEMM), Q4_K, Q5_K and Q6_K.
+static bool gemv16_shape(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {
+  return (w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q5_K || w_type == COGNI_TYPE_Q6_K) && tokens >= 1 && tokens <= 16 &&
+         gemv_mt_supported(w_type, 2, in_dim);
+}
+int cogni_gemv_pack16_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t image, void* stream) {
+  if (!gemv16_shape(w_type, in_dim, tokens))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack16_dev: Q4_K, Q5_K or Q6_K, 1..16 tokens, in_dim a multiple of 256 up to 12288");
+  if (!x || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack16_dev: null device pointer");
+  void* params[] = {&x, &image, &tokens, &in_dim};
+  return launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_mt16_q6k_f16" : "pack_x_mt16_q4k_f16", 4 * gemv_mt_padded_sb(in_dim), 256, 0, params, stream);
+}
+int cogni_gemv_packed16_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,
+                            const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream) {
+  const char* who = "cogni_gemv_packed16_dev";
+  if (!w_raw || !out || !out_dims || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null argument");
+  if (count == 0 || count > 8) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": count must be 1..8");
+  if (!gemv16_shape(w_type, in_dim, tokens))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": Q4_K, Q5_K or Q6_K, 1..16 tokens, in_dim a multiple of 256 up to 12288");
+  if (residual && count != 1) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": a residual goes with a single matrix");
+  for (uint32_t i = 0; i < count; i++)
+    if (!w_raw[i] || !out[i] || out_dims[i] == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null pointer or zero rows");
+  // up to three matrices per launch, as cogni_gemv_packed_dev
+  for (uint32_t i0 = 0; i0 < count;) {
+    uint64_t w[3] = {0, 0, 0}, o[3] = {0, 0, 0}, none = residual;
+    uint32_t rows[3] = {0, 0, 0}, n = 0;
+    uint64_t total = 0;
+    while (n < 3 && i0 + n < count) {
+      w[n] = w_raw[i0 + n], o[n] = out[i0 + n], rows[n] = out_dims[i0 + n];
+      total += rows[n];
+      n++;
+      if (rows[n - 1] % 16 != 0) break;
+    }
+    if (total > 0x7FFFFFFFull) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": too many rows");
+    void* params[] = {&w[0], &w[1], &w[2], &image, &none, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2], &tokens};
+    const int rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt16_f32" : (w_type == COGNI_TYPE_Q5_K ? "q5_k_gemv_mt16_f32" : "q4_k_gemv_mt16_f32"), gemv_mt_grid(w_type, in_dim, (uint32_t)total),
+                          GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type) + GEMV_MT_X16_LDS_EXTRA, params, stream);
+    if (rc != 0) return rc;
+    i0 += n;
+  }
+  return 0;
+}
+
 int cogni_gemv_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t image, uint64_t out, uint32_t in_dim,
                                  uint32_t out_dim, uint32_t tokens, void* stream) {
   if (!w_gate || !w_up || !image || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: null device pointer");
@@ -1266,8 +1310,21 @@ int32_t cogni_get_gemm_threshold(void) {
 
 int cogni_matmul_dev(uint64_t w_raw, uint32_t w_type, uint64_t x, uint64_t bias, uint64_t out, uint32_t in_dim,
                      uint32_t out_dim, uint32_t tokens, uint64_t workspace, size_t workspace_bytes, void* stream) {
-  if (gemm_type(w_type) && tokens > (uint32_t)cogni_get_gemm_threshold())
+  if (gemm_type(w_type) && tokens > (uint32_t)cogni_get_gemm_threshold()) {
+    // up to sixteen tokens of a Q4_K, Q5_K or Q6_K matrix without a bias: one pass over the weights on the decode kernels with
+    // sixteen single-term tokens (the GEMM's precision class) costs about half of pack + GEMM + plane sum; the image goes
+    // where the GEMM's packed activations would (COGNI_MATMUL_X16=0 keeps the GEMM: a measurement knob)
+    bool x16 = tokens <= 16 && !bias && gemv16_shape(w_type, in_dim, tokens) && workspace &&
+               workspace_bytes >= (size_t)gemv_mt_image_bytes(w_type, in_dim);
+    if (const char* e = std::getenv("COGNI_MATMUL_X16"))
+      if (e[0] == '0') x16 = false;
+    if (x16) {
+      if (!w_raw || !x || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_matmul_dev: null device pointer");
+      if (int rc = cogni_gemv_pack16_dev(x, w_type, in_dim, tokens, workspace, stream)) return rc;
+      return cogni_gemv_packed16_dev(&w_raw, w_type, workspace, 0, &out, &out_dim, 1, in_dim, tokens, stream);
+    }
     return cogni_gemm_dev(w_raw, w_type, x, bias, out, in_dim, out_dim, tokens, workspace, workspace_bytes, stream);
+  }
   if (bias && tokens != 1)
     return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_matmul_dev: a [out_dim] bias is only accepted with one token or on the GEMM path; "
                                             "pass a [tokens][out_dim] residual to cogni_gemv_dev");

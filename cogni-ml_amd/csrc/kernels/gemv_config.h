@@ -241,6 +241,8 @@ static inline unsigned gemv_mt_grid(unsigned type, unsigned in_dim, unsigned tot
 }
 // the k-slices' partial sums, then per wavefront the slots of its units: 6 x (16 rows x 144 B) for Q4_K, 6 x (16 rows x
 // 176 B) for Q5_K, 4 x (16 rows x 240 B) for Q6_K, 4 x (16 rows x 272 B) for Q8_0
+// (the sixteen-token kernels keep twice the partial sums)
+#define GEMV_MT_X16_LDS_EXTRA (GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u)
 static inline unsigned gemv_mt_lds_bytes(unsigned type) {
   return GEMV_MT_WAVES * GEMV_MT_TMAX * 8u * 16u * 4u +
          GEMV_MT_WAVES * (type == 14 ? 4u * 3840u : (type == 8 ? 4u * 4352u : (type == 13 ? 6u * 2816u : 6u * 2304u)));

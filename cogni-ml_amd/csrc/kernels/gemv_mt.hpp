@@ -167,6 +167,67 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float*
   mt_pack_store_q4k(image, nsbp, sb, tok, lane, v, present);
 }
 
+// The image for sixteen single-term tokens (MtK45<Q5, true>): the same bytes per super-block with row = token, the halves
+// binary16(x) as they are; behind the operands, per (super-block, lane = 16 kg + token), the sums of sub-blocks
+// 4 kg + (0,2,1,3) of the rounded values / 32 as hi (halves 0..3) and lo (halves 4..7) binary16 terms, zeros for kg >= 2.
+// (x, image, tokens <= 16, in_dim): block 256, grid 4 * gemv_mt_padded_sb(in_dim). |x| has to stay inside the binary16
+// range, as for the prefill GEMM.
+extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q4k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
+                                                                      u32 tokens, u32 in_dim) {
+  const u32 lane = threadIdx.x & 63;
+  const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const u32 nsb = in_dim >> 8, nsbp = gemv_mt_padded_sb(in_dim);
+  const u32 sb = unit >> 4, tok = unit & 15;
+  if (sb >= nsbp) return;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tok < tokens && sb < nsb) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  const _Float16 h0 = (_Float16)v.x, h1 = (_Float16)v.y, h2 = (_Float16)v.z, h3 = (_Float16)v.w;
+  // element 4 l sits in instruction j = l / 8, k-group (l / 2) % 4, upper half of the lane's eight if l is odd (mt_pack_store_q4k)
+  const u32 j = lane >> 3, kg = (lane >> 1) & 3;
+  *reinterpret_cast<mt_half4*>(image + ((size_t)(sb * 8 + j) * 64 + kg * 16 + tok) * 16 + 8 * (lane & 1)) = (mt_half4){h0, h2, h1, h3};
+  float sm = ((float)h0 + (float)h1) + ((float)h2 + (float)h3);
+  sm += MT_DPP(sm, MT_QUAD_1032);
+  sm += MT_DPP(sm, MT_QUAD_2301);
+  sm += MT_DPP(sm, MT_ROW_HALF_MIRROR);
+  const float s32 = 0.03125f;
+  const _Float16 sh = (_Float16)(sm * s32), sl = (_Float16)fmaf(sm, s32, -(float)sh);
+  uint8_t* aux = image + (size_t)nsbp * 8192 + (size_t)sb * 1024;
+  if ((lane & 3) == 0) {
+    const u32 sj = lane >> 3, zero = (lane >> 2) & 1;
+    const u32 slot = ((sj & 1) << 1) | ((sj >> 1) & 1);
+    _Float16* ap = reinterpret_cast<_Float16*>(aux + (((sj >> 2) + 2 * zero) * 16 + tok) * 16) + slot;
+    ap[0] = zero ? (_Float16)0.0f : sh;
+    ap[4] = zero ? (_Float16)0.0f : sl;
+  }
+}
+
+// The same for the Q6_K order: sums of sub-blocks 4 kg .. 4 kg + 3 / 16 as hi (halves 0..3) and lo (halves 4..7).
+extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q6k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
+                                                                      u32 tokens, u32 in_dim) {
+  const u32 lane = threadIdx.x & 63;
+  const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const u32 nsb = in_dim >> 8, nsbp = gemv_mt_padded_sb(in_dim);
+  const u32 sb = unit >> 4, tok = unit & 15;
+  if (sb >= nsbp) return;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tok < tokens && sb < nsb) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  const _Float16 h0 = (_Float16)v.x, h1 = (_Float16)v.y, h2 = (_Float16)v.z, h3 = (_Float16)v.w;
+  // element 4 l sits in sub-block s = l / 4, k-group l % 4 (mt_pack_store_q6k)
+  const u32 s = lane >> 2, kg = lane & 3;
+  *reinterpret_cast<mt_half4*>(image + ((size_t)(sb * 8 + (s >> 1)) * 64 + kg * 16 + tok) * 16 + 8 * (s & 1)) = (mt_half4){h0, h2, h1, h3};
+  float sm = ((float)h0 + (float)h1) + ((float)h2 + (float)h3);
+  sm += MT_DPP(sm, MT_QUAD_1032);
+  sm += MT_DPP(sm, MT_QUAD_2301);
+  const float s16 = 0.0625f;
+  const _Float16 sh = (_Float16)(sm * s16), sl = (_Float16)fmaf(sm, s16, -(float)sh);
+  uint8_t* aux = image + (size_t)nsbp * 8192 + (size_t)sb * 1024;
+  if ((lane & 3) == 0) {
+    _Float16* ap = reinterpret_cast<_Float16*>(aux + ((s >> 2) * 16 + tok) * 16) + (s & 3);
+    ap[0] = sh;
+    ap[4] = sl;
+  }
+}
+
 // Q6_K image: [super-block][sub-block pair p][lane = 16 kg + row][2 x 4 halves]: the halves of lane (kg, row = 2 token +
 // part) for sub-block s = 2 p + (0 | 1) are part of x[token][256 sb + 16 s + 4 kg + (0,2,1,3)] * 2^e. Behind the operands:
 // [super-block][lane = 16 kg + row][16 bytes]: four halves, part of sum(x[token] over sub-block 4 kg + (0,1,2,3)) * 2^(e-4)
@@ -249,9 +310,13 @@ __device__ __forceinline__ void mt_pin(mt_u32x4& v) { asm volatile("" : "+v"(v))
 // Q4_K (144 B: d, dmin, scales[12], qs[128]) and Q5_K (176 B: d, dmin, scales[12], qh[32], qs[128]): byte l of qs[32 g ..
 // 32 g + 32) holds element 64 g + l (low nibble, sub-block 2 g) and element 64 g + 32 + l (high nibble, sub-block 2 g + 1);
 // Q5_K adds bit 2 g / 2 g + 1 of qh[l] as the fifth bit of the two. Both read the same activation image (the Q4_K one).
-template <bool Q5>
+// X16: the sixteen rows of the activation operand are sixteen tokens in one binary16 term each (the precision of the prefill
+// GEMM: x rounded to half, no scaling) instead of eight tokens x (hi, lo) - the kernel for 9..16 tokens (image from
+// pack_x_mt16_q4k_f16: no token scales, the sub-block sums as hi and lo operands).
+template <bool Q5, bool X16 = false>
 struct MtK45 {
   static constexpr unsigned TYPE = Q5 ? 13 : 12;
+  static constexpr int NTOK = X16 ? 16 : 8;   // tokens a launch covers
   static constexpr int BB = Q5 ? 176 : 144, P = BB / 16, NCOPY = 3, LAST = 16 * P - 128, NAUX = 1, NSLOT = 6, TMAX = 3;
   static constexpr int QOFF = Q5 ? 48 : 16;   // where qs starts in the block
   static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 64 * 16;
@@ -262,10 +327,12 @@ struct MtK45 {
 
   // the scales of the lane's two tokens and, as the matrix-core operand of lane (kg, row), the sums of sub-blocks
   // 4 kg + (0,2,1,3) of that row's (token, part) (zeros for kg >= 2)
-  struct Aux { float fsc[2]; mt_u32x2 sums; };
+  // (X16: no scales; the second half of the 16 bytes is the low term of the sums, a second operand)
+  struct Aux { float fsc[2]; mt_u32x2 sums, sums_lo; };
   static __device__ __forceinline__ Aux aux(const mt_u32x4 (&r)[NAUX]) {
     Aux a;
     a.sums = (mt_u32x2){r[0].x, r[0].y};
+    a.sums_lo = (mt_u32x2){r[0].z, r[0].w};
     a.fsc[0] = __uint_as_float(r[0].z), a.fsc[1] = __uint_as_float(r[0].w);
     return a;
   }
@@ -338,18 +405,23 @@ struct MtK45 {
     //     bytes of k-groups 0 and 1 read as binary16 (m * 2^-24, in the order bytes 0, 2, 1, 3 of the masked dword)
     const u32 msel = w.kg == 0 ? mA : (w.kg == 1 ? mB : 0u);
     const mt_u32x2 mb = {msel & 0x00FF00FFu, (msel >> 8) & 0x00FF00FFu};
-    const mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), __builtin_bit_cast(mt_half4, mb),
-                                                                (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), __builtin_bit_cast(mt_half4, mb),
+                                                          (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    if constexpr (X16)
+      off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums_lo), __builtin_bit_cast(mt_half4, mb), off, 0, 0, 0);
     const float d24 = dd * MT_TWO_P24, d20 = dd * MT_TWO_P20, dm29 = dmin * -536870912.0f;   // 2^24 * 2^5
 #pragma unroll
     for (int k = 0; k < 4; k++) {
       const float in = fmaf(d24, ev[k], fmaf(dm29, off[k], d20 * od[k]));
-      acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
+      if constexpr (X16) acc[k] += in;   // (rows 4 rg .. 4 rg + 3 are four tokens)
+      else acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
     }
   }
 };
 typedef MtK45<false> MtQ4K;
 typedef MtK45<true> MtQ5K;
+typedef MtK45<false, true> MtQ4Kx16;
+typedef MtK45<true, true> MtQ5Kx16;
 
 // Q8_0 (34 B per 32 values: d, qs:i8[32]). Eight blocks are taken together as one 272-byte "super-block" of 256 values
 // (17 pieces of 16 bytes; in_dim a multiple of 256 makes every row a whole number of them, 16-byte aligned when the matrix
@@ -363,6 +435,7 @@ typedef MtK45<true> MtQ5K;
 // v_alignbyte_b32.
 struct MtQ80 {
   static constexpr unsigned TYPE = 8;
+  static constexpr int NTOK = 8;
   static constexpr int BB = 272, P = 17, NCOPY = 5, LAST = 16, NAUX = 1, NSLOT = 4, TMAX = 2;
   static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 64 * 16;
   static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece * 16; }
@@ -426,7 +499,10 @@ struct MtQ80 {
 // is 15 pieces (240 bytes: rows 60 dwords apart hit 16 different bank groups): pieces 0..12 are bytes 0..207 of the block,
 // piece 13 is bytes 194..209 (shifted back so that nothing past the end of the matrix is read: d sits at byte 222 of
 // the row) and piece 14 repeats piece 13.
-struct MtQ6K {
+// (X16: sixteen single-term tokens, as MtK45's)
+template <bool X16 = false>
+struct MtQ6KT {
+  static constexpr int NTOK = X16 ? 16 : 8;
   static constexpr unsigned TYPE = 14;
   static constexpr int BB = 210, P = 15, NCOPY = 4, LAST = 48, NAUX = 1, NSLOT = 4, TMAX = 2;
   static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 64 * 16;
@@ -435,10 +511,11 @@ struct MtQ6K {
 
   // the scales of the lane's two tokens and, as the matrix-core operand of lane (kg, row), the sums of sub-blocks
   // 4 kg .. 4 kg + 3 of that row's (token, part)
-  struct Aux { float fsc[2]; mt_u32x2 sums; };
+  struct Aux { float fsc[2]; mt_u32x2 sums, sums_lo; };
   static __device__ __forceinline__ Aux aux(const mt_u32x4 (&r)[NAUX]) {
     Aux a;
     a.sums = (mt_u32x2){r[0].x, r[0].y};
+    a.sums_lo = (mt_u32x2){r[0].z, r[0].w};
     a.fsc[0] = __uint_as_float(r[0].z), a.fsc[1] = __uint_as_float(r[0].w);
     return a;
   }
@@ -494,16 +571,20 @@ struct MtQ6K {
     // sum (q - 32) x = sum q x - 32 sum x: per sub-block that is sc * sum(x), sixteen of them: one more instruction, the
     // sums (times 2^(e-4), hi and lo) against the scales as exact binary16 integers
     const mt_half4 scb = {(_Float16)sbyte_f(w.sck, 0), (_Float16)sbyte_f(w.sck, 1), (_Float16)sbyte_f(w.sck, 2), (_Float16)sbyte_f(w.sck, 3)};
-    const mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), scb,
-                                                                (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), scb,
+                                                          (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    if constexpr (X16) off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums_lo), scb, off, 0, 0, 0);
     const float dd = h2f(w.d), d24 = dd * MT_TWO_P24, d20 = dd * MT_TWO_P20, d512 = dd * -512.0f;   // 32 * 2^4
 #pragma unroll
     for (int k = 0; k < 4; k++) {
       const float in = fmaf(d24, lo[k], fmaf(d512, off[k], d20 * hi[k]));
-      acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
+      if constexpr (X16) acc[k] += in;
+      else acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
     }
   }
 };
+typedef MtQ6KT<false> MtQ6K;
+typedef MtQ6KT<true> MtQ6Kx16;
 
 // ---- the GEMV ------------------------------------------------------------------------------------------------------------
 struct MtArgs {
@@ -527,6 +608,8 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
                                              const float* __restrict__ residual, u32 in_dim, u32 tokens,
                                              u32* __restrict__ top_ids = nullptr) {
   constexpr bool STREAM = SBW > 2;
+  constexpr int NTOK = F::NTOK;   // token rows of the partial sums: 8, or 16 single-term tokens
+  static_assert(NTOK == 8 || (NTOK == 16 && !SWIGLU && !TOP1), "sixteen tokens: plain rows only");
   static_assert(!TOP1 || (!SWIGLU && T * 16 * GEMV_MT_MAX_TOKENS <= GEMV_MT_WAVES * 64), "TOP1: a thread owns one (tile, token, row) of a row group");
   static_assert(!SWIGLU || T == (STREAM ? 1 : 2), "SWIGLU pairs a gate tile with an up tile");
   static_assert(!STREAM || T == 1, "streamed operands: one tile per wavefront");
@@ -541,9 +624,9 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
   const u32 total_rows = a.rows[0] + a.rows[1] + a.rows[2];
   const u32 ntiles = (total_rows + 15) >> 4;
   const u32 ngroups = SWIGLU ? (a.rows[0] + 15) >> 4 : (ntiles + T - 1) / T;
-  // LDS: partial[wave][GEMV_MT_TMAX][8 tokens][16 rows] f32 | slots[wave][NSLOT units]
+  // LDS: partial[wave][GEMV_MT_TMAX][NTOK tokens][16 rows] f32 | slots[wave][NSLOT units]
   float* part = reinterpret_cast<float*>(lds);
-  constexpr u32 SLOTS_OFF = GEMV_MT_WAVES * GEMV_MT_TMAX * 8 * 16 * 4;
+  constexpr u32 SLOTS_OFF = GEMV_MT_WAVES * GEMV_MT_TMAX * NTOK * 16 * 4;
   const char* slots = lds + SLOTS_OFF + wave * (F::NSLOT * F::UNIT_BYTES);
   const u32 slots_lds = (u32)(size_t)(mt_lds_void*)mt_lds4 + SLOTS_OFF + wave * (F::NSLOT * F::UNIT_BYTES);
 
@@ -623,8 +706,13 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
 
   // k-slices through LDS in wavefront order: partial[wave][tile][token][row]; hi + lo of a token first
   auto store_part = [&](int t, const float (&acc)[4]) {
-    part[((wave * GEMV_MT_TMAX + t) * 8 + 2 * rg) * 16 + ar] = acc[0] + acc[1];
-    part[((wave * GEMV_MT_TMAX + t) * 8 + 2 * rg + 1) * 16 + ar] = acc[2] + acc[3];
+    if constexpr (NTOK == 16) {
+#pragma unroll
+      for (int k = 0; k < 4; k++) part[((wave * GEMV_MT_TMAX + t) * 16 + 4 * rg + k) * 16 + ar] = acc[k];
+    } else {
+      part[((wave * GEMV_MT_TMAX + t) * 8 + 2 * rg) * 16 + ar] = acc[0] + acc[1];
+      part[((wave * GEMV_MT_TMAX + t) * 8 + 2 * rg + 1) * 16 + ar] = acc[2] + acc[3];
+    }
   };
   auto finish = [&]() {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -647,7 +735,7 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
         const u32 r = o & 15, m = (o >> 4) % tokens, t = o / (16 * tokens);
         float v = 0.f;
 #pragma unroll
-        for (u32 k = 0; k < GEMV_MT_WAVES; k++) v += part[((k * GEMV_MT_TMAX + t) * 8 + m) * 16 + r];
+        for (u32 k = 0; k < GEMV_MT_WAVES; k++) v += part[((k * GEMV_MT_TMAX + t) * NTOK + m) * 16 + r];
         const u32 row = (grp * T + t) * 16 + r;
         if constexpr (TOP1) {
           // (the groups a thread walks ascend, so do its rows: among equal values the first one stays; a row past the end
@@ -835,6 +923,11 @@ GEMV_MT_ENTRY(q4_k_gemv_mt_f32, MtQ4K)
 GEMV_MT_ENTRY(q5_k_gemv_mt_f32, MtQ5K)
 GEMV_MT_ENTRY(q6_k_gemv_mt_f32, MtQ6K)
 GEMV_MT_ENTRY(q8_0_gemv_mt_f32, MtQ80)
+// 9..16 tokens against the image of pack_x_mt16_q4k_f16 (activations as one binary16 term per token); same parameters,
+// grid and block, dynamic shared memory gemv_mt_lds_bytes(type) + GEMV_MT_X16_LDS_EXTRA
+GEMV_MT_ENTRY(q4_k_gemv_mt16_f32, MtQ4Kx16)
+GEMV_MT_ENTRY(q5_k_gemv_mt16_f32, MtQ5Kx16)
+GEMV_MT_ENTRY(q6_k_gemv_mt16_f32, MtQ6Kx16)
 
 // (w, image, partial_ids, partial_values, in_dim, out_dim, tokens): the output head's arg-max for 2..8 tokens in one pass
 // over the weights. Grid, block and dynamic shared memory as q4_k_gemv_mt_f32 | q6_k_gemv_mt_f32 for out_dim rows;

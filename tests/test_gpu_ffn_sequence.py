@@ -85,11 +85,13 @@ def test_ffn_half_of_a_layer(gpu, oracle, hidden, ffn_dim, tokens):
 
 
 @pytest.mark.parametrize("hidden,ffn_dim,tokens,block", [(1024, 1536, 64, False), (2048, 768, 130, True), (4096, 12288, 64, True),
-                                                         (4096, 12288, 512, True), (4096, 12288, 512, False)])
+                                                         (4096, 12288, 512, True), (4096, 12288, 512, False),
+                                                         (4096, 12288, 16, True), (2048, 768, 9, False), (1024, 1536, 13, True)])
 def test_prefill_form_of_the_ffn_block(gpu, oracle, hidden, ffn_dim, tokens, block):
     """More tokens than the GEMM threshold: pack, gate | up GEMM with SwiGLU inside, pack, down GEMM with the residual inside
     (block: add + RMSNorm in front, as in a decoder layer). A sample of tokens against the CPU form to the fp16-path bar, and
-    the first eight tokens against the decode path of the same runner class (fp32 GEMVs) to the same bar."""
+    the first eight tokens against the decode path of the same runner class (fp32 GEMVs) to the same bar. Up to sixteen tokens
+    the block runs on the one-pass decode kernels with sixteen single-term tokens: the same bars."""
     rng = np.random.default_rng(5 * tokens + hidden)
     gate_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
     up_raw = synth.make_weights(rng, Q4_K, ffn_dim, hidden)
@@ -111,7 +113,7 @@ def test_prefill_form_of_the_ffn_block(gpu, oracle, hidden, ffn_dim, tokens, blo
             r_.read_outputs()
         assert runner._ws_x is not None and small._ws_x is None
         zero_f = np.zeros(ffn_dim, dtype=np.float32)
-        for tok in sorted({0, 1, 7, 31, 32, tokens // 2, tokens - 1}):
+        for tok in sorted(t_ for t_ in {0, 1, 7, 31, 32, tokens // 2, tokens - 1} if t_ < tokens):
             x = xs[tok * hidden:(tok + 1) * hidden]
             o = other[tok * hidden:(tok + 1) * hidden]
             r = x + o if block else o
@@ -131,7 +133,7 @@ def test_prefill_form_of_the_ffn_block(gpu, oracle, hidden, ffn_dim, tokens, blo
             lean.reset_sequence()
             lean.run_sequence()
             lean.read_outputs()
-            assert lean.combined is None and runner.combined is not None
+            assert (lean.combined is None) == (tokens > 16) and runner.combined is not None
             assert np.array_equal(lean.out, runner.out)
         finally:
             lean.close()

@@ -460,3 +460,81 @@ def test_a_ninth_stream_is_counted_and_a_captured_image_stays_pinned(gpu, oracle
         graph.close()
     for a in [w, xd] + outs:
         a.close()
+
+
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("in_dim,dims,tokens", [(4096, [12288], 16), (4096, [4096, 1024, 1024], 9), (2048, [130], 12), (12288, [4096], 16),
+                                                (1024, [48, 1000], 11), (5120, [257], 13), (256, [16], 1), (4096, [16 * 700], 10),
+                                                (2048, [32, 64, 7, 4000], 15)])
+def test_nine_to_sixteen_tokens_in_one_pass(gpu, oracle, t, in_dim, dims, tokens):
+    """cogni_gemv_pack16_dev + cogni_gemv_packed16_dev: the one-pass kernels with sixteen single-term tokens. The activations
+    are rounded to binary16 (the prefill GEMM's precision class) and everything behind that is exact codes and fp32 sums, so
+    the result is held to the one-pass bars against the CPU form of the rounded activations (2e-5 of a token's largest output);
+    resident and streamed operands, rows that do not fill their k-slices, lists, row counts that are no multiple of 16,
+    workgroups that walk row groups, a single token."""
+    rng = np.random.default_rng(in_dim + 31 * tokens + sum(dims) + int(t))
+    raws = [synth.make_weights(rng, t, d, in_dim) for d in dims]
+    x = synth.make_activations(rng, tokens, in_dim)
+    x16 = x.astype(np.float16).astype(np.float32)
+    image = DevArray(np.full(quant.gemv_image_bytes(t, in_dim, 8), 0xFF, dtype=np.uint8))
+    xd, wd = DevArray(x), [DevArray(r) for r in raws]
+    outs = [DevArray(np.full(tokens * d, np.float32(-9.0))) for d in dims]
+    quant.gemv_pack16_dev(xd.ptr, t, in_dim, tokens, image.ptr)
+    quant.gemv_packed16_dev([w.ptr for w in wd], t, image.ptr, [o.ptr for o in outs], dims, in_dim, tokens)
+    for raw, o, d in zip(raws, outs, dims):
+        want, tol = oracle_rows(oracle, raw, x16, in_dim, d, tokens, t)
+        assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, "type %d in=%d M=%d rows=%d" % (t, in_dim, tokens, d))
+    with pytest.raises(quant.QuantError, match="1..16 tokens"):
+        quant.gemv_pack16_dev(xd.ptr, t, in_dim, 17, image.ptr)
+    with pytest.raises(quant.QuantError, match="Q4_K, Q5_K or Q6_K"):
+        quant.gemv_packed16_dev([w.ptr for w in wd], Q8_0, image.ptr, [o.ptr for o in outs], dims, in_dim, tokens)
+    # a residual with a single matrix
+    res = rng.standard_normal(tokens * dims[0]).astype(np.float32)
+    rd, o2 = DevArray(res), DevArray(nbytes=4 * tokens * dims[0])
+    quant.gemv_packed16_dev([wd[0].ptr], t, image.ptr, [o2.ptr], [dims[0]], in_dim, tokens, rd.ptr)
+    assert np.array_equal(o2.read(np.float32, tokens * dims[0]), outs[0].read(np.float32, tokens * dims[0]) + res)
+    if len(dims) > 1:
+        with pytest.raises(quant.QuantError, match="a residual goes with a single matrix"):
+            quant.gemv_packed16_dev([w.ptr for w in wd], t, image.ptr, [o.ptr for o in outs], dims, in_dim, tokens, rd.ptr)
+    rd.close()
+    o2.close()
+    for a in [image, xd] + wd + outs:
+        a.close()
+
+
+def test_router_sends_nine_to_sixteen_tokens_to_the_one_pass_kernels(gpu):
+    """cogni_matmul_dev between the GEMM threshold and sixteen tokens without a bias: the bits of cogni_gemv_pack16_dev +
+    cogni_gemv_packed16_dev (Q4_K; Q6_K the same path); with a bias or with seventeen tokens it stays on the GEMM."""
+    rng = np.random.default_rng(77)
+    in_dim, out_dim = 2048, 520
+    raw = synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    raw6 = synth.make_weights(rng, Q6_K, out_dim, in_dim)
+    bias = rng.standard_normal(out_dim).astype(np.float32)
+    w, w6, bd = DevArray(raw), DevArray(raw6), DevArray(bias)
+    for tokens in (9, 16, 17):
+        x = synth.make_activations(rng, tokens, in_dim)
+        xd = DevArray(x)
+        wsb = quant.gemm_workspace_bytes(Q4_K, in_dim, tokens, out_dim)
+        ws, img = DevArray(nbytes=wsb), DevArray(nbytes=quant.gemv_image_bytes(Q4_K, in_dim, 8))
+        routed, direct, gemm, biased = (DevArray(nbytes=4 * tokens * out_dim) for _ in range(4))
+        quant.matmul_dev(w.ptr, Q4_K, xd.ptr, routed.ptr, in_dim, out_dim, tokens, ws.ptr, wsb)
+        quant.gemm_dev(w.ptr, Q4_K, xd.ptr, gemm.ptr, in_dim, out_dim, tokens, ws.ptr, wsb)
+        r, g = routed.read(np.float32, tokens * out_dim), gemm.read(np.float32, tokens * out_dim)
+        if tokens <= 16:
+            quant.gemv_pack16_dev(xd.ptr, Q4_K, in_dim, tokens, img.ptr)
+            quant.gemv_packed16_dev([w.ptr], Q4_K, img.ptr, [direct.ptr], [out_dim], in_dim, tokens)
+            assert np.array_equal(r, direct.read(np.float32, tokens * out_dim))
+            assert not np.array_equal(r, g) and np.max(np.abs(r - g)) <= 2e-3 * np.max(np.abs(g))
+            quant.matmul_dev(w.ptr, Q4_K, xd.ptr, biased.ptr, in_dim, out_dim, tokens, ws.ptr, wsb, bd.ptr)
+            want = (g.reshape(tokens, out_dim) + bias).reshape(-1)
+            assert np.max(np.abs(biased.read(np.float32, tokens * out_dim) - want)) <= 1e-5 * np.max(np.abs(want))
+        else:
+            assert np.array_equal(r, g)
+        quant.matmul_dev(w6.ptr, Q6_K, xd.ptr, routed.ptr, in_dim, out_dim, tokens, ws.ptr, wsb)
+        quant.gemm_dev(w6.ptr, Q6_K, xd.ptr, gemm.ptr, in_dim, out_dim, tokens, ws.ptr, wsb)
+        r6, g6 = routed.read(np.float32, tokens * out_dim), gemm.read(np.float32, tokens * out_dim)
+        assert (not np.array_equal(r6, g6) and np.max(np.abs(r6 - g6)) <= 2e-3 * np.max(np.abs(g6))) if tokens <= 16 else np.array_equal(r6, g6)
+        for a in (xd, ws, img, routed, direct, gemm, biased):
+            a.close()
+    for a in (w, w6, bd):
+        a.close()

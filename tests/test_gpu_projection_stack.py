@@ -48,10 +48,11 @@ def test_stack_matches_oracle(gpu, oracle, weights, tokens, threshold):
         stream.close()
 
 
-@pytest.mark.parametrize("tokens", [11, 64, 200])
+@pytest.mark.parametrize("tokens", [11, 16, 64, 200])
 def test_prefill_route_of_the_stack(gpu, oracle, weights, tokens):
     """More tokens than the router's threshold: every distinct input packed once, every projection one GEMM over all the
-    tokens (k-split where a projection has few tiles). Each projection against the oracle on the input it consumed, to
+    tokens (k-split where a projection has few tiles; lists of projections that share their input in one launch; up to sixteen
+    tokens the Q4_K projections on the one-pass kernels with sixteen single-term tokens). Each projection against the oracle on the input it consumed, to
     the fp16-path bar; the active-token prefix below the threshold falls back to the decode kernels."""
     rng = np.random.default_rng(1000 + tokens)
     xs = synth.make_activations(rng, tokens, weights.hidden)
