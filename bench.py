@@ -671,9 +671,33 @@ def main():
                 tokens, layers[0].raw_bytes, steps, r["us"], rec["gbps"], rec["frac_hbm"], r1["us"]))
         for r_ in runners:
             r_.close()
+    # sixteen tokens through the router: between the GEMM threshold and sixteen tokens cogni_matmul_dev takes the one-pass decode
+    # kernels with sixteen single-term tokens (image + kernel), the GEMM's precision class
+    mraw = synth.make_weights(rng, Q4_K, 12288, 4096)
+    mcopies = int(max(2, min(24, -(-int(1.2 * LLC_BYTES) // mraw.nbytes))))
+    mbufs = []
+    for c in range(mcopies):
+        b = hip.DeviceBuffer(mraw.nbytes)
+        hip.copy_htod(b.ptr, mraw if c == 0 else np.roll(mraw, 4096 * c + 17), mraw.nbytes, "w")
+        mbufs.append(b)
+    mx = synth.make_activations(rng, 16, 4096)
+    mwsb = quant.gemm_workspace_bytes(Q4_K, 4096, 16, 12288)
+    mdev = [hip.DeviceBuffer(n) for n in (mx.nbytes, 4 * 16 * 12288, mwsb)]
+    hip.copy_htod(mdev[0].ptr, mx, mx.nbytes, "x")
+
+    def m16(copy, st):
+        quant.matmul_dev(mbufs[copy].ptr, Q4_K, mdev[0].ptr, mdev[1].ptr, 4096, 12288, 16, mdev[2].ptr, mwsb, 0, st.handle)
+    r = measure(hip, stream, Rotating(m16, mcopies, mraw.nbytes), max(5, min(100, args.steps)), min(5, args.warmup))
+    m16_bytes = mraw.nbytes + 4 * 16 * (4096 + 12288)
+    rec = gemv_record(r, m16_bytes)
+    rec["launches"] = "pack_x_mt16_q4k_f16, q4_k_gemv_mt16_f32"
+    cases["q4_k matmul 12288x4096 M=16 (router: sixteen tokens in one pass)"] = rec
+    log("case=q4_k matmul M=16\nhip_us=%.3f\ngbps_hbm=%.1f\nfrac_hbm=%.4f\n" % (r["us"], rec["gbps"], rec["frac_hbm"]))
+    for b in mbufs + mdev:
+        b.close()
     # the same stack beyond the GEMM threshold (its prefill route): x packed once, q | k | v | gate | up as one list GEMM, o and
     # the Q6_K down projection behind their own packs
-    for tokens in (64, 512):
+    for tokens in (16, 64, 512):
         xs = rng.uniform(-1.0, 1.0, tokens * layers[0].hidden).astype(np.float32)
         runners = [QwenProjectionStackRunner.from_weights(w, tokens, xs) for w in layers]
         for r_ in runners:
@@ -689,7 +713,8 @@ def main():
         cases["cfg5 projection stack prefill M=%d" % tokens] = {
             "us": round(r["us"], 2), "tflops": round(pflops / r["us"] / 1e6, 1),
             "frac_mfma_f16": round(pflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "flops": pflops, "steps": steps,
-            "launches": "pack x, list GEMM q|k|v|gate|up, pack q, o GEMM, pack gate, Q6_K down GEMM (+ plane sums where the k range is split)"}
+            "launches": ("images of x, q and gate for sixteen single-term tokens; q|k|v, gate|up, o, down on the one-pass decode kernels" if tokens <= 16 else
+                         "pack x, list GEMM q|k|v|gate|up, pack q, o GEMM, pack gate, Q6_K down GEMM (+ plane sums where the k range is split)")}
         log("case=projection stack prefill\ntokens=%d\nhip_us=%.2f\ntflops=%.1f\nfrac_mfma_f16_peak=%.4f\n" % (
             tokens, r["us"], pflops / r["us"] / 1e6, pflops / r["us"] / 1e6 / MFMA_F16_PEAK_TFLOPS))
         for r_ in runners:
