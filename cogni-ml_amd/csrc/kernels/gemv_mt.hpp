@@ -10,6 +10,10 @@
 //   q4_k_gemv_mt_f32 | q5_k_gemv_mt_f32 | q6_k_gemv_mt_f32 | q8_0_gemv_mt_f32 (w0, w1, w2, image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens)
 //     (Q5_K and Q8_0 read the image pack_x_mt_q4k_f16 writes)
 //     block 512 (8 wavefronts), grid and dynamic shared memory from gemv_config.h (gemv_mt_grid, gemv_mt_lds_bytes).
+//   pack_x_mt16_q4k_f16 | pack_x_mt16_q6k_f16 and q4_k_gemv_mt16_f32 | q5_k_gemv_mt16_f32 | q6_k_gemv_mt16_f32 (same parameters)
+//     the same for up to sixteen tokens, each as ONE binary16 term (x rounded to half: the precision class of the prefill GEMM,
+//     which these kernels stand in for between 9 and 16 tokens); grid 4 * gemv_mt_padded_sb(in_dim) for the pack, shared memory
+//     gemv_mt_lds_bytes + GEMV_MT_X16_LDS_EXTRA for the GEMV.
 //     rows1 / rows2 may be 0 (then w1 / w2 / out1 / out2 are not read); residual (may be null) belongs to the first
 //     matrix. Row counts of all but the last matrix present must be multiples of 16. in_dim must be a multiple of 256
 //     up to 12288 (8 k-slices of 1..6 super-blocks; see "Rows that are not a multiple of 2048 values" below). out_i rows at stride rows_i (the reference's multi-token kernel
