@@ -127,7 +127,7 @@ class FFNSequenceRunner:
 
     def _launch_prefill16(self, count):
         """9..16 tokens: every projection in one pass over its weights on the decode kernels with sixteen single-term tokens
-        (the GEMM's precision class at half its time): norm, image of x, gate | up as one list, SwiGLU, image of the products
+        (the GEMM's precision class at half its time): norm, image of x, gate | up | SwiGLU in one launch, image of the products
         in the down matrix's order, down with the residual."""
         st = hip.current_stream_handle()
         h, f = self.hidden, self.ffn_dim
@@ -136,9 +136,13 @@ class FFNSequenceRunner:
             quant.add_rmsnorm_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, self._normed.ptr, h, count, self._eps, st)
             x = self._normed.ptr
         quant.gemv_pack16_dev(x, TensorType.Q4_K, h, count, self._img16_x.ptr, st)
-        quant.gemv_packed16_dev([self._w["gate"].ptr, self._w["up"].ptr], TensorType.Q4_K, self._img16_x.ptr,
-                                [self._gate.ptr, self._up.ptr], [f, f], h, count, 0, st)
-        quant.swiglu_dev(self._gate.ptr, self._up.ptr, self._act.ptr, count * f, st)
+        if f % 16 == 0:
+            quant.gemv_packed16_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, self._img16_x.ptr, self._act.ptr,
+                                           h, f, count, st)
+        else:
+            quant.gemv_packed16_dev([self._w["gate"].ptr, self._w["up"].ptr], TensorType.Q4_K, self._img16_x.ptr,
+                                    [self._gate.ptr, self._up.ptr], [f, f], h, count, 0, st)
+            quant.swiglu_dev(self._gate.ptr, self._up.ptr, self._act.ptr, count * f, st)
         quant.gemv_pack16_dev(self._act.ptr, self.down_type, f, count, self._img16_act.ptr, st)
         quant.gemv_packed16_dev([self._w["down"].ptr], self.down_type, self._img16_act.ptr, [self._out.ptr], [h], f, count,
                                 self._res.ptr if self._res is not None else 0, st)

@@ -335,6 +335,13 @@ def gemv_packed16_dev(w_ptrs, w_type, image_ptr, out_ptrs, out_dims, in_dim, tok
                                              ctypes.c_uint32(in_dim), ctypes.c_uint32(tokens), stream))
 
 
+def gemv_packed16_swiglu_dev(w_gate_ptr, w_up_ptr, w_type, image_ptr, out_ptr, in_dim, out_dim, tokens, stream=None):
+    """silu(gate . x) * (up . x) for up to sixteen tokens against a sixteen-token image (Q4_K), one pass over both matrices."""
+    _check(hip.lib().cogni_gemv_packed16_swiglu_dev(ctypes.c_uint64(w_gate_ptr), ctypes.c_uint64(w_up_ptr), ctypes.c_uint32(int(w_type)),
+                                                    ctypes.c_uint64(image_ptr), ctypes.c_uint64(out_ptr), ctypes.c_uint32(in_dim),
+                                                    ctypes.c_uint32(out_dim), ctypes.c_uint32(tokens), stream))
+
+
 def gemm_packed_many_dev(w_ptrs, w_type, workspace_ptr, workspace_bytes, out_ptrs, out_dims, in_dim, tokens, stream=None):
     """One GEMM launch for up to six matrices of one type and row length against the same packed activations (no k split)."""
     n = len(w_ptrs)

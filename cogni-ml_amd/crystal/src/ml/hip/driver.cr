@@ -117,6 +117,8 @@ lib LibCogniHIP
   fun cogni_gemv_pack16_dev(x : UInt64, w_type : UInt32, in_dim : UInt32, tokens : UInt32, image : UInt64, stream : Void*) : Int32
   fun cogni_gemv_packed16_dev(w_raw : UInt64*, w_type : UInt32, image : UInt64, residual : UInt64, out : UInt64*, out_dims : UInt32*,
                               count : UInt32, in_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
+  fun cogni_gemv_packed16_swiglu_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, image : UInt64, out : UInt64, in_dim : UInt32,
+                                     out_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemm_packed_many_dev(w_raw : UInt64*, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT, outs : UInt64*,
                                  out_dims : UInt32*, count : UInt32, in_dim : UInt32, tokens : UInt32, stream : Void*) : Int32
   fun cogni_gemm_packed_swiglu_pack_dev(w_gate : UInt64, w_up : UInt64, w_type : UInt32, workspace : UInt64, workspace_bytes : LibC::SizeT,

@@ -486,6 +486,19 @@ int cogni_gemv_packed16_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t ima
   return 0;
 }
 
+int cogni_gemv_packed16_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t image, uint64_t out, uint32_t in_dim,
+                                   uint32_t out_dim, uint32_t tokens, void* stream) {
+  const char* who = "cogni_gemv_packed16_swiglu_dev";
+  if (!w_gate || !w_up || !image || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null device pointer");
+  if (out_dim == 0 || out_dim > 0x7FFFFFFFu) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": bad out_dim");
+  if (w_type != COGNI_TYPE_Q4_K || !gemv16_shape(w_type, in_dim, tokens))
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": Q4_K, 1..16 tokens, in_dim a multiple of 256 up to 12288");
+  const uint32_t groups = (out_dim + 15) / 16;
+  void* params[] = {&w_gate, &w_up, &image, &out, &in_dim, &out_dim, &tokens};
+  return launch("q4_k_gemv_mt16_swiglu_f32", groups < 256u ? groups : 256u, GEMV_MT_WAVES * 64,
+                gemv_mt_lds_bytes(w_type) + GEMV_MT_X16_LDS_EXTRA, params, stream);
+}
+
 int cogni_gemv_packed_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t image, uint64_t out, uint32_t in_dim,
                                  uint32_t out_dim, uint32_t tokens, void* stream) {
   if (!w_gate || !w_up || !image || !out) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_packed_swiglu_dev: null device pointer");

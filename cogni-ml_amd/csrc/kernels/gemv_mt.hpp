@@ -613,7 +613,7 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
                                              u32* __restrict__ top_ids = nullptr) {
   constexpr bool STREAM = SBW > 2;
   constexpr int NTOK = F::NTOK;   // token rows of the partial sums: 8, or 16 single-term tokens
-  static_assert(NTOK == 8 || (NTOK == 16 && !SWIGLU && !TOP1), "sixteen tokens: plain rows only");
+  static_assert(NTOK == 8 || (NTOK == 16 && !TOP1), "sixteen tokens: rows or SwiGLU, no top-1");
   static_assert(!TOP1 || (!SWIGLU && T * 16 * GEMV_MT_MAX_TOKENS <= GEMV_MT_WAVES * 64), "TOP1: a thread owns one (tile, token, row) of a row group");
   static_assert(!SWIGLU || T == (STREAM ? 1 : 2), "SWIGLU pairs a gate tile with an up tile");
   static_assert(!STREAM || T == 1, "streamed operands: one tile per wavefront");
@@ -728,8 +728,8 @@ __device__ __forceinline__ void gemv_mt_core(const MtArgs& a, const uint8_t* __r
         float g = 0.f, u = 0.f;
 #pragma unroll
         for (u32 k = 0; k < GEMV_MT_WAVES; k++) {
-          g += part[((k * GEMV_MT_TMAX + 0) * 8 + m) * 16 + r];
-          u += part[((k * GEMV_MT_TMAX + 1) * 8 + m) * 16 + r];
+          g += part[((k * GEMV_MT_TMAX + 0) * NTOK + m) * 16 + r];
+          u += part[((k * GEMV_MT_TMAX + 1) * NTOK + m) * 16 + r];
         }
         const u32 row = grp * 16 + r;
         if (row < a.rows[0]) a.out[0][(size_t)m * a.rows[0] + row] = swiglu_one(g, u);
@@ -955,15 +955,25 @@ GEMV_MT_TOP1_ENTRY(q6_k_gemv_mt_top1_partial_f32, MtQ6K)
 // (w_gate, w_up, image, out, in_dim, out_dim, tokens): out[m][o] = silu(gate . x) * (up . x); block 512, grid = min(256,
 // ceil(out_dim / 16)), dynamic shared memory as q4_k_gemv_mt_f32. The parameter list of q4_k_dual_gemv_swiglu_f32 with the
 // image in the place of x and the token count behind.
-extern "C" __global__ __launch_bounds__(GEMV_MT_WAVES * 64) void q4_k_gemv_mt_swiglu_f32(
-    const uint8_t* w_gate, const uint8_t* w_up, const uint8_t* image, float* out, u32 in_dim, u32 out_dim, u32 tokens) {
+template <class F>
+__device__ __forceinline__ void gemv_mt_swiglu_dispatch(const uint8_t* w_gate, const uint8_t* w_up, const uint8_t* image, float* out,
+                                                        u32 in_dim, u32 out_dim, u32 tokens) {
   const MtArgs a = {{w_gate, w_up, nullptr}, {out, nullptr, nullptr}, {out_dim, out_dim, 0u}};
   switch (gemv_mt_padded_sb(in_dim) >> 3) {
-    case 1: gemv_mt_core<MtQ4K, 1, 2, true>(a, image, nullptr, in_dim, tokens); break;
-    case 2: gemv_mt_core<MtQ4K, 2, 2, true>(a, image, nullptr, in_dim, tokens); break;
-    case 3: gemv_mt_core<MtQ4K, 3, 1, true>(a, image, nullptr, in_dim, tokens); break;
-    case 4: gemv_mt_core<MtQ4K, 4, 1, true>(a, image, nullptr, in_dim, tokens); break;
-    case 5: gemv_mt_core<MtQ4K, 5, 1, true>(a, image, nullptr, in_dim, tokens); break;
-    default: gemv_mt_core<MtQ4K, 6, 1, true>(a, image, nullptr, in_dim, tokens); break;
+    case 1: gemv_mt_core<F, 1, 2, true>(a, image, nullptr, in_dim, tokens); break;
+    case 2: gemv_mt_core<F, 2, 2, true>(a, image, nullptr, in_dim, tokens); break;
+    case 3: gemv_mt_core<F, 3, 1, true>(a, image, nullptr, in_dim, tokens); break;
+    case 4: gemv_mt_core<F, 4, 1, true>(a, image, nullptr, in_dim, tokens); break;
+    case 5: gemv_mt_core<F, 5, 1, true>(a, image, nullptr, in_dim, tokens); break;
+    default: gemv_mt_core<F, 6, 1, true>(a, image, nullptr, in_dim, tokens); break;
   }
+}
+extern "C" __global__ __launch_bounds__(GEMV_MT_WAVES * 64) void q4_k_gemv_mt_swiglu_f32(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint8_t* image, float* out, u32 in_dim, u32 out_dim, u32 tokens) {
+  gemv_mt_swiglu_dispatch<MtQ4K>(w_gate, w_up, image, out, in_dim, out_dim, tokens);
+}
+// the same against the image of pack_x_mt16_q4k_f16, up to sixteen tokens (shared memory + GEMV_MT_X16_LDS_EXTRA)
+extern "C" __global__ __launch_bounds__(GEMV_MT_WAVES * 64) void q4_k_gemv_mt16_swiglu_f32(
+    const uint8_t* w_gate, const uint8_t* w_up, const uint8_t* image, float* out, u32 in_dim, u32 out_dim, u32 tokens) {
+  gemv_mt_swiglu_dispatch<MtQ4Kx16>(w_gate, w_up, image, out, in_dim, out_dim, tokens);
 }

@@ -202,6 +202,11 @@ int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image
  * shared memory). The reference has no counterpart: its router sends every M > 8 to the prefill GEMM
  * (src/ml/gguf/qwen35_cpu.cr:1478-1490); cogni_matmul_dev takes this path by itself for 9..16 tokens without a bias. */
 int cogni_gemv_pack16_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t image, void* stream);
+/* (cogni_gemv_packed16_swiglu_dev, below: gate | up | SwiGLU against the same image, as cogni_gemv_packed_swiglu_dev does for up
+ * to eight tokens - kernel "q4_k_gemv_mt16_swiglu_f32", the parameters of "q4_k_gemv_mt_swiglu_f32"; the bits of
+ * cogni_gemv_packed16_dev on the pair followed by cogni_swiglu_dev) */
+int cogni_gemv_packed16_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t image, uint64_t out, uint32_t in_dim,
+                                   uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemv_packed16_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,
                             const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream);
 /* The gate and up projections and the SwiGLU against an image, one launch:

@@ -538,3 +538,25 @@ def test_router_sends_nine_to_sixteen_tokens_to_the_one_pass_kernels(gpu):
             a.close()
     for a in (w, w6, bd):
         a.close()
+
+
+@pytest.mark.parametrize("in_dim,out_dim,tokens", [(4096, 12288, 16), (2048, 130, 9), (12288, 48, 12), (1024, 1000, 11), (6144, 40, 10)])
+def test_swiglu_for_nine_to_sixteen_tokens(gpu, in_dim, out_dim, tokens):
+    """cogni_gemv_packed16_swiglu_dev: gate | up | SwiGLU against a sixteen-token image - the bits of cogni_gemv_packed16_dev on
+    the pair followed by cogni_swiglu_dev (resident and streamed operands, row counts that are no multiple of 16)."""
+    rng = np.random.default_rng(in_dim + out_dim + tokens)
+    raw_g, raw_u = synth.make_weights(rng, Q4_K, out_dim, in_dim), synth.make_weights(rng, Q4_K, out_dim, in_dim)
+    x = synth.make_activations(rng, tokens, in_dim)
+    n = tokens * out_dim
+    wg, wu, xd = DevArray(raw_g), DevArray(raw_u), DevArray(x)
+    image = DevArray(nbytes=quant.gemv_image_bytes(Q4_K, in_dim, 8))
+    g, u, two_step, fused = DevArray(nbytes=4 * n), DevArray(nbytes=4 * n), DevArray(nbytes=4 * n), DevArray(np.full(n, np.float32(5.0)))
+    quant.gemv_pack16_dev(xd.ptr, Q4_K, in_dim, tokens, image.ptr)
+    quant.gemv_packed16_dev([wg.ptr, wu.ptr], Q4_K, image.ptr, [g.ptr, u.ptr], [out_dim, out_dim], in_dim, tokens)
+    quant.swiglu_dev(g.ptr, u.ptr, two_step.ptr, n)
+    quant.gemv_packed16_swiglu_dev(wg.ptr, wu.ptr, Q4_K, image.ptr, fused.ptr, in_dim, out_dim, tokens)
+    assert np.array_equal(fused.read(np.float32, n), two_step.read(np.float32, n))
+    with pytest.raises(quant.QuantError, match="Q4_K, 1..16 tokens"):
+        quant.gemv_packed16_swiglu_dev(wg.ptr, wu.ptr, Q5_K, image.ptr, fused.ptr, in_dim, out_dim, tokens)
+    for a in (wg, wu, xd, image, g, u, two_step, fused):
+        a.close()
