@@ -132,10 +132,15 @@ class FFNSequenceRunner:
         st = hip.current_stream_handle()
         h, f = self.hidden, self.ffn_dim
         x = self._x.ptr
-        if self._norm is not None:
-            quant.add_rmsnorm_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, self._normed.ptr, h, count, self._eps, st)
-            x = self._normed.ptr
-        quant.gemv_pack16_dev(x, TensorType.Q4_K, h, count, self._img16_x.ptr, st)
+        if self._norm is not None and h <= 4096:
+            # r = x + add, and rmsnorm(r) written straight as the image gate | up read
+            quant.add_rmsnorm_pack16_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, 0, TensorType.Q4_K, self._img16_x.ptr, h,
+                                         count, self._eps, st)
+        else:
+            if self._norm is not None:
+                quant.add_rmsnorm_dev(x, self._add.ptr, self._norm.ptr, self._res.ptr, self._normed.ptr, h, count, self._eps, st)
+                x = self._normed.ptr
+            quant.gemv_pack16_dev(x, TensorType.Q4_K, h, count, self._img16_x.ptr, st)
         if f % 16 == 0:
             quant.gemv_packed16_swiglu_dev(self._w["gate"].ptr, self._w["up"].ptr, TensorType.Q4_K, self._img16_x.ptr, self._act.ptr,
                                            h, f, count, st)

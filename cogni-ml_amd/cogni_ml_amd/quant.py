@@ -244,6 +244,22 @@ def add_rmsnorm_pack_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_
                                                 ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
 
 
+def rmsnorm_pack16_dev(x_ptr, norm_ptr, out_ptr, w_type, image_ptr, dim, tokens, eps=1.0e-6, stream=None):
+    """rmsnorm_dev that writes the normalised rows as the image of the sixteen-token one-pass kernels (out_ptr may be 0)."""
+    _check(hip.lib().cogni_rmsnorm_pack16_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(out_ptr),
+                                              ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr), ctypes.c_uint32(dim),
+                                              ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
+
+def add_rmsnorm_pack16_dev(x_ptr, add_ptr, norm_ptr, residual_out_ptr, normed_out_ptr, w_type, image_ptr, dim, tokens, eps=1.0e-6,
+                           stream=None):
+    """add_rmsnorm_dev that writes the normalised rows as the image of the sixteen-token one-pass kernels (normed_out_ptr may be 0)."""
+    _check(hip.lib().cogni_add_rmsnorm_pack16_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(add_ptr), ctypes.c_uint64(norm_ptr),
+                                                  ctypes.c_uint64(residual_out_ptr), ctypes.c_uint64(normed_out_ptr),
+                                                  ctypes.c_uint32(int(w_type)), ctypes.c_uint64(image_ptr), ctypes.c_uint32(dim),
+                                                  ctypes.c_uint32(tokens), ctypes.c_float(eps), stream))
+
+
 def rmsnorm_gemm_pack_dev(x_ptr, norm_ptr, out_ptr, w_type, workspace_ptr, workspace_bytes, dim, tokens, eps=1.0e-6, stream=None):
     """rmsnorm_dev whose rows leave as the packed activations of the prefill GEMMs (what gemm_pack_dev would write); out_ptr may be 0."""
     _check(hip.lib().cogni_rmsnorm_gemm_pack_dev(ctypes.c_uint64(x_ptr), ctypes.c_uint64(norm_ptr), ctypes.c_uint64(out_ptr),

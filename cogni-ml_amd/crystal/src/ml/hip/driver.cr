@@ -87,6 +87,11 @@ lib LibCogniHIP
   fun cogni_add_rmsnorm_pack_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,
                                  w_type : UInt32, image : UInt64, dim : UInt32, tokens : UInt32, eps : Float32,
                                  stream : Void*) : Int32
+  fun cogni_rmsnorm_pack16_dev(x : UInt64, norm : UInt64, out : UInt64, w_type : UInt32, image : UInt64, dim : UInt32,
+                               tokens : UInt32, eps : Float32, stream : Void*) : Int32
+  fun cogni_add_rmsnorm_pack16_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,
+                                   w_type : UInt32, image : UInt64, dim : UInt32, tokens : UInt32, eps : Float32,
+                                   stream : Void*) : Int32
   fun cogni_rmsnorm_gemm_pack_dev(x : UInt64, norm : UInt64, out : UInt64, w_type : UInt32, workspace : UInt64,
                                   workspace_bytes : LibC::SizeT, dim : UInt32, tokens : UInt32, eps : Float32, stream : Void*) : Int32
   fun cogni_add_rmsnorm_gemm_pack_dev(x : UInt64, add : UInt64, norm : UInt64, residual_out : UInt64, normed_out : UInt64,

@@ -998,6 +998,31 @@ int cogni_add_rmsnorm_pack_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t
   return launch(w_type == COGNI_TYPE_Q6_K ? "add_rmsnorm_pack_q6k_f32" : "add_rmsnorm_pack_q4k_f32", GEMV_MT_MAX_TOKENS, 256, 0, params, stream);
 }
 
+// the same norms in front of the sixteen-token one-pass kernels (the image of cogni_gemv_pack16_dev)
+static int norm_pack16_check(const char* who, uint32_t w_type, uint32_t dim, uint32_t tokens) {
+  if (!(w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q5_K || w_type == COGNI_TYPE_Q6_K) || tokens == 0 || tokens > 16 ||
+      !gemv_mt_supported(w_type, 2, dim) || dim > 4096u)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": needs 1..16 tokens of a Q4_K, Q5_K or Q6_K row length that is a multiple of 256 "
+                                                               "up to 4096 - got type " + type_name(w_type) + ", dim " + std::to_string(dim) +
+                                                ", " + std::to_string(tokens) + " tokens");
+  return 0;
+}
+int cogni_rmsnorm_pack16_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t w_type, uint64_t image, uint32_t dim, uint32_t tokens,
+                             float eps, void* stream) {
+  if (!x || !norm || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_rmsnorm_pack16_dev: null device pointer");
+  if (int rc = norm_pack16_check("cogni_rmsnorm_pack16_dev", w_type, dim, tokens)) return rc;
+  void* params[] = {&x, &norm, &out, &image, &dim, &tokens, &eps};
+  return launch(w_type == COGNI_TYPE_Q6_K ? "rmsnorm_pack_x16_q6k_f32" : "rmsnorm_pack_x16_q4k_f32", 16, 256, 0, params, stream);
+}
+int cogni_add_rmsnorm_pack16_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t w_type,
+                                 uint64_t image, uint32_t dim, uint32_t tokens, float eps, void* stream) {
+  if (!x || !add || !norm || !residual_out || !image)
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_add_rmsnorm_pack16_dev: null device pointer");
+  if (int rc = norm_pack16_check("cogni_add_rmsnorm_pack16_dev", w_type, dim, tokens)) return rc;
+  void* params[] = {&x, &add, &norm, &residual_out, &normed_out, &image, &dim, &tokens, &eps};
+  return launch(w_type == COGNI_TYPE_Q6_K ? "add_rmsnorm_pack_x16_q6k_f32" : "add_rmsnorm_pack_x16_q4k_f32", 16, 256, 0, params, stream);
+}
+
 int g_gemm_threshold = -1;   // -1: not resolved yet
 
 static bool gemm_type(uint32_t t) { return t == COGNI_TYPE_Q4_K || t == COGNI_TYPE_Q5_K || t == COGNI_TYPE_Q6_K; }

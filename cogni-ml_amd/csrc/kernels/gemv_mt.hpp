@@ -176,15 +176,9 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt_q4k_f16(const float*
 // 4 kg + (0,2,1,3) of the rounded values / 32 as hi (halves 0..3) and lo (halves 4..7) binary16 terms, zeros for kg >= 2.
 // (x, image, tokens <= 16, in_dim): block 256, grid 4 * gemv_mt_padded_sb(in_dim). |x| has to stay inside the binary16
 // range, as for the prefill GEMM.
-extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q4k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
-                                                                      u32 tokens, u32 in_dim) {
-  const u32 lane = threadIdx.x & 63;
-  const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const u32 nsb = in_dim >> 8, nsbp = gemv_mt_padded_sb(in_dim);
-  const u32 sb = unit >> 4, tok = unit & 15;
-  if (sb >= nsbp) return;
-  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (tok < tokens && sb < nsb) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+// One wavefront's share of that image: (token slot tok < 16, super-block sb) from the lane's four values v (zeros for a token or
+// super-block that is not there).
+__device__ __forceinline__ void mt_pack16_store_q4k(uint8_t* __restrict__ image, u32 nsbp, u32 sb, u32 tok, u32 lane, float4 v) {
   const _Float16 h0 = (_Float16)v.x, h1 = (_Float16)v.y, h2 = (_Float16)v.z, h3 = (_Float16)v.w;
   // element 4 l sits in instruction j = l / 8, k-group (l / 2) % 4, upper half of the lane's eight if l is odd (mt_pack_store_q4k)
   const u32 j = lane >> 3, kg = (lane >> 1) & 3;
@@ -204,9 +198,7 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q4k_f16(const floa
     ap[4] = zero ? (_Float16)0.0f : sl;
   }
 }
-
-// The same for the Q6_K order: sums of sub-blocks 4 kg .. 4 kg + 3 / 16 as hi (halves 0..3) and lo (halves 4..7).
-extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q6k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
+extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q4k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
                                                                       u32 tokens, u32 in_dim) {
   const u32 lane = threadIdx.x & 63;
   const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -215,6 +207,11 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q6k_f16(const floa
   if (sb >= nsbp) return;
   float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
   if (tok < tokens && sb < nsb) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  mt_pack16_store_q4k(image, nsbp, sb, tok, lane, v);
+}
+
+// The same for the Q6_K order: sums of sub-blocks 4 kg .. 4 kg + 3 / 16 as hi (halves 0..3) and lo (halves 4..7).
+__device__ __forceinline__ void mt_pack16_store_q6k(uint8_t* __restrict__ image, u32 nsbp, u32 sb, u32 tok, u32 lane, float4 v) {
   const _Float16 h0 = (_Float16)v.x, h1 = (_Float16)v.y, h2 = (_Float16)v.z, h3 = (_Float16)v.w;
   // element 4 l sits in sub-block s = l / 4, k-group l % 4 (mt_pack_store_q6k)
   const u32 s = lane >> 2, kg = lane & 3;
@@ -230,6 +227,17 @@ extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q6k_f16(const floa
     ap[0] = sh;
     ap[4] = sl;
   }
+}
+extern "C" __global__ __launch_bounds__(256) void pack_x_mt16_q6k_f16(const float* __restrict__ x, uint8_t* __restrict__ image,
+                                                                      u32 tokens, u32 in_dim) {
+  const u32 lane = threadIdx.x & 63;
+  const u32 unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const u32 nsb = in_dim >> 8, nsbp = gemv_mt_padded_sb(in_dim);
+  const u32 sb = unit >> 4, tok = unit & 15;
+  if (sb >= nsbp) return;
+  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tok < tokens && sb < nsb) __builtin_memcpy(&v, x + (size_t)tok * in_dim + (size_t)sb * 256 + 4 * lane, 16);
+  mt_pack16_store_q6k(image, nsbp, sb, tok, lane, v);
 }
 
 // Q6_K image: [super-block][sub-block pair p][lane = 16 kg + row][2 x 4 halves]: the halves of lane (kg, row = 2 token +

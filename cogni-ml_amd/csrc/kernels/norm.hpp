@@ -18,7 +18,8 @@
 #define NORM_BLOCK 256
 #define NORM_KEEP 4   // float4 a thread keeps across the reduction on the short-row path
 
-// IMG: 0 = no image, 12 = the Q4_K (and Q5_K) image, 14 = the Q6_K image. With an image the grid is the image's eight token
+// IMG: 0 = no image, 12 = the Q4_K (and Q5_K) image, 14 = the Q6_K image, 112 / 114 = the images for sixteen single-term tokens
+// (pack_x_mt16_q4k_f16 / pack_x_mt16_q6k_f16). With an image the grid is the image's eight (sixteen) token
 // slots, the workgroups of slots at and above `tokens` write the zeros of an absent token, dim is a multiple of 256 up to
 // 4096 (the short-row path), and `out` may be null (the normalised rows then exist only as the image).
 // GP: 0, or the packed GEMM activations in the Q4_K / Q5_K order (12) or the Q6_K order (14) behind `image`: the grid is the
@@ -69,7 +70,9 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
       const u32 lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
       for (u32 sb = from + wave; sb < gemv_mt_padded_sb(dim); sb += NORM_BLOCK / WAVE) {
         if constexpr (IMG == 14) mt_pack_store_q6k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
-        else mt_pack_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
+        else if constexpr (IMG == 12) mt_pack_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f), false);
+        else if constexpr (IMG == 114) mt_pack16_store_q6k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f));
+        else mt_pack16_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, lane, make_float4(0.f, 0.f, 0.f, 0.f));
       }
     }
   };
@@ -127,14 +130,16 @@ __device__ __forceinline__ void rmsnorm_core(const float* x, const float* __rest
           // (i < dim holds for whole wavefronts: dim is a multiple of 256)
           const u32 sb = 4u * (u32)k + (tid >> 6);
           if constexpr (IMG == 14) mt_pack_store_q6k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, tid & 63, o, true);
-          else mt_pack_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, tid & 63, o, true);
+          else if constexpr (IMG == 12) mt_pack_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, tid & 63, o, true);
+          else if constexpr (IMG == 114) mt_pack16_store_q6k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, tid & 63, o);
+          else mt_pack16_store_q4k(image, gemv_mt_padded_sb(dim), sb, blockIdx.x, tid & 63, o);
         }
       }
     }
     zero_image(dim >> 8);
     return;
   }
-  static_assert(IMG == 0 || IMG == 12 || IMG == 14, "image kinds");
+  static_assert(IMG == 0 || IMG == 12 || IMG == 14 || IMG == 112 || IMG == 114, "image kinds");
   static_assert(GP == 0 || GP == 12 || GP == 14, "packed layouts");
   if constexpr (IMG != 0 || GP != 0) return;   // (the host launches the pack forms for the short-row shapes only)
   if (vec) {
@@ -211,6 +216,10 @@ extern "C" __global__ __launch_bounds__(NORM_BLOCK) void add_rmsnorm_f32(const f
   }
 NORM_PACK_ENTRIES(q4k, 12)
 NORM_PACK_ENTRIES(q6k, 14)
+// the images of the sixteen-token kernels: rmsnorm_pack_x16_q4k_f32 | ..._x16_q6k_f32, add_rmsnorm_pack_x16_q4k_f32 | ..._x16_q6k_f32,
+// the same parameters, grid.x = 16
+NORM_PACK_ENTRIES(x16_q4k, 112)
+NORM_PACK_ENTRIES(x16_q6k, 114)
 
 // The same with the normalised rows written as the packed fp16 activations of the prefill GEMMs:
 //   rmsnorm_gemm_pack_q4k_f32 | rmsnorm_gemm_pack_q6k_f32 (x, norm, out | null, xp, dim, tokens, eps)

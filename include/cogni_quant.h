@@ -205,6 +205,14 @@ int cogni_gemv_pack16_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t
 /* (cogni_gemv_packed16_swiglu_dev, below: gate | up | SwiGLU against the same image, as cogni_gemv_packed_swiglu_dev does for up
  * to eight tokens - kernel "q4_k_gemv_mt16_swiglu_f32", the parameters of "q4_k_gemv_mt_swiglu_f32"; the bits of
  * cogni_gemv_packed16_dev on the pair followed by cogni_swiglu_dev) */
+/* (cogni_rmsnorm_pack16_dev, cogni_add_rmsnorm_pack16_dev: the norms that write this image themselves, as cogni_rmsnorm_pack_dev /
+ * cogni_add_rmsnorm_pack_dev write the eight-token one - 1..16 tokens, rows of a multiple of 256 up to 4096 values, byte for byte
+ * what cogni_gemv_pack16_dev makes of the normalised rows; kernels "rmsnorm_pack_x16_q4k_f32" | "rmsnorm_pack_x16_q6k_f32" and
+ * "add_rmsnorm_pack_x16_q4k_f32" | "add_rmsnorm_pack_x16_q6k_f32", the parameters of the eight-token ones, grid 16) */
+int cogni_rmsnorm_pack16_dev(uint64_t x, uint64_t norm, uint64_t out, uint32_t w_type, uint64_t image, uint32_t dim, uint32_t tokens,
+                             float eps, void* stream);
+int cogni_add_rmsnorm_pack16_dev(uint64_t x, uint64_t add, uint64_t norm, uint64_t residual_out, uint64_t normed_out, uint32_t w_type,
+                                 uint64_t image, uint32_t dim, uint32_t tokens, float eps, void* stream);
 int cogni_gemv_packed16_swiglu_dev(uint64_t w_gate, uint64_t w_up, uint32_t w_type, uint64_t image, uint64_t out, uint32_t in_dim,
                                    uint32_t out_dim, uint32_t tokens, void* stream);
 int cogni_gemv_packed16_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,

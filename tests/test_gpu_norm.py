@@ -173,3 +173,39 @@ def test_norm_gemm_pack_argument_errors(gpu):
     with pytest.raises(quant.QuantError, match="null device pointer"):
         quant.add_rmsnorm_gemm_pack_dev(p, p, p, 0, p, 12, p, n, 1024, 16)
     buf.close()
+
+
+@pytest.mark.parametrize("w_type", [12, 13, 14])
+@pytest.mark.parametrize("dim,tokens", [(4096, 16), (4096, 9), (2048, 12), (1024, 1), (2560, 13), (256, 16)])
+def test_norms_that_write_the_sixteen_token_image(gpu, w_type, dim, tokens):
+    """cogni_rmsnorm_pack16_dev / cogni_add_rmsnorm_pack16_dev: every byte of the image cogni_gemv_pack16_dev makes of the plain
+    norm's output (zeros for the absent tokens and the super-blocks past the row's end), the residual stream and, when asked
+    for, the normalised rows bit for bit the plain kernels'."""
+    rng = np.random.default_rng(dim + 17 * tokens + w_type)
+    x = (rng.standard_normal(tokens * dim) * 2.5).astype(np.float32)
+    add = rng.standard_normal(tokens * dim).astype(np.float32)
+    w = (1.0 + 0.1 * rng.standard_normal(dim)).astype(np.float32)
+    eps = 1.0e-6
+    nbytes = quant.gemv_image_bytes(w_type, dim, 8)
+    ff = np.full(nbytes, 0xFF, dtype=np.uint8)
+    xd, ad, wd = DevArray(x), DevArray(add), DevArray(w)
+    od, rd, nd, od2, rd2 = (DevArray(nbytes=x.nbytes) for _ in range(5))
+    i_ref, i_a, i_b = DevArray(ff), DevArray(ff), DevArray(ff)
+    try:
+        quant.rmsnorm_dev(xd.ptr, wd.ptr, od.ptr, dim, tokens, eps)
+        quant.gemv_pack16_dev(od.ptr, w_type, dim, tokens, i_ref.ptr)
+        quant.rmsnorm_pack16_dev(xd.ptr, wd.ptr, od2.ptr, w_type, i_a.ptr, dim, tokens, eps)
+        assert np.array_equal(i_a.read(np.uint8, nbytes), i_ref.read(np.uint8, nbytes))
+        assert np.array_equal(od2.read(np.float32, x.size), od.read(np.float32, x.size))
+        quant.add_rmsnorm_dev(xd.ptr, ad.ptr, wd.ptr, rd.ptr, nd.ptr, dim, tokens, eps)
+        quant.gemv_pack16_dev(nd.ptr, w_type, dim, tokens, i_ref.ptr)
+        quant.add_rmsnorm_pack16_dev(xd.ptr, ad.ptr, wd.ptr, rd2.ptr, 0, w_type, i_b.ptr, dim, tokens, eps)
+        assert np.array_equal(i_b.read(np.uint8, nbytes), i_ref.read(np.uint8, nbytes))
+        assert np.array_equal(rd2.read(np.float32, x.size), rd.read(np.float32, x.size))
+        with pytest.raises(quant.QuantError, match="1..16 tokens"):
+            quant.rmsnorm_pack16_dev(xd.ptr, wd.ptr, od2.ptr, w_type, i_a.ptr, dim, 17, eps)
+        with pytest.raises(quant.QuantError, match="1..16 tokens"):
+            quant.rmsnorm_pack16_dev(xd.ptr, wd.ptr, od2.ptr, 8, i_a.ptr, dim, tokens, eps)
+    finally:
+        for d in (xd, ad, wd, od, rd, nd, od2, rd2, i_ref, i_a, i_b):
+            d.close()
