@@ -445,12 +445,12 @@ int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image
 // Nine to sixteen tokens in one pass over the weights: the one-pass kernels with their sixteen activation rows as sixteen
 // tokens in one binary16 term each (the precision class of the prefill GEMM), Q4_K, Q5_K and Q6_K.
 static bool gemv16_shape(uint32_t w_type, uint32_t in_dim, uint32_t tokens) {
-  return (w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q5_K || w_type == COGNI_TYPE_Q6_K) && tokens >= 1 && tokens <= 16 &&
-         gemv_mt_supported(w_type, 2, in_dim);
+  return (w_type == COGNI_TYPE_Q4_K || w_type == COGNI_TYPE_Q5_K || w_type == COGNI_TYPE_Q6_K || w_type == COGNI_TYPE_Q8_0) && tokens >= 1 &&
+         tokens <= 16 && gemv_mt_supported(w_type, 2, in_dim);
 }
 int cogni_gemv_pack16_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t image, void* stream) {
   if (!gemv16_shape(w_type, in_dim, tokens))
-    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack16_dev: Q4_K, Q5_K or Q6_K, 1..16 tokens, in_dim a multiple of 256 up to 12288");
+    return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack16_dev: Q4_K, Q5_K, Q6_K or Q8_0, 1..16 tokens, in_dim a multiple of 256 up to 12288");
   if (!x || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, "cogni_gemv_pack16_dev: null device pointer");
   void* params[] = {&x, &image, &tokens, &in_dim};
   return launch(w_type == COGNI_TYPE_Q6_K ? "pack_x_mt16_q6k_f16" : "pack_x_mt16_q4k_f16", 4 * gemv_mt_padded_sb(in_dim), 256, 0, params, stream);
@@ -461,7 +461,7 @@ int cogni_gemv_packed16_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t ima
   if (!w_raw || !out || !out_dims || !image) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null argument");
   if (count == 0 || count > 8) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": count must be 1..8");
   if (!gemv16_shape(w_type, in_dim, tokens))
-    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": Q4_K, Q5_K or Q6_K, 1..16 tokens, in_dim a multiple of 256 up to 12288");
+    return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": Q4_K, Q5_K, Q6_K or Q8_0, 1..16 tokens, in_dim a multiple of 256 up to 12288");
   if (residual && count != 1) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": a residual goes with a single matrix");
   for (uint32_t i = 0; i < count; i++)
     if (!w_raw[i] || !out[i] || out_dims[i] == 0) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": null pointer or zero rows");
@@ -478,7 +478,8 @@ int cogni_gemv_packed16_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t ima
     }
     if (total > 0x7FFFFFFFull) return fail(COGNI_ERR_INVALID_ARGUMENT, std::string(who) + ": too many rows");
     void* params[] = {&w[0], &w[1], &w[2], &image, &none, &o[0], &o[1], &o[2], &in_dim, &rows[0], &rows[1], &rows[2], &tokens};
-    const int rc = launch(w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt16_f32" : (w_type == COGNI_TYPE_Q5_K ? "q5_k_gemv_mt16_f32" : "q4_k_gemv_mt16_f32"), gemv_mt_grid(w_type, in_dim, (uint32_t)total),
+    const char* kernel = w_type == COGNI_TYPE_Q6_K ? "q6_k_gemv_mt16_f32" : (w_type == COGNI_TYPE_Q5_K ? "q5_k_gemv_mt16_f32" : (w_type == COGNI_TYPE_Q8_0 ? "q8_0_gemv_mt16_f32" : "q4_k_gemv_mt16_f32"));
+    const int rc = launch(kernel, gemv_mt_grid(w_type, in_dim, (uint32_t)total),
                           GEMV_MT_WAVES * 64, gemv_mt_lds_bytes(w_type) + GEMV_MT_X16_LDS_EXTRA, params, stream);
     if (rc != 0) return rc;
     i0 += n;

@@ -10,7 +10,7 @@
 //   q4_k_gemv_mt_f32 | q5_k_gemv_mt_f32 | q6_k_gemv_mt_f32 | q8_0_gemv_mt_f32 (w0, w1, w2, image, residual, out0, out1, out2, in_dim, rows0, rows1, rows2, tokens)
 //     (Q5_K and Q8_0 read the image pack_x_mt_q4k_f16 writes)
 //     block 512 (8 wavefronts), grid and dynamic shared memory from gemv_config.h (gemv_mt_grid, gemv_mt_lds_bytes).
-//   pack_x_mt16_q4k_f16 | pack_x_mt16_q6k_f16 and q4_k_gemv_mt16_f32 | q5_k_gemv_mt16_f32 | q6_k_gemv_mt16_f32 (same parameters)
+//   pack_x_mt16_q4k_f16 | pack_x_mt16_q6k_f16 and q4_k_gemv_mt16_f32 | q5_k_ | q6_k_ | q8_0_gemv_mt16_f32 (same parameters)
 //     the same for up to sixteen tokens, each as ONE binary16 term (x rounded to half: the precision class of the prefill GEMM,
 //     which these kernels stand in for between 9 and 16 tokens); grid 4 * gemv_mt_padded_sb(in_dim) for the pack, shared memory
 //     gemv_mt_lds_bytes + GEMV_MT_X16_LDS_EXTRA for the GEMV.
@@ -445,9 +445,10 @@ typedef MtK45<true, true> MtQ5Kx16;
 // In LDS a row is its 272 bytes as they are: d of block j at 34 j, its codes at 34 j + 2. The codes of the odd blocks start
 // on a multiple of 4 (two dword reads); the even blocks' are 2 bytes off and come out of three dwords through
 // v_alignbyte_b32.
-struct MtQ80 {
+template <bool X16 = false>   // (X16: sixteen single-term tokens, as MtK45's; the image of pack_x_mt16_q4k_f16)
+struct MtQ80T {
   static constexpr unsigned TYPE = 8;
-  static constexpr int NTOK = 8;
+  static constexpr int NTOK = X16 ? 16 : 8;
   static constexpr int BB = 272, P = 17, NCOPY = 5, LAST = 16, NAUX = 1, NSLOT = 4, TMAX = 2;
   static constexpr u32 UNIT_BYTES = 16 * P * 16, AUX_SB_BYTES = 64 * 16;
   static __device__ __forceinline__ u32 piece_offset(u32 piece) { return piece * 16; }
@@ -493,15 +494,20 @@ struct MtQ80 {
     const u32 dA = w.kg == 0 ? (w.d[0] | (w.d[2] << 16)) : (w.d[4] | (w.d[6] << 16));
     const u32 dB = w.kg == 0 ? (w.d[1] | (w.d[3] << 16)) : (w.d[5] | (w.d[7] << 16));
     const mt_u32x2 db = w.kg < 2 ? (mt_u32x2){dA, dB} : (mt_u32x2){0u, 0u};
-    const mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), __builtin_bit_cast(mt_half4, db),
-                                                                (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    mt_float4 off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums), __builtin_bit_cast(mt_half4, db),
+                                                          (mt_float4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    if constexpr (X16)
+      off = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(mt_half4, ax.sums_lo), __builtin_bit_cast(mt_half4, db), off, 0, 0, 0);
 #pragma unroll
     for (int k = 0; k < 4; k++) {
       const float in = fmaf(MT_TWO_P24, sum[k], -4096.0f * off[k]);   // 128 * 2^5
-      acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
+      if constexpr (X16) acc[k] += in;
+      else acc[k] = fmaf(ax.fsc[k >> 1], in, acc[k]);
     }
   }
 };
+typedef MtQ80T<false> MtQ80;
+typedef MtQ80T<true> MtQ80x16;
 
 
 // Q6_K (210 B: ql[128], qh[64], scales:i8[16], d). Element 128 n + 32 k + l (half n, quarter k, l < 32) has its low four bits
@@ -940,6 +946,7 @@ GEMV_MT_ENTRY(q8_0_gemv_mt_f32, MtQ80)
 GEMV_MT_ENTRY(q4_k_gemv_mt16_f32, MtQ4Kx16)
 GEMV_MT_ENTRY(q5_k_gemv_mt16_f32, MtQ5Kx16)
 GEMV_MT_ENTRY(q6_k_gemv_mt16_f32, MtQ6Kx16)
+GEMV_MT_ENTRY(q8_0_gemv_mt16_f32, MtQ80x16)
 
 // (w, image, partial_ids, partial_values, in_dim, out_dim, tokens): the output head's arg-max for 2..8 tokens in one pass
 // over the weights. Grid, block and dynamic shared memory as q4_k_gemv_mt_f32 | q6_k_gemv_mt_f32 for out_dim rows;

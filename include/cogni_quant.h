@@ -191,16 +191,17 @@ int cogni_gemv_packed_launch_dims(uint32_t w_type, uint32_t in_dim, uint32_t tot
 int cogni_gemv_pack_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t image, void* stream);
 int cogni_gemv_packed_dev(const uint64_t* w_raw, uint32_t w_type, uint64_t image, uint64_t residual, const uint64_t* out,
                           const uint32_t* out_dims, uint32_t count, uint32_t in_dim, uint32_t tokens, void* stream);
-/* Nine to sixteen tokens in one pass over the weights (Q4_K, Q5_K, Q6_K): the one-pass kernels with their sixteen activation rows
+/* Nine to sixteen tokens in one pass over the weights (Q4_K, Q5_K, Q6_K, Q8_0): the one-pass kernels with their sixteen activation rows
  * as sixteen tokens in ONE binary16 term each instead of eight tokens x (hi, lo) - the precision class of the prefill GEMM (x
  * rounded to half, |x| < 65504; fp32 sums), at the cost of a decode launch where pack + GEMM + plane sum take twice as long.
  * cogni_gemv_pack16_dev writes the image (cogni_gemv_image_bytes(type, in_dim, 8) bytes: the same size; Q4_K and Q5_K
  * share one, Q6_K has its own; kernels "pack_x_mt16_q4k_f16" | "pack_x_mt16_q6k_f16" (x, image, tokens:u32, in_dim:u32), block
  * 256, grid 4 * ceil(in_dim / 2048) * 8); cogni_gemv_packed16_dev runs up to eight matrices of one type and row length
  * against it, three per launch, a [tokens][out_dim] residual (may be 0) with a single matrix (kernels "q4_k_gemv_mt16_f32" |
- * "q5_k_gemv_mt16_f32" | "q6_k_gemv_mt16_f32", parameters, grid and block of "<type>_gemv_mt_f32", 12 KiB more dynamic
+ * "q5_k_gemv_mt16_f32" | "q6_k_gemv_mt16_f32" | "q8_0_gemv_mt16_f32" - Q8_0 reads the Q4_K image -, parameters, grid and block of "<type>_gemv_mt_f32", 12 KiB more dynamic
  * shared memory). The reference has no counterpart: its router sends every M > 8 to the prefill GEMM
- * (src/ml/gguf/qwen35_cpu.cr:1478-1490); cogni_matmul_dev takes this path by itself for 9..16 tokens without a bias. */
+ * (src/ml/gguf/qwen35_cpu.cr:1478-1490); cogni_matmul_dev takes this path by itself for 9..16 tokens of a K-quant matrix without a bias (Q8_0, whose reference path stays in
+ * fp32 at every token count, only on request). */
 int cogni_gemv_pack16_dev(uint64_t x, uint32_t w_type, uint32_t in_dim, uint32_t tokens, uint64_t image, void* stream);
 /* (cogni_gemv_packed16_swiglu_dev, below: gate | up | SwiGLU against the same image, as cogni_gemv_packed_swiglu_dev does for up
  * to eight tokens - kernel "q4_k_gemv_mt16_swiglu_f32", the parameters of "q4_k_gemv_mt_swiglu_f32"; the bits of

@@ -462,7 +462,7 @@ def test_a_ninth_stream_is_counted_and_a_captured_image_stays_pinned(gpu, oracle
         a.close()
 
 
-@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_K, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("in_dim,dims,tokens", [(4096, [12288], 16), (4096, [4096, 1024, 1024], 9), (2048, [130], 12), (12288, [4096], 16),
                                                 (1024, [48, 1000], 11), (5120, [257], 13), (256, [16], 1), (4096, [16 * 700], 10),
                                                 (2048, [32, 64, 7, 4000], 15)])
@@ -486,8 +486,8 @@ def test_nine_to_sixteen_tokens_in_one_pass(gpu, oracle, t, in_dim, dims, tokens
         assert_bars(o.read(np.float32, tokens * d), want, tol, tokens, d, "type %d in=%d M=%d rows=%d" % (t, in_dim, tokens, d))
     with pytest.raises(quant.QuantError, match="1..16 tokens"):
         quant.gemv_pack16_dev(xd.ptr, t, in_dim, 17, image.ptr)
-    with pytest.raises(quant.QuantError, match="Q4_K, Q5_K or Q6_K"):
-        quant.gemv_packed16_dev([w.ptr for w in wd], Q8_0, image.ptr, [o.ptr for o in outs], dims, in_dim, tokens)
+    with pytest.raises(quant.QuantError, match="Q4_K, Q5_K, Q6_K or Q8_0"):
+        quant.gemv_packed16_dev([w.ptr for w in wd], 2, image.ptr, [o.ptr for o in outs], dims, in_dim, tokens)
     # a residual with a single matrix
     res = rng.standard_normal(tokens * dims[0]).astype(np.float32)
     rd, o2 = DevArray(res), DevArray(nbytes=4 * tokens * dims[0])
