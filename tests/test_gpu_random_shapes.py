@@ -195,3 +195,42 @@ def test_random_gemm_lists(gpu, seed):
             assert np.array_equal(o2.read(np.float32, tokens * d), o1.read(np.float32, tokens * d)), what + " member %d" % d
         for a in [ws, xd] + wd + singles + lists:
             a.close()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_sixteen_token_shapes(gpu, oracle, seed):
+    """The one-pass kernels with sixteen single-term tokens at drawn sizes: any of the four block types, rows of 256..12288
+    values, 1..16 tokens, one to four matrices of 1..1500 rows, with a residual on single matrices; against the CPU form of
+    the activations rounded to binary16, to the one-pass bars."""
+    from test_gpu_gemv_one_pass import assert_bars, oracle_rows
+    rng = np.random.default_rng(9900 + seed)
+    for case in range(8):
+        t = [Q4_K, Q5_K, Q6_K, Q8_0][int(rng.integers(0, 4))]
+        in_dim = 2048 * int(rng.integers(1, 7)) if rng.integers(0, 2) else 256 * int(rng.integers(1, 49))
+        tokens = int(rng.integers(1, 17))
+        count = int(rng.integers(1, 5))
+        dims = [int(rng.integers(1, 1500)) if rng.integers(0, 3) else 16 * int(rng.integers(1, 90)) for _ in range(count)]
+        what = "seed %d case %d: type %d in=%d M=%d dims=%s" % (seed, case, t, in_dim, tokens, dims)
+        print(what, flush=True)
+        raws = [synth.make_weights(rng, t, d, in_dim) for d in dims]
+        x = synth.make_activations(rng, tokens, in_dim)
+        x16 = x.astype(np.float16).astype(np.float32)
+        res = rng.standard_normal(tokens * dims[0]).astype(np.float32) if count == 1 and rng.integers(0, 2) else None
+        image = DevArray(np.full(quant.gemv_image_bytes(t, in_dim, 8), 0xFF, dtype=np.uint8))
+        xd, wd = DevArray(x), [DevArray(r) for r in raws]
+        rd = DevArray(res) if res is not None else None
+        outs = [DevArray(np.full(tokens * d, np.float32(-9.0))) for d in dims]
+        quant.gemv_pack16_dev(xd.ptr, t, in_dim, tokens, image.ptr)
+        quant.gemv_packed16_dev([w.ptr for w in wd], t, image.ptr, [o.ptr for o in outs], dims, in_dim, tokens, rd.ptr if rd else 0)
+        for raw, o, d in zip(raws, outs, dims):
+            want, tol = oracle_rows(oracle, raw, x16, in_dim, d, tokens, t)
+            got = o.read(np.float32, tokens * d)
+            if res is not None:
+                got = got - res   # (the residual is added last, in fp32: taking it off again costs one rounding of the sum)
+                tol = tol + 1e-6 * (np.abs(res) + np.abs(want))
+                err = np.abs(got.astype(np.float64) - want)
+                assert np.all(err <= tol + 2e-5 * np.max(np.abs(want))), what
+            else:
+                assert_bars(got, want, tol, tokens, d, what + " member %d" % d)
+        for a in [image, xd] + wd + outs + ([rd] if rd else []):
+            a.close()
