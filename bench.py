@@ -565,6 +565,31 @@ def main():
         gemv_case("q6_k gemv output head 151936x4096 M=2", Q6_K, 151936, 4096, 2)
         gemv_case("q6_k gemv output head 151936x4096 M=8", Q6_K, 151936, 4096, 8)
 
+    # bulk dequantize (Dequant.dequantize_* on device pointers): a 12288x4096 matrix of each block format to float32, three
+    # rotating sets of input and output (690 MB per rotation: nothing comes out of or stays in the last-level cache)
+    dq_n = 12288 * 4096
+    dq_out = [hip.DeviceBuffer(4 * dq_n) for _ in range(3)]
+    for w_type in (Q8_0, Q4_K, Q5_K, Q6_K):
+        draw = synth.make_weights(rng, w_type, 12288, 4096)
+        dws = []
+        for c in range(3):
+            b = hip.DeviceBuffer(draw.nbytes)
+            hip.copy_htod(b.ptr, draw if c == 0 else np.roll(draw, 4096 * c + 34), draw.nbytes, "w")
+            dws.append(b)
+
+        def deq(copy, st, dws=dws, w_type=w_type):
+            quant.dequantize_dev(dws[copy].ptr, w_type, dq_n, dq_out[copy].ptr, st.handle)
+        r = measure(hip, stream, Rotating(deq, 3, draw.nbytes + 4 * dq_n), max(5, min(30, args.steps)), 3)
+        rec = gemv_record(r, draw.nbytes + 4 * dq_n)
+        rec["kernel"] = quant.dequantize_kernel_name(w_type)
+        cases["%s dequantize 12288x4096 (50.3 M values to float32)" % TYPE_NAME[w_type].lower()] = rec
+        log("case=dequantize\ntype=%s\nelements=%d\nhip_us=%.2f\ngbps_hbm=%.1f\nfrac_hbm=%.4f\n" % (
+            TYPE_NAME[w_type], dq_n, r["us"], rec["gbps"], rec["frac_hbm"]))
+        for b in dws:
+            b.close()
+    for b in dq_out:
+        b.close()
+
     # config 4: prefill GEMM
     gemm = {}
     for tokens in (64, 512, 2048):

@@ -16,6 +16,17 @@
 #define DEQ_BLOCK 256
 #define DEQ_WAVES (DEQ_BLOCK / WAVE)
 
+// The output of a bulk dequantize is written once and not read again by the kernel: a streaming (non-temporal) store.
+#ifndef DEQ_STREAM_STORES
+#define DEQ_STREAM_STORES 1
+#endif
+typedef float deq_f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void deq_store4(float* p, float4 y) {
+  const deq_f32x4 v = {y.x, y.y, y.z, y.w};
+  if (DEQ_STREAM_STORES) __builtin_nontemporal_store(v, reinterpret_cast<deq_f32x4*>(p));
+  else *reinterpret_cast<deq_f32x4*>(p) = v;
+}
+
 // Elements past the last whole block stay zero, as in the reference's zero-initialised result.
 __device__ __forceinline__ void zero_tail(float* out, u64 from, u64 n) {
   u64 tid = (u64)blockIdx.x * blockDim.x + threadIdx.x;
@@ -47,7 +58,7 @@ extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q4_k_f32(cons
   const u64 nb = n >> 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (u64 b = (u64)blockIdx.x * DEQ_WAVES + wave; b < nb; b += (u64)gridDim.x * DEQ_WAVES)
-    *reinterpret_cast<float4*>(out + b * 256 + 4 * lane) = deq4_q4_k(w + b * 144, lane);
+    deq_store4(out + b * 256 + 4 * lane, deq4_q4_k(w + b * 144, lane));
   zero_tail(out, nb << 8, n);
 }
 
@@ -73,7 +84,7 @@ extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q5_k_f32(cons
     y.y = d1 * ubyte_f<1>(q) - m1;
     y.z = d1 * ubyte_f<2>(q) - m1;
     y.w = d1 * ubyte_f<3>(q) - m1;
-    *reinterpret_cast<float4*>(out + b * 256 + 4 * lane) = y;
+    deq_store4(out + b * 256 + 4 * lane, y);
   }
   zero_tail(out, nb << 8, n);
 }
@@ -100,7 +111,7 @@ extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q6_k_f32(cons
   const u64 nb = n >> 8;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (u64 b = (u64)blockIdx.x * DEQ_WAVES + wave; b < nb; b += (u64)gridDim.x * DEQ_WAVES)
-    *reinterpret_cast<float4*>(out + b * 256 + 4 * lane) = deq4_q6_k(w + b * 210, lane);
+    deq_store4(out + b * 256 + 4 * lane, deq4_q6_k(w + b * 210, lane));
   zero_tail(out, nb << 8, n);
 }
 
@@ -144,7 +155,7 @@ extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_q8_0_f32(cons
     y[2] = d * (float)(int)(signed char)((q >> 16) & 0xFFu);
     y[3] = d * (float)(int)(signed char)((q >> 24) & 0xFFu);
     if (e + 4 <= n) {
-      *reinterpret_cast<float4*>(out + e) = make_float4(y[0], y[1], y[2], y[3]);
+      deq_store4(out + e, make_float4(y[0], y[1], y[2], y[3]));
     } else {
       for (int c = 0; c < 4; c++)
         if (e + c < n) out[e + c] = y[c];
@@ -173,7 +184,7 @@ extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_iq4_nl_f32(co
     y[2] = d * kIq4nlValues[(q >> 16) & 0xFFu];
     y[3] = d * kIq4nlValues[(q >> 24) & 0xFFu];
     if (e + 4 <= n) {
-      *reinterpret_cast<float4*>(out + e) = make_float4(y[0], y[1], y[2], y[3]);
+      deq_store4(out + e, make_float4(y[0], y[1], y[2], y[3]));
     } else {
       for (int c = 0; c < 4; c++)
         if (e + c < n) out[e + c] = y[c];
