@@ -416,6 +416,20 @@ def main():
         for tokens in (512, 2048):
             rec = bench_gemm(hip, quant, synth, rng, stream, Q4_K, tokens, 12288, 4096, max(4, n // 4), 2, graph=False)
             log("pmc mode: prefill GEMM M=%d -> %s (pack_x_f16_q4k in front), %d weight copies" % (tokens, rec["kernel"], rec["weight_copies_rotated"]))
+        # the bulk dequantize of a 12288x4096 matrix, Q4_K and Q6_K (the copy kernel's 512 MiB destination takes the output)
+        for w_type in (Q4_K, Q6_K):
+            draw = synth.make_weights(rng, w_type, 12288, 4096)
+            dbufs = []
+            for c in range(3):
+                b = hip.DeviceBuffer(draw.nbytes)
+                hip.copy_htod(b.ptr, draw, draw.nbytes, "w")
+                dbufs.append(b)
+            for i in range(max(6, n // 4)):
+                quant.dequantize_dev(dbufs[i % 3].ptr, w_type, 12288 * 4096, dst.ptr + (i % 2) * (256 << 20), stream.handle)
+            stream.synchronize()
+            log("pmc mode: %d x %s of a 12288x4096 matrix" % (max(6, n // 4), quant.dequantize_kernel_name(w_type)))
+            for b in dbufs:
+                b.close()
         with hip.with_stream(stream):
             for i in range(8):
                 hip.launch(copy_fn, 8192, 1, 1, 256, 1, 1, params, "copy_bytes_16")
@@ -582,6 +596,7 @@ def main():
         r = measure(hip, stream, Rotating(deq, 3, draw.nbytes + 4 * dq_n), max(5, min(30, args.steps)), 3)
         rec = gemv_record(r, draw.nbytes + 4 * dq_n)
         rec["kernel"] = quant.dequantize_kernel_name(w_type)
+        rec["traffic"] = traffic_field(rec["kernel"], draw.nbytes + 4 * dq_n)
         cases["%s dequantize 12288x4096 (50.3 M values to float32)" % TYPE_NAME[w_type].lower()] = rec
         log("case=dequantize\ntype=%s\nelements=%d\nhip_us=%.2f\ngbps_hbm=%.1f\nfrac_hbm=%.4f\n" % (
             TYPE_NAME[w_type], dq_n, r["us"], rec["gbps"], rec["frac_hbm"]))
