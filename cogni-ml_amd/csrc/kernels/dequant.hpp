@@ -198,8 +198,7 @@ extern "C" __global__ __launch_bounds__(DEQ_BLOCK) void dequantize_f16_f32(const
   for (u64 e = tid * 4; e < n; e += step * 4) {
     if (e + 4 <= n) {
       const uint2 h = ld8(w + 2 * e);
-      *reinterpret_cast<float4*>(out + e) =
-          make_float4(h2f_canonical(h.x), h2f_canonical(h.x >> 16), h2f_canonical(h.y), h2f_canonical(h.y >> 16));
+      deq_store4(out + e, make_float4(h2f_canonical(h.x), h2f_canonical(h.x >> 16), h2f_canonical(h.y), h2f_canonical(h.y >> 16)));
     } else {
       for (u64 c = e; c < n; c++) out[c] = h2f_canonical(ld2(w + 2 * c));
     }
