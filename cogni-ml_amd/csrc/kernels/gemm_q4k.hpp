@@ -46,6 +46,7 @@
 // consumed (two 64 KiB buffers); the raw weight bytes of the next super-block are copied into the one 28 KiB
 // buffer as soon as every wavefront has taken the current ones into registers.
 #pragma once
+#include <type_traits>
 #include "common.hpp"
 #include "gemv_config.h"
 
@@ -244,8 +245,9 @@ __device__ __forceinline__ void gemm_epilogue(float16_t (&acc)[MT][NT], const fl
 
 // Epilogue of the gate | up kernel: the nh = 0 wavefronts hold 96 gate rows, the nh = 1 wavefronts the same 96 rows of up,
 // in the same lane layout. First the two k halves are added as above, each wavefront finishing its two token tiles in
-// place; then the up wavefronts hand their sums to the gate wavefronts (same kh) through LDS, which store
-// silu(gate) * up: 128 tokens x 96 outputs per workgroup, four consecutive floats per register quad.
+// place; then the gate and the up wavefront of the same kh exchange half of their sums through LDS and each stores
+// silu(gate) * up for its half of the column quads: 128 tokens x 96 outputs per workgroup, four consecutive floats per
+// register quad.
 // PACK (12: the Q4_K / Q5_K order, 14: the Q6_K order): the products also leave as fp16 in the packed layout the GEMM
 // kernels read their activations from (what pack_x_f16_q4k | pack_x_f16_q6k would make of `out`, bit for bit), so that the
 // GEMM behind this one - the down projection - needs no pack launch and `out` may be null. A lane's four consecutive
@@ -281,72 +283,85 @@ __device__ __forceinline__ void gemm_epilogue_swiglu_half(float16_t (&acc)[MT][3
         t[4 * g4 + 2] = KH ? p.z + t[4 * g4 + 2] : t[4 * g4 + 2] + p.z;
         t[4 * g4 + 3] = KH ? p.w + t[4 * g4 + 3] : t[4 * g4 + 3] + p.w;
       }
-  __syncthreads();   // the hand-over regions have been read: they carry the up sums next
-  float4* up = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + lane;
-  if (nh == 1) {
+  __syncthreads();   // the hand-over regions have been read: they carry the exchanged sums next
+  // silu(gate) * up costs some thirty instructions a value, so both wavefronts of a pair finish half of the cells each:
+  // the gate wavefront keeps column quads g4 = 0, 1 of every (token tile, column group) and gives 2, 3 to the up
+  // wavefront, which gives its 0, 1 in return. Region nh of the buffer holds what wavefront nh gives.
+  float4* xch = reinterpret_cast<float4*>(KH ? gemm_xbuf1 : gemm_xbuf0) + lane;
+  const bool vec = (out_dim & 3u) == 0;
+  auto give = [&](auto nhc) {
+    constexpr int NH = decltype(nhc)::value;
 #pragma unroll
     for (int rr = 0; rr < RH; rr++)
 #pragma unroll
       for (int c = 0; c < 3; c++)
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
+        for (int gg = 0; gg < 2; gg++) {
+          const int g4 = NH == 0 ? 2 + gg : gg;   // the quad given away
           const float16_t& t = acc[RH * KH + rr][c];
-          up[((rr * 3 + c) * 4 + g4) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
+          xch[(NH * (RH * 6) + (rr * 3 + c) * 2 + gg) * 64] = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
         }
-  }
-  __syncthreads();
-  if (nh != 0) return;
-  const bool vec = (out_dim & 3u) == 0;
+  };
+  auto finish = [&](auto nhc) {
+    constexpr int NH = decltype(nhc)::value;
 #pragma unroll
-  for (int rr = 0; rr < RH; rr++) {
-    const u32 token = mt * GEMM_BM + 32 * (RH * KH + rr) + j;
+    for (int rr = 0; rr < RH; rr++) {
+      const u32 token = mt * GEMM_BM + 32 * (RH * KH + rr) + j;
 #pragma unroll
-    for (int c = 0; c < 3; c++)
+      for (int c = 0; c < 3; c++)
 #pragma unroll
-      for (int g4 = 0; g4 < 4; g4++) {
-        const float16_t& t = acc[RH * KH + rr][c];
-        const float4 u = up[((rr * 3 + c) * 4 + g4) * 64];
-        const float4 o = make_float4(swiglu_one(t[4 * g4], u.x), swiglu_one(t[4 * g4 + 1], u.y), swiglu_one(t[4 * g4 + 2], u.z),
-                                     swiglu_one(t[4 * g4 + 3], u.w));
-        const u32 n = nt * (GEMM_BN / 2) + 32 * c + 8 * g4 + 4 * kg;
-        if ((PACK == 0 || out) && token < m && n < out_dim) {
-          float* dst = out + (size_t)token * out_dim + n;
-          if (vec && n + 4 <= out_dim) {
-            *reinterpret_cast<float4*>(dst) = o;
-          } else {
-            const float ov[4] = {o.x, o.y, o.z, o.w};
-            for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e];
-          }
-        }
-        if constexpr (PACK != 0) {
-          // the eight consecutive rows n8 .. n8 + 7 of the lane pair are k values of the next GEMM: super-block n8 / 256,
-          // cell (k-step, k-group) by the inverse of gemm_k_element | gemm_k_element_q6k (as in pack_x_core), all
-          // uniform over the wavefront; the absent tokens of the last tile are zeros, as the pack kernel writes them
-          const u32 n8 = nt * (GEMM_BN / 2) + 32 * c + 8 * g4;
-          if (n8 < out_dim) {
-            const u32 kb = n8 >> 8, k = n8 & 255u;
-            u32 ks, kgr;
-            if (PACK == 14) {
-              ks = 8 * (k >> 7) + 2 * ((k >> 5) & 3) + ((k >> 3) & 1);
-              kgr = (k >> 4) & 1;
+        for (int gg = 0; gg < 2; gg++) {
+          const int g4 = NH == 0 ? gg : 2 + gg;   // the quad finished here
+          const float16_t& t = acc[RH * KH + rr][c];
+          const float4 other = xch[((1 - NH) * (RH * 6) + (rr * 3 + c) * 2 + gg) * 64];
+          const float4 mine4 = make_float4(t[4 * g4], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]);
+          const float4 g = NH == 0 ? mine4 : other, u = NH == 0 ? other : mine4;
+          const float4 o = make_float4(swiglu_one(g.x, u.x), swiglu_one(g.y, u.y), swiglu_one(g.z, u.z), swiglu_one(g.w, u.w));
+          const u32 n = nt * (GEMM_BN / 2) + 32 * c + 8 * g4 + 4 * kg;
+          if ((PACK == 0 || out) && token < m && n < out_dim) {
+            float* dst = out + (size_t)token * out_dim + n;
+            if (vec && n + 4 <= out_dim) {
+              *reinterpret_cast<float4*>(dst) = o;
             } else {
-              const u32 g = k >> 6;
-              ks = 8 * (g >> 1) + 4 * ((k >> 4) & 1) + 2 * ((k >> 5) & 1) + ((k >> 3) & 1);
-              kgr = g & 1;
+              const float ov[4] = {o.x, o.y, o.z, o.w};
+              for (u32 e = 0; e < 4 && n + e < out_dim; e++) dst[e] = ov[e];
             }
-            const float4 z = token < m ? o : make_float4(0.f, 0.f, 0.f, 0.f);
-            const __half2 p0 = __floats2half2_rn(z.x, z.z), p1 = __floats2half2_rn(z.y, z.w);   // slot order 0,2,1,3
-            uint2 q;
-            q.x = *reinterpret_cast<const u32*>(&p0);
-            q.y = *reinterpret_cast<const u32*>(&p1);
-            uint2* cell = xq + (((size_t)mt * (out_dim >> 8) + kb) * 4096 + (ks * 2 + kgr) * 128 + 32 * (RH * KH + rr) + j) * 2 + kg;
-            *cell = q;
-            // (64 tokens: the upper half of the token tile is nobody's; it gets the zeros the pack kernel writes there)
-            if constexpr (MT == 2) cell[2 * 64] = make_uint2(0u, 0u);
+          }
+          if constexpr (PACK != 0) {
+            // the eight consecutive rows n8 .. n8 + 7 of the lane pair are k values of the next GEMM: super-block n8 / 256,
+            // cell (k-step, k-group) by the inverse of gemm_k_element | gemm_k_element_q6k (as in pack_x_core), all
+            // uniform over the wavefront; the absent tokens of the last tile are zeros, as the pack kernel writes them
+            const u32 n8 = nt * (GEMM_BN / 2) + 32 * c + 8 * g4;
+            if (n8 < out_dim) {
+              const u32 kb = n8 >> 8, k = n8 & 255u;
+              u32 ks, kgr;
+              if (PACK == 14) {
+                ks = 8 * (k >> 7) + 2 * ((k >> 5) & 3) + ((k >> 3) & 1);
+                kgr = (k >> 4) & 1;
+              } else {
+                const u32 g6 = k >> 6;
+                ks = 8 * (g6 >> 1) + 4 * ((k >> 4) & 1) + 2 * ((k >> 5) & 1) + ((k >> 3) & 1);
+                kgr = g6 & 1;
+              }
+              const float4 z = token < m ? o : make_float4(0.f, 0.f, 0.f, 0.f);
+              const __half2 p0 = __floats2half2_rn(z.x, z.z), p1 = __floats2half2_rn(z.y, z.w);   // slot order 0,2,1,3
+              uint2 q;
+              q.x = *reinterpret_cast<const u32*>(&p0);
+              q.y = *reinterpret_cast<const u32*>(&p1);
+              uint2* cell = xq + (((size_t)mt * (out_dim >> 8) + kb) * 4096 + (ks * 2 + kgr) * 128 + 32 * (RH * KH + rr) + j) * 2 + kg;
+              *cell = q;
+              // (64 tokens: the upper half of the token tile is nobody's; it gets the zeros the pack kernel writes there)
+              if constexpr (MT == 2) cell[2 * 64] = make_uint2(0u, 0u);
+            }
           }
         }
-      }
-  }
+    }
+  };
+  if (nh == 0) give(std::integral_constant<int, 0>{});
+  else give(std::integral_constant<int, 1>{});
+  __syncthreads();
+  if (nh == 0) finish(std::integral_constant<int, 0>{});
+  else finish(std::integral_constant<int, 1>{});
 }
 
 // Up to GEMM_MANY_MAX matrices of one type and row length against the same packed activations, as one launch: the tiles of
